@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized decode product on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: the
+Q4_0 decode GEMV y = x . W^T at the Llama-3-8B gate/up shape (W 14336 x 4096,
+batch 1), inputs resident in HBM. Successive steps read different copies of W
+(more of them than the last-level cache holds) so that every step streams its
+weights from HBM, as a decode loop over a whole model does.
+
+Prints one JSON line: whole-job throughput in algorithmic GB/s, the roofline
+object of the kernel, and a CPU baseline (the oracle's restatement of the
+reference's CPU path, timed on this host's cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def gemv_bytes(n: int, k: int, block_bytes: int = 18) -> int:
+    """Algorithmic bytes of one batch-1 product: W once, x in, y out."""
+    return n * (k // 32) * block_bytes + 4 * k + 4 * n
+
+
+def bench_blocks_q4_0(rng, n_elems):
+    nb = n_elems // 32
+    b = np.empty((nb, 18), np.uint8)
+    d = np.abs(rng.normal(0, 0.02, nb)).astype(np.float32).astype(np.float16).view(np.uint16)
+    b[:, 0] = d & 0xff
+    b[:, 1] = d >> 8
+    b[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
+    return b.reshape(-1)
+
+
+def time_gemv(lib, capi, torch, dt, n, k, steps, warmup, n_bufs, seed=0, check=True):
+    """Times `steps` launches after `warmup`, rotating over n_bufs copies of W.
+    Returns (ms per step by wall clock, ms per launch by HIP events)."""
+    rng = np.random.default_rng(seed)
+    raw = bench_blocks_q4_0(rng, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    w0 = torch.from_numpy(raw).to("cuda:0")
+    bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
+    xd = torch.from_numpy(x).to("cuda:0")
+    y = torch.empty(n, dtype=torch.float32, device="cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def launch(i):
+        capi.check(lib.mi355x_qgemv(dt, bufs[i % n_bufs].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, st))
+
+    if check:  # the result is checked against the oracle before anything is timed
+        import oracle as O
+        launch(0)
+        capi.check(lib.mi355x_sync(st))
+        want = O.qmatmul(O.Q4_0, raw, x, n, k)
+        got = y.cpu().numpy()
+        err = np.abs(got - want) / np.maximum(1, np.abs(want))
+        if not np.all(err <= 1e-3):
+            raise SystemExit(f"bench: GEMV {n}x{k} differs from the oracle: worst {err.max():.3e}")
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        launch(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
+    return wall_ms, ev_ms
+
+
+def time_gemv_graph(lib, capi, torch, dt, n, k, steps, warmup, n_bufs, seed=0):
+    """The same launches captured once into a HIP graph and replayed, which
+    takes the host's launch cost out of the device timeline."""
+    rng = np.random.default_rng(seed)
+    raw = bench_blocks_q4_0(rng, n * k)
+    w0 = torch.from_numpy(raw).to("cuda:0")
+    bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
+    xd = torch.from_numpy(rng.normal(size=k).astype(np.float32)).to("cuda:0")
+    y = torch.empty(n, dtype=torch.float32, device="cuda:0")
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    per_graph = n_bufs
+    with torch.cuda.stream(s):
+        for i in range(3):
+            capi.check(lib.mi355x_qgemv(dt, bufs[i % n_bufs].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, s.cuda_stream))
+        s.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            for i in range(per_graph):
+                capi.check(lib.mi355x_qgemv(dt, bufs[i].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, s.cuda_stream))
+        reps = max(1, steps // per_graph)
+        for _ in range(max(1, warmup // per_graph)):
+            g.replay()
+        s.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(s)
+        for _ in range(reps):
+            g.replay()
+        e1.record(s)
+        s.synchronize()
+    return e0.elapsed_time(e1) / (reps * per_graph)
+
+
+def stream_ceiling(lib, capi, torch, nbytes, n_bufs, steps):
+    """GB/s of a plain 128-bit streaming read of nbytes, rotating buffers."""
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").random_(0, 255) for _ in range(n_bufs)]
+    grid, threads = 2048, 512
+    scratch = torch.empty(grid * threads // 64, dtype=torch.float32, device="cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    for i in range(20):
+        capi.check(lib.mi355x_stream_read(bufs[i % n_bufs].data_ptr(), nbytes, scratch.data_ptr(), grid, threads, st))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        capi.check(lib.mi355x_stream_read(bufs[i % n_bufs].data_ptr(), nbytes, scratch.data_ptr(), grid, threads, st))
+    e1.record()
+    torch.cuda.synchronize()
+    return nbytes / (e0.elapsed_time(e1) / steps * 1e-3) / 1e9
+
+
+def cpu_baseline(n, k, seconds=2.0):
+    """The reference's CPU route for a Q4_0 linear, restated by the oracle:
+    weights decoded to float32 once (untimed), then the float32 GEMV over all
+    host cores. Throughput is quoted in the same algorithmic bytes as the GPU's."""
+    import oracle as O
+    rng = np.random.default_rng(0)
+    raw = bench_blocks_q4_0(rng, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    wf = O.dequantize(O.Q4_0, raw).reshape(n, k)
+    threads = O.lib().mo_num_threads()
+    O.sgemv(wf, x)  # warm
+    iters, t0 = 0, time.perf_counter()
+    while True:
+        O.sgemv(wf, x)
+        iters += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds and iters >= 5:
+            break
+    per = dt / iters
+    return {
+        "value": round(gemv_bytes(n, k) / per / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"{iters} float32 GEMVs {n}x{k} over weights decoded once from Q4_0 ({wf.nbytes / 1e6:.0f} MB read per GEMV, "
+                  f"{per * 1e3:.2f} ms each; {wf.nbytes / per / 1e9:.1f} GB/s of float32 reads), {dt:.1f} s wall",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--bufs", type=int, default=16, help="copies of W to rotate over (16 x 33 MB > the 256 MB last-level cache)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives or sharding are built)")
+
+    import torch
+    from mimir_amd import capi
+    lib = capi.load()  # raises if the HIP library is not built: there is no fallback
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+    capi.check(lib.mi355x_init(0))
+
+    n, k = 14336, 4096
+    wall_ms, ev_ms = time_gemv(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, args.bufs)
+    bytes_ = gemv_bytes(n, k)
+    value = bytes_ / (wall_ms * 1e-3) / 1e9
+    achieved = bytes_ / (ev_ms * 1e-3) / 1e9
+    out = {
+        "metric": "Q4_0 GEMV HBM GB/s (% of peak); decode tok/s, 8B-shape, batch 1",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "Q4_0 decode GEMV 4096->14336 (Llama-3-8B gate/up), batch 1, W rotated over "
+                               f"{args.bufs} HBM-resident copies", "N": n, "K": k, "M": 1},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "qgemv_q4_0_kernel", "bytes_per_launch": bytes_, "us_per_launch": round(ev_ms * 1e3, 3)},
+    }
+    extra = {}
+    if args.all_shapes:
+        for name, (nn, kk) in {"down_14336->4096": (4096, 14336), "qo_4096->4096": (4096, 4096), "kv_4096->1024": (1024, 4096)}.items():
+            nb = max(args.bufs, int(600e6 // gemv_bytes(nn, kk)) + 1)
+            w, e = time_gemv(lib, capi, torch, capi.Q4_0, nn, kk, args.steps, args.warmup, min(nb, 256))
+            extra[name] = {"us_per_launch": round(e * 1e3, 3), "GBps": round(gemv_bytes(nn, kk) / (e * 1e-3) / 1e9, 1)}
+        extra["gate_up_hot_1buf"] = {"us_per_launch": round(time_gemv(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, 1, check=False)[1] * 1e3, 3)}
+        extra["gate_up_graph"] = {"us_per_launch": round(time_gemv_graph(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, args.bufs) * 1e3, 3)}
+        extra["stream_read_33MB_GBps"] = round(stream_ceiling(lib, capi, torch, 33030144, args.bufs, args.steps), 1)
+        extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
+        out["extra"] = extra
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(n, k)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

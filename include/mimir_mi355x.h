@@ -1,0 +1,116 @@
+/*
+ * C ABI of libmimir_mi355x.so: the MI355X (gfx950) implementation of mimir's
+ * quantized-matmul decode path. A host binds these symbols with dlopen/dlsym
+ * (purego's Dlopen + RegisterFunc in Go, ctypes in Python); the signatures use
+ * plain pointers and integers only.
+ *
+ * Conventions
+ *  - Every function returns a status word: 0 on success, a hipError_t value
+ *    (1..1999) when the HIP runtime failed, or one of the MI355X_ERR_* codes,
+ *    which map one to one onto the reference's sentinel errors
+ *    (backend/backend.go:31-54). mi355x_last_error gives the message of the
+ *    calling thread's last failure.
+ *  - Device pointers come from mi355x_alloc or from any other HIP allocation
+ *    of the same process (hipMalloc, a torch tensor's data_ptr).
+ *  - `stream` is a hipStream_t passed as a pointer; NULL is the device's
+ *    default stream. Launches return once queued, like Backend.Run
+ *    (backend/backend.go:152-168); mi355x_sync waits and reports device-side
+ *    errors, like Backend.Sync (backend/rocm/rocm_linux.go:349-375).
+ *  - dtype codes are the reference's DType enumeration
+ *    (backend/backend.go:72-90) with Q4_0 appended.
+ *  - Block-quantized buffers hold ggml's block layout unchanged
+ *    (backend/backend.go:66-71); kernels read it in place.
+ */
+#ifndef MIMIR_MI355X_H
+#define MIMIR_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported from the shared library, whose other symbols are hidden. */
+#define MI355X_API __attribute__((visibility("default")))
+
+typedef uint32_t mi355x_status;
+
+enum {
+    MI355X_OK = 0,
+    MI355X_ERR_OUT_OF_MEMORY = 2,     /* hipErrorOutOfMemory -> backend.ErrOutOfMemory (rocm_linux.go:194-203) */
+    MI355X_ERR_SHAPE = 0x1001,        /* backend.ErrShape */
+    MI355X_ERR_DTYPE = 0x1002,        /* backend.ErrDType */
+    MI355X_ERR_INDEX = 0x1003,        /* backend.ErrIndex */
+    MI355X_ERR_INTERNAL = 0x1005      /* backend.ErrInternal */
+};
+
+enum {
+    MI355X_F32 = 1, MI355X_I32 = 2, MI355X_BF16 = 3, MI355X_F16 = 4,
+    MI355X_Q8_0 = 5, MI355X_Q4_K = 6, MI355X_Q6_K = 7, MI355X_Q4_0 = 8
+};
+
+/* ---- device, memory, ordering: Backend.Alloc/Free/Upload/Download/Sync ----
+ * (backend/backend.go:141-171; backend/rocm/rocm_linux.go:88,220-375) */
+
+/* Selects the device, creates the library's state on it (once per device) and
+ * checks that it is a gfx950. */
+MI355X_API mi355x_status mi355x_init(int device);
+/* Copies the calling thread's last error message into buf (NUL-terminated,
+ * truncated to n); returns its length. */
+MI355X_API size_t mi355x_last_error(char* buf, size_t n);
+/* Elements per block and bytes per block of a dtype (backend/quant.go:24-48);
+ * 0 bytes for an unknown dtype. */
+MI355X_API int mi355x_block_size(int dtype);
+MI355X_API int mi355x_block_bytes(int dtype);
+/* Bytes of n elements of dtype, or -1 when n is not whole blocks
+ * (backend/quant.go:53-59). */
+MI355X_API int64_t mi355x_bytes(int dtype, int64_t n);
+
+MI355X_API mi355x_status mi355x_alloc(void** out, size_t bytes);
+MI355X_API mi355x_status mi355x_free(void* ptr);
+MI355X_API mi355x_status mi355x_upload(void* dst, const void* src, size_t bytes, void* stream);
+MI355X_API mi355x_status mi355x_download(void* dst, const void* src, size_t bytes, void* stream);
+/* Waits for the stream, then reports and clears the device error word:
+ * MI355X_ERR_INDEX if a gather read an index out of range. */
+MI355X_API mi355x_status mi355x_sync(void* stream);
+
+/* ---- the hot path: OpQMatMul ------------------------------------------------
+ * y[m, :] = x[m, :] . W^T for m < M. W is [N, K] of a block-quantized dtype,
+ * contiguous from a block boundary (any 2-byte aligned address); x rows are
+ * x_row_stride floats apart; y is [M, N] float32, contiguous.
+ * Replaces the generated kernel of backend/internal/gen/quant.go:163-209 and
+ * computes what the CPU backend's runQMatMul computes
+ * (backend/cpu/qmatmul.go:310-405): for Q8_0, Q4_K and Q6_K each block of a
+ * row of x is rounded to int8 first and the dot products are integer; for
+ * Q4_0 it is the float32 product with the dequantized weights, the route the
+ * reference takes for that file dtype (io/mim/dtype.go:118-123). */
+MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
+                           int64_t x_row_stride, void* stream);
+
+/* ---- OpCast / OpGather of a block-quantized input ---------------------------
+ * (backend/cpu/quant.go:198-327; replaced kernels gen/quant.go:140-150 and
+ * gen/gen.go:751-756). Bit-exact with the CPU backend. */
+/* out[i] = element first + i of the blocks at W, i < n, rounded to out_dtype
+ * (F32, BF16 or F16). */
+MI355X_API mi355x_status mi355x_dequant(int dtype, const void* W, int64_t first, int64_t n, void* out, int out_dtype, void* stream);
+/* out[r, :] = row idx[r] of the [rows, K] table, dequantized; an index outside
+ * [0, rows) writes zeros and makes the next mi355x_sync fail with
+ * MI355X_ERR_INDEX. */
+MI355X_API mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_t rows, int64_t K, const int32_t* idx, int64_t n,
+                                 float* out, void* stream);
+
+/* ---- measurement aids (no counterpart in the reference) ---------------------
+ * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
+ * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds"; 0 restores the
+ * built-in choice. */
+MI355X_API mi355x_status mi355x_tune(const char* key, int value);
+/* Reads `bytes` bytes at p with 128-bit loads from `grid` workgroups of
+ * `threads` threads and folds them into scratch (at least grid*threads/64
+ * floats): the practical ceiling of a streaming read on this device. */
+MI355X_API mi355x_status mi355x_stream_read(const void* p, size_t bytes, float* scratch, int grid, int threads, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIMIR_MI355X_H */

@@ -1,0 +1,73 @@
+"""ctypes binding of libmimir_mi355x.so, the C ABI of include/mimir_mi355x.h.
+
+This is the same binding a Go host makes with purego (Dlopen + RegisterFunc):
+symbols are looked up by name and called with plain pointers and integers.
+The library is built ahead of time by mimir_amd.build; loading fails loudly
+when it is missing, and there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libmimir_mi355x.so")
+
+OK = 0
+ERR_OUT_OF_MEMORY, ERR_SHAPE, ERR_DTYPE, ERR_INDEX, ERR_INTERNAL = 2, 0x1001, 0x1002, 0x1003, 0x1005
+F32, I32, BF16, F16, Q8_0, Q4_K, Q6_K, Q4_0 = 1, 2, 3, 4, 5, 6, 7, 8
+
+_vp, _i64, _int, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
+
+# name -> (restype, argtypes): every symbol include/mimir_mi355x.h declares.
+SYMBOLS = {
+    "mi355x_init": (C.c_uint32, [_int]),
+    "mi355x_last_error": (_sz, [C.c_char_p, _sz]),
+    "mi355x_block_size": (_int, [_int]),
+    "mi355x_block_bytes": (_int, [_int]),
+    "mi355x_bytes": (_i64, [_int, _i64]),
+    "mi355x_alloc": (C.c_uint32, [C.POINTER(_vp), _sz]),
+    "mi355x_free": (C.c_uint32, [_vp]),
+    "mi355x_upload": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "mi355x_download": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "mi355x_sync": (C.c_uint32, [_vp]),
+    "mi355x_qgemv": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "mi355x_dequant": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _int, _vp]),
+    "mi355x_gather_rows": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp]),
+    "mi355x_tune": (C.c_uint32, [C.c_char_p, _int]),
+    "mi355x_stream_read": (C.c_uint32, [_vp, _sz, _vp, _int, _int, _vp]),
+}
+
+
+class Mi355xError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"[{status:#x}] {message}")
+        self.status = status
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads the library and declares every symbol; raises if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(f"{LIB_PATH} is not built: run `python -m mimir_amd.build`")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)  # AttributeError if the symbol is missing
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    buf = C.create_string_buffer(1024)
+    load().mi355x_last_error(buf, 1024)
+    return buf.value.decode(errors="replace")
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise Mi355xError(status, last_error())

@@ -1,0 +1,218 @@
+// The C ABI declared in include/mimir_mi355x.h: argument checks on the host
+// (so that a launch never sees a shape its kernel does not expect), the
+// per-device state, and the mapping of failures onto status codes.
+#include "../../include/mimir_mi355x.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+mi355x_status fail(mi355x_status code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+mi355x_status hip_fail(hipError_t e, const char* what) {
+    return fail((mi355x_status)e, "mi355x: %s: %s", what, hipGetErrorName(e));
+}
+
+#define HIP_TRY(expr, what)                         \
+    do {                                            \
+        hipError_t e_ = (expr);                     \
+        if (e_ != hipSuccess) return hip_fail(e_, what); \
+    } while (0)
+
+constexpr int kMaxDevices = 16;
+
+// Per-device state: the error word kernels OR bits into, read back at sync.
+struct DeviceState {
+    bool ready = false;
+    uint32_t* err_dev = nullptr;
+    uint32_t* err_host = nullptr;  // pinned
+};
+
+std::mutex g_mu;
+DeviceState g_dev[kMaxDevices];
+int g_tune_q4[4] = {0, 0, 0, 0};
+
+mi355x_status current_state(DeviceState** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(MI355X_ERR_INTERNAL, "mi355x: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& s = g_dev[dev];
+    if (!s.ready) {
+        hipDeviceProp_t prop;
+        HIP_TRY(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return fail(MI355X_ERR_INTERNAL, "mi355x: device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+        HIP_TRY(hipMalloc((void**)&s.err_dev, 256), "hipMalloc(error word)");
+        HIP_TRY(hipMemset(s.err_dev, 0, 256), "hipMemset(error word)");
+        HIP_TRY(hipHostMalloc((void**)&s.err_host, 256, hipHostMallocDefault), "hipHostMalloc(error word)");
+        s.ready = true;
+    }
+    *out = &s;
+    return MI355X_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+mi355x_status mi355x_init(int device) {
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    if (device < 0 || device >= n) return fail(MI355X_ERR_INTERNAL, "mi355x: device %d of %d", device, n);
+    HIP_TRY(hipSetDevice(device), "hipSetDevice");
+    DeviceState* s;
+    return current_state(&s);
+}
+
+size_t mi355x_last_error(char* buf, size_t n) {
+    if (buf && n) {
+        size_t c = g_last_error.size() < n - 1 ? g_last_error.size() : n - 1;
+        memcpy(buf, g_last_error.data(), c);
+        buf[c] = 0;
+    }
+    return g_last_error.size();
+}
+
+int mi355x_block_size(int dtype) { return mimir::block_size(dtype); }
+int mi355x_block_bytes(int dtype) { return mimir::block_bytes(dtype); }
+
+int64_t mi355x_bytes(int dtype, int64_t n) {
+    int bs = mimir::block_size(dtype), bb = mimir::block_bytes(dtype);
+    if (bb == 0 || n < 0 || n % bs != 0 || n / bs > INT64_MAX / bb) return -1;
+    return n / bs * bb;
+}
+
+mi355x_status mi355x_alloc(void** out, size_t bytes) {
+    if (!out) return fail(MI355X_ERR_INTERNAL, "mi355x: alloc: null result pointer");
+    *out = nullptr;
+    // at least 4 bytes, as the reference's Alloc (backend/rocm/rocm_linux.go:220-240)
+    hipError_t e = hipMalloc(out, bytes < 4 ? 4 : bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_free(void* ptr) {
+    if (!ptr) return MI355X_OK;
+    HIP_TRY(hipFree(ptr), "hipFree");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_upload(void* dst, const void* src, size_t bytes, void* stream) {
+    if (bytes == 0) return MI355X_OK;
+    if (!dst || !src) return fail(MI355X_ERR_INTERNAL, "mi355x: upload: null pointer");
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(H2D)");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_download(void* dst, const void* src, size_t bytes, void* stream) {
+    if (bytes == 0) return MI355X_OK;
+    if (!dst || !src) return fail(MI355X_ERR_INTERNAL, "mi355x: download: null pointer");
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(D2H)");
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_sync(void* stream) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    HIP_TRY(hipMemcpyAsync(s->err_host, s->err_dev, 4, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(error word)");
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    uint32_t bits = *s->err_host;
+    if (bits) {
+        HIP_TRY(hipMemsetAsync(s->err_dev, 0, 4, (hipStream_t)stream), "hipMemsetAsync(error word)");
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+        if (bits & mimir::kErrIndex) return fail(MI355X_ERR_INDEX, "mi355x: a gather read an index out of range");
+        return fail(MI355X_ERR_INTERNAL, "mi355x: device error bits %#x", bits);
+    }
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
+                           int64_t x_row_stride, void* stream) {
+    if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by weights of dtype %d", dtype);
+    int bs = mimir::block_size(dtype);
+    if (M < 0 || N < 0 || K < 0 || K % bs != 0)
+        return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv of [%lld, %lld] by [%lld, %lld] in blocks of %d", (long long)M,
+                    (long long)K, (long long)N, (long long)K, bs);
+    if (M == 0 || N == 0) return MI355X_OK;
+    if (!W || !x || !y) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv: null pointer");
+    if (M > 65535 || N > (int64_t)1 << 30 || K > (int64_t)1 << 30)
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv of %lld rows by [%lld, %lld]: too large", (long long)M, (long long)N,
+                    (long long)K);
+    if (M > 1 && x_row_stride < K && x_row_stride != 0)
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv: rows of x %lld apart overlap (K = %lld)", (long long)x_row_stride, (long long)K);
+    if (K == 0) {  // an empty sum: zeros (backend/cpu/qmatmul.go:336-339)
+        HIP_TRY(mimir::fill_u32(y, 0, M * N, (hipStream_t)stream), "launch fill");
+        return MI355X_OK;
+    }
+    mimir::QGemvArgs a{W, x, y, M, N, K, x_row_stride, 0};
+    switch (dtype) {
+    case MI355X_Q4_0:
+        HIP_TRY(mimir::qgemv_q4_0(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
+        return MI355X_OK;
+    default:
+        return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by dtype %d is not built yet", dtype);
+    }
+}
+
+mi355x_status mi355x_dequant(int dtype, const void* W, int64_t first, int64_t n, void* out, int out_dtype, void* stream) {
+    if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: dequantize dtype %d", dtype);
+    if (out_dtype != MI355X_F32 && out_dtype != MI355X_BF16 && out_dtype != MI355X_F16)
+        return fail(MI355X_ERR_DTYPE, "mi355x: dequantize into dtype %d", out_dtype);  // backend/cpu/quant.go:288-290
+    if (first < 0 || n < 0) return fail(MI355X_ERR_INTERNAL, "mi355x: dequantize elements [%lld, +%lld)", (long long)first, (long long)n);
+    if (n == 0) return MI355X_OK;
+    if (!W || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: dequantize: null pointer");
+    HIP_TRY(mimir::dequantize(dtype, W, first, n, out, out_dtype, (hipStream_t)stream), "launch dequantize");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_t rows, int64_t K, const int32_t* idx, int64_t n,
+                                 float* out, void* stream) {
+    if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: gather from dtype %d", dtype);
+    if (rows < 0 || K < 0 || n < 0 || K % mimir::block_size(dtype) != 0 || n > 65535)
+        return fail(MI355X_ERR_SHAPE, "mi355x: gather %lld rows of [%lld, %lld]", (long long)n, (long long)rows, (long long)K);
+    if (n == 0 || K == 0) return MI355X_OK;
+    if (!table || !idx || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: gather: null pointer");
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    HIP_TRY(mimir::gather_rows(dtype, table, rows, K, idx, n, out, s->err_dev, (hipStream_t)stream), "launch gather_rows");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_tune(const char* key, int value) {
+    static const char* keys[4] = {"q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds"};
+    for (int i = 0; i < 4; i++)
+        if (key && strcmp(key, keys[i]) == 0) {
+            g_tune_q4[i] = value;
+            return MI355X_OK;
+        }
+    return fail(MI355X_ERR_INTERNAL, "mi355x: unknown tuning key %s", key ? key : "(null)");
+}
+
+mi355x_status mi355x_stream_read(const void* p, size_t bytes, float* scratch, int grid, int threads, void* stream) {
+    if (!p || !scratch || grid <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0 || ((uintptr_t)p & 15))
+        return fail(MI355X_ERR_INTERNAL, "mi355x: stream_read: bad arguments");
+    HIP_TRY(mimir::stream_read(p, bytes, scratch, grid, threads, (hipStream_t)stream), "launch stream_read");
+    return MI355X_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+// Host-side entry points of the gfx950 kernels. Each launches on the given
+// stream and returns the launch status; none of them synchronises.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mimir {
+
+// dtype codes: the reference's DType enumeration (backend/backend.go:72-90)
+// with Q4_0 appended, so that IsQuantized stays the range test Q8_0..Q4_0.
+enum DType : int { kInvalid = 0, kF32 = 1, kI32 = 2, kBF16 = 3, kF16 = 4, kQ8_0 = 5, kQ4_K = 6, kQ6_K = 7, kQ4_0 = 8 };
+
+inline bool is_quantized(int dt) { return dt >= kQ8_0 && dt <= kQ4_0; }
+inline int block_size(int dt) { return (dt == kQ8_0 || dt == kQ4_0) ? 32 : (dt == kQ4_K || dt == kQ6_K) ? 256 : 1; }
+inline int block_bytes(int dt) {
+    switch (dt) {
+    case kQ8_0: return 34;
+    case kQ4_0: return 18;
+    case kQ4_K: return 144;
+    case kQ6_K: return 210;
+    case kF32: case kI32: return 4;
+    case kBF16: case kF16: return 2;
+    default: return 0;
+    }
+}
+
+// y[m, :] = x[m, :] . W^T for m < M: W is [N, K] blocks read in place, x rows
+// are x_row_stride floats apart, y rows N floats apart.
+struct QGemvArgs {
+    const void* W;
+    const float* x;
+    float* y;
+    int64_t M, N, K;
+    int64_t x_row_stride;
+    int rows_per_wg;  // 0 = derived from the launch shape
+};
+
+// tune: {R, C, waves, no_lds}; zeros pick the built-in plan.
+hipError_t qgemv_q4_0(const QGemvArgs& a, const int* tune, hipStream_t st);
+
+// A plain streaming read of `bytes` bytes, summed into out[0..grid): the
+// practical ceiling of HBM reads to compare the products against.
+hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);
+int stream_read_out_len(int grid, int threads);
+
+// p[i] = v for i < n 32-bit words, as a kernel.
+hipError_t fill_u32(void* p, uint32_t v, int64_t n, hipStream_t st);
+
+// Bits a kernel ORs into the device error word, read back at sync, as the
+// reference's kernels report theirs (backend/rocm/rocm_linux.go:349-375).
+enum : uint32_t { kErrIndex = 1u, kErrInternal = 2u };
+
+// out[i] = element first + i of the blocks at data, i < n, as out_dt
+// (kF32, kBF16 or kF16): OpCast of a contiguous view.
+hipError_t dequantize(int dt, const void* data, int64_t first, int64_t n, void* out, int out_dt, hipStream_t st);
+
+// out[r, :] = dequantized row idx[r] of a [rows, k] table: OpGather on axis 0.
+hipError_t gather_rows(int dt, const void* table, int64_t rows, int64_t k, const int32_t* idx, int64_t n, float* out,
+                       uint32_t* err, hipStream_t st);
+
+}  // namespace mimir

@@ -1,0 +1,34 @@
+"""The C-ABI library loads and exports every symbol include/mimir_mi355x.h
+declares. No compute call is made: this runs without a GPU."""
+import os
+import re
+
+from mimir_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mimir_mi355x.h")).read()
+    return set(re.findall(r"MI355X_API\s+[\w\s\*]+?\b(mi355x_\w+)\s*\(", text))
+
+
+def test_header_and_binding_agree():
+    declared = _declared()
+    assert declared, "no declarations found"
+    assert declared == set(capi.SYMBOLS), declared ^ set(capi.SYMBOLS)
+
+
+def test_library_exports_every_symbol():
+    lib = capi.load()
+    for name in _declared():
+        assert getattr(lib, name) is not None
+
+
+def test_block_accounting_without_a_device():
+    lib = capi.load()
+    # backend/quant.go:24-59 with Q4_0 added
+    assert [(lib.mi355x_block_size(d), lib.mi355x_block_bytes(d)) for d in (capi.Q8_0, capi.Q4_K, capi.Q6_K, capi.Q4_0)] == \
+        [(32, 34), (256, 144), (256, 210), (32, 18)]
+    assert lib.mi355x_bytes(capi.Q4_0, 4096 * 14336) == 4096 * 14336 // 32 * 18
+    assert lib.mi355x_bytes(capi.Q8_0, 33) == -1 and lib.mi355x_bytes(capi.F32, 5) == 20 and lib.mi355x_bytes(0, 4) == -1

@@ -1,0 +1,172 @@
+"""Parity of the HIP path with the oracle, through the C ABI, on a real
+MI355X: dequantization bit for bit, products within the stated tolerance.
+
+Tolerances: dequantized weights 0 (bit-exact). Products: the conformance rule
+of the reference, |got - want| <= tol * max(1, |want|), with tol = 1e-3 (the
+bar this build is given for GEMV outputs) and, for Q4_0, also 1e-4 on inputs
+the reference's own GPU conformance cases use (kerneltest/quant.go:142)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from mimir_amd import capi
+from mimir_amd.mimfile import golden_cases
+from tests import gpu
+from tests.helpers import bench_blocks, bits_equal, check_close, exact_rows, random_blocks, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+
+
+@pytest.mark.parametrize("dt", [O.Q8_0, O.Q4_K, O.Q6_K, O.Q4_0])
+@pytest.mark.parametrize("out_dt", [O.F32, O.BF16, O.F16])
+def test_dequantize_bit_exact(dt, out_dt):
+    rng = np.random.default_rng(100 + dt)
+    n = 10 * 1280  # kerneltest/quant.go:85: 9+1 rows of 1280
+    raw = random_blocks(rng, dt, n)
+    gpu.say(f"dequant dt={dt} out={out_dt} n={n}")
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    got = gpu.dequant(dt, ptr, 0, n, out_dt)
+    want = O.dequantize(dt, raw, out_dt)
+    assert bits_equal(got, want) if out_dt == O.F32 else np.array_equal(got, want)
+    # rows 1..9: a view that starts a row in (the "shrunk" case)
+    got = gpu.dequant(dt, ptr, 1280, 9 * 1280, out_dt)
+    assert np.array_equal(got.view(np.uint32 if out_dt == O.F32 else np.uint16), want[1280:].view(np.uint32 if out_dt == O.F32 else np.uint16))
+
+
+def test_dequantize_golden(golden_dir):
+    cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
+    for kind, dt in (("q8_0", O.Q8_0), ("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
+        c = cases[f"{kind}_dequantize"]
+        raw = c["in"][-1].data.reshape(-1)
+        gpu.say(f"golden dequant {kind}")
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        got = gpu.dequant(dt, ptr, 0, c["out"].data.size)
+        assert bits_equal(got, c["out"].data.reshape(-1))
+
+
+@pytest.mark.parametrize("dt", [O.Q8_0, O.Q4_K, O.Q6_K, O.Q4_0])
+def test_gather_rows(dt):
+    rng = np.random.default_rng(200 + dt)
+    k = 1280
+    raw = random_blocks(rng, dt, 10 * k)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    l = gpu.lib()
+    for idx, ok in (([2, 0, 9], True), ([2, 10, 0], False)):  # kerneltest/quant.go:97
+        gpu.say(f"gather dt={dt} idx={idx}")
+        ti = gpu.dev(np.array(idx, np.int32))
+        out = torch.zeros((3, k), dtype=torch.float32, device="cuda:0")
+        capi.check(l.mi355x_gather_rows(dt, ptr, 10, k, ti.data_ptr(), 3, out.data_ptr(), gpu.stream()))
+        st = l.mi355x_sync(gpu.stream())
+        if ok:
+            assert st == 0
+            assert bits_equal(out.cpu().numpy(), O.gather_rows(dt, raw, 10, k, idx))
+        else:
+            assert st == capi.ERR_INDEX
+            assert l.mi355x_sync(gpu.stream()) == 0  # the error is reported once
+
+
+# ---- products ---------------------------------------------------------------
+
+Q4_SHAPES = [  # (N, K): the decode shapes of an 8B Llama, and ragged ones
+    (14336, 4096), (4096, 14336), (4096, 4096), (1024, 4096),
+    (9, 1280), (1, 32), (5, 64), (130, 2048 + 32), (257, 4096 + 64), (33, 17 * 32), (3, 16384 + 256),
+]
+
+
+@pytest.mark.parametrize("n,k", Q4_SHAPES)
+def test_q4_0_gemv_matches_oracle(n, k):
+    rng = np.random.default_rng(n * 31 + k)
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    gpu.say(f"q4_0 gemv N={n} K={k}")
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    check_close(got, want, TOL, f"q4_0 {n}x{k}")
+    assert rel_l2(got, want) < 1e-5
+
+
+def test_q4_0_gemv_random_scales_and_unaligned_start():
+    """Weights that start a row into a buffer, 18 bytes past a 256-byte
+    boundary (kerneltest/quant.go:89-92), with scales of either sign,
+    subnormal and zero; activations the int8 path would keep exactly."""
+    rng = np.random.default_rng(5)
+    n, k = 9, 1280
+    raw = random_blocks(rng, O.Q4_0, (n + 1) * k)
+    row = k // 32 * 18
+    for m, shape in ((1, (k,)), (1, (1, k)), (6, (2, 3, k))):
+        x = exact_rows(rng, O.Q4_0, m, k).reshape(shape)
+        gpu.say(f"q4_0 gemv shrunk rows, x shape {shape}")
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        got = gpu.qgemv(O.Q4_0, ptr + row, gpu.dev(x), n, k)
+        want = O.qmatmul(O.Q4_0, raw[row:], x, n, k)
+        check_close(got, want, 1e-4, f"q4_0 shrunk {shape}")
+
+
+def test_q4_0_gemv_without_lds_staging():
+    rng = np.random.default_rng(6)
+    n, k = 64, 4096
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    try:
+        capi.check(l.mi355x_tune(b"q4_0.no_lds", 1))
+        gpu.say("q4_0 gemv no-lds path")
+        check_close(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k), want, TOL)
+    finally:
+        capi.check(l.mi355x_tune(b"q4_0.no_lds", 0))
+
+
+@pytest.mark.parametrize("rows,cols,waves", [(1, 1, 1), (2, 1, 4), (4, 2, 8), (7, 2, 8), (8, 2, 2), (4, 4, 4), (2, 7, 8), (1, 7, 1), (16, 1, 2)])
+def test_q4_0_gemv_every_launch_shape(rows, cols, waves):
+    rng = np.random.default_rng(7)
+    n, k = 203, 4096 + 32 * 5
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    try:
+        for key, v in ((b"q4_0.rows", rows), (b"q4_0.cols", cols), (b"q4_0.waves", waves)):
+            capi.check(l.mi355x_tune(key, v))
+        gpu.say(f"q4_0 gemv plan R={rows} C={cols} waves={waves}")
+        check_close(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k), want, TOL)
+    finally:
+        for key in (b"q4_0.rows", b"q4_0.cols", b"q4_0.waves"):
+            capi.check(l.mi355x_tune(key, 0))
+
+
+def test_q4_0_gemv_linearity_at_full_size():
+    """Size-independent property at the benchmark's shape: the product is
+    linear in x, and a one-hot x picks a column of the dequantized W."""
+    rng = np.random.default_rng(8)
+    n, k = 14336, 4096
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    a = rng.normal(size=k).astype(np.float32); b = rng.normal(size=k).astype(np.float32)
+    gpu.say("q4_0 gemv linearity 14336x4096")
+    ya, yb, yab = (gpu.qgemv(O.Q4_0, ptr, gpu.dev(v), n, k) for v in (a, b, a + b))
+    assert np.abs(yab - (ya + yb)).max() <= 1e-4 * max(1, np.abs(yab).max())
+    e = np.zeros(k, np.float32); e[1234] = 1
+    col = gpu.qgemv(O.Q4_0, ptr, gpu.dev(e), n, k)
+    assert bits_equal(col, O.dequantize(O.Q4_0, raw).reshape(n, k)[:, 1234])
+
+
+def test_qgemv_argument_errors():
+    l = gpu.lib()
+    x = torch.zeros(64, device="cuda:0"); y = torch.zeros(4, device="cuda:0"); w = torch.zeros(1024, dtype=torch.uint8, device="cuda:0")
+    assert l.mi355x_qgemv(capi.F32, w.data_ptr(), x.data_ptr(), y.data_ptr(), 1, 4, 64, 64, 0) == capi.ERR_DTYPE
+    assert l.mi355x_qgemv(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), 1, 4, 48, 48, 0) == capi.ERR_INTERNAL  # K not whole blocks (qmatmul.go:329-332)
+    assert "blocks of 32" in capi.last_error()
+    assert l.mi355x_qgemv(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), 0, 4, 64, 64, 0) == 0  # empty output
+    y.fill_(7)
+    assert l.mi355x_qgemv(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), 1, 4, 0, 0, 0) == 0    # K = 0: zeros
+    gpu.sync()
+    assert not y.cpu().numpy().any()
