@@ -88,6 +88,17 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
 
+/* The Q4_0 product in two steps, for callers that multiply one x by several
+ * matrices (q, k and v; gate and up): mi355x_q4_0_convert_act turns each row of
+ * x (K a multiple of 64) into the fixed-point form the fast kernel reads,
+ * mi355x_q4_0_act_bytes(K) bytes per row at a 16-byte aligned `act`, and
+ * mi355x_qgemv_q4_0_act multiplies by a dword-aligned W. mi355x_qgemv does both
+ * through a scratch buffer of its own when W and K qualify. No counterpart in
+ * the reference, whose kernels take float32 activations only. */
+MI355X_API size_t mi355x_q4_0_act_bytes(int64_t K);
+MI355X_API mi355x_status mi355x_q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
+MI355X_API mi355x_status mi355x_qgemv_q4_0_act(const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* ---- OpCast / OpGather of a block-quantized input ---------------------------
  * (backend/cpu/quant.go:198-327; replaced kernels gen/quant.go:140-150 and
  * gen/gen.go:751-756). Bit-exact with the CPU backend. */
@@ -102,8 +113,8 @@ MI355X_API mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_
 
 /* ---- measurement aids (no counterpart in the reference) ---------------------
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
- * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds"; 0 restores the
- * built-in choice. */
+ * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
+ * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice. */
 MI355X_API mi355x_status mi355x_tune(const char* key, int value);
 /* Reads `bytes` bytes at p with 128-bit loads from `grid` workgroups of
  * `threads` threads and folds them into scratch (at least grid*threads/64

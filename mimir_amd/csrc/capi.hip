@@ -44,11 +44,16 @@ struct DeviceState {
     bool ready = false;
     uint32_t* err_dev = nullptr;
     uint32_t* err_host = nullptr;  // pinned
+    // Converted activations of mi355x_qgemv's fixed-point path: grown on
+    // demand, shared by every call on this device (calls that overlap on two
+    // streams of one device race on it).
+    void* act = nullptr;
+    size_t act_bytes = 0;
 };
 
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
-int g_tune_q4[4] = {0, 0, 0, 0};
+int g_tune_q4[5] = {0, 0, 0, 0, 0};
 
 mi355x_status current_state(DeviceState** out) {
     int dev = 0;
@@ -67,6 +72,23 @@ mi355x_status current_state(DeviceState** out) {
         s.ready = true;
     }
     *out = &s;
+    return MI355X_OK;
+}
+
+// Returns the device's activation scratch, at least `bytes` long.
+mi355x_status act_scratch(size_t bytes, void** out) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (s->act_bytes < bytes) {
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        void* p = nullptr;
+        HIP_TRY(hipMalloc(&p, want), "hipMalloc(activation scratch)");
+        if (s->act) HIP_TRY(hipFree(s->act), "hipFree(activation scratch)");  // waits for work that reads it
+        s->act = p;
+        s->act_bytes = want;
+    }
+    *out = s->act;
     return MI355X_OK;
 }
 
@@ -164,14 +186,45 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         HIP_TRY(mimir::fill_u32(y, 0, M * N, (hipStream_t)stream), "launch fill");
         return MI355X_OK;
     }
-    mimir::QGemvArgs a{W, x, y, M, N, K, x_row_stride, 0};
+    mimir::QGemvArgs a{W, x, nullptr, y, M, N, K, x_row_stride, 0};
     switch (dtype) {
     case MI355X_Q4_0:
+        if (g_tune_q4[4] != 1 && mimir::q4_0_fixed_point_ok(W, K)) {
+            void* act;
+            if (mi355x_status st = act_scratch(mimir::q4_0_act_bytes(K) * (size_t)M, &act)) return st;
+            HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
+            a.act = act;
+            HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
+            return MI355X_OK;
+        }
         HIP_TRY(mimir::qgemv_q4_0(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
         return MI355X_OK;
     default:
         return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by dtype %d is not built yet", dtype);
     }
+}
+
+size_t mi355x_q4_0_act_bytes(int64_t K) { return K > 0 && K % 32 == 0 ? mimir::q4_0_act_bytes(K) : 0; }
+
+mi355x_status mi355x_q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream) {
+    if (M < 0 || K <= 0 || K % 64 != 0 || M > 65535)
+        return fail(MI355X_ERR_SHAPE, "mi355x: convert activations [%lld, %lld]: K must be a positive multiple of 64", (long long)M, (long long)K);
+    if (M == 0) return MI355X_OK;
+    if (!x || !act || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: convert activations: null or misaligned pointer");
+    HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_qgemv_q4_0_act(const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (M < 0 || N < 0 || K <= 0 || M > 65535 || N > (int64_t)1 << 30)
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_q4_0_act of %lld rows by [%lld, %lld]", (long long)M, (long long)N, (long long)K);
+    if (M == 0 || N == 0) return MI355X_OK;
+    if (!W || !act || !y || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv_q4_0_act: null or misaligned pointer");
+    if (!mimir::q4_0_fixed_point_ok(W, K))
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_q4_0_act needs K a multiple of 64 up to 24448 and W dword aligned (K = %lld)", (long long)K);
+    mimir::QGemvArgs a{W, nullptr, act, y, M, N, K, 0, 0};
+    HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
+    return MI355X_OK;
 }
 
 mi355x_status mi355x_dequant(int dtype, const void* W, int64_t first, int64_t n, void* out, int out_dtype, void* stream) {
@@ -199,8 +252,8 @@ mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_t rows, int
 }
 
 mi355x_status mi355x_tune(const char* key, int value) {
-    static const char* keys[4] = {"q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds"};
-    for (int i = 0; i < 4; i++)
+    static const char* keys[5] = {"q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path"};
+    for (int i = 0; i < 5; i++)
         if (key && strcmp(key, keys[i]) == 0) {
             g_tune_q4[i] = value;
             return MI355X_OK;

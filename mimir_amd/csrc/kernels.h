@@ -29,15 +29,25 @@ inline int block_bytes(int dt) {
 // are x_row_stride floats apart, y rows N floats apart.
 struct QGemvArgs {
     const void* W;
-    const float* x;
+    const float* x;    // float32 activations, or
+    const void* act;   // activations converted for the fixed-point Q4_0 kernel
     float* y;
     int64_t M, N, K;
     int64_t x_row_stride;
     int rows_per_wg;  // 0 = derived from the launch shape
 };
 
-// tune: {R, C, waves, no_lds}; zeros pick the built-in plan.
+// The float32 Q4_0 product, any shape. tune: {rows, cols, waves, no_lds}; zeros
+// pick the built-in plan.
 hipError_t qgemv_q4_0(const QGemvArgs& a, const int* tune, hipStream_t st);
+
+// The fixed-point Q4_0 product: x is converted once (q4_0_convert_act, into
+// q4_0_act_bytes(K) bytes per row) and multiplied with v_dot8_i32_i4.
+// q4_0_fixed_point_ok says whether a W and K qualify.
+bool q4_0_fixed_point_ok(const void* W, int64_t K);
+size_t q4_0_act_bytes(int64_t K);
+hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.

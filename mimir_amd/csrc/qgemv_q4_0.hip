@@ -1,0 +1,549 @@
+// Decode products by Q4_0 weights, y = x . W^T with few rows of x, for gfx950.
+// They replace the reference's generated qmatmul kernel
+// (backend/internal/gen/quant.go:152-209). What the reference's CPU computes
+// for a Q4_0 linear is the float32 product with the dequantized weights: it
+// decodes Q4_0 to float32 at load (io/mim/dtype.go:118-123) and multiplies in
+// float32 (backend/cpu/gemv.go:73-104).
+//
+// W stays in ggml's layout (18-byte blocks: binary16 scale, 16 bytes of
+// nibbles), read in place. A wavefront owns R rows of W at a time and splits K
+// across its 64 lanes; every load of a tile is issued before the first is
+// used; the activations are staged once per workgroup in LDS, laid out so that
+// the lanes' 128-bit LDS reads are conflict-free; row sums are reduced over
+// the wavefront with DPP.
+//
+// Two kernels:
+//
+//  qgemv_q4_0_i4_kernel   the fast path. The kernel is bound by vector-ALU
+//    issue as much as by HBM (a 16-lane SIMD needs four cycles per wavefront
+//    instruction), so it multiplies eight weights per instruction with
+//    v_dot8_i32_i4: XOR 0x88888888 turns a dword of offset-binary nibbles n
+//    into two's-complement (n - 8), and each block of 32 activations is held
+//    as a 20-bit fixed-point number per element, split into five planes of
+//    signed 4-bit digits, with one float32 scale per block. The integer sums
+//    are exact; the only error is the fixed-point rounding of x, at most
+//    2^-20 of the block's largest magnitude per element (about 1e-6 relative
+//    on the result, the size of float32 rounding itself, a thousand times
+//    below the 1e-3 bar). Lanes own pairs of blocks (36 bytes, dword aligned)
+//    and fetch them with aligned 128-bit loads. Needs K a multiple of 64 and W
+//    dword aligned.
+//
+//  qgemv_q4_0_kernel      any shape and any 2-byte aligned W: float32
+//    multiply-adds through v_fma_mix_f32 on nibbles masked in place as
+//    binary16 subnormals.
+#include "device_util.h"
+#include "kernels.h"
+
+namespace mimir {
+
+// LDS layout of the staged activations of one row of x with nb blocks:
+//   float4 xs[8][nbp]   part j of block b at xs[j * nbp + b]; nbp = nb | 1
+//   float  xsum[nb]     sum of the block's 32 values
+__host__ __device__ inline int q4_nbp(int nb) { return nb | 1; }
+__host__ __device__ inline size_t q4_lds_bytes(int nb) { return (size_t)q4_nbp(nb) * 8 * 16 + (size_t)nb * 4; }
+
+// ---- Q4_0 -------------------------------------------------------------------
+//
+// The nibbles are multiplied without an integer-to-float conversion: masked
+// in place, a nibble at bits 0-3 (or 4-7) of a 16-bit half is the binary16
+// subnormal n * 2^-24 (or 16n * 2^-24), which v_fma_mix_f32 widens for free.
+// Per dword of 8 nibbles that is 5 bit operations and 8 fused multiply-adds.
+// The factors 2^-24 and 16 are powers of two and are taken out exactly when
+// the block's scale is applied; the offset 8 is applied through the block sum
+// of x: sum (n-8) x = sum n x - 8 sum x.
+// x values a thread parks in registers between their global load and their
+// LDS store, so that the weights' loads can be issued in between.
+constexpr int kStage = 8;
+
+__device__ __forceinline__ f32x4 load_f32x4(const float* p) {
+    f32x4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+
+template <int R, int C>
+struct Q4Tile {
+    u32x4 q[R][C];
+    uint16_t d[R][C];
+};
+
+template <int R, int C>
+__device__ __forceinline__ void q4_load_tile(Q4Tile<R, C>& t, const uint8_t* __restrict__ W, int64_t row_bytes, int N, int nb,
+                                             int row0, int c0, int lane) {
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        int b = lane + 64 * (c0 + c);
+        int bc = b < nb ? b : nb - 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = row0 + r;
+            row = row < N ? row : N - 1;
+            const uint8_t* p = W + (int64_t)row * row_bytes + (int64_t)bc * 18;
+            t.d[r][c] = load_u16(p);
+            t.q[r][c] = load_u32x4_unaligned(p + 2);
+        }
+    }
+}
+
+template <int R, int C, bool XLDS>
+__global__ __launch_bounds__(512) void qgemv_q4_0_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x,
+                                                         float* __restrict__ y, int N, int nb, int64_t x_row_stride,
+                                                         int rows_per_wg) {
+    extern __shared__ f32x4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int m = blockIdx.y;
+    const float* xr = x + (int64_t)m * x_row_stride;
+    float* yr = y + (int64_t)m * N;
+    const int nbp = q4_nbp(nb);
+    float* xsum = (float*)(lds + 8 * nbp);
+    const int64_t row_bytes = (int64_t)nb * 18;
+    const int wg_row0 = blockIdx.x * rows_per_wg;
+    const int ncol = (nb + 63) >> 6;
+    const int nf = nb * 8;  // float4s of x
+
+    Q4Tile<R, C> tile;
+    int r0 = wave * R;
+    // The first tile's loads go out between the loads of x and its LDS stores.
+    f32x4 park[kStage];
+    if (XLDS) {
+#pragma unroll
+        for (int i = 0; i < kStage; i++) {
+            int f = tid + i * (int)blockDim.x;
+            if (f < nf) park[i] = load_f32x4(xr + 4 * (int64_t)f);
+        }
+    }
+    const bool first_live = r0 < rows_per_wg && wg_row0 + r0 < N;
+    if (first_live) q4_load_tile<R, C>(tile, W, row_bytes, N, nb, wg_row0 + r0, 0, lane);
+    if (XLDS) {
+#pragma unroll
+        for (int i = 0; i < kStage; i++) {
+            int f = tid + i * (int)blockDim.x;
+            if (f < nf) {
+                f32x4 v = park[i];
+                int b = f >> 3, j = f & 7;
+                lds[j * nbp + b] = v;
+                // all 8 lanes of a block are live together: nf is a multiple of 8 and so is the stride
+                float s = group8_sum((v[0] + v[1]) + (v[2] + v[3]));
+                if (j == 7) xsum[b] = s;
+            }
+        }
+        for (int f = tid + kStage * (int)blockDim.x; f < nf; f += (int)blockDim.x) {
+            f32x4 v = load_f32x4(xr + 4 * (int64_t)f);
+            int b = f >> 3, j = f & 7;
+            lds[j * nbp + b] = v;
+            float s = group8_sum((v[0] + v[1]) + (v[2] + v[3]));
+            if (j == 7) xsum[b] = s;
+        }
+        __syncthreads();
+    }
+
+    bool loaded = first_live;
+    for (; r0 < rows_per_wg; r0 += waves * R) {
+        const int row0 = wg_row0 + r0;
+        if (row0 >= N) break;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+        for (int c0 = 0; c0 < ncol; c0 += C) {
+            if (!loaded) q4_load_tile<R, C>(tile, W, row_bytes, N, nb, row0, c0, lane);
+            loaded = false;
+#pragma unroll
+            for (int c = 0; c < C; c++) {
+                int b = lane + 64 * (c0 + c);
+                bool live = b < nb;
+                int bc = live ? b : nb - 1;
+                f32x4 xv[8];
+                float xs;
+                if (XLDS) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) xv[j] = lds[j * nbp + bc];
+                    xs = xsum[bc];
+                } else {
+                    xs = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        xv[j] = load_f32x4(xr + 32 * (int64_t)bc + 4 * j);
+                        xs += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
+                    }
+                }
+                if (!live) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) xv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    xs = 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    float lo = 0.f, hi = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        uint32_t w = tile.q[r][c][i], s = w >> 8;
+                        f16x2 p0 = as_f16x2(w & 0x000F000Fu), p1 = as_f16x2(w & 0x00F000F0u);
+                        f16x2 p2 = as_f16x2(s & 0x000F000Fu), p3 = as_f16x2(s & 0x00F000F0u);
+                        // byte k of the dword holds elements 4i+k (low nibble) and 16+4i+k (high)
+                        lo = fmaf((float)p0[0], xv[i][0], lo);
+                        lo = fmaf((float)p2[0], xv[i][1], lo);
+                        lo = fmaf((float)p0[1], xv[i][2], lo);
+                        lo = fmaf((float)p2[1], xv[i][3], lo);
+                        hi = fmaf((float)p1[0], xv[4 + i][0], hi);
+                        hi = fmaf((float)p3[0], xv[4 + i][1], hi);
+                        hi = fmaf((float)p1[1], xv[4 + i][2], hi);
+                        hi = fmaf((float)p3[1], xv[4 + i][3], hi);
+                    }
+                    // lo = 2^-24 sum n x over the low nibbles, hi = 2^-20 sum n x over the high ones
+                    float t = fmaf(hi, 0.0625f, lo);
+                    t = fmaf(xs, -8.0f * 0x1p-24f, t);
+                    float d = f16_bits_to_f32(tile.d[r][c]) * 0x1p24f;
+                    acc[r] = fmaf(d, t, acc[r]);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float s = wave_sum(acc[r]);
+            if (lane == 0 && row0 + r < N) yr[row0 + r] = s;
+        }
+    }
+}
+
+template <int R, int C>
+static hipError_t launch_q4_0(const QGemvArgs& a, int waves, bool xlds, hipStream_t st) {
+    int rows_per_wg = a.rows_per_wg > 0 ? a.rows_per_wg : R * waves;
+    dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
+    size_t lds = xlds ? q4_lds_bytes((int)(a.K / 32)) : 0;
+    if (xlds)
+        hipLaunchKernelGGL((qgemv_q4_0_kernel<R, C, true>), grid, dim3(64 * waves), lds, st, (const uint8_t*)a.W, a.x, a.y,
+                           (int)a.N, (int)(a.K / 32), a.x_row_stride, rows_per_wg);
+    else
+        hipLaunchKernelGGL((qgemv_q4_0_kernel<R, C, false>), grid, dim3(64 * waves), lds, st, (const uint8_t*)a.W, a.x, a.y,
+                           (int)a.N, (int)(a.K / 32), a.x_row_stride, rows_per_wg);
+    return hipGetLastError();
+}
+
+// ---- fixed-point activations, v_dot8_i32_i4 ---------------------------------
+//
+// One row of x with nb blocks, converted (nbp = nb | 1; q4_0_act_bytes(K) bytes):
+//   u32x4 plane[5][nbp]  digit plane j of block b at plane[j * nbp + b]: dword i
+//                        holds, nibble for nibble as dword i of the block's
+//                        weights does (byte k: low nibble element 4i+k, high
+//                        nibble element 16+4i+k), digit j of those elements
+//   float scale[nb]      x[e] ~ scale * sum_j 16^j digit_j[e]
+// The conversion runs once per x (q4_0_convert_act), not once per workgroup
+// of the product: a decode step multiplies the same x by several matrices.
+constexpr int kDigits = 5;
+constexpr int kFixMax = 489335;  // 7 * (16^5 - 1) / 15: the largest balanced 5-digit number
+
+size_t q4_0_act_bytes(int64_t K) {
+    int64_t nb = K / 32;
+    return (size_t)(((nb | 1) * kDigits * 16 + nb * 4 + 15) / 16 * 16);
+}
+
+// The eight values a thread holds (elements 4i..4i+3 and 16+4i..16+4i+3 of a
+// block) to five dwords of digits. Z = (X + 0x88888) ^ 0x88888 has the
+// two's-complement balanced digit j of X in nibble j.
+__device__ __forceinline__ void fix_digits(const float lo[4], const float hi[4], float inv, uint32_t out[kDigits]) {
+    uint32_t z[8];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        z[2 * k] = ((uint32_t)((int)__builtin_rintf(lo[k] * inv) + 0x88888)) ^ 0x88888u;      // nibble position 2k
+        z[2 * k + 1] = ((uint32_t)((int)__builtin_rintf(hi[k] * inv) + 0x88888)) ^ 0x88888u;  // nibble position 2k+1
+    }
+#pragma unroll
+    for (int j = 0; j < kDigits; j++) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int p = 0; p < 8; p++) w |= ((z[p] >> (4 * j)) & 15u) << (4 * p);
+        out[j] = w;
+    }
+}
+
+// Thread t of a row takes item t: block t / 4, dword t % 4. The block's four
+// items sit in consecutive lanes (the item count and the stride are multiples
+// of 4), so its largest magnitude is a quad reduction.
+__global__ __launch_bounds__(256) void q4_0_convert_act_kernel(const float* __restrict__ x, int64_t x_row_stride, int nb,
+                                                               uint8_t* __restrict__ act, int64_t act_row_bytes) {
+    const float* xr = x + (int64_t)blockIdx.y * x_row_stride;
+    u32x4* plane = (u32x4*)(act + (int64_t)blockIdx.y * act_row_bytes);
+    const int nbp = nb | 1;
+    float* xscale = (float*)(plane + kDigits * nbp);
+    const int nq = nb * 4;
+    for (int t = blockIdx.x * blockDim.x + threadIdx.x; t < nq; t += gridDim.x * blockDim.x) {
+        int b = t >> 2, d = t & 3;
+        f32x4 vlo = load_f32x4(xr + 32 * (int64_t)b + 4 * d), vhi = load_f32x4(xr + 32 * (int64_t)b + 16 + 4 * d);
+        float lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
+        float amax = 0.f;
+        bool finite = true;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float a0 = __builtin_fabsf(lo[k]), a1 = __builtin_fabsf(hi[k]);
+            finite = finite && a0 < __builtin_inff() && a1 < __builtin_inff();  // false for NaN too
+            amax = fmaxf(amax, fmaxf(a0, a1));
+        }
+        amax = fmaxf(amax, dpp_f32<0xb1>(amax));
+        amax = fmaxf(amax, dpp_f32<0x4e>(amax));
+        float bad = finite ? 0.f : 1.f;
+        bad = fmaxf(bad, dpp_f32<0xb1>(bad));
+        bad = fmaxf(bad, dpp_f32<0x4e>(bad));
+        float scale, inv;
+        if (bad != 0.f) {  // a NaN or an infinity in the block: its products are NaN
+            scale = __builtin_nanf("");
+            inv = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) lo[k] = hi[k] = 0.f;
+        } else if (amax < 0x1p-100f) {  // nothing to represent (and 1/amax would overflow)
+            scale = 0.f;
+            inv = 0.f;
+        } else {
+            scale = amax / (float)kFixMax;
+            inv = (float)kFixMax / amax;
+        }
+        uint32_t dig[kDigits];
+        fix_digits(lo, hi, inv, dig);
+#pragma unroll
+        for (int j = 0; j < kDigits; j++) ((uint32_t*)(plane + j * nbp + b))[d] = dig[j];
+        if (d == 0) xscale[b] = scale;
+    }
+}
+
+hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
+    int nb = (int)(K / 32);
+    int gx = (nb * 4 + 255) / 256;
+    hipLaunchKernelGGL(q4_0_convert_act_kernel, dim3((unsigned)gx, (unsigned)M), dim3(256), 0, st, x, x_row_stride, nb,
+                       (uint8_t*)act, (int64_t)q4_0_act_bytes(K));
+    return hipGetLastError();
+}
+
+// A 128-bit load that is only dword aligned (gfx950 serves it at full rate).
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
+template <int R, int PC>
+struct Q4PairTile {
+    u32x4 a[R][PC], b[R][PC];
+    uint32_t c[R][PC];
+};
+
+// Lane `lane` owns blocks 2p, 2p+1 with p = lane + 64 * pc: nine aligned
+// dwords. Plain (cached) loads: the three touch the same cache lines, which
+// must stay cached between them.
+template <int R, int PC>
+__device__ __forceinline__ void q4_load_pairs(Q4PairTile<R, PC>& t, const uint8_t* __restrict__ W, int64_t row_bytes, int N,
+                                              int npairs, int row0, int pc0, int lane) {
+#pragma unroll
+    for (int pc = 0; pc < PC; pc++) {
+        int p = lane + 64 * (pc0 + pc);
+        p = p < npairs ? p : npairs - 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = row0 + r;  // wave-uniform
+            row = row < N ? row : N - 1;
+            const uint32_t* src = (const uint32_t*)(W + (int64_t)row * row_bytes) + p * 9;
+            t.a[r][pc] = *(const u32x4_a4*)src;
+            t.b[r][pc] = *(const u32x4_a4*)(src + 4);
+            t.c[r][pc] = src[8];
+        }
+    }
+}
+
+// For the two blocks of a pair: sum over the block of (n - 8) * X, X the
+// fixed-point activations. Digit planes run from the most significant down,
+// each four v_dot8 accumulating on sixteen times the sum so far; the two
+// blocks' chains are independent and interleaved so that neither waits on
+// its own previous result.
+__device__ __forceinline__ void q4_pair_dot(const uint32_t q0[4], const uint32_t q1[4], const u32x4 d0[kDigits],
+                                            const u32x4 d1[kDigits], int& out0, int& out1) {
+    int w0[4], w1[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        w0[i] = (int)(q0[i] ^ 0x88888888u);
+        w1[i] = (int)(q1[i] ^ 0x88888888u);
+    }
+    int t0 = 0, t1 = 0;
+#pragma unroll
+    for (int j = kDigits - 1; j >= 0; j--) {
+        t0 *= 16;
+        t1 *= 16;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            t0 = __builtin_amdgcn_sdot8(w0[i], (int)d0[j][i], t0, false);
+            t1 = __builtin_amdgcn_sdot8(w1[i], (int)d1[j][i], t1, false);
+        }
+    }
+    out0 = t0;  // |t| <= 32 * 8 * 489335 < 2^27
+    out1 = t1;
+}
+
+template <int R, int PC>
+__global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+                                                             float* __restrict__ y, int N, int nb, int64_t act_row_bytes,
+                                                             int rows_per_wg) {
+    extern __shared__ u32x4 lds_i4[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+    const int m = blockIdx.y;
+    float* yr = y + (int64_t)m * N;
+    const int nbp = nb | 1;
+    const float* xscale = (const float*)(lds_i4 + kDigits * nbp);
+    const int64_t row_bytes = (int64_t)nb * 18;
+    const int wg_row0 = blockIdx.x * rows_per_wg;
+    const int npairs = nb >> 1;
+    const int npc = (npairs + 63) >> 6;
+
+    // Loads return in order, so the activations' loads go out first: they come
+    // back from L2 well before the weights do from HBM, and the LDS stores and
+    // the barrier are then over by the time the first weights arrive.
+    constexpr int kPark = PC == 1 ? 2 : 5;
+    const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
+    const int n16 = (int)(act_row_bytes >> 4);
+    u32x4 park[kPark];
+#pragma unroll
+    for (int i = 0; i < kPark; i++) {
+        int idx = tid + i * (int)blockDim.x;
+        if (idx < n16) park[i] = act_row[idx];
+    }
+    Q4PairTile<R, PC> tile;
+    int r0 = wave * R;
+    // Unconditional (rows are clamped into W): a branch here would make the
+    // wait before the LDS stores below cover the weights' loads as well.
+    q4_load_pairs<R, PC>(tile, W, row_bytes, N, npairs, wg_row0 + r0, 0, lane);
+#pragma unroll
+    for (int i = 0; i < kPark; i++) {
+        int idx = tid + i * (int)blockDim.x;
+        if (idx < n16) lds_i4[idx] = park[i];
+    }
+    for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_i4[idx] = act_row[idx];
+    __syncthreads();
+
+    bool loaded = true;
+    for (; r0 < rows_per_wg; r0 += waves * R) {
+        const int row0 = wg_row0 + r0;
+        if (row0 >= N) break;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
+        for (int pc0 = 0; pc0 < npc; pc0 += PC) {
+            if (!loaded) q4_load_pairs<R, PC>(tile, W, row_bytes, N, npairs, row0, pc0, lane);
+            loaded = false;
+#pragma unroll
+            for (int pc = 0; pc < PC; pc++) {
+                int p = lane + 64 * (pc0 + pc);
+                const bool live = p < npairs;
+                p = live ? p : npairs - 1;
+                u32x4 d0[kDigits], d1[kDigits];
+#pragma unroll
+                for (int j = 0; j < kDigits; j++) {
+                    d0[j] = lds_i4[j * nbp + 2 * p];
+                    d1[j] = lds_i4[j * nbp + 2 * p + 1];
+                }
+                const float s0 = live ? xscale[2 * p] : 0.f, s1 = live ? xscale[2 * p + 1] : 0.f;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const u32x4 a = tile.a[r][pc], b = tile.b[r][pc];
+                    const uint32_t c = tile.c[r][pc];
+                    // block 0: scale in the low half of a[0], nibbles at bytes 2..17
+                    const uint32_t q0[4] = {__builtin_amdgcn_alignbyte(a[1], a[0], 2), __builtin_amdgcn_alignbyte(a[2], a[1], 2),
+                                            __builtin_amdgcn_alignbyte(a[3], a[2], 2), __builtin_amdgcn_alignbyte(b[0], a[3], 2)};
+                    // block 1: scale in the high half of b[0], nibbles at bytes 20..35
+                    const uint32_t q1[4] = {b[1], b[2], b[3], c};
+                    int i0, i1;
+                    q4_pair_dot(q0, q1, d0, d1, i0, i1);
+                    const float f0 = (float)i0, f1 = (float)i1;
+                    const float w0 = f16_bits_to_f32((uint16_t)(a[0] & 0xffffu)) * s0;
+                    const float w1 = f16_bits_to_f32((uint16_t)(b[0] >> 16)) * s1;
+                    acc[r] = fmaf(w0, f0, acc[r]);
+                    acc[r] = fmaf(w1, f1, acc[r]);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float s = wave_sum(acc[r]);
+            if (lane == 0 && row0 + r < N) yr[row0 + r] = s;
+        }
+    }
+}
+
+template <int R, int PC>
+static hipError_t launch_q4_0_i4(const QGemvArgs& a, int waves, hipStream_t st) {
+    int rows_per_wg = R * waves;
+    dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
+    size_t act_bytes = q4_0_act_bytes(a.K);
+    hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
+                       (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+    return hipGetLastError();
+}
+
+// Shape of a launch: R rows per wavefront, C column steps in flight, waves
+// per workgroup. A 16-lane SIMD issues a wavefront instruction over four
+// cycles, so the tiles must cover all four SIMDs of each of the 256 CUs: the
+// plan aims at 2048 tiles or more (8 wavefronts per CU), with up to 16
+// 128-bit loads in flight per lane, in workgroups as large as leaves at
+// least one per CU, which share one staging of x.
+struct Q4Plan { int R, C, waves; };
+
+static int floor_to_instantiated_rows(int64_t r, int c) {
+    static const int rows1[] = {16, 8, 4, 2, 1}, rows2[] = {8, 7, 4, 2, 1}, rows4[] = {4, 2, 1}, rows7[] = {2, 1};
+    const int* set = c == 1 ? rows1 : c == 2 ? rows2 : c == 4 ? rows4 : rows7;
+    int n = c == 1 ? 5 : c == 2 ? 5 : c == 4 ? 3 : 2;
+    for (int i = 0; i < n; i++)
+        if (set[i] <= r) return set[i];
+    return 1;
+}
+
+static Q4Plan plan_q4_0(int64_t N, int64_t K, const int* tune) {
+    Q4Plan p;
+    int ncol = (int)((K / 32 + 63) / 64);
+    p.C = ncol <= 1 ? 1 : ncol <= 2 ? 2 : ncol <= 4 ? 4 : 7;
+    if (tune[1] > 0) p.C = tune[1];
+    p.R = floor_to_instantiated_rows(N / 2048 > 0 ? N / 2048 : 1, p.C);
+    if (p.R == 8 && p.C == 2 && N % 7 == 0) p.R = 7;
+    if (tune[0] > 0) p.R = tune[0];
+    int64_t tiles = (N + p.R - 1) / p.R;
+    p.waves = 8;
+    while (p.waves > 1 && tiles / p.waves < 256) p.waves >>= 1;
+    if (tune[2] > 0) p.waves = tune[2];
+    return p;
+}
+
+bool q4_0_fixed_point_ok(const void* W, int64_t K) {
+    int64_t nb = K / 32;
+    return nb > 0 && nb % 2 == 0 && ((uintptr_t)W & 3) == 0 && q4_0_act_bytes(K) <= 64 * 1024;
+}
+
+// The fixed-point product from converted activations (a.act). Needs
+// q4_0_fixed_point_ok. tune: {rows, pair steps, waves}.
+hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
+    int nb = (int)(a.K / 32);
+    int npc = (nb / 2 + 63) / 64;  // steps of 64 pairs of blocks that cover a row
+    int PC = npc <= 1 ? 1 : 2;
+    if (tune[1] > 0) PC = tune[1];
+    // Many small tiles: measured on MI355X, two rows per wavefront in
+    // workgroups of eight wavefronts stream best at the decode shapes.
+    int R = a.N >= 4096 ? 2 : 1;
+    if (tune[0] > 0) R = tune[0];
+    int64_t tiles = (a.N + R - 1) / R;
+    int waves = 8;
+    while (waves > 1 && tiles / waves < 256) waves >>= 1;
+    if (tune[2] > 0) waves = tune[2];
+#define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP>(a, waves, st)
+    Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(3, 1); Q4ICASE(4, 1); Q4ICASE(7, 1); Q4ICASE(8, 1);
+    Q4ICASE(1, 2); Q4ICASE(2, 2); Q4ICASE(4, 2);
+#undef Q4ICASE
+    return launch_q4_0_i4<1, 1>(a, waves, st);
+}
+
+// The float32 product, any shape. tune: {rows, cols, waves, no_lds}.
+hipError_t qgemv_q4_0(const QGemvArgs& a, const int* tune, hipStream_t st) {
+    int nb = (int)(a.K / 32);
+    Q4Plan p = plan_q4_0(a.N, a.K, tune);
+    bool xlds = q4_lds_bytes(nb) <= 64 * 1024 && tune[3] == 0;
+#define Q4CASE(RR, CC) if (p.R == RR && p.C == CC) return launch_q4_0<RR, CC>(a, p.waves, xlds, st)
+    Q4CASE(1, 1); Q4CASE(2, 1); Q4CASE(4, 1); Q4CASE(8, 1); Q4CASE(16, 1);
+    Q4CASE(1, 2); Q4CASE(2, 2); Q4CASE(4, 2); Q4CASE(7, 2); Q4CASE(8, 2);
+    Q4CASE(1, 4); Q4CASE(2, 4); Q4CASE(4, 4);
+    Q4CASE(1, 7); Q4CASE(2, 7);
+#undef Q4CASE
+    // any other shape: one row per wavefront, one step at a time
+    return launch_q4_0<1, 1>(a, p.waves, xlds, st);
+}
+
+}  // namespace mimir

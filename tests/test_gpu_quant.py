@@ -108,6 +108,51 @@ def test_q4_0_gemv_random_scales_and_unaligned_start():
         check_close(got, want, 1e-4, f"q4_0 shrunk {shape}")
 
 
+@pytest.mark.parametrize("rows,cols,waves", [(1, 1, 1), (2, 1, 4), (4, 1, 8), (7, 1, 8), (8, 1, 2), (1, 2, 4), (2, 2, 8), (4, 2, 2)])
+def test_q4_0_fixed_point_kernel_every_launch_shape(rows, cols, waves):
+    rng = np.random.default_rng(9)
+    n, k = 203, 4096 + 64 * 3
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    try:
+        for key, v in ((b"q4_0.path", 2), (b"q4_0.rows", rows), (b"q4_0.cols", cols), (b"q4_0.waves", waves)):
+            capi.check(l.mi355x_tune(key, v))
+        gpu.say(f"q4_0 fixed-point gemv plan R={rows} PC={cols} waves={waves}")
+        got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+        check_close(got, want, TOL)
+        assert rel_l2(got, want) < 1e-5
+    finally:
+        for key in (b"q4_0.path", b"q4_0.rows", b"q4_0.cols", b"q4_0.waves"):
+            capi.check(l.mi355x_tune(key, 0))
+
+
+def test_q4_0_fixed_point_kernel_special_values():
+    """Blocks of x that are all zero, tiny, huge, or hold an infinity or a NaN:
+    zeros contribute nothing, and a non-finite block makes its rows NaN, as a
+    float product does (Inf - Inf or 0 * Inf)."""
+    rng = np.random.default_rng(10)
+    n, k = 40, 512
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    x = rng.normal(size=k).astype(np.float32)
+    x[0:32] = 0
+    x[32:64] *= 1e-36
+    x[64:96] *= 1e30
+    x[96:128] = np.float32(1e-42)  # subnormal
+    gpu.say("q4_0 fixed-point gemv special values")
+    got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    x[200] = np.inf
+    got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    assert np.isnan(got).all()
+    x[200] = np.nan
+    assert np.isnan(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)).all()
+
+
 def test_q4_0_gemv_without_lds_staging():
     rng = np.random.default_rng(6)
     n, k = 64, 4096
@@ -118,10 +163,12 @@ def test_q4_0_gemv_without_lds_staging():
     want = O.qmatmul(O.Q4_0, raw, x, n, k)
     try:
         capi.check(l.mi355x_tune(b"q4_0.no_lds", 1))
+        capi.check(l.mi355x_tune(b"q4_0.path", 1))
         gpu.say("q4_0 gemv no-lds path")
         check_close(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k), want, TOL)
     finally:
         capi.check(l.mi355x_tune(b"q4_0.no_lds", 0))
+        capi.check(l.mi355x_tune(b"q4_0.path", 0))
 
 
 @pytest.mark.parametrize("rows,cols,waves", [(1, 1, 1), (2, 1, 4), (4, 2, 8), (7, 2, 8), (8, 2, 2), (4, 4, 4), (2, 7, 8), (1, 7, 1), (16, 1, 2)])
@@ -134,12 +181,12 @@ def test_q4_0_gemv_every_launch_shape(rows, cols, waves):
     buf, ptr = gpu.dev_bytes_at(raw, 0)
     want = O.qmatmul(O.Q4_0, raw, x, n, k)
     try:
-        for key, v in ((b"q4_0.rows", rows), (b"q4_0.cols", cols), (b"q4_0.waves", waves)):
+        for key, v in ((b"q4_0.path", 1), (b"q4_0.rows", rows), (b"q4_0.cols", cols), (b"q4_0.waves", waves)):
             capi.check(l.mi355x_tune(key, v))
         gpu.say(f"q4_0 gemv plan R={rows} C={cols} waves={waves}")
         check_close(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k), want, TOL)
     finally:
-        for key in (b"q4_0.rows", b"q4_0.cols", b"q4_0.waves"):
+        for key in (b"q4_0.path", b"q4_0.rows", b"q4_0.cols", b"q4_0.waves"):
             capi.check(l.mi355x_tune(key, 0))
 
 
@@ -156,7 +203,14 @@ def test_q4_0_gemv_linearity_at_full_size():
     assert np.abs(yab - (ya + yb)).max() <= 1e-4 * max(1, np.abs(yab).max())
     e = np.zeros(k, np.float32); e[1234] = 1
     col = gpu.qgemv(O.Q4_0, ptr, gpu.dev(e), n, k)
-    assert bits_equal(col, O.dequantize(O.Q4_0, raw).reshape(n, k)[:, 1234])
+    wcol = O.dequantize(O.Q4_0, raw).reshape(n, k)[:, 1234]
+    assert np.abs(col - wcol).max() <= 1e-6 * np.abs(wcol).max()  # a few float32 roundings of the scales
+    l = gpu.lib()
+    try:  # the float32 kernel multiplies by exactly 1: the column itself
+        capi.check(l.mi355x_tune(b"q4_0.path", 1))
+        assert bits_equal(gpu.qgemv(O.Q4_0, ptr, gpu.dev(e), n, k), wcol)
+    finally:
+        capi.check(l.mi355x_tune(b"q4_0.path", 0))
 
 
 def test_qgemv_argument_errors():
