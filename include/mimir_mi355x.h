@@ -88,16 +88,19 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
 
-/* The Q4_0 product in two steps, for callers that multiply one x by several
- * matrices (q, k and v; gate and up): mi355x_q4_0_convert_act turns each row of
- * x (K a multiple of 64) into the fixed-point form the fast kernel reads,
- * mi355x_q4_0_act_bytes(K) bytes per row at a 16-byte aligned `act`, and
- * mi355x_qgemv_q4_0_act multiplies by a dword-aligned W. mi355x_qgemv does both
- * through a scratch buffer of its own when W and K qualify. No counterpart in
- * the reference, whose kernels take float32 activations only. */
-MI355X_API size_t mi355x_q4_0_act_bytes(int64_t K);
-MI355X_API mi355x_status mi355x_q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
-MI355X_API mi355x_status mi355x_qgemv_q4_0_act(const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
+/* The product in two steps, for callers that multiply one x by several
+ * matrices (q, k and v; gate and up). mi355x_convert_act turns each row of x
+ * into the form the kernels of `dtype` read, mi355x_act_bytes(dtype, K) bytes
+ * per row at a 16-byte aligned `act` (0 when that dtype and K have no such
+ * form); mi355x_qgemv_act multiplies by W. mi355x_qgemv does both through a
+ * scratch buffer of its own.
+ *   Q8_0: quantizeRow's int8 blocks (backend/cpu/qmatmul.go:208-254).
+ *   Q4_0: 20-bit fixed point per block of 32 (K a multiple of 64, W dword
+ *         aligned); no counterpart in the reference, whose kernels take
+ *         float32 activations only. */
+MI355X_API size_t mi355x_act_bytes(int dtype, int64_t K);
+MI355X_API mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
+MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
 
 /* ---- OpCast / OpGather of a block-quantized input ---------------------------
  * (backend/cpu/quant.go:198-327; replaced kernels gen/quant.go:140-150 and

@@ -32,9 +32,9 @@ SYMBOLS = {
     "mi355x_download": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "mi355x_sync": (C.c_uint32, [_vp]),
     "mi355x_qgemv": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "mi355x_q4_0_act_bytes": (_sz, [_i64]),
-    "mi355x_q4_0_convert_act": (C.c_uint32, [_vp, _i64, _i64, _i64, _vp, _vp]),
-    "mi355x_qgemv_q4_0_act": (C.c_uint32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_act_bytes": (_sz, [_int, _i64]),
+    "mi355x_convert_act": (C.c_uint32, [_int, _vp, _i64, _i64, _i64, _vp, _vp]),
+    "mi355x_qgemv_act": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_dequant": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _int, _vp]),
     "mi355x_gather_rows": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp]),
     "mi355x_tune": (C.c_uint32, [C.c_char_p, _int]),

@@ -199,31 +199,56 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         }
         HIP_TRY(mimir::qgemv_q4_0(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
         return MI355X_OK;
+    case MI355X_Q8_0: {
+        if (!mimir::q8_act_fits(K)) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv by q8_0 with K = %lld: rows longer than 57344 are not supported", (long long)K);
+        void* act;
+        if (mi355x_status st = act_scratch(mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
+        HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
+        a.act = act;
+        HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0_act");
+        return MI355X_OK;
+    }
     default:
         return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by dtype %d is not built yet", dtype);
     }
 }
 
-size_t mi355x_q4_0_act_bytes(int64_t K) { return K > 0 && K % 32 == 0 ? mimir::q4_0_act_bytes(K) : 0; }
+size_t mi355x_act_bytes(int dtype, int64_t K) {
+    if (K <= 0) return 0;
+    if (dtype == MI355X_Q4_0 && K % 64 == 0) return mimir::q4_0_act_bytes(K);
+    if (dtype == MI355X_Q8_0 && K % 32 == 0) return mimir::q8_act_bytes(K);
+    return 0;
+}
 
-mi355x_status mi355x_q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream) {
-    if (M < 0 || K <= 0 || K % 64 != 0 || M > 65535)
-        return fail(MI355X_ERR_SHAPE, "mi355x: convert activations [%lld, %lld]: K must be a positive multiple of 64", (long long)M, (long long)K);
+mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream) {
+    if (mi355x_act_bytes(dtype, K) == 0 || M < 0 || M > 65535)
+        return fail(MI355X_ERR_SHAPE, "mi355x: convert activations [%lld, %lld] for weights of dtype %d", (long long)M, (long long)K, dtype);
     if (M == 0) return MI355X_OK;
     if (!x || !act || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: convert activations: null or misaligned pointer");
-    HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
+    if (dtype == MI355X_Q4_0)
+        HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
+    else
+        HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
     return MI355X_OK;
 }
 
-mi355x_status mi355x_qgemv_q4_0_act(const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
     if (M < 0 || N < 0 || K <= 0 || M > 65535 || N > (int64_t)1 << 30)
-        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_q4_0_act of %lld rows by [%lld, %lld]", (long long)M, (long long)N, (long long)K);
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act of %lld rows by [%lld, %lld]", (long long)M, (long long)N, (long long)K);
     if (M == 0 || N == 0) return MI355X_OK;
-    if (!W || !act || !y || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv_q4_0_act: null or misaligned pointer");
-    if (!mimir::q4_0_fixed_point_ok(W, K))
-        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_q4_0_act needs K a multiple of 64 up to 24448 and W dword aligned (K = %lld)", (long long)K);
+    if (!W || !act || !y || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv_act: null or misaligned pointer");
     mimir::QGemvArgs a{W, nullptr, act, y, M, N, K, 0, 0};
-    HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
+    if (dtype == MI355X_Q4_0) {
+        if (!mimir::q4_0_fixed_point_ok(W, K))
+            return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by q4_0 needs K a multiple of 64 up to 24448 and W dword aligned (K = %lld)", (long long)K);
+        HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
+    } else if (dtype == MI355X_Q8_0) {
+        if (K % 32 != 0 || !mimir::q8_act_fits(K))
+            return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by q8_0 needs K a multiple of 32 up to 57344 (K = %lld)", (long long)K);
+        HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0_act");
+    } else {
+        return fail(MI355X_ERR_DTYPE, "mi355x: qgemv_act by dtype %d", dtype);
+    }
     return MI355X_OK;
 }
 

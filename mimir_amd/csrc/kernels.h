@@ -49,6 +49,14 @@ size_t q4_0_act_bytes(int64_t K);
 hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 
+// The Q8_0 product as the reference's CPU computes it: x rounded to int8 per
+// block of 32 (q8_convert_act, q8_act_bytes(K) bytes per row), integer dot
+// products. q8_act_fits says whether the converted row fits the LDS.
+bool q8_act_fits(int64_t K);
+size_t q8_act_bytes(int64_t K);
+hipError_t q8_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
+
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);

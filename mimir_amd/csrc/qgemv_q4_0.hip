@@ -447,8 +447,9 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
                     int i0, i1;
                     q4_pair_dot(q0, q1, d0, d1, i0, i1);
                     const float f0 = (float)i0, f1 = (float)i1;
-                    const float w0 = f16_bits_to_f32((uint16_t)(a[0] & 0xffffu)) * s0;
-                    const float w1 = f16_bits_to_f32((uint16_t)(b[0] >> 16)) * s1;
+                    // a lane past the row's end re-reads the last pair: it must add exactly zero
+                    const float w0 = live ? f16_bits_to_f32((uint16_t)(a[0] & 0xffffu)) * s0 : 0.f;
+                    const float w1 = live ? f16_bits_to_f32((uint16_t)(b[0] >> 16)) * s1 : 0.f;
                     acc[r] = fmaf(w0, f0, acc[r]);
                     acc[r] = fmaf(w1, f1, acc[r]);
                 }

@@ -1,0 +1,245 @@
+// Decode products by Q8_0 weights, y = x . W^T with few rows of x, for gfx950.
+// They replace the reference's generated qmatmul kernel
+// (backend/internal/gen/quant.go:152-209) and compute what its CPU backend
+// computes (backend/cpu/qmatmul.go:310-405): each block of 32 activations is
+// rounded to int8 with a float32 scale (quantizeRow, qmatmul.go:208-254), the
+// products of a block are summed in four int32 lanes, value p into lane
+// p/4 mod 4, each lane times the product of the two scales is added to a
+// float32 lane of its own (a multiply, then an add: never fused), and the lanes
+// are added (0+2)+(1+3) (qdotQ8_0Go, qmatmul.go:125-139). The integer sums are
+// exact; the result differs from the CPU's only in the order in which the
+// blocks of a row are added, a few units in the last place.
+//
+// W stays in ggml's layout (34-byte blocks: binary16 scale, 32 int8), read in
+// place. A lane owns a pair of blocks, 68 bytes, dword aligned, fetched with
+// four aligned 128-bit loads and one dword; the second block's quants are
+// dword aligned, the first's are realigned with v_alignbyte. The activations
+// are converted once per x by q8_convert_act and staged in LDS per workgroup.
+#include "device_util.h"
+#include "kernels.h"
+
+namespace mimir {
+
+#pragma clang fp contract(off)
+
+// One row of x with nb blocks, converted (nbp = nb | 1):
+//   u32x4 q[2][nbp]   quants 16h..16h+15 of block b at q[h * nbp + b]
+//   float d[nb]       the block's scale
+size_t q8_act_bytes(int64_t K) {
+    int64_t nb = K / 32;
+    return (size_t)(((nb | 1) * 2 * 16 + nb * 4 + 15) / 16 * 16);
+}
+
+// quantizeRow (backend/cpu/qmatmul.go:208-254) for blocks of 32. Thread t takes
+// four values: block t / 8, dword t % 8; a block's eight threads are
+// consecutive lanes.
+__global__ __launch_bounds__(256) void q8_convert_act_kernel(const float* __restrict__ x, int64_t x_row_stride, int nb,
+                                                             uint8_t* __restrict__ act, int64_t act_row_bytes) {
+    const float* xr = x + (int64_t)blockIdx.y * x_row_stride;
+    uint32_t* q = (uint32_t*)(act + (int64_t)blockIdx.y * act_row_bytes);
+    const int nbp = nb | 1;
+    float* dscale = (float*)(q + 2 * nbp * 4);
+    const int nq = nb * 8;
+    for (int t = blockIdx.x * blockDim.x + threadIdx.x; t < nq; t += gridDim.x * blockDim.x) {
+        int b = t >> 3, i = t & 7;
+        f32x4 v;
+        __builtin_memcpy(&v, xr + 32 * (int64_t)b + 4 * i, 16);
+        float amax = 0.f;
+        bool finite = true;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float a = __builtin_fabsf(v[k]);
+            finite = finite && a < __builtin_inff();  // false for NaN too
+            if (a > amax) amax = a;
+        }
+        amax = group8_max(amax);
+        float bad = group8_max(finite ? 0.f : 1.f);
+        float d = 0.f;
+        uint32_t packed = 0;
+        if (bad != 0.f) {
+            d = __builtin_nanf("");
+        } else if (amax != 0.f) {
+            d = amax / 127.0f;
+            float id = 127.0f / amax;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                int r = (int)__builtin_rintf(v[k] * id);  // nearest, ties to even
+                r = r > 127 ? 127 : r < -127 ? -127 : r;
+                packed |= (uint32_t)(r & 0xff) << (8 * k);
+            }
+        }
+        q[((i >> 2) * nbp + b) * 4 + (i & 3)] = packed;
+        if (i == 0) dscale[b] = d;
+    }
+}
+
+hipError_t q8_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
+    int nb = (int)(K / 32);
+    int gx = (nb * 8 + 255) / 256;
+    hipLaunchKernelGGL(q8_convert_act_kernel, dim3((unsigned)gx, (unsigned)M), dim3(256), 0, st, x, x_row_stride, nb,
+                       (uint8_t*)act, (int64_t)q8_act_bytes(K));
+    return hipGetLastError();
+}
+
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+
+// The 17 dwords of a pair of blocks, or, for an odd last block or a W that is
+// only 2-byte aligned, one block at a time through unaligned loads.
+struct Q8Pair {
+    u32x4 v[4];
+    uint32_t tail;
+};
+
+// acc[l] += (d_w * d_x) * float(s_l) for the four lane sums of one block,
+// with the reference's roundings: the scales' product, its product with each
+// sum, and the addition are each rounded to float32.
+__device__ __forceinline__ void q8_block(const uint32_t w[8], const u32x4 xa, const u32x4 xb, float dw, float dx, float acc[4]) {
+    const float dd = dw * dx;
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+        int s = __builtin_amdgcn_sdot4((int)w[l], (int)xa[l], 0, false);
+        s = __builtin_amdgcn_sdot4((int)w[l + 4], (int)xb[l], s, false);
+        float t = dd * (float)s;
+        acc[l] = acc[l] + t;
+    }
+}
+
+template <int R, bool ALIGNED>
+__global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+                                                         float* __restrict__ y, int N, int nb, int64_t act_row_bytes,
+                                                         int rows_per_wg) {
+    extern __shared__ u32x4 lds_q8[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+    const int m = blockIdx.y;
+    float* yr = y + (int64_t)m * N;
+    const int nbp = nb | 1;
+    const float* xd = (const float*)(lds_q8 + 2 * nbp);
+    const int64_t row_bytes = (int64_t)nb * 34;
+    const int wg_row0 = blockIdx.x * rows_per_wg;
+    // ALIGNED: lanes own pairs of blocks; otherwise single blocks.
+    const int nunits = ALIGNED ? nb >> 1 : nb;
+    const int nsteps = (nunits + 63) >> 6;
+
+    // Stage the converted activations (see qgemv_q4_0_i4_kernel for the order).
+    constexpr int kPark = 2;
+    const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
+    const int n16 = (int)(act_row_bytes >> 4);
+    u32x4 park[kPark];
+#pragma unroll
+    for (int i = 0; i < kPark; i++) {
+        int idx = tid + i * (int)blockDim.x;
+        if (idx < n16) park[i] = act_row[idx];
+    }
+#pragma unroll
+    for (int i = 0; i < kPark; i++) {
+        int idx = tid + i * (int)blockDim.x;
+        if (idx < n16) lds_q8[idx] = park[i];
+    }
+    for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_q8[idx] = act_row[idx];
+    __syncthreads();
+
+    for (int r0 = wave * R; r0 < rows_per_wg; r0 += waves * R) {
+        const int row0 = wg_row0 + r0;
+        if (row0 >= N) break;
+        float acc[R][4];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int l = 0; l < 4; l++) acc[r][l] = 0.f;
+        for (int step = 0; step < nsteps; step++) {
+            int u = lane + 64 * step;
+            const bool live = u < nunits;
+            u = live ? u : nunits - 1;
+            Q8Pair pr[R];
+            uint32_t single[R][9];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                int row = row0 + r;
+                row = row < N ? row : N - 1;
+                const uint8_t* rowp = W + (int64_t)row * row_bytes;
+                if (ALIGNED) {
+                    const uint32_t* src = (const uint32_t*)rowp + u * 17;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) pr[r].v[k] = *(const u32x4_a4*)(src + 4 * k);
+                    pr[r].tail = src[16];
+                } else {
+                    const uint8_t* src = rowp + (int64_t)u * 34;
+                    u32x4 a = *(const u32x4_a2*)(src + 2), b = *(const u32x4_a2*)(src + 18);
+                    single[r][0] = load_u16(src);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        single[r][1 + k] = a[k];
+                        single[r][5 + k] = b[k];
+                    }
+                }
+            }
+            if (ALIGNED) {
+                const u32x4 xa0 = lds_q8[2 * u], xb0 = lds_q8[nbp + 2 * u];
+                const u32x4 xa1 = lds_q8[2 * u + 1], xb1 = lds_q8[nbp + 2 * u + 1];
+                const float dx0 = live ? xd[2 * u] : 0.f, dx1 = live ? xd[2 * u + 1] : 0.f;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    uint32_t d[17];
+#pragma unroll
+                    for (int k = 0; k < 16; k++) d[k] = pr[r].v[k >> 2][k & 3];
+                    d[16] = pr[r].tail;
+                    // block 0: scale in the low half of d[0], quants at bytes 2..33
+                    uint32_t w0[8], w1[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        w0[k] = __builtin_amdgcn_alignbyte(d[k + 1], d[k], 2);
+                        w1[k] = d[9 + k];  // block 1: scale in the high half of d[8], quants at bytes 36..67
+                    }
+                    // a lane past the row's end re-reads the last pair: it must add exactly zero
+                    q8_block(w0, xa0, xb0, live ? f16_bits_to_f32((uint16_t)(d[0] & 0xffffu)) : 0.f, dx0, acc[r]);
+                    q8_block(w1, xa1, xb1, live ? f16_bits_to_f32((uint16_t)(d[8] >> 16)) : 0.f, dx1, acc[r]);
+                }
+            } else {
+                const u32x4 xa = lds_q8[u], xb = lds_q8[nbp + u];
+                const float dx = live ? xd[u] : 0.f;
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                    q8_block(&single[r][1], xa, xb, live ? f16_bits_to_f32((uint16_t)single[r][0]) : 0.f, dx, acc[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float a0 = wave_sum(acc[r][0]), a1 = wave_sum(acc[r][1]), a2 = wave_sum(acc[r][2]), a3 = wave_sum(acc[r][3]);
+            float s02 = a0 + a2, s13 = a1 + a3;
+            if (lane == 0 && row0 + r < N) yr[row0 + r] = s02 + s13;
+        }
+    }
+}
+
+bool q8_act_fits(int64_t K) { return q8_act_bytes(K) <= 64 * 1024; }
+
+template <int R, bool ALIGNED>
+static hipError_t launch_q8(const QGemvArgs& a, int waves, hipStream_t st) {
+    int rows_per_wg = R * waves;
+    dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
+    size_t act_bytes = q8_act_bytes(a.K);
+    hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
+                       (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+    return hipGetLastError();
+}
+
+// tune: {rows, -, waves}. Needs q8_act_fits(K).
+hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
+    int nb = (int)(a.K / 32);
+    const bool aligned = nb % 2 == 0 && ((uintptr_t)a.W & 3) == 0;
+    int R = a.N >= 4096 ? 2 : 1;
+    if (tune[0] > 0) R = tune[0];
+    int64_t tiles = (a.N + R - 1) / R;
+    int waves = 8;
+    while (waves > 1 && tiles / waves < 256) waves >>= 1;
+    if (tune[2] > 0) waves = tune[2];
+#define Q8CASE(RR)                                                           \
+    if (R == RR) return aligned ? launch_q8<RR, true>(a, waves, st) : launch_q8<RR, false>(a, waves, st)
+    Q8CASE(1); Q8CASE(2); Q8CASE(4);
+#undef Q8CASE
+    return aligned ? launch_q8<1, true>(a, waves, st) : launch_q8<1, false>(a, waves, st);
+}
+
+}  // namespace mimir

@@ -62,3 +62,29 @@ def dequant(dt, w_ptr, first: int, n: int, out_dt=capi.F32) -> np.ndarray:
     sync()
     r = out.cpu().numpy()
     return r if out_dt == capi.F32 else r.view(np.uint16)
+
+
+def convert_act(dt, x: torch.Tensor, k: int) -> np.ndarray:
+    """The converted activations of the rows of x, as raw bytes [m, act_bytes]."""
+    l = lib()
+    x2 = x.reshape(-1, k)
+    m = x2.shape[0]
+    nbytes = l.mi355x_act_bytes(dt, k)
+    assert nbytes > 0
+    act = torch.zeros((m, nbytes), dtype=torch.uint8, device="cuda:0")
+    capi.check(l.mi355x_convert_act(dt, x2.data_ptr(), m, k, x2.stride(0) if m > 1 else k, act.data_ptr(), stream()))
+    sync()
+    return act.cpu().numpy()
+
+
+def qgemv_act(dt, w_ptr, x: torch.Tensor, n: int, k: int) -> np.ndarray:
+    """The two-step product: convert once, multiply."""
+    l = lib()
+    x2 = x.reshape(-1, k)
+    m = x2.shape[0]
+    act = torch.zeros((m, l.mi355x_act_bytes(dt, k)), dtype=torch.uint8, device="cuda:0")
+    y = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(l.mi355x_convert_act(dt, x2.data_ptr(), m, k, x2.stride(0) if m > 1 else k, act.data_ptr(), stream()))
+    capi.check(l.mi355x_qgemv_act(dt, w_ptr, act.data_ptr(), y.data_ptr(), m, n, k, stream()))
+    sync()
+    return y.cpu().numpy().reshape(tuple(x.shape[:-1]) + (n,))

@@ -213,6 +213,135 @@ def test_q4_0_gemv_linearity_at_full_size():
         capi.check(l.mi355x_tune(b"q4_0.path", 0))
 
 
+# ---- Q8_0: the int8-activation product of the CPU backend -------------------
+
+def _unpack_q8_act(raw, k):
+    """The device's converted row (q[2][nbp] of 16 bytes, then float scales) as
+    quantizeRow's blocks: f32 d | int8 q[32]."""
+    nb = k // 32; nbp = nb | 1
+    q = raw[:2 * nbp * 16].reshape(2, nbp, 16)
+    d = raw[2 * nbp * 16:2 * nbp * 16 + 4 * nb].view(np.float32)
+    out = np.zeros((nb, 36), np.uint8)
+    out[:, :4] = d.view(np.uint8).reshape(nb, 4)
+    out[:, 4:20] = q[0, :nb]
+    out[:, 20:36] = q[1, :nb]
+    return out.reshape(-1)
+
+
+def test_q8_activation_rounding_is_bit_exact():
+    """quantizeRow on the device against the oracle's, byte for byte: normal
+    values, ties under an amax of 127, tiny and huge magnitudes, zeros, an
+    infinity and a NaN (backend/cpu/quant_test.go:523-558)."""
+    rng = np.random.default_rng(17)
+    bs, nblk = 32, 64
+    x = np.empty(nblk * bs, np.float32)
+    for b in range(nblk):
+        v = x[b * bs:(b + 1) * bs]
+        if b % 4 == 0:
+            v[:] = rng.random(bs, dtype=np.float32) * 2 - 1
+        elif b % 4 == 1:
+            v[:] = (rng.integers(0, 254, bs) - 127) / 2
+            v[0] = 127
+        elif b % 4 == 2:
+            v[:] = rng.normal(size=bs) * 1e-30
+        else:
+            v[:] = rng.normal(size=bs) * 1e30
+    x[7 * bs:8 * bs] = 0
+    x[5 * bs + 3] = np.inf
+    x[9 * bs] = np.nan
+    gpu.say("q8 convert_act vs quantize_row")
+    got = _unpack_q8_act(gpu.convert_act(O.Q8_0, gpu.dev(x), x.size)[0], x.size).reshape(nblk, 36)
+    want = O.quantize_row(x, 32, False).reshape(nblk, 36)
+    for b in range(nblk):
+        gd, wd = got[b, :4].view(np.float32)[0], want[b, :4].view(np.float32)[0]
+        assert (np.isnan(gd) and np.isnan(wd)) or got[b, :4].tobytes() == want[b, :4].tobytes(), b
+        assert np.array_equal(got[b, 4:], want[b, 4:]), b
+
+
+def test_q8_0_gemv_baseline_config():
+    """W 4096 x 4096 int8 uniform in [-127, 127], one binary16 scale |N(0, 0.02)|
+    per block, x ~ N(0, 1), seed 0, against the CPU path (int8 activations)."""
+    rng = np.random.default_rng(0)
+    n = k = 4096
+    raw = bench_blocks(rng, O.Q8_0, n * k)
+    x = rng.normal(size=(1, k)).astype(np.float32)
+    gpu.say("q8_0 gemv 4096x4096")
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+    want = O.qmatmul(O.Q8_0, raw, x, n, k)
+    check_close(got, want, TOL, "q8_0 4096x4096")
+    assert rel_l2(got, want) < 1e-6  # only the order of the blocks' additions differs
+    assert np.array_equal(got, gpu.qgemv_act(O.Q8_0, ptr, gpu.dev(x), n, k))  # the two-step entry is the same product
+
+
+@pytest.mark.parametrize("n,k,offset", [(9, 1280, 0), (9, 1280, 2), (7, 32 * 5, 0), (1, 32, 0), (300, 4096 + 96, 0), (64, 14336, 0), (5, 32768, 2)])
+def test_q8_0_gemv_shapes(n, k, offset):
+    """Ragged shapes, an odd number of blocks, and a W that is only 2-byte
+    aligned (the single-block path)."""
+    rng = np.random.default_rng(n * 7 + k + offset)
+    raw = random_blocks(rng, O.Q8_0, n * k)
+    for m, shape in ((1, (k,)), (6, (2, 3, k))):
+        x = rng.normal(size=shape).astype(np.float32)
+        gpu.say(f"q8_0 gemv N={n} K={k} offset={offset} x{shape}")
+        buf, ptr = gpu.dev_bytes_at(raw, offset)
+        got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+        want = O.qmatmul(O.Q8_0, raw, x, n, k)
+        # Same integers, same per-block roundings; only the order of the blocks'
+        # float32 additions differs, so the error scales with sum |w||x|.
+        mag = np.abs(x.reshape(-1, k)).astype(np.float64) @ np.abs(O.dequantize(O.Q8_0, raw).reshape(n, k)).astype(np.float64).T
+        assert np.all(np.abs(got.reshape(-1, n) - want.reshape(-1, n)) <= 2e-6 * mag + 1e-30), f"q8_0 {n}x{k}+{offset}"
+
+
+def test_q8_0_gemv_golden_and_exact_rows(golden_dir):
+    c = golden_cases(os.path.join(golden_dir, "quant.mim"))["q8_0_matmul"]
+    x, raw = c["in"][0].data, c["in"][1].data.reshape(-1)
+    n, k = c["in"][1].shape[0], c["in"][1].shape[1] // 34 * 32
+    gpu.say("q8_0 golden matmul")
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+    assert np.all(np.abs(got - c["out"].data) <= 1e-5 + 1e-5 * np.abs(c["out"].data))  # tensor/quant_test.go:321
+    # kerneltest/quant.go:113-139: rows 1..9 of a 10-row table, exact activations, Tol 1e-4 against the CPU
+    rng = np.random.default_rng(13)
+    n, k = 9, 1280
+    raw = random_blocks(rng, O.Q8_0, (n + 1) * k)
+    row = k // 32 * 34
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    for shape in ((k,), (1, k), (2, 3, k)):
+        x = exact_rows(rng, O.Q8_0, int(np.prod(shape[:-1])), k).reshape(shape)
+        got = gpu.qgemv(O.Q8_0, ptr + row, gpu.dev(x), n, k)
+        check_close(got, O.qmatmul(O.Q8_0, raw[row:], x, n, k), 1e-4)
+
+
+def test_q8_0_gemv_nan_and_inf_blocks():
+    """A block of x that holds a NaN or an infinity makes every product NaN
+    (backend/cpu/qmatmul.go:205-207)."""
+    rng = np.random.default_rng(3)
+    n, k = 16, 256
+    raw = bench_blocks(rng, O.Q8_0, n * k)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    x = rng.normal(size=k).astype(np.float32)
+    for bad in (np.inf, -np.inf, np.nan):
+        x2 = x.copy(); x2[77] = bad
+        got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x2), n, k)
+        want = O.qmatmul(O.Q8_0, raw, x2, n, k)
+        assert np.isnan(got).all() and np.isnan(want).all()
+
+
+def test_q8_0_lm_head_shape_sampled():
+    """The output projection of an 8B model, 128256 x 4096 (558 MB), against
+    the oracle on every row."""
+    rng = np.random.default_rng(11)
+    n, k = 128256, 4096
+    raw = bench_blocks(rng, O.Q8_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    gpu.say("q8_0 gemv lm_head 128256x4096")
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+    want = O.qmatmul(O.Q8_0, raw, x, n, k, simd=True)
+    check_close(got, want, 1e-4, "lm_head")
+    assert O.argmax(got) == O.argmax(want)
+
+
 def test_qgemv_argument_errors():
     l = gpu.lib()
     x = torch.zeros(64, device="cuda:0"); y = torch.zeros(4, device="cuda:0"); w = torch.zeros(1024, dtype=torch.uint8, device="cuda:0")
