@@ -95,6 +95,7 @@ MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, 
  * form); mi355x_qgemv_act multiplies by W. mi355x_qgemv does both through a
  * scratch buffer of its own.
  *   Q8_0: quantizeRow's int8 blocks (backend/cpu/qmatmul.go:208-254).
+ *   Q4_K, Q6_K: quantizeRow's int8 super-blocks of 256 with their sums.
  *   Q4_0: 20-bit fixed point per block of 32 (K a multiple of 64, W dword
  *         aligned); no counterpart in the reference, whose kernels take
  *         float32 activations only. */

@@ -208,8 +208,17 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0_act");
         return MI355X_OK;
     }
+    case MI355X_Q4_K:
+    case MI355X_Q6_K: {
+        void* act;
+        if (mi355x_status st = act_scratch(mimir::kq_act_bytes(K) * (size_t)M, &act)) return st;
+        HIP_TRY(mimir::kq_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch kq_convert_act");
+        a.act = act;
+        HIP_TRY(mimir::qgemv_kquant_act(dtype, a, (hipStream_t)stream), "launch qgemv_kquant_act");
+        return MI355X_OK;
+    }
     default:
-        return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by dtype %d is not built yet", dtype);
+        return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by weights of dtype %d", dtype);
     }
 }
 
@@ -217,6 +226,7 @@ size_t mi355x_act_bytes(int dtype, int64_t K) {
     if (K <= 0) return 0;
     if (dtype == MI355X_Q4_0 && K % 64 == 0) return mimir::q4_0_act_bytes(K);
     if (dtype == MI355X_Q8_0 && K % 32 == 0) return mimir::q8_act_bytes(K);
+    if ((dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) && K % 256 == 0) return mimir::kq_act_bytes(K);
     return 0;
 }
 
@@ -227,8 +237,10 @@ mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K
     if (!x || !act || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: convert activations: null or misaligned pointer");
     if (dtype == MI355X_Q4_0)
         HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
-    else
+    else if (dtype == MI355X_Q8_0)
         HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
+    else
+        HIP_TRY(mimir::kq_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch kq_convert_act");
     return MI355X_OK;
 }
 
@@ -246,6 +258,9 @@ mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float*
         if (K % 32 != 0 || !mimir::q8_act_fits(K))
             return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by q8_0 needs K a multiple of 32 up to 57344 (K = %lld)", (long long)K);
         HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0_act");
+    } else if (dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) {
+        if (K % 256 != 0) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by a K-quant needs K a multiple of 256 (K = %lld)", (long long)K);
+        HIP_TRY(mimir::qgemv_kquant_act(dtype, a, (hipStream_t)stream), "launch qgemv_kquant_act");
     } else {
         return fail(MI355X_ERR_DTYPE, "mi355x: qgemv_act by dtype %d", dtype);
     }

@@ -57,6 +57,13 @@ size_t q8_act_bytes(int64_t K);
 hipError_t q8_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 
+// The Q4_K and Q6_K products as the reference's CPU computes them: x rounded
+// to int8 in super-blocks of 256 with the sums of each 16 quants
+// (kq_convert_act, kq_act_bytes(K) bytes per row), integer dot products.
+size_t kq_act_bytes(int64_t K);
+hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
+
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);

@@ -342,6 +342,63 @@ def test_q8_0_lm_head_shape_sampled():
     assert O.argmax(got) == O.argmax(want)
 
 
+# ---- Q4_K / Q6_K -------------------------------------------------------------
+
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+def test_kquant_activation_rounding_is_bit_exact(dt):
+    rng = np.random.default_rng(21)
+    k = 256 * 6
+    x = rng.normal(size=k).astype(np.float32)
+    x[256:512] = 0
+    x[512:768] = (rng.integers(0, 254, 256) - 127) / 2; x[512] = 127  # ties
+    x[1300] = np.nan
+    gpu.say(f"kquant convert_act dt={dt}")
+    raw = gpu.convert_act(dt, gpu.dev(x), k)[0]
+    nsb = k // 256
+    want = O.quantize_row(x, 256, True).reshape(nsb, 292)
+    assert np.array_equal(raw[:nsb * 256].reshape(nsb, 256), want[:, 4:260])
+    assert np.array_equal(raw[nsb * 256:nsb * 288].reshape(nsb, 32), want[:, 260:292])
+    gd, wd = raw[nsb * 288:nsb * 292].view(np.float32), want[:, :4].copy().view(np.float32).reshape(-1)
+    assert np.array_equal(np.isnan(gd), np.isnan(wd)) and np.array_equal(gd[~np.isnan(gd)], wd[~np.isnan(wd)])
+
+
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("n,k,offset", [(9, 1280, 0), (5, 256, 2), (33, 256 * 17, 0), (300, 4096, 0)])
+def test_kquant_gemv_matches_oracle(dt, n, k, offset):
+    rng = np.random.default_rng(n + k + dt)
+    raw = random_blocks(rng, dt, n * k)
+    wabs = np.abs(O.dequantize(dt, raw).reshape(n, k)).astype(np.float64)
+    for shape in ((k,), (2, 3, k)):
+        x = rng.normal(size=shape).astype(np.float32)
+        gpu.say(f"kquant gemv dt={dt} N={n} K={k} offset={offset} x{shape}")
+        buf, ptr = gpu.dev_bytes_at(raw, offset)
+        got = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
+        want = O.qmatmul(dt, raw, x, n, k)
+        mag = np.abs(x.reshape(-1, k)).astype(np.float64) @ wabs.T
+        assert np.all(np.abs(got.reshape(-1, n) - want.reshape(-1, n)) <= 4e-6 * mag + 1e-30)
+        assert np.array_equal(got, gpu.qgemv_act(dt, ptr, gpu.dev(x), n, k))
+
+
+def test_kquant_gemv_golden_and_exact_rows(golden_dir):
+    cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
+    for kind, dt in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
+        c = cases[f"{kind}_matmul"]
+        x, raw = c["in"][0].data, c["in"][1].data.reshape(-1)
+        n, k = c["in"][1].shape[0], c["in"][1].shape[1] // O.block_bytes(dt) * 256
+        gpu.say(f"{kind} golden matmul")
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        got = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
+        assert np.all(np.abs(got - c["out"].data) <= 1e-5 + 1e-5 * np.abs(c["out"].data))
+        rng = np.random.default_rng(13)
+        n2, k2 = 9, 1280
+        raw2 = random_blocks(rng, dt, (n2 + 1) * k2)
+        row = k2 // 256 * O.block_bytes(dt)
+        buf2, ptr2 = gpu.dev_bytes_at(raw2, 0)
+        for shape in ((k2,), (1, k2), (2, 3, k2)):
+            xx = exact_rows(rng, dt, int(np.prod(shape[:-1])), k2).reshape(shape)
+            check_close(gpu.qgemv(dt, ptr2 + row, gpu.dev(xx), n2, k2), O.qmatmul(dt, raw2[row:], xx, n2, k2), 1e-4)
+
+
 def test_qgemv_argument_errors():
     l = gpu.lib()
     x = torch.zeros(64, device="cuda:0"); y = torch.zeros(4, device="cuda:0"); w = torch.zeros(1024, dtype=torch.uint8, device="cuda:0")
