@@ -115,6 +115,44 @@ MI355X_API mi355x_status mi355x_dequant(int dtype, const void* W, int64_t first,
 MI355X_API mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_t rows, int64_t K, const int32_t* idx, int64_t n,
                                  float* out, void* stream);
 
+/* ---- the other kernels of a decoding step -----------------------------------
+ * On the reference these are runs of generated elementwise and reduction
+ * kernels plus OpAttention; each is one launch here, so a whole step is queued
+ * without a host round trip. */
+
+/* RMSNorm.Forward (nn/transformer.go:50-61; llm/decode.go:376-385):
+ * y[r, :] = (x[r, :] * recip(sqrt(mean(x[r, :]^2) + eps))) * w; w may be NULL. */
+MI355X_API mi355x_status mi355x_rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, void* stream);
+/* RotaryEmbedding.Apply (nn/transformer.go:225-257). x is [rows, S, head_dim]
+ * read with strides in floats; position s of every row turns by row
+ * offset + s of cos_table and sin_table, [table_len, rope_dim/2] float32, which
+ * the host computes in float64 as the reference does (transformer.go:146-164).
+ * interleaved pairs features (2i, 2i+1), else (i, i + rope_dim/2). y may be x. */
+MI355X_API mi355x_status mi355x_rope(const float* x, float* y, int64_t rows, int64_t S, int head_dim, int rope_dim, int interleaved,
+                          int64_t x_row_stride, int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride,
+                          const float* cos_table, const float* sin_table, int64_t table_len, int64_t offset, void* stream);
+/* KVCache.Append's write (nn/transformer.go:397-423): src [B, heads, S, dim],
+ * read with strides, lands at positions [pos, pos + S) of cache
+ * [B, heads, capacity, dim], cast to cache_dtype (F32 or F16). */
+MI355X_API mi355x_status mi355x_kv_write(const float* src, void* cache, int cache_dtype, int64_t B, int heads, int64_t S, int dim,
+                              int64_t capacity, int64_t pos, int64_t src_b_stride, int64_t src_h_stride, int64_t src_p_stride,
+                              void* stream);
+/* OpAttention (backend/op.go:117-129; backend/attention.go:25-143) without a
+ * mask: queries [B, H, Q, D], keys and values [B, HK, K, D] of kv_dtype (F32 or
+ * F16), out [B, H, Q, D], each read through strides {batch, head, position}
+ * with contiguous features; lse, if not NULL, [B, H, Q] contiguous. Key j is
+ * hidden from query i when causal and j > i + causal_offset. D at most 256. */
+MI355X_API mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const void* v, int kv_dtype,
+                               const int64_t* kv_strides, float* out, const int64_t* out_strides, float* lse, int64_t B, int H,
+                               int HK, int64_t Q, int64_t K, int D, double scale, int causal, int64_t causal_offset, void* stream);
+/* Block.mlp's activation (llm/model.go:446-448): out = SiLU(gate) * up, rows of
+ * gate and up in_row_stride floats apart, out contiguous. */
+MI355X_API mi355x_status mi355x_swiglu(const float* gate, const float* up, float* out, int64_t rows, int64_t n, int64_t in_row_stride, void* stream);
+MI355X_API mi355x_status mi355x_add(const float* a, const float* b, float* out, int64_t n, void* stream);
+/* Sampler.Sample at temperature 0 (examples/llama/generate.go:44-53): the first
+ * index of each row's largest value, into device memory. */
+MI355X_API mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, void* stream);
+
 /* ---- measurement aids (no counterpart in the reference) ---------------------
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces

@@ -49,6 +49,9 @@ struct DeviceState {
     // streams of one device race on it).
     void* act = nullptr;
     size_t act_bytes = 0;
+    // Partial results of split attention, grown and shared likewise.
+    void* attn = nullptr;
+    size_t attn_bytes = 0;
 };
 
 std::mutex g_mu;
@@ -89,6 +92,22 @@ mi355x_status act_scratch(size_t bytes, void** out) {
         s->act_bytes = want;
     }
     *out = s->act;
+    return MI355X_OK;
+}
+
+mi355x_status attn_scratch(size_t bytes, void** out) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (s->attn_bytes < bytes) {
+        size_t want = bytes < (4u << 20) ? (4u << 20) : bytes;
+        void* p = nullptr;
+        HIP_TRY(hipMalloc(&p, want), "hipMalloc(attention scratch)");
+        if (s->attn) HIP_TRY(hipFree(s->attn), "hipFree(attention scratch)");
+        s->attn = p;
+        s->attn_bytes = want;
+    }
+    *out = s->attn;
     return MI355X_OK;
 }
 
@@ -288,6 +307,95 @@ mi355x_status mi355x_gather_rows(int dtype, const void* table, int64_t rows, int
     DeviceState* s;
     if (mi355x_status st = current_state(&s)) return st;
     HIP_TRY(mimir::gather_rows(dtype, table, rows, K, idx, n, out, s->err_dev, (hipStream_t)stream), "launch gather_rows");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, void* stream) {
+    if (rows < 0 || d < 0 || rows > INT32_MAX || d > INT32_MAX) return fail(MI355X_ERR_SHAPE, "mi355x: rmsnorm of [%lld, %lld]", (long long)rows, (long long)d);
+    if (rows == 0 || d == 0) return MI355X_OK;
+    if (!x || !y) return fail(MI355X_ERR_INTERNAL, "mi355x: rmsnorm: null pointer");
+    HIP_TRY(mimir::rmsnorm(x, w, y, rows, d, eps, (hipStream_t)stream), "launch rmsnorm");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_rope(const float* x, float* y, int64_t rows, int64_t S, int head_dim, int rope_dim, int interleaved,
+                          int64_t x_row_stride, int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride,
+                          const float* cos_table, const float* sin_table, int64_t table_len, int64_t offset, void* stream) {
+    // nn/transformer.go:229-231
+    if (rows < 0 || S < 0 || head_dim <= 0 || rope_dim <= 0 || rope_dim % 2 != 0 || rope_dim > head_dim || offset < 0 ||
+        offset + S > table_len)
+        return fail(MI355X_ERR_SHAPE, "mi355x: rotary embedding of %d of %d features at positions [%lld, %lld) of a table of %lld",
+                    rope_dim, head_dim, (long long)offset, (long long)(offset + S), (long long)table_len);
+    if (rows == 0 || S == 0) return MI355X_OK;
+    if (!x || !y || !cos_table || !sin_table) return fail(MI355X_ERR_INTERNAL, "mi355x: rope: null pointer");
+    HIP_TRY(mimir::rope(x, y, rows, S, head_dim, rope_dim, interleaved, x_row_stride, x_pos_stride, y_row_stride, y_pos_stride,
+                        cos_table, sin_table, offset, (hipStream_t)stream), "launch rope");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_kv_write(const float* src, void* cache, int cache_dtype, int64_t B, int heads, int64_t S, int dim,
+                              int64_t capacity, int64_t pos, int64_t src_b_stride, int64_t src_h_stride, int64_t src_p_stride,
+                              void* stream) {
+    if (cache_dtype != MI355X_F32 && cache_dtype != MI355X_F16) return fail(MI355X_ERR_DTYPE, "mi355x: KV cache of dtype %d", cache_dtype);
+    // nn/transformer.go:405-411
+    if (B < 0 || heads <= 0 || S < 0 || dim <= 0 || pos < 0 || pos + S > capacity)
+        return fail(MI355X_ERR_SHAPE, "mi355x: write %lld positions at %lld to a cache of %lld", (long long)S, (long long)pos, (long long)capacity);
+    if (B == 0 || S == 0) return MI355X_OK;
+    if (!src || !cache) return fail(MI355X_ERR_INTERNAL, "mi355x: kv_write: null pointer");
+    HIP_TRY(mimir::kv_write(src, cache, cache_dtype, B, heads, S, dim, capacity, pos, src_b_stride, src_h_stride, src_p_stride,
+                            (hipStream_t)stream), "launch kv_write");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const void* v, int kv_dtype,
+                               const int64_t* kv_strides, float* out, const int64_t* out_strides, float* lse, int64_t B, int H,
+                               int HK, int64_t Q, int64_t K, int D, double scale, int causal, int64_t causal_offset, void* stream) {
+    if (kv_dtype != MI355X_F32 && kv_dtype != MI355X_F16) return fail(MI355X_ERR_DTYPE, "mi355x: attention over keys of dtype %d", kv_dtype);
+    // backend/attention.go:36-62
+    if (B < 0 || Q < 0 || K < 0 || H <= 0 || HK <= 0 || H % HK != 0 || D <= 0 || D > 256)
+        return fail(MI355X_ERR_SHAPE, "mi355x: attention of %d heads on %d key heads of %d features (at most 256)", H, HK, D);
+    if (B == 0 || Q == 0) return MI355X_OK;
+    if (B * Q > 65535 || (int64_t)HK * ((H / HK + 3) / 4) > 65535)
+        return fail(MI355X_ERR_SHAPE, "mi355x: attention of %lld query rows: too many for one launch", (long long)(B * Q));
+    if (!q || !out || !q_strides || !kv_strides || !out_strides || (K > 0 && (!k || !v))) return fail(MI355X_ERR_INTERNAL, "mi355x: attention: null pointer");
+    mimir::AttnArgs a;
+    a.q = q; a.k = k; a.v = v; a.kv_dtype = kv_dtype; a.out = out; a.lse = lse;
+    for (int i = 0; i < 3; i++) {
+        a.q_strides[i] = q_strides[i];
+        a.k_strides[i] = a.v_strides[i] = kv_strides[i];
+        a.o_strides[i] = out_strides[i];
+    }
+    a.B = B; a.Q = Q; a.K = K; a.H = H; a.HK = HK; a.D = D;
+    a.scale = scale; a.causal = causal; a.causal_offset = causal_offset;
+    mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
+    void* ws = nullptr;
+    if (size_t need = mimir::attention_workspace_bytes(B, H, Q, D, a.nsplit))
+        if (mi355x_status st = attn_scratch(need, &ws)) return st;
+    HIP_TRY(mimir::attention(a, ws, (hipStream_t)stream), "launch attention");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_swiglu(const float* gate, const float* up, float* out, int64_t rows, int64_t n, int64_t in_row_stride, void* stream) {
+    if (rows < 0 || n < 0) return fail(MI355X_ERR_SHAPE, "mi355x: swiglu of [%lld, %lld]", (long long)rows, (long long)n);
+    if (rows == 0 || n == 0) return MI355X_OK;
+    if (!gate || !up || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: swiglu: null pointer");
+    HIP_TRY(mimir::swiglu(gate, up, out, rows, n, in_row_stride, (hipStream_t)stream), "launch swiglu");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_add(const float* a, const float* b, float* out, int64_t n, void* stream) {
+    if (n < 0) return fail(MI355X_ERR_SHAPE, "mi355x: add of %lld elements", (long long)n);
+    if (n == 0) return MI355X_OK;
+    if (!a || !b || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: add: null pointer");
+    HIP_TRY(mimir::add(a, b, out, n, (hipStream_t)stream), "launch add");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, void* stream) {
+    if (rows < 0 || n <= 0 || n > INT32_MAX || rows > 65535) return fail(MI355X_ERR_SHAPE, "mi355x: argmax of [%lld, %lld]", (long long)rows, (long long)n);
+    if (rows == 0) return MI355X_OK;
+    if (!logits || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: argmax: null pointer");
+    HIP_TRY(mimir::argmax(logits, rows, n, out, (hipStream_t)stream), "launch argmax");
     return MI355X_OK;
 }
 

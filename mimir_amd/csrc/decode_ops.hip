@@ -1,0 +1,218 @@
+// The small kernels of a decoding step, for gfx950: RMSNorm, rotary
+// embedding, the KV-cache write, SwiGLU, the residual add and greedy argmax.
+// On the reference's ROCm backend these arrive as runs of generated
+// elementwise and reduction kernels (backend/internal/gen/gen.go:556+); here
+// each is one launch, so that a whole step is queued with no host round trip.
+// The arithmetic follows the reference operation by operation (each product
+// rounded to float32 on its own, no fused multiply-adds) except for the order
+// of RMSNorm's sum of squares, which a parallel reduction fixes differently.
+#include "device_util.h"
+#include "kernels.h"
+
+namespace mimir {
+
+#pragma clang fp contract(off)
+
+// ---- RMSNorm: nn/transformer.go:50-61; llm/decode.go:376-385 -----------------
+// y = (x * recip(sqrt(mean(x^2) + eps))) * w, one workgroup per row. mean is
+// sum * float32(1/d); eps is added as a float32; the reciprocal and the square
+// root are correctly rounded.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      float* __restrict__ y, int d, float inv_d, float eps) {
+    __shared__ float part[4];
+    const float* xr = x + (int64_t)blockIdx.x * d;
+    float* yr = y + (int64_t)blockIdx.x * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = xr[i];
+        float sq = v * v;
+        ss = ss + sq;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = (part[0] + part[1]) + (part[2] + part[3]);
+    float ms = total * inv_d;
+    float scale = 1.0f / __builtin_sqrtf(ms + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = xr[i] * scale;
+        yr[i] = w ? v * w[i] : v;
+    }
+}
+
+hipError_t rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, hipStream_t st) {
+    if (rows == 0 || d == 0) return hipSuccess;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, w, y, (int)d, (float)(1.0 / (double)d), (float)eps);
+    return hipGetLastError();
+}
+
+// ---- RoPE: nn/transformer.go:225-257 -------------------------------------------
+// x is [rows, S, head_dim] with explicit strides; position s of every row
+// turns by the angles of table row offset + s (cos and sin are [len, dim/2],
+// computed on the host in float64 as the reference does, transformer.go:146-164).
+// a' = a*cos - b*sin, b' = a*sin + b*cos for interleaved pairs (2i, 2i+1), and
+// for halves (i, i + dim/2) a' = a*cos - b*sin, b' = b*cos + a*sin.
+__global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x, float* __restrict__ y, int64_t rows, int s,
+                                                   int head_dim, int dim, int interleaved, int64_t x_row_stride,
+                                                   int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride,
+                                                   const float* __restrict__ cosv, const float* __restrict__ sinv, int offset) {
+    const int half = dim >> 1, per = half + (head_dim - dim);  // work items per (row, position)
+    int64_t total = rows * s * per;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        int i = (int)(t % per);
+        int64_t rp = t / per;
+        int q = (int)(rp % s);
+        int64_t r = rp / s;
+        const float* xi = x + r * x_row_stride + q * x_pos_stride;
+        float* yo = y + r * y_row_stride + q * y_pos_stride;
+        if (i >= half) {  // features past dim pass through
+            int f = dim + (i - half);
+            yo[f] = xi[f];
+            continue;
+        }
+        int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+        float a = xi[ia], b = xi[ib];
+        float c = cosv[(int64_t)(offset + q) * half + i], sn = sinv[(int64_t)(offset + q) * half + i];
+        float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;
+        yo[ia] = ac - bs;
+        yo[ib] = interleaved ? as + bc : bc + as;
+    }
+}
+
+hipError_t rope(const float* x, float* y, int64_t rows, int64_t s, int head_dim, int dim, int interleaved, int64_t x_row_stride,
+                int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride, const float* cosv, const float* sinv,
+                int64_t offset, hipStream_t st) {
+    int64_t total = rows * s * (dim / 2 + head_dim - dim);
+    if (total == 0) return hipSuccess;
+    int64_t groups = (total + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)groups), dim3(256), 0, st, x, y, rows, (int)s, head_dim, dim, interleaved,
+                       x_row_stride, x_pos_stride, y_row_stride, y_pos_stride, cosv, sinv, (int)offset);
+    return hipGetLastError();
+}
+
+// ---- KV cache write: nn/transformer.go:397-423 (Append) ---------------------------
+// src is [B, heads, S, dim] read with strides; it lands at positions
+// [pos, pos + S) of a cache [B, heads, cap, dim], cast to the cache's dtype
+// (float32 kept, binary16 rounded to nearest even).
+__global__ __launch_bounds__(256) void kv_write_kernel(const float* __restrict__ src, void* __restrict__ cache, int cache_dt,
+                                                       int64_t total, int heads, int s, int dim, int64_t cap, int64_t pos,
+                                                       int64_t src_b, int64_t src_h, int64_t src_p) {
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        int d = (int)(t % dim);
+        int64_t r = t / dim;
+        int q = (int)(r % s);
+        r /= s;
+        int h = (int)(r % heads);
+        int64_t b = r / heads;
+        float v = src[b * src_b + h * src_h + q * src_p + d];
+        int64_t at = ((b * heads + h) * cap + pos + q) * dim + d;
+        if (cache_dt == kF32)
+            ((float*)cache)[at] = v;
+        else
+            ((uint16_t*)cache)[at] = f32_to_f16_bits(v);
+    }
+}
+
+hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int heads, int64_t s, int dim, int64_t cap,
+                    int64_t pos, int64_t src_b, int64_t src_h, int64_t src_p, hipStream_t st) {
+    int64_t total = B * heads * s * dim;
+    if (total == 0) return hipSuccess;
+    int64_t groups = (total + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(kv_write_kernel, dim3((unsigned)groups), dim3(256), 0, st, src, cache, cache_dt, total, heads, (int)s, dim,
+                       cap, pos, src_b, src_h, src_p);
+    return hipGetLastError();
+}
+
+// ---- SwiGLU: llm/model.go:446-448; tensor/elementwise.go:520-525,583-585 ----------
+// out = (g * recip(1 + exp2(g * -log2e))) * u, each step a float32. Rows of g
+// and u are `stride` floats apart (they may be the halves of one fused
+// product); out is contiguous.
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                     float* __restrict__ out, int64_t rows, int64_t n, int64_t stride) {
+    const float nl2e = (float)(-1.4426950408889634);
+    int64_t total = rows * n;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = t / n, i = t % n;
+        float gv = g[r * stride + i];
+        float e = __builtin_exp2f(gv * nl2e);
+        float s = 1.0f / (1.0f + e);
+        float a = gv * s;
+        out[t] = a * u[r * stride + i];
+    }
+}
+
+hipError_t swiglu(const float* g, const float* u, float* out, int64_t rows, int64_t n, int64_t stride, hipStream_t st) {
+    if (rows * n == 0) return hipSuccess;
+    int64_t groups = (rows * n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)groups), dim3(256), 0, st, g, u, out, rows, n, stride);
+    return hipGetLastError();
+}
+
+// ---- residual add ------------------------------------------------------------
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+                                                  int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) out[i] = a[i] + b[i];
+}
+
+hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    int64_t groups = (n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)groups), dim3(256), 0, st, a, b, out, n);
+    return hipGetLastError();
+}
+
+// ---- greedy argmax: examples/llama/generate.go:44-53 -----------------------------
+// The first index of the largest value per row. The reference scans with
+// `v > logits[best]` from best = 0, so a NaN never wins, and a NaN at index 0
+// is never beaten.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int64_t n, int32_t* __restrict__ out) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const float* row = logits + (int64_t)blockIdx.x * n;
+    float best = -__builtin_inff();
+    int at = 0x7fffffff;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = row[i];
+        if (v > best || (v == best && (int)i < at)) {
+            best = v;
+            at = (int)i;
+        }
+    }
+    // over the wavefront, then over the wavefronts: larger value, then smaller index
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off);
+        int oi = __shfl_xor(at, off);
+        if (ov > best || (ov == best && oi < at)) {
+            best = ov;
+            at = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        bv[threadIdx.x >> 6] = best;
+        bi[threadIdx.x >> 6] = at;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < at)) {
+                best = bv[w];
+                at = bi[w];
+            }
+        float first = row[0];
+        if (first != first || at == 0x7fffffff) at = 0;  // NaN at 0, or nothing but NaNs
+        out[blockIdx.x] = at;
+    }
+}
+
+hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, hipStream_t st) {
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, n, out);
+    return hipGetLastError();
+}
+
+}  // namespace mimir

@@ -64,6 +64,39 @@ size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
 
+// ---- the other kernels of a decoding step ------------------------------------
+hipError_t rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, hipStream_t st);
+hipError_t rope(const float* x, float* y, int64_t rows, int64_t s, int head_dim, int dim, int interleaved, int64_t x_row_stride,
+                int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride, const float* cosv, const float* sinv,
+                int64_t offset, hipStream_t st);
+hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int heads, int64_t s, int dim, int64_t cap,
+                    int64_t pos, int64_t src_b, int64_t src_h, int64_t src_p, hipStream_t st);
+hipError_t swiglu(const float* g, const float* u, float* out, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
+hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st);
+hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, hipStream_t st);
+
+// Attention of queries [B, H, Q, D] over keys and values [B, HK, K, D], each
+// read through strides {batch, head, position} (features contiguous). chunk
+// and nsplit come from attention_plan; workspace holds
+// attention_workspace_bytes(...) bytes when nsplit > 1.
+struct AttnArgs {
+    const float* q;
+    const void *k, *v;
+    int kv_dtype;  // kF32 or kF16
+    float* out;
+    float* lse;    // [B, H, Q] contiguous, or null
+    int64_t q_strides[3], k_strides[3], v_strides[3], o_strides[3];
+    int64_t B, Q, K;
+    int H, HK, D;
+    double scale;
+    int causal;
+    int64_t causal_offset;
+    int chunk, nsplit;
+};
+void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, int* nsplit);
+size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit);
+hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
+
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);

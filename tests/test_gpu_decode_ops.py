@@ -1,0 +1,225 @@
+"""Parity of the decode-step kernels with the oracle and with the reference's
+golden attention.mim, through the C ABI, on a real MI355X.
+
+Tolerances: the reference's own for these ops, atol 1e-5 + rtol 1e-4
+(nn/transformer_test.go:139); RoPE, the KV write, SwiGLU's operations and
+argmax are compared bit for bit where the arithmetic order is fixed."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from mimir_amd import capi
+from mimir_amd.mimfile import golden_cases
+from tests import gpu
+from tests.helpers import bits_equal
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 1e-5, 1e-4
+
+
+def close(got, want, what=""):
+    assert got.shape == want.shape, (got.shape, want.shape)
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= ATOL + RTOL * np.abs(want)), f"{what}: worst {err.max():.3e}"
+
+
+@pytest.fixture(scope="module")
+def cases(golden_dir):
+    return golden_cases(os.path.join(golden_dir, "attention.mim"))
+
+
+def rmsnorm(x, w, eps):
+    l = gpu.lib()
+    xd = gpu.dev(x); y = torch.empty_like(xd)
+    wd = gpu.dev(w) if w is not None else None
+    d = x.shape[-1]
+    capi.check(l.mi355x_rmsnorm(xd.data_ptr(), wd.data_ptr() if wd is not None else None, y.data_ptr(), x.size // d, d, eps, gpu.stream()))
+    gpu.sync()
+    return y.cpu().numpy()
+
+
+def test_rmsnorm(cases):
+    gpu.say("rmsnorm golden + 8B shape")
+    c = cases["rms_norm"]
+    close(rmsnorm(c["in"][0].data, c["in"][1].data, 1e-6), c["out"].data)
+    c = cases["rms_norm_default_eps"]
+    close(rmsnorm(c["in"][0].data, c["in"][1].data, 2.0 ** -23), c["out"].data)
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=(8, 4096)).astype(np.float32) * 3; w = rng.normal(1, 0.02, 4096).astype(np.float32)
+    got = rmsnorm(x, w, 1e-5)
+    want = O.rmsnorm(x, w, 1e-5)
+    assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max()  # only the order of the sum of squares differs
+    assert np.abs(rmsnorm(x, None, 1e-5) - O.rmsnorm(x, None, 1e-5)).max() <= 2e-6 * 4
+
+
+def rope(x, cos, sin, dim, inter, offset, table_len=None):
+    """x [..., S, head_dim] contiguous."""
+    l = gpu.lib()
+    s, hd = x.shape[-2], x.shape[-1]
+    xd = gpu.dev(x); y = torch.empty_like(xd)
+    cd, sd = gpu.dev(cos), gpu.dev(sin)
+    capi.check(l.mi355x_rope(xd.data_ptr(), y.data_ptr(), x.size // (s * hd), s, hd, dim, int(inter), s * hd, hd, s * hd, hd,
+                             cd.data_ptr(), sd.data_ptr(), cos.shape[0], offset, gpu.stream()))
+    gpu.sync()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("name,dim,inter,off,scaling,params", [
+    ("rope_neox", 8, False, 3, O.ROPE_NONE, ()),
+    ("rope_interleaved", 8, True, 3, O.ROPE_NONE, ()),
+    ("rope_partial_scaled", 8, False, 2, O.ROPE_LLAMA3, (8, 1, 4, 64)),
+])
+def test_rope_golden(cases, name, dim, inter, off, scaling, params):
+    c = cases[name]
+    x = c["in"][0].data
+    n = off + x.shape[-2]
+    cos, sin = O.rope_angles(dim, 10000.0, 0, n, scaling, params)  # the whole table; the kernel reads rows off..
+    gpu.say(name)
+    got = rope(x, cos, sin, dim, inter, off)
+    close(got, c["out"].data)
+    assert bits_equal(got, O.rope_apply(x, cos[off:], sin[off:], dim, inter))
+
+
+def test_rope_decode_shape_bit_exact_and_strided():
+    """40 heads of 128 features at position 2048 of a table for theta 500000,
+    interleaved; and q read in place from a [S, heads * dim] product (position
+    stride heads * dim, head stride dim)."""
+    rng = np.random.default_rng(1)
+    cos, sin = O.rope_angles(128, 500000.0, 0, 2100)
+    x = rng.normal(size=(40, 1, 128)).astype(np.float32)
+    gpu.say("rope decode shape")
+    assert bits_equal(rope(x, cos, sin, 128, True, 2048), O.rope_apply(x, cos[2048:2049], sin[2048:2049], 128, True))
+    S, H, D = 5, 4, 128
+    tok_major = rng.normal(size=(S, H * D)).astype(np.float32)
+    l = gpu.lib()
+    xd = gpu.dev(tok_major); cd, sd = gpu.dev(cos), gpu.dev(sin)
+    capi.check(l.mi355x_rope(xd.data_ptr(), xd.data_ptr(), H, S, D, D, 1, D, H * D, D, H * D, cd.data_ptr(), sd.data_ptr(), 2100, 7, gpu.stream()))
+    gpu.sync()
+    heads_major = tok_major.reshape(S, H, D).transpose(1, 0, 2).copy()
+    want = O.rope_apply(heads_major, cos[7:12], sin[7:12], D, True).transpose(1, 0, 2).reshape(S, H * D)
+    assert bits_equal(xd.cpu().numpy(), want)
+    assert l.mi355x_rope(xd.data_ptr(), xd.data_ptr(), H, S, D, D, 1, D, H * D, D, H * D, cd.data_ptr(), sd.data_ptr(), 2100, 2098, gpu.stream()) == capi.ERR_SHAPE
+
+
+def test_kv_write_casts_like_the_reference():
+    rng = np.random.default_rng(2)
+    B, KVH, S, D, cap, pos = 2, 8, 3, 128, 64, 5
+    src = (rng.normal(size=(B, KVH, S, D)) * np.array([1e-6, 1, 300, 70000])[rng.integers(0, 4, (B, KVH, S, D))]).astype(np.float32)
+    l = gpu.lib()
+    sd = gpu.dev(src)
+    for dt, tdt in ((capi.F16, torch.int16), (capi.F32, torch.float32)):
+        cache = torch.zeros((B, KVH, cap, D), dtype=tdt, device="cuda:0")
+        gpu.say(f"kv_write dt={dt}")
+        capi.check(l.mi355x_kv_write(sd.data_ptr(), cache.data_ptr(), dt, B, KVH, S, D, cap, pos, KVH * S * D, S * D, D, gpu.stream()))
+        gpu.sync()
+        got = cache.cpu().numpy()
+        if dt == capi.F16:
+            got = got.view(np.uint16)
+            assert np.array_equal(got[:, :, pos:pos + S], O.f32_to_f16(src))  # round to nearest even, overflow to infinity
+        else:
+            assert bits_equal(got[:, :, pos:pos + S], src)
+        assert not got[:, :, :pos].any() and not got[:, :, pos + S:].any()
+    assert l.mi355x_kv_write(sd.data_ptr(), cache.data_ptr(), capi.F32, B, KVH, S, D, cap, cap - 2, KVH * S * D, S * D, D, gpu.stream()) == capi.ERR_SHAPE
+
+
+def attention(q, k, v, scale, causal=False, offset=0, kv_dt=capi.F32, k_len=None, want_lse=True):
+    """q [B,H,Q,D], k/v [B,HK,cap,D] contiguous numpy (uint16 bits for F16)."""
+    l = gpu.lib()
+    B, H, Q, D = q.shape
+    HK, cap = k.shape[1], k.shape[2]
+    K = cap if k_len is None else k_len
+    qd = gpu.dev(q)
+    kd = gpu.dev(k.view(np.int16) if kv_dt == capi.F16 else k); vd = gpu.dev(v.view(np.int16) if kv_dt == capi.F16 else v)
+    out = torch.full((B, H, Q, D), float("nan"), dtype=torch.float32, device="cuda:0")
+    lse = torch.full((B, H, Q), float("nan"), dtype=torch.float32, device="cuda:0")
+    arr = lambda *a: (C.c_int64 * 3)(*a)
+    capi.check(l.mi355x_attention(qd.data_ptr(), arr(H * Q * D, Q * D, D), kd.data_ptr(), vd.data_ptr(), kv_dt, arr(HK * cap * D, cap * D, D),
+                                  out.data_ptr(), arr(H * Q * D, Q * D, D), lse.data_ptr() if want_lse else None, B, H, HK, Q, K, D,
+                                  scale, int(causal), offset, gpu.stream()))
+    gpu.sync()
+    return out.cpu().numpy(), lse.cpu().numpy()
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("sdpa_causal", {"causal": True}),
+    ("sdpa_causal_offset", {"causal": True, "offset": 4}),
+    ("sdpa_gqa", {"causal": True, "offset": 2}),
+])
+def test_attention_golden(cases, name, kw):
+    c = cases[name]
+    q, k, v = (t.data for t in c["in"][:3])
+    gpu.say(name)
+    out, lse = attention(q, k, v, 1 / np.sqrt(q.shape[-1]), **kw)
+    close(out, c["out"].data, name)
+    wo, wl = O.attention(q, k, v, 1 / np.sqrt(q.shape[-1]), causal=kw.get("causal", False), causal_offset=kw.get("offset", 0))
+    close(lse, wl, name + " lse")
+
+
+@pytest.mark.parametrize("B,H,HK,D,cap,n", [(1, 32, 8, 128, 2304, 2049), (8, 32, 8, 128, 2304, 2049), (2, 8, 2, 64, 64, 37), (1, 4, 1, 64, 300, 300),
+                                            (1, 6, 1, 16, 40, 1), (3, 5, 5, 8, 33, 33)])
+def test_decode_attention_f16_cache(B, H, HK, D, cap, n):
+    """One query per head over a binary16 cache holding n of cap positions: the
+    decode step's shape (32 heads on 8 key heads of 128, 2049 keys) and small
+    and ragged ones, groups of 4, 6 and 1 query heads per key head."""
+    rng = np.random.default_rng(B * 1000 + n)
+    q = rng.normal(size=(B, H, 1, D)).astype(np.float32)
+    kh = O.f32_to_f16(rng.normal(size=(B, HK, cap, D)).astype(np.float32)); vh = O.f32_to_f16(rng.normal(size=(B, HK, cap, D)).astype(np.float32))
+    gpu.say(f"decode attention B={B} H={H} HK={HK} D={D} n={n}")
+    out, lse = attention(q, kh, vh, 1 / np.sqrt(D), kv_dt=capi.F16, k_len=n)
+    wo, wl = O.attention(q, kh, vh, 1 / np.sqrt(D), kv_dt=O.F16, k_len=n)
+    close(out, wo); close(lse, wl)
+    out2, _ = attention(q, kh, vh, 1 / np.sqrt(D), causal=True, offset=n - 1, kv_dt=capi.F16, want_lse=False)  # the same keys, hidden causally
+    assert bits_equal(out2, out)
+
+
+def test_prompt_attention_f32_cache_and_empty_rows():
+    rng = np.random.default_rng(5)
+    B, H, HK, Q, D = 1, 8, 2, 17, 64
+    q = rng.normal(size=(B, H, Q, D)).astype(np.float32); k = rng.normal(size=(B, HK, Q + 3, D)).astype(np.float32); v = rng.normal(size=(B, HK, Q + 3, D)).astype(np.float32)
+    gpu.say("prompt attention causal offset 3, then offset -2")
+    out, lse = attention(q, k, v, 0.3, causal=True, offset=3)
+    wo, wl = O.attention(q, k, v, 0.3, causal=True, causal_offset=3)
+    close(out, wo); close(lse, wl)
+    out, lse = attention(q, k, v, 0.3, causal=True, offset=-2)  # rows 0 and 1 see no key
+    wo, wl = O.attention(q, k, v, 0.3, causal=True, causal_offset=-2)
+    assert not out[:, :, :2].any() and np.all(lse[:, :, :2] == -np.inf)
+    close(out, wo); close(lse[:, :, 2:], wl[:, :, 2:])
+
+
+def test_swiglu_add_argmax():
+    l = gpu.lib()
+    rng = np.random.default_rng(6)
+    n = 14336
+    g = (rng.normal(size=(2, n)) * 4).astype(np.float32); u = rng.normal(size=(2, n)).astype(np.float32)
+    g[0, :5] = [-200, 200, 0, -88.5, 1e-30]
+    gd, ud = gpu.dev(g), gpu.dev(u)
+    out = torch.empty((2, n), dtype=torch.float32, device="cuda:0")
+    gpu.say("swiglu")
+    capi.check(l.mi355x_swiglu(gd.data_ptr(), ud.data_ptr(), out.data_ptr(), 2, n, n, gpu.stream())); gpu.sync()
+    want = O.silu_mul(g, u)
+    got = out.cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()  # exp2 differs in the last bits between libraries
+    assert got[0, 0] == 0
+    # halves of one fused [2, 2n] product
+    both = np.concatenate([g, u], axis=1)
+    bd = gpu.dev(both)
+    capi.check(l.mi355x_swiglu(bd.data_ptr(), bd.data_ptr() + 4 * n, out.data_ptr(), 2, n, 2 * n, gpu.stream())); gpu.sync()
+    assert bits_equal(out.cpu().numpy(), got)
+    gpu.say("add")
+    capi.check(l.mi355x_add(gd.data_ptr(), ud.data_ptr(), out.data_ptr(), 2 * n, gpu.stream())); gpu.sync()
+    assert bits_equal(out.cpu().numpy(), g + u)
+    gpu.say("argmax")
+    logits = rng.normal(size=(4, 128256)).astype(np.float32)
+    logits[1, 777] = logits[1, 90000] = 50.0          # a tie: the first index wins
+    logits[2, 0] = np.nan                              # NaN at 0 is never beaten
+    logits[3, 5] = np.nan; logits[3, 100000] = 60.0    # a NaN elsewhere never wins
+    ld = gpu.dev(logits); idx = torch.full((4,), -1, dtype=torch.int32, device="cuda:0")
+    capi.check(l.mi355x_argmax(ld.data_ptr(), 4, 128256, idx.data_ptr(), gpu.stream())); gpu.sync()
+    assert idx.cpu().tolist() == [O.argmax(r) for r in logits] == [int(np.argmax(logits[0])), 777, 0, 100000]
+    tiny = gpu.dev(np.array([[-np.inf, -np.inf], [np.nan, np.nan]], np.float32))
+    capi.check(l.mi355x_argmax(tiny.data_ptr(), 2, 2, idx.data_ptr(), gpu.stream())); gpu.sync()
+    assert idx.cpu().tolist()[:2] == [0, 0]
