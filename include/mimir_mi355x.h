@@ -96,7 +96,7 @@ MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, 
  * scratch buffer of its own.
  *   Q8_0: quantizeRow's int8 blocks (backend/cpu/qmatmul.go:208-254).
  *   Q4_K, Q6_K: quantizeRow's int8 super-blocks of 256 with their sums.
- *   Q4_0: 20-bit fixed point per block of 32 (K a multiple of 64, W dword
+ *   Q4_0: 24-bit fixed point per block of 32 (K a multiple of 64, W dword
  *         aligned); no counterpart in the reference, whose kernels take
  *         float32 activations only. */
 MI355X_API size_t mi355x_act_bytes(int dtype, int64_t K);
@@ -152,6 +152,46 @@ MI355X_API mi355x_status mi355x_add(const float* a, const float* b, float* out, 
 /* Sampler.Sample at temperature 0 (examples/llama/generate.go:44-53): the first
  * index of each row's largest value, into device memory. */
 MI355X_API mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, void* stream);
+
+/* ---- the decoder: llm.Model, its caches and the greedy loop ------------------
+ * (llm/model.go:216-455; nn/transformer.go:348-423;
+ * examples/llama/generate.go:44-53,162-202). Weights keep their block dtypes on
+ * the device, a step is queued without host synchronisation, and the next
+ * token is chosen on the device. batch sequences are decoded in lockstep (the
+ * reference's llm fixes batch 1). */
+typedef struct mi355x_llama_config {
+    int32_t embed, hidden, layers, heads, kv_heads, head_dim, rope_dim, vocab;
+    int32_t context;      /* capacity of the KV caches, in positions */
+    int32_t interleaved;  /* rotate pairs (2i, 2i+1): arch "llama"; else halves: "qwen2" (llm/model.go:321) */
+    int32_t cache_dtype;  /* MI355X_F32 or MI355X_F16 */
+    int32_t batch;
+    double rope_base, rope_scale, eps;
+} mi355x_llama_config;
+
+MI355X_API mi355x_status mi355x_llama_create(const mi355x_llama_config* cfg, void** model);
+MI355X_API mi355x_status mi355x_llama_destroy(void* model);
+/* Uploads one tensor from host bytes in its file layout (ggml blocks for the
+ * quantized dtypes). Names are llama.cpp's, as llm.Load reads them
+ * (llm/model.go:268-310): token_embd.weight, output_norm.weight, output.weight
+ * (absent: tied to the embeddings), blk.N.{attn_norm,attn_q,attn_k,attn_v,
+ * attn_output,ffn_norm,ffn_gate,ffn_up,ffn_down}.weight. */
+MI355X_API mi355x_status mi355x_llama_set_tensor(void* model, const char* name, int dtype, const void* host_data, int64_t n_elems);
+/* rope_freqs.weight: divisors of each pair's frequency (llm/model.go:318-346). */
+MI355X_API mi355x_status mi355x_llama_set_rope_factors(void* model, const float* factors, int32_t n);
+/* Checks the tensors, builds the rotary table, allocates the caches (zeroed)
+ * and the activations of calls of up to max_tokens tokens per sequence. */
+MI355X_API mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens);
+/* Empties the caches (KVCache.Reset). */
+MI355X_API mi355x_status mi355x_llama_reset(void* model);
+MI355X_API int64_t mi355x_llama_cache_len(void* model);
+/* Model.Logits: runs tokens [batch, n], which follow the positions the caches
+ * hold, appends their keys and values, and copies to the host the logits of the
+ * last token [batch, vocab], or of every token [batch, n, vocab] if all. */
+MI355X_API mi355x_status mi355x_llama_logits(void* model, const int32_t* tokens, int64_t n, int all, float* logits_host);
+/* Greedy generation: prompt [batch, n_prompt], then n_new tokens a sequence into
+ * out_tokens [batch, n_new]. seconds, if not NULL, gets the device time of the
+ * prompt pass (with the first token) and of the n_new - 1 decoding steps. */
+MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t n_prompt, int64_t n_new, int32_t* out_tokens, double* seconds);
 
 /* ---- measurement aids (no counterpart in the reference) ---------------------
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of

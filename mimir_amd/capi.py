@@ -44,9 +44,24 @@ SYMBOLS = {
     "mi355x_swiglu": (C.c_uint32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_add": (C.c_uint32, [_vp, _vp, _vp, _i64, _vp]),
     "mi355x_argmax": (C.c_uint32, [_vp, _i64, _i64, _vp, _vp]),
+    "mi355x_llama_create": (C.c_uint32, [_vp, C.POINTER(_vp)]),
+    "mi355x_llama_destroy": (C.c_uint32, [_vp]),
+    "mi355x_llama_set_tensor": (C.c_uint32, [_vp, C.c_char_p, _int, _vp, _i64]),
+    "mi355x_llama_set_rope_factors": (C.c_uint32, [_vp, _vp, C.c_int32]),
+    "mi355x_llama_finalize": (C.c_uint32, [_vp, _i64]),
+    "mi355x_llama_reset": (C.c_uint32, [_vp]),
+    "mi355x_llama_cache_len": (_i64, [_vp]),
+    "mi355x_llama_logits": (C.c_uint32, [_vp, _vp, _i64, _int, _vp]),
+    "mi355x_llama_generate": (C.c_uint32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "mi355x_tune": (C.c_uint32, [C.c_char_p, _int]),
     "mi355x_stream_read": (C.c_uint32, [_vp, _sz, _vp, _int, _int, _vp]),
 }
+
+
+class LlamaConfig(C.Structure):
+    """mi355x_llama_config."""
+    _fields_ = [(n, C.c_int32) for n in ("embed", "hidden", "layers", "heads", "kv_heads", "head_dim", "rope_dim", "vocab", "context",
+                                          "interleaved", "cache_dtype", "batch")] + [(n, C.c_double) for n in ("rope_base", "rope_scale", "eps")]
 
 
 class Mi355xError(RuntimeError):

@@ -113,6 +113,23 @@ mi355x_status attn_scratch(size_t bytes, void** out) {
 
 }  // namespace
 
+// For the other host files of the library.
+namespace mimir {
+mi355x_status capi_fail(mi355x_status code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+uint32_t* device_error_word() {
+    DeviceState* s;
+    return current_state(&s) == MI355X_OK ? s->err_dev : nullptr;
+}
+}  // namespace mimir
+
 extern "C" {
 
 mi355x_status mi355x_init(int device) {
@@ -271,7 +288,7 @@ mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float*
     mimir::QGemvArgs a{W, nullptr, act, y, M, N, K, 0, 0};
     if (dtype == MI355X_Q4_0) {
         if (!mimir::q4_0_fixed_point_ok(W, K))
-            return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by q4_0 needs K a multiple of 64 up to 24448 and W dword aligned (K = %lld)", (long long)K);
+            return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act by q4_0 needs K a multiple of 64 up to 20928 and W dword aligned (K = %lld)", (long long)K);
         HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
     } else if (dtype == MI355X_Q8_0) {
         if (K % 32 != 0 || !mimir::q8_act_fits(K))

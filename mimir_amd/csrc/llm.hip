@@ -1,0 +1,500 @@
+// Host-side decoder of the llama architecture over the kernels of this
+// library: the counterpart of the reference's llm.Model (llm/model.go:216-455:
+// Load, NewCaches, Logits, project, mlp), nn.KVCache (nn/transformer.go:348-423)
+// and the greedy loop of examples/llama (generate.go:44-53,162-202), with the
+// same error behaviour (shape and index errors before anything is queued).
+//
+// Differences that are the point of this build: weights stay in their block
+// dtypes on the device, Q4_0 included (the reference decodes Q4_0 to float32
+// when the model opens); a step is queued as a fixed run of launches with no
+// host synchronisation in between (the reference's GPU path realizes and
+// syncs twice per block, llm/model.go:409-427); the next token is chosen on
+// the device and fed to the next step's embedding lookup from device memory,
+// so generation downloads nothing until it ends; several sequences may be
+// decoded in lockstep (llm fixes batch 1, llm/model.go:378-385,408).
+#include "../../include/mimir_mi355x.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+
+namespace mimir {
+
+mi355x_status capi_fail(mi355x_status code, const char* fmt, ...);  // capi.hip
+
+namespace {
+
+#define LLM_HIP(expr, what)                                                          \
+    do {                                                                             \
+        hipError_t e_ = (expr);                                                      \
+        if (e_ != hipSuccess) return capi_fail((mi355x_status)e_, "mi355x: llama: %s: %s", what, hipGetErrorName(e_)); \
+    } while (0)
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t alloc(size_t n) {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        bytes = n;
+        return hipMalloc(&p, n < 4 ? 4 : n);
+    }
+    template <typename T>
+    T* as() const { return (T*)p; }
+};
+
+struct Weight {
+    int dtype = 0;
+    int64_t n = 0, k = 0;
+    DevBuf buf;
+    bool set() const { return buf.p != nullptr; }
+};
+
+// The form of converted activations a weight's product reads.
+enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3 };
+
+struct Block {
+    Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down;
+};
+
+struct Model {
+    mi355x_llama_config c{};
+    Weight embed, norm, output;
+    bool tied = false;
+    std::vector<Block> blocks;
+    std::vector<float> rope_factors;
+    bool ready = false;
+
+    DevBuf cos_t, sin_t;                 // [context, rope_dim/2]
+    std::vector<DevBuf> keys, values;    // per block: [batch, kv_heads, context, head_dim]
+    int64_t cache_len = 0;
+
+    // activations of up to max_rows rows (batch x tokens of one call)
+    int64_t max_rows = 0;
+    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[4], tokens_dev, next_tok;
+    hipStream_t stream = nullptr;
+};
+
+int act_class(const Weight& w) {
+    switch (w.dtype) {
+    case kQ4_0: return q4_0_fixed_point_ok(w.buf.p, w.k) ? kActQ4 : kActNone;
+    case kQ8_0: return q8_act_fits(w.k) ? kActQ8 : kActNone;
+    case kQ4_K: case kQ6_K: return kActKQ;
+    default: return kActNone;
+    }
+}
+
+size_t act_row_bytes(int cls, int64_t K) {
+    switch (cls) {
+    case kActQ4: return q4_0_act_bytes(K);
+    case kActQ8: return q8_act_bytes(K);
+    case kActKQ: return kq_act_bytes(K);
+    default: return 0;
+    }
+}
+
+const int kNoTune[5] = {0, 0, 0, 0, 0};
+
+// Converts rows of x once for every activation form that `ws` need.
+mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[4]) {
+    for (int i = 0; i < 4; i++) done[i] = false;
+    for (const Weight* w : ws) {
+        int cls = act_class(*w);
+        if (cls == kActNone || done[cls]) continue;
+        size_t need = act_row_bytes(cls, K) * (size_t)rows;
+        if (m.act[cls].bytes < need) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: activation scratch of %zu bytes, need %zu", m.act[cls].bytes, need);
+        hipError_t e = cls == kActQ4   ? q4_0_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
+                       : cls == kActQ8 ? q8_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
+                                       : kq_convert_act(x, rows, K, K, m.act[cls].p, m.stream);
+        LLM_HIP(e, "convert activations");
+        done[cls] = true;
+    }
+    return MI355X_OK;
+}
+
+// y[rows, n] = x[rows, k] . W^T (nn/layers.go:49-55 -> tensor/quant.go:35-56).
+mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows) {
+    int cls = act_class(w);
+    QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
+    hipError_t e;
+    switch (w.dtype) {
+    case kQ4_0: e = cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream) : qgemv_q4_0(a, kNoTune, m.stream); break;
+    case kQ8_0:
+        if (cls != kActQ8) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: q8_0 rows of %lld are too long", (long long)w.k);
+        e = qgemv_q8_0_act(a, kNoTune, m.stream);
+        break;
+    case kQ4_K: case kQ6_K: e = qgemv_kquant_act(w.dtype, a, m.stream); break;
+    case kF32: case kF16: case kBF16: e = gemv_float(w.dtype, w.buf.p, x, y, rows, w.n, w.k, w.k, m.stream); break;
+    default: return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: a linear weight of dtype %d", w.dtype);
+    }
+    LLM_HIP(e, "linear");
+    return MI355X_OK;
+}
+
+mi355x_status embed_rows(Model& m, const int32_t* idx_dev, int64_t rows, float* out, uint32_t* err) {
+    const Weight& w = m.embed;
+    if (is_quantized(w.dtype)) {
+        LLM_HIP(gather_rows(w.dtype, w.buf.p, w.n, w.k, idx_dev, rows, out, err, m.stream), "embedding");
+        return MI355X_OK;
+    }
+    return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: token_embd.weight of dtype %d (block-quantized tables only)", w.dtype);
+}
+
+}  // namespace
+
+uint32_t* device_error_word();  // capi.hip
+
+// One pass of s tokens per sequence over the blocks (llm/model.go:391-437),
+// tokens already on the device at m.tokens_dev [batch, s]. Leaves the final
+// hidden state in m.x; advances the caches.
+static mi355x_status forward(Model& m, int64_t s) {
+    const auto& c = m.c;
+    const int64_t B = c.batch, rows = B * s, past = m.cache_len;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
+    float *x = m.x.as<float>(), *h = m.h.as<float>(), *q = m.q.as<float>(), *k = m.k.as<float>(), *v = m.v.as<float>();
+    float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
+    bool done[4];
+    if (mi355x_status st = embed_rows(m, m.tokens_dev.as<int32_t>(), rows, x, device_error_word())) return st;
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m.blocks[i];
+        LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, rows, c.embed, c.eps, m.stream), "attn_norm");
+        if (mi355x_status st = convert_for(m, h, rows, c.embed, {&b.q, &b.k, &b.v}, done)) return st;
+        if (mi355x_status st = linear(m, b.q, h, q, rows)) return st;
+        if (mi355x_status st = linear(m, b.k, h, k, rows)) return st;
+        if (mi355x_status st = linear(m, b.v, h, v, rows)) return st;
+        // q and k are [B, s, heads, dim]. One position: every head of every
+        // sequence is a row `dim` apart. More: per sequence, heads are rows
+        // `dim` apart and positions heads * dim apart.
+        if (s == 1) {
+            LLM_HIP(rope(q, q, B * c.heads, 1, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, qd, c.head_dim, qd,
+                         m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope q");
+            LLM_HIP(rope(k, k, B * c.kv_heads, 1, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, kvd, c.head_dim, kvd,
+                         m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope k");
+        } else {
+            for (int64_t bb = 0; bb < B; bb++) {
+                LLM_HIP(rope(q + bb * s * qd, q + bb * s * qd, c.heads, s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, qd,
+                             c.head_dim, qd, m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope q");
+                LLM_HIP(rope(k + bb * s * kvd, k + bb * s * kvd, c.kv_heads, s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim,
+                             kvd, c.head_dim, kvd, m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope k");
+            }
+        }
+        LLM_HIP(kv_write(k, m.keys[i].p, c.cache_dtype, B, c.kv_heads, s, c.head_dim, c.context, past, s * kvd, c.head_dim, kvd, m.stream), "cache keys");
+        LLM_HIP(kv_write(v, m.values[i].p, c.cache_dtype, B, c.kv_heads, s, c.head_dim, c.context, past, s * kvd, c.head_dim, kvd, m.stream), "cache values");
+        AttnArgs at;
+        at.q = q; at.k = m.keys[i].p; at.v = m.values[i].p; at.kv_dtype = c.cache_dtype; at.out = a; at.lse = nullptr;
+        at.q_strides[0] = s * qd; at.q_strides[1] = c.head_dim; at.q_strides[2] = qd;
+        at.k_strides[0] = at.v_strides[0] = (int64_t)c.kv_heads * c.context * c.head_dim;
+        at.k_strides[1] = at.v_strides[1] = (int64_t)c.context * c.head_dim;
+        at.k_strides[2] = at.v_strides[2] = c.head_dim;
+        for (int j = 0; j < 3; j++) at.o_strides[j] = at.q_strides[j];
+        at.B = B; at.Q = s; at.K = past + s; at.H = c.heads; at.HK = c.kv_heads; at.D = c.head_dim;
+        at.scale = 1.0 / std::sqrt((double)c.head_dim);
+        at.causal = 1; at.causal_offset = past;
+        attention_plan(B, c.heads, c.kv_heads, s, at.K, &at.chunk, &at.nsplit);
+        size_t need = attention_workspace_bytes(B, c.heads, s, c.head_dim, at.nsplit);
+        if (need > m.act[0].bytes) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: attention scratch of %zu bytes, need %zu", m.act[0].bytes, need);
+        LLM_HIP(attention(at, m.act[0].p, m.stream), "attention");
+        if (mi355x_status st = convert_for(m, a, rows, qd, {&b.o}, done)) return st;
+        if (mi355x_status st = linear(m, b.o, a, o, rows)) return st;
+        LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
+        LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, rows, c.embed, c.eps, m.stream), "ffn_norm");
+        if (mi355x_status st = convert_for(m, h, rows, c.embed, {&b.gate, &b.up}, done)) return st;
+        if (mi355x_status st = linear(m, b.gate, h, gate, rows)) return st;
+        if (mi355x_status st = linear(m, b.up, h, up, rows)) return st;
+        LLM_HIP(swiglu(gate, up, sw, rows, c.hidden, c.hidden, m.stream), "swiglu");
+        if (mi355x_status st = convert_for(m, sw, rows, c.hidden, {&b.down}, done)) return st;
+        if (mi355x_status st = linear(m, b.down, sw, o, rows)) return st;
+        LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
+    }
+    m.cache_len = past + s;
+    return MI355X_OK;
+}
+
+// Norm and output projection of `rows` rows of hidden states at xin, which are
+// row_stride floats apart, into m.logits [rows, vocab].
+static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_stride) {
+    const auto& c = m.c;
+    float* hl = m.hlast.as<float>();
+    if (row_stride == c.embed) {
+        LLM_HIP(rmsnorm(xin, m.norm.buf.as<float>(), hl, rows, c.embed, c.eps, m.stream), "output_norm");
+    } else {
+        for (int64_t r = 0; r < rows; r++)
+            LLM_HIP(rmsnorm(xin + r * row_stride, m.norm.buf.as<float>(), hl + r * c.embed, 1, c.embed, c.eps, m.stream), "output_norm");
+    }
+    const Weight& w = m.tied ? m.embed : m.output;
+    bool done[4];
+    if (mi355x_status st = convert_for(m, hl, rows, c.embed, {&w}, done)) return st;
+    return linear(m, w, hl, m.logits.as<float>(), rows);
+}
+
+}  // namespace mimir
+
+using mimir::Model;
+
+extern "C" {
+
+mi355x_status mi355x_llama_create(const mi355x_llama_config* cfg, void** out) {
+    using namespace mimir;
+    if (!cfg || !out) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_create: null pointer");
+    const auto& c = *cfg;
+    // readConfig's checks (llm/model.go:97-171)
+    if (c.embed <= 0 || c.hidden <= 0 || c.layers <= 0 || c.layers > 1024 || c.heads <= 0 || c.kv_heads <= 0 || c.heads % c.kv_heads != 0 ||
+        c.head_dim <= 0 || c.head_dim > 256 || c.rope_dim <= 0 || c.rope_dim > c.head_dim || c.rope_dim % 2 != 0 || c.vocab <= 0 || c.context <= 0 ||
+        c.batch <= 0 || !(c.rope_base > 1) || !(c.rope_scale > 0) || !(c.eps > 0))
+        return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: model hyperparameters: %d layers, %d heads and %d key heads of %d features, %d rotated",
+                         c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim);
+    if (c.cache_dtype != MI355X_F32 && c.cache_dtype != MI355X_F16) return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: KV cache of dtype %d", c.cache_dtype);
+    auto m = std::make_unique<Model>();
+    m->c = c;
+    m->blocks.resize(c.layers);
+    *out = m.release();
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_llama_destroy(void* model) {
+    delete (Model*)model;
+    return MI355X_OK;
+}
+
+// Names are llama.cpp's, as the reference reads them (llm/model.go:268-310).
+mi355x_status mi355x_llama_set_tensor(void* model, const char* name, int dtype, const void* host, int64_t n_elems) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || !name || !host) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_set_tensor: null pointer");
+    const auto& c = m->c;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
+    Weight* w = nullptr;
+    int64_t n = 0, k = 0;
+    std::string s(name);
+    if (s == "token_embd.weight") { w = &m->embed; n = c.vocab; k = c.embed; }
+    else if (s == "output_norm.weight") { w = &m->norm; n = 1; k = c.embed; }
+    else if (s == "output.weight") { w = &m->output; n = c.vocab; k = c.embed; }
+    else if (s.rfind("blk.", 0) == 0) {
+        size_t dot = s.find('.', 4);
+        int i = atoi(s.substr(4, dot - 4).c_str());
+        if (dot == std::string::npos || i < 0 || i >= c.layers) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: tensor %s of a model of %d blocks", name, c.layers);
+        std::string leaf = s.substr(dot + 1);
+        Block& b = m->blocks[i];
+        if (leaf == "attn_norm.weight") { w = &b.attn_norm; n = 1; k = c.embed; }
+        else if (leaf == "ffn_norm.weight") { w = &b.ffn_norm; n = 1; k = c.embed; }
+        else if (leaf == "attn_q.weight") { w = &b.q; n = qd; k = c.embed; }
+        else if (leaf == "attn_k.weight") { w = &b.k; n = kvd; k = c.embed; }
+        else if (leaf == "attn_v.weight") { w = &b.v; n = kvd; k = c.embed; }
+        else if (leaf == "attn_output.weight") { w = &b.o; n = c.embed; k = qd; }
+        else if (leaf == "ffn_gate.weight") { w = &b.gate; n = c.hidden; k = c.embed; }
+        else if (leaf == "ffn_up.weight") { w = &b.up; n = c.hidden; k = c.embed; }
+        else if (leaf == "ffn_down.weight") { w = &b.down; n = c.embed; k = c.hidden; }
+    }
+    if (!w) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: unknown tensor %s", name);
+    if (n * k != n_elems) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %s of %lld elements, want [%lld, %lld]", name, (long long)n_elems, (long long)n, (long long)k);
+    int bs = block_size(dtype), bb = block_bytes(dtype);
+    if (bb == 0 || k % bs != 0) return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: %s of dtype %d", name, dtype);
+    if ((w == &m->norm || s.find("_norm.weight") != std::string::npos) && dtype != kF32)
+        return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: %s of dtype %d, want float32", name, dtype);
+    size_t bytes = (size_t)(n_elems / bs) * bb;
+    LLM_HIP(w->buf.alloc(bytes), "hipMalloc(weight)");
+    LLM_HIP(hipMemcpy(w->buf.p, host, bytes, hipMemcpyHostToDevice), "hipMemcpy(weight)");
+    w->dtype = dtype; w->n = n; w->k = k;
+    m->ready = false;
+    return MI355X_OK;
+}
+
+// Divisors of each pair's frequency (rope_freqs.weight, llm/model.go:318-346).
+mi355x_status mi355x_llama_set_rope_factors(void* model, const float* factors, int32_t n) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || (n > 0 && !factors)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_set_rope_factors: null pointer");
+    if (n != 0 && n != m->c.rope_dim / 2) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %d rope frequency factors, want %d", n, m->c.rope_dim / 2);
+    for (int i = 0; i < n; i++)
+        if (!(factors[i] > 0) || std::isinf(factors[i])) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: rope frequency factor %g", factors[i]);
+    m->rope_factors.assign(factors, factors + n);
+    m->ready = false;
+    return MI355X_OK;
+}
+
+// Checks that every tensor is there, builds the rotary table and allocates
+// the caches and the activations of calls of up to max_tokens tokens per
+// sequence.
+mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || max_tokens <= 0) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_finalize: bad arguments");
+    const auto& c = m->c;
+    if (!m->embed.set() || !m->norm.set()) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: token_embd.weight or output_norm.weight missing");
+    m->tied = !m->output.set();  // llm/model.go:283-288
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m->blocks[i];
+        for (const Weight* w : {&b.attn_norm, &b.ffn_norm, &b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down})
+            if (!w->set()) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: block %d is missing a tensor", i);
+    }
+    // nn/transformer.go:146-164 with llm/model.go:332-346: float64 angles, rounded to float32
+    const int half = c.rope_dim / 2;
+    std::vector<float> cosv((size_t)c.context * half), sinv((size_t)c.context * half);
+    std::vector<double> inv(half);
+    for (int i = 0; i < half; i++) {
+        double f = std::pow(c.rope_base, -(double)(2 * i) / (double)c.rope_dim);
+        f = f / c.rope_scale;
+        if (!m->rope_factors.empty()) f /= (double)m->rope_factors[i];
+        inv[i] = f;
+    }
+    for (int64_t p = 0; p < c.context; p++)
+        for (int i = 0; i < half; i++) {
+            double ang = (double)p * inv[i];
+            cosv[p * half + i] = (float)std::cos(ang);
+            sinv[p * half + i] = (float)std::sin(ang);
+        }
+    LLM_HIP(m->cos_t.alloc(cosv.size() * 4), "hipMalloc(rope table)");
+    LLM_HIP(m->sin_t.alloc(sinv.size() * 4), "hipMalloc(rope table)");
+    LLM_HIP(hipMemcpy(m->cos_t.p, cosv.data(), cosv.size() * 4, hipMemcpyHostToDevice), "hipMemcpy(rope table)");
+    LLM_HIP(hipMemcpy(m->sin_t.p, sinv.data(), sinv.size() * 4, hipMemcpyHostToDevice), "hipMemcpy(rope table)");
+
+    const size_t esz = c.cache_dtype == kF32 ? 4 : 2;
+    const size_t cache_bytes = (size_t)c.batch * c.kv_heads * c.context * c.head_dim * esz;
+    m->keys.clear(); m->values.clear();
+    m->keys.resize(c.layers); m->values.resize(c.layers);
+    for (int i = 0; i < c.layers; i++) {
+        LLM_HIP(m->keys[i].alloc(cache_bytes), "hipMalloc(KV cache)");
+        LLM_HIP(m->values[i].alloc(cache_bytes), "hipMalloc(KV cache)");
+        LLM_HIP(hipMemset(m->keys[i].p, 0, cache_bytes), "hipMemset(KV cache)");    // NewKVCache starts from zeros
+        LLM_HIP(hipMemset(m->values[i].p, 0, cache_bytes), "hipMemset(KV cache)");
+    }
+    m->cache_len = 0;
+    const int64_t rows = (int64_t)c.batch * max_tokens;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
+    m->max_rows = rows;
+    LLM_HIP(m->x.alloc(rows * c.embed * 4), "hipMalloc"); LLM_HIP(m->h.alloc(rows * c.embed * 4), "hipMalloc");
+    LLM_HIP(m->q.alloc(rows * qd * 4), "hipMalloc"); LLM_HIP(m->k.alloc(rows * kvd * 4), "hipMalloc"); LLM_HIP(m->v.alloc(rows * kvd * 4), "hipMalloc");
+    LLM_HIP(m->a.alloc(rows * qd * 4), "hipMalloc"); LLM_HIP(m->o.alloc(rows * c.embed * 4), "hipMalloc");
+    LLM_HIP(m->gate.alloc(rows * c.hidden * 4), "hipMalloc"); LLM_HIP(m->up.alloc(rows * c.hidden * 4), "hipMalloc"); LLM_HIP(m->s.alloc(rows * c.hidden * 4), "hipMalloc");
+    LLM_HIP(m->hlast.alloc(rows * c.embed * 4), "hipMalloc");
+    LLM_HIP(m->logits.alloc((size_t)rows * c.vocab * 4), "hipMalloc(logits)");
+    LLM_HIP(m->tokens_dev.alloc(rows * 4), "hipMalloc"); LLM_HIP(m->next_tok.alloc(c.batch * 4), "hipMalloc");
+    const int64_t kmax = c.hidden > qd ? (c.hidden > c.embed ? c.hidden : c.embed) : (qd > c.embed ? qd : c.embed);
+    for (int cls = 1; cls < 4; cls++) {
+        int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : (kmax + 63) / 64 * 64;
+        LLM_HIP(m->act[cls].alloc(act_row_bytes(cls, kk) * rows + 64), "hipMalloc(activations)");
+    }
+    int chunk, nsplit;
+    attention_plan(c.batch, c.heads, c.kv_heads, max_tokens, c.context, &chunk, &nsplit);
+    size_t attn_ws = 0;  // the most splits come from the smallest chunk
+    for (int cc = 32; cc <= 256; cc <<= 1) {
+        size_t b = attention_workspace_bytes(c.batch, c.heads, max_tokens, c.head_dim, (int)((c.context + cc - 1) / cc));
+        attn_ws = b > attn_ws ? b : attn_ws;
+    }
+    LLM_HIP(m->act[0].alloc(attn_ws + 64), "hipMalloc(attention scratch)");
+    m->ready = true;
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_llama_reset(void* model) {
+    Model* m = (Model*)model;
+    if (!m) return mimir::capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_reset: null pointer");
+    m->cache_len = 0;  // KVCache.Reset (nn/transformer.go:377)
+    return MI355X_OK;
+}
+
+int64_t mi355x_llama_cache_len(void* model) { return model ? ((Model*)model)->cache_len : -1; }
+
+static mi355x_status check_tokens(Model* m, const int32_t* tokens, int64_t n) {
+    using namespace mimir;
+    const auto& c = m->c;
+    if (!m->ready) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: model is not finalized");
+    // llm/model.go:393-400
+    if (n <= 0 || (int64_t)c.batch * n > m->max_rows) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %lld tokens a sequence, at most %lld a call", (long long)n, (long long)(m->max_rows / c.batch));
+    if (m->cache_len + n > c.context)
+        return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: append %lld positions to a cache holding %lld of %d", (long long)n, (long long)m->cache_len, c.context);
+    for (int64_t i = 0; i < (int64_t)c.batch * n; i++)
+        if (tokens[i] < 0 || tokens[i] >= c.vocab) return capi_fail(MI355X_ERR_INDEX, "mi355x: llama: token %d of a vocabulary of %d", tokens[i], c.vocab);
+    return MI355X_OK;
+}
+
+// Model.Logits (llm/model.go:391-437): runs tokens [batch, n], which follow the
+// positions the caches hold, and copies to the host the logits of the last
+// token, [batch, vocab], or of every token, [batch, n, vocab], if all is set.
+mi355x_status mi355x_llama_logits(void* model, const int32_t* tokens, int64_t n, int all, float* logits_host) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || !tokens || !logits_host) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_logits: null pointer");
+    if (mi355x_status st = check_tokens(m, tokens, n)) return st;
+    const auto& c = m->c;
+    const int64_t rows = (int64_t)c.batch * n;
+    LLM_HIP(hipMemcpyAsync(m->tokens_dev.p, tokens, rows * 4, hipMemcpyHostToDevice, m->stream), "upload tokens");
+    if (mi355x_status st = forward(*m, n)) return st;
+    int64_t out_rows = all ? rows : c.batch;
+    if (mi355x_status st = all ? head(*m, m->x.as<float>(), rows, c.embed) : head(*m, m->x.as<float>() + (n - 1) * c.embed, c.batch, n * c.embed)) return st;
+    LLM_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)out_rows * c.vocab * 4, hipMemcpyDeviceToHost, m->stream), "download logits");
+    return mi355x_sync(m->stream);
+}
+
+// Greedy generation (examples/llama/generate.go:162-202 with Sample at :44-53):
+// the prompt [batch, n_prompt], then n_new steps. Each step's token is chosen on
+// the device and read by the next step's embedding lookup from device memory;
+// out_tokens [batch, n_new] comes back once at the end. seconds, if not NULL,
+// gets the wall time of the prompt pass and of the n_new - 1 decoding steps.
+mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t n_prompt, int64_t n_new, int32_t* out_tokens, double* seconds) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || !prompt || !out_tokens || n_new <= 0) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_generate: bad arguments");
+    if (mi355x_status st = check_tokens(m, prompt, n_prompt)) return st;
+    const auto& c = m->c;
+    if (m->cache_len + n_prompt + n_new - 1 > c.context)
+        return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %lld positions for a context of %d", (long long)(m->cache_len + n_prompt + n_new - 1), c.context);
+    const int64_t B = c.batch;
+    DevBuf picked;  // [n_new, batch]
+    LLM_HIP(picked.alloc((size_t)n_new * B * 4), "hipMalloc(tokens)");
+    hipEvent_t e0, e1, e2;
+    LLM_HIP(hipEventCreate(&e0), "hipEventCreate"); LLM_HIP(hipEventCreate(&e1), "hipEventCreate"); LLM_HIP(hipEventCreate(&e2), "hipEventCreate");
+    LLM_HIP(hipMemcpyAsync(m->tokens_dev.p, prompt, B * n_prompt * 4, hipMemcpyHostToDevice, m->stream), "upload tokens");
+    LLM_HIP(hipEventRecord(e0, m->stream), "hipEventRecord");
+    mi355x_status st = forward(*m, n_prompt);
+    if (!st) st = head(*m, m->x.as<float>() + (n_prompt - 1) * c.embed, B, n_prompt * c.embed);
+    if (!st) {
+        hipError_t e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>(), m->stream);
+        if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: argmax: %s", hipGetErrorName(e));
+    }
+    if (!st) (void)hipEventRecord(e1, m->stream);
+    for (int64_t t = 1; t < n_new && !st; t++) {
+        // the step reads its tokens where the last step's argmax wrote them
+        hipError_t e = hipMemcpyAsync(m->tokens_dev.p, picked.as<int32_t>() + (t - 1) * B, B * 4, hipMemcpyDeviceToDevice, m->stream);
+        if (e != hipSuccess) { st = capi_fail((mi355x_status)e, "mi355x: llama: token copy: %s", hipGetErrorName(e)); break; }
+        st = forward(*m, 1);
+        if (!st) st = head(*m, m->x.as<float>(), B, c.embed);
+        if (!st) {
+            e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>() + t * B, m->stream);
+            if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: argmax: %s", hipGetErrorName(e));
+        }
+    }
+    if (!st) (void)hipEventRecord(e2, m->stream);
+    std::vector<int32_t> host((size_t)n_new * B);
+    if (!st) {
+        hipError_t e = hipMemcpyAsync(host.data(), picked.p, host.size() * 4, hipMemcpyDeviceToHost, m->stream);
+        if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: download tokens: %s", hipGetErrorName(e));
+    }
+    if (!st) st = mi355x_sync(m->stream);
+    if (!st) {
+        for (int64_t t = 0; t < n_new; t++)
+            for (int64_t b = 0; b < B; b++) out_tokens[b * n_new + t] = host[t * B + b];
+        if (seconds) {
+            float ms01 = 0, ms12 = 0;
+            (void)hipEventElapsedTime(&ms01, e0, e1);
+            (void)hipEventElapsedTime(&ms12, e1, e2);
+            seconds[0] = ms01 * 1e-3;
+            seconds[1] = ms12 * 1e-3;
+        }
+    }
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipEventDestroy(e2);
+    return st;
+}
+
+}  // extern "C"

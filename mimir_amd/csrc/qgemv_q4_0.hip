@@ -19,12 +19,11 @@
 //    instruction), so it multiplies eight weights per instruction with
 //    v_dot8_i32_i4: XOR 0x88888888 turns a dword of offset-binary nibbles n
 //    into two's-complement (n - 8), and each block of 32 activations is held
-//    as a 20-bit fixed-point number per element, split into five planes of
+//    as a 24-bit fixed-point number per element, split into six planes of
 //    signed 4-bit digits, with one float32 scale per block. The integer sums
 //    are exact; the only error is the fixed-point rounding of x, at most
-//    2^-20 of the block's largest magnitude per element (about 1e-6 relative
-//    on the result, the size of float32 rounding itself, a thousand times
-//    below the 1e-3 bar). Lanes own pairs of blocks (36 bytes, dword aligned)
+//    2^-23 of the block's largest magnitude per element: float32's own
+//    precision for the block's large values, and below 1e-7 of the result. Lanes own pairs of blocks (36 bytes, dword aligned)
 //    and fetch them with aligned 128-bit loads. Needs K a multiple of 64 and W
 //    dword aligned.
 //
@@ -223,15 +222,16 @@ static hipError_t launch_q4_0(const QGemvArgs& a, int waves, bool xlds, hipStrea
 // ---- fixed-point activations, v_dot8_i32_i4 ---------------------------------
 //
 // One row of x with nb blocks, converted (nbp = nb | 1; q4_0_act_bytes(K) bytes):
-//   u32x4 plane[5][nbp]  digit plane j of block b at plane[j * nbp + b]: dword i
+//   u32x4 plane[6][nbp]  digit plane j of block b at plane[j * nbp + b]: dword i
 //                        holds, nibble for nibble as dword i of the block's
 //                        weights does (byte k: low nibble element 4i+k, high
 //                        nibble element 16+4i+k), digit j of those elements
 //   float scale[nb]      x[e] ~ scale * sum_j 16^j digit_j[e]
 // The conversion runs once per x (q4_0_convert_act), not once per workgroup
 // of the product: a decode step multiplies the same x by several matrices.
-constexpr int kDigits = 5;
-constexpr int kFixMax = 489335;  // 7 * (16^5 - 1) / 15: the largest balanced 5-digit number
+constexpr int kDigits = 6;
+constexpr int kFixMax = 7829367;       // 7 * (16^6 - 1) / 15: the largest balanced 6-digit number
+constexpr uint32_t kFixBias = 0x888888;  // 8 in every digit
 
 size_t q4_0_act_bytes(int64_t K) {
     int64_t nb = K / 32;
@@ -239,14 +239,18 @@ size_t q4_0_act_bytes(int64_t K) {
 }
 
 // The eight values a thread holds (elements 4i..4i+3 and 16+4i..16+4i+3 of a
-// block) to five dwords of digits. Z = (X + 0x88888) ^ 0x88888 has the
+// block) to kDigits dwords of digits. Z = (X + kFixBias) ^ kFixBias has the
 // two's-complement balanced digit j of X in nibble j.
 __device__ __forceinline__ void fix_digits(const float lo[4], const float hi[4], float inv, uint32_t out[kDigits]) {
     uint32_t z[8];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        z[2 * k] = ((uint32_t)((int)__builtin_rintf(lo[k] * inv) + 0x88888)) ^ 0x88888u;      // nibble position 2k
-        z[2 * k + 1] = ((uint32_t)((int)__builtin_rintf(hi[k] * inv) + 0x88888)) ^ 0x88888u;  // nibble position 2k+1
+        // x * inv may round half a unit past kFixMax for the block's largest value: clamp
+        int a = (int)__builtin_rintf(lo[k] * inv), b = (int)__builtin_rintf(hi[k] * inv);
+        a = a > kFixMax ? kFixMax : a < -kFixMax ? -kFixMax : a;
+        b = b > kFixMax ? kFixMax : b < -kFixMax ? -kFixMax : b;
+        z[2 * k] = ((uint32_t)(a + (int)kFixBias)) ^ kFixBias;      // nibble position 2k
+        z[2 * k + 1] = ((uint32_t)(b + (int)kFixBias)) ^ kFixBias;  // nibble position 2k+1
     }
 #pragma unroll
     for (int j = 0; j < kDigits; j++) {
@@ -368,7 +372,7 @@ __device__ __forceinline__ void q4_pair_dot(const uint32_t q0[4], const uint32_t
             t1 = __builtin_amdgcn_sdot8(w1[i], (int)d1[j][i], t1, false);
         }
     }
-    out0 = t0;  // |t| <= 32 * 8 * 489335 < 2^27
+    out0 = t0;  // |t| <= 32 * 8 * 7829367 < 2^31
     out1 = t1;
 }
 
@@ -391,7 +395,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
     // Loads return in order, so the activations' loads go out first: they come
     // back from L2 well before the weights do from HBM, and the LDS stores and
     // the barrier are then over by the time the first weights arrive.
-    constexpr int kPark = PC == 1 ? 2 : 5;
+    constexpr int kPark = PC == 1 ? 2 : 6;
     const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
     const int n16 = (int)(act_row_bytes >> 4);
     u32x4 park[kPark];

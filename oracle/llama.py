@@ -256,7 +256,7 @@ def tensor_seed(seed: int, name: str) -> int:
     return h
 
 
-def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: int = O.Q8_0) -> Model:
+def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: int = O.Q8_0, output_dt: int | None = None) -> Model:
     """A random-init Llama: linear weights of linear_dt, embeddings and the
     output projection of table_dt, norm weights N(1, 0.02); block scales
     |N(0, 0.02)| as binary16, quants uniform over their range."""
@@ -267,7 +267,7 @@ def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: 
         return np.random.default_rng(tensor_seed(seed, name))
 
     m.embed = _q_blocks(rng("token_embd.weight"), table_dt, c.vocab, c.embed)
-    m.output = _q_blocks(rng("output.weight"), table_dt, c.vocab, c.embed)
+    m.output = _q_blocks(rng("output.weight"), table_dt if output_dt is None else output_dt, c.vocab, c.embed)
     m.norm = rng("output_norm.weight").normal(1, 0.02, c.embed).astype(np.float32)
     qd, kvd = c.heads * c.head_dim, c.kv_heads * c.head_dim
     for i in range(c.layers):
