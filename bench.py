@@ -131,6 +131,70 @@ def stream_ceiling(lib, capi, torch, nbytes, n_bufs, steps):
     return nbytes / (e0.elapsed_time(e1) / steps * 1e-3) / 1e9
 
 
+def tensor_seed(seed: int, name: str) -> int:
+    h = 1469598103934665603
+    for ch in f"{seed}/{name}".encode():
+        h = ((h ^ ch) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def q_blocks(rng, kind, n_elems):
+    """Blocks as the configurations draw them: quants uniform over their range,
+    one binary16 scale |N(0, 0.02)| per block of 32."""
+    nb = n_elems // 32
+    bb = 18 if kind == "q4_0" else 34
+    b = np.empty((nb, bb), np.uint8)
+    d = np.abs(rng.normal(0, 0.02, nb)).astype(np.float32).astype(np.float16).view(np.uint16)
+    b[:, 0], b[:, 1] = d & 0xff, d >> 8
+    if kind == "q4_0":
+        b[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
+    else:
+        b[:, 2:] = rng.integers(-127, 128, (nb, 32)).astype(np.int8).view(np.uint8)
+    return b.reshape(-1)
+
+
+def build_llama(capi, layers=32, batch=1, context=1024, max_tokens=512, seed=0, embed=4096, hidden=14336, heads=32, kv_heads=8,
+                head_dim=128, vocab=128256):
+    """A random-init Llama-3-8B-shaped decoder on the device: Q4_0 linears, Q8_0
+    embeddings and output, norm weights N(1, 0.02), binary16 KV cache. Each
+    tensor's generator is seeded from its name."""
+    from mimir_amd.llama import Llama
+    c = capi.LlamaConfig()
+    c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = embed, hidden, layers, heads, kv_heads, head_dim, head_dim, vocab
+    c.context, c.interleaved, c.cache_dtype, c.batch = context, 1, capi.F16, batch
+    c.rope_base, c.rope_scale, c.eps = 500000.0, 1.0, 1e-5
+    m = Llama(c)
+    rng = lambda name: np.random.default_rng(tensor_seed(seed, name))
+    m.set_tensor("token_embd.weight", capi.Q8_0, q_blocks(rng("token_embd.weight"), "q8_0", vocab * embed), vocab * embed)
+    m.set_tensor("output.weight", capi.Q8_0, q_blocks(rng("output.weight"), "q8_0", vocab * embed), vocab * embed)
+    m.set_tensor("output_norm.weight", capi.F32, rng("output_norm.weight").normal(1, 0.02, embed).astype(np.float32), embed)
+    qd, kvd = heads * head_dim, kv_heads * head_dim
+    for i in range(layers):
+        p = f"blk.{i}."
+        for leaf in ("attn_norm", "ffn_norm"):
+            m.set_tensor(p + leaf + ".weight", capi.F32, rng(p + leaf + ".weight").normal(1, 0.02, embed).astype(np.float32), embed)
+        for leaf, n, k in (("attn_q", qd, embed), ("attn_k", kvd, embed), ("attn_v", kvd, embed), ("attn_output", embed, qd),
+                           ("ffn_gate", hidden, embed), ("ffn_up", hidden, embed), ("ffn_down", embed, hidden)):
+            m.set_tensor(p + leaf + ".weight", capi.Q4_0, q_blocks(rng(p + leaf + ".weight"), "q4_0", n * k), n * k)
+    m.finalize(max_tokens)
+    return m
+
+
+def decode_bench(capi, layers=32, batch=1, prompt=512, new=256):
+    """Whole-model greedy decoding: a prompt of uniform-random token ids, then
+    `new` tokens a sequence. Returns tokens/s of the decoding steps."""
+    t0 = time.perf_counter()
+    m = build_llama(capi, layers=layers, batch=batch, context=prompt + new, max_tokens=prompt)
+    build_s = time.perf_counter() - t0
+    toks = np.random.default_rng(0).integers(0, m.config.vocab, (batch, prompt))
+    out, (t_prompt, t_decode) = m.generate(toks, new)
+    per_tok_bytes = layers * 218103808 * 0.5625 + 128256 * 4096 * 1.0625
+    return {"layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
+            "decode_tok_per_s": round(batch * (new - 1) / t_decode, 1), "ms_per_step": round(t_decode / (new - 1) * 1e3, 4),
+            "weight_GBps": round(per_tok_bytes / (t_decode / (new - 1)) / 1e9, 1), "build_s": round(build_s, 1),
+            "first_tokens": out[0, :8].tolist()}
+
+
 def cpu_baseline(n, k, seconds=2.0):
     """The reference's CPU route for a Q4_0 linear, restated by the oracle:
     weights decoded to float32 once (untimed), then the float32 GEMV over all
@@ -165,6 +229,9 @@ def main():
     ap.add_argument("--bufs", type=int, default=16, help="copies of W to rotate over (16 x 33 MB > the 256 MB last-level cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
+    ap.add_argument("--decode", action="store_true", help="also decode with the whole random-init 8B-shaped model (batch 1)")
+    ap.add_argument("--decode-layers", type=int, default=32)
+    ap.add_argument("--decode-batch", type=int, default=1)
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives or sharding are built)")
@@ -203,6 +270,8 @@ def main():
         extra["stream_read_33MB_GBps"] = round(stream_ceiling(lib, capi, torch, 33030144, args.bufs, args.steps), 1)
         extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
         out["extra"] = extra
+    if args.decode:
+        out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n, k)
     print(json.dumps(out), flush=True)

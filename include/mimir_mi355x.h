@@ -103,6 +103,18 @@ MI355X_API size_t mi355x_act_bytes(int dtype, int64_t K);
 MI355X_API mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
 MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The fused products of a decoding step, over converted activations (Q4_0
+ * weights that qualify for mi355x_qgemv_act). The reference fuses the same
+ * products on its CPU path by concatenating the weights (fusedFor,
+ * llm/decode.go:240-266); here the matrices stay where they are.
+ *   _add     y = resid + x . W^T                     (attn_output, ffn_down + residual)
+ *   _multi   y = x . [W0; W1; W2]^T, rows n0+n1+n2   (attn_q, attn_k, attn_v)
+ *   _swiglu  y = SiLU(x . gate^T) * (x . up^T)        (Block.mlp, llm/model.go:446-448) */
+MI355X_API mi355x_status mi355x_qgemv_act_add(int dtype, const void* W, const void* act, const float* resid, float* y, int64_t M, int64_t N, int64_t K, void* stream);
+MI355X_API mi355x_status mi355x_qgemv_act_multi(int dtype, const void* W0, const void* W1, const void* W2, int64_t n0, int64_t n1, int64_t n2,
+                                     const void* act, float* y, int64_t M, int64_t K, void* stream);
+MI355X_API mi355x_status mi355x_qgemv_act_swiglu(int dtype, const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* ---- OpCast / OpGather of a block-quantized input ---------------------------
  * (backend/cpu/quant.go:198-327; replaced kernels gen/quant.go:140-150 and
  * gen/gen.go:751-756). Bit-exact with the CPU backend. */

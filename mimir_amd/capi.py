@@ -35,6 +35,9 @@ SYMBOLS = {
     "mi355x_act_bytes": (_sz, [_int, _i64]),
     "mi355x_convert_act": (C.c_uint32, [_int, _vp, _i64, _i64, _i64, _vp, _vp]),
     "mi355x_qgemv_act": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_qgemv_act_add": (C.c_uint32, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_qgemv_act_multi": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
+    "mi355x_qgemv_act_swiglu": (C.c_uint32, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_dequant": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _int, _vp]),
     "mi355x_gather_rows": (C.c_uint32, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp]),
     "mi355x_rmsnorm": (C.c_uint32, [_vp, _vp, _vp, _i64, _i64, C.c_double, _vp]),

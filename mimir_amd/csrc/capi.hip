@@ -303,6 +303,53 @@ mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float*
     return MI355X_OK;
 }
 
+// The fused products of a decoding step. The reference fuses the same ones on
+// its CPU path by concatenating weights (fusedFor, llm/decode.go:240-266).
+static mi355x_status fused_args_ok(const char* what, int dtype, const void* act, const float* y, int64_t M, int64_t K) {
+    if (dtype != MI355X_Q4_0) return fail(MI355X_ERR_DTYPE, "mi355x: %s by weights of dtype %d (q4_0 only)", what, dtype);
+    if (M < 0 || M > 65535 || K <= 0) return fail(MI355X_ERR_SHAPE, "mi355x: %s of [%lld, %lld]", what, (long long)M, (long long)K);
+    if (!act || !y || ((uintptr_t)act & 15)) return fail(MI355X_ERR_INTERNAL, "mi355x: %s: null or misaligned pointer", what);
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_qgemv_act_add(int dtype, const void* W, const void* act, const float* resid, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (mi355x_status st = fused_args_ok("qgemv_act_add", dtype, act, y, M, K)) return st;
+    if (N < 0 || N > (int64_t)1 << 30) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_add of %lld rows", (long long)N);
+    if (M == 0 || N == 0) return MI355X_OK;
+    if (!W || !resid || !mimir::q4_0_fixed_point_ok(W, K)) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_add needs K a multiple of 64 up to 20928 and W dword aligned");
+    mimir::QGemvArgs a{W, nullptr, act, y, M, N, K, 0, 0};
+    a.resid = resid;
+    HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_qgemv_act_multi(int dtype, const void* W0, const void* W1, const void* W2, int64_t n0, int64_t n1, int64_t n2,
+                                     const void* act, float* y, int64_t M, int64_t K, void* stream) {
+    if (mi355x_status st = fused_args_ok("qgemv_act_multi", dtype, act, y, M, K)) return st;
+    const void* W[3] = {W0, W1, W2};
+    const int64_t n[3] = {n0, n1, n2};
+    for (int i = 0; i < 3; i++) {
+        if (n[i] < 0 || n[i] > (int64_t)1 << 28) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_multi: matrix %d of %lld rows", i, (long long)n[i]);
+        if (n[i] > 0 && (!W[i] || !mimir::q4_0_fixed_point_ok(W[i], K)))
+            return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_multi needs K a multiple of 64 up to 20928 and every W dword aligned");
+    }
+    if (n0 == 0 && (n1 > 0 || n2 > 0)) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_multi: the first matrix is empty");
+    if (n1 == 0 && n2 > 0) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_multi: the second matrix is empty");
+    if (M == 0 || n0 + n1 + n2 == 0) return MI355X_OK;
+    HIP_TRY(mimir::qgemv_q4_0_act_multi(W, n, act, y, M, K, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act_multi");
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_qgemv_act_swiglu(int dtype, const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (mi355x_status st = fused_args_ok("qgemv_act_swiglu", dtype, act, y, M, K)) return st;
+    if (N < 0 || N > (int64_t)1 << 28) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_swiglu of %lld rows", (long long)N);
+    if (M == 0 || N == 0) return MI355X_OK;
+    if (!gate || !up || !mimir::q4_0_fixed_point_ok(gate, K) || !mimir::q4_0_fixed_point_ok(up, K))
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_swiglu needs K a multiple of 64 up to 20928 and both W dword aligned");
+    HIP_TRY(mimir::qgemv_q4_0_act_swiglu(gate, up, act, y, M, N, K, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act_swiglu");
+    return MI355X_OK;
+}
+
 mi355x_status mi355x_dequant(int dtype, const void* W, int64_t first, int64_t n, void* out, int out_dtype, void* stream) {
     if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: dequantize dtype %d", dtype);
     if (out_dtype != MI355X_F32 && out_dtype != MI355X_BF16 && out_dtype != MI355X_F16)

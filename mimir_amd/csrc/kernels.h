@@ -34,7 +34,8 @@ struct QGemvArgs {
     float* y;
     int64_t M, N, K;
     int64_t x_row_stride;
-    int rows_per_wg;  // 0 = derived from the launch shape
+    int rows_per_wg;            // 0 = derived from the launch shape
+    const float* resid = nullptr;  // [M, N] added to the product (fixed-point Q4_0 kernel only)
 };
 
 // The float32 Q4_0 product, any shape. tune: {rows, cols, waves, no_lds}; zeros
@@ -48,6 +49,12 @@ bool q4_0_fixed_point_ok(const void* W, int64_t K);
 size_t q4_0_act_bytes(int64_t K);
 hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
+// Up to three matrices that share x and K in one launch, their rows
+// concatenated in y; and a SwiGLU pair: y = SiLU(x . gate^T) * (x . up^T).
+hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                const int* tune, hipStream_t st);
+hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
+                                 const int* tune, hipStream_t st);
 
 // The Q8_0 product as the reference's CPU computes it: x rounded to int8 per
 // block of 32 (q8_convert_act, q8_act_bytes(K) bytes per row), integer dot

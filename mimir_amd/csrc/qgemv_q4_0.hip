@@ -309,6 +309,9 @@ __global__ __launch_bounds__(256) void q4_0_convert_act_kernel(const float* __re
     }
 }
 
+// A 128-bit load that is only dword aligned (gfx950 serves it at full rate).
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
 hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
     int nb = (int)(K / 32);
     int gx = (nb * 4 + 255) / 256;
@@ -317,30 +320,24 @@ hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_
     return hipGetLastError();
 }
 
-// A 128-bit load that is only dword aligned (gfx950 serves it at full rate).
-typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
-
-template <int R, int PC>
+template <int RR, int PC>
 struct Q4PairTile {
-    u32x4 a[R][PC], b[R][PC];
-    uint32_t c[R][PC];
+    u32x4 a[RR][PC], b[RR][PC];
+    uint32_t c[RR][PC];
 };
 
-// Lane `lane` owns blocks 2p, 2p+1 with p = lane + 64 * pc: nine aligned
-// dwords. Plain (cached) loads: the three touch the same cache lines, which
-// must stay cached between them.
-template <int R, int PC>
-__device__ __forceinline__ void q4_load_pairs(Q4PairTile<R, PC>& t, const uint8_t* __restrict__ W, int64_t row_bytes, int N,
-                                              int npairs, int row0, int pc0, int lane) {
+// Lane `lane` owns blocks 2p, 2p+1 with p = lane + 64 * pc of each row: nine
+// aligned dwords. Plain (cached) loads: the three touch the same cache lines,
+// which must stay cached between them.
+template <int RR, int PC>
+__device__ __forceinline__ void q4_load_pairs(Q4PairTile<RR, PC>& t, const uint8_t* const rowp[RR], int npairs, int pc0, int lane) {
 #pragma unroll
     for (int pc = 0; pc < PC; pc++) {
         int p = lane + 64 * (pc0 + pc);
         p = p < npairs ? p : npairs - 1;
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            int row = row0 + r;  // wave-uniform
-            row = row < N ? row : N - 1;
-            const uint32_t* src = (const uint32_t*)(W + (int64_t)row * row_bytes) + p * 9;
+        for (int r = 0; r < RR; r++) {
+            const uint32_t* src = (const uint32_t*)rowp[r] + p * 9;
             t.a[r][pc] = *(const u32x4_a4*)src;
             t.b[r][pc] = *(const u32x4_a4*)(src + 4);
             t.c[r][pc] = src[8];
@@ -376,14 +373,31 @@ __device__ __forceinline__ void q4_pair_dot(const uint32_t q0[4], const uint32_t
     out1 = t1;
 }
 
-template <int R, int PC>
-__global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                             float* __restrict__ y, int N, int nb, int64_t act_row_bytes,
-                                                             int rows_per_wg) {
+// What one launch of the fixed-point kernel computes, for each row m of x:
+//   kPlain    y[m, :] = x[m, :] . W0^T (+ resid[m, :])
+//   kMulti    y[m, :] = x[m, :] . [W0; W1; W2]^T: up to three matrices that share
+//             K, their rows concatenated (queries, keys and values of a block)
+//   kSwiGLU   y[m, r] = SiLU(x[m, :] . W0[r]) * (x[m, :] . W1[r]): gate and up
+//             of a SwiGLU feed-forward (llm/model.go:446-448), the activation
+//             applied as tensor/elementwise.go:520-525,583-585 computes it
+enum Q4Mode { kPlain = 0, kMulti = 1, kSwiGLU = 2 };
+
+struct Q4Job {
+    const uint8_t* W[3];
+    int n[3];
+    int total;           // rows of y
+    const float* resid;  // [M, total] or null
+};
+
+template <int R, int PC, int MODE>
+__global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y,
+                                                             int nb, int64_t act_row_bytes, int rows_per_wg) {
+    constexpr int RR = MODE == kSwiGLU ? 2 * R : R;  // rows of weights a tile reads
     extern __shared__ u32x4 lds_i4[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
     const int m = blockIdx.y;
+    const int N = job.total;
     float* yr = y + (int64_t)m * N;
     const int nbp = nb | 1;
     const float* xscale = (const float*)(lds_i4 + kDigits * nbp);
@@ -391,6 +405,23 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
     const int wg_row0 = blockIdx.x * rows_per_wg;
     const int npairs = nb >> 1;
     const int npc = (npairs + 63) >> 6;
+
+    // The address of the weights behind row t of the tile at row0; rows past
+    // the end are clamped into the matrix (their sums are never stored).
+    auto row_ptr = [&](int row0, int t) -> const uint8_t* {
+        if (MODE == kSwiGLU) {
+            int r = row0 + (t < R ? t : t - R);
+            r = r < N ? r : N - 1;
+            return job.W[t < R ? 0 : 1] + (int64_t)r * row_bytes;
+        }
+        int g = row0 + t;
+        g = g < N ? g : N - 1;
+        if (MODE == kMulti) {
+            if (g >= job.n[0] + job.n[1]) return job.W[2] + (int64_t)(g - job.n[0] - job.n[1]) * row_bytes;
+            if (g >= job.n[0]) return job.W[1] + (int64_t)(g - job.n[0]) * row_bytes;
+        }
+        return job.W[0] + (int64_t)g * row_bytes;
+    };
 
     // Loads return in order, so the activations' loads go out first: they come
     // back from L2 well before the weights do from HBM, and the LDS stores and
@@ -404,11 +435,14 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
         int idx = tid + i * (int)blockDim.x;
         if (idx < n16) park[i] = act_row[idx];
     }
-    Q4PairTile<R, PC> tile;
+    Q4PairTile<RR, PC> tile;
     int r0 = wave * R;
+    const uint8_t* rowp[RR];
+#pragma unroll
+    for (int t = 0; t < RR; t++) rowp[t] = row_ptr(wg_row0 + r0, t);
     // Unconditional (rows are clamped into W): a branch here would make the
     // wait before the LDS stores below cover the weights' loads as well.
-    q4_load_pairs<R, PC>(tile, W, row_bytes, N, npairs, wg_row0 + r0, 0, lane);
+    q4_load_pairs<RR, PC>(tile, rowp, npairs, 0, lane);
 #pragma unroll
     for (int i = 0; i < kPark; i++) {
         int idx = tid + i * (int)blockDim.x;
@@ -421,11 +455,15 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
     for (; r0 < rows_per_wg; r0 += waves * R) {
         const int row0 = wg_row0 + r0;
         if (row0 >= N) break;
-        float acc[R];
+        if (!loaded) {
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = 0.f;
+            for (int t = 0; t < RR; t++) rowp[t] = row_ptr(row0, t);
+        }
+        float acc[RR];
+#pragma unroll
+        for (int r = 0; r < RR; r++) acc[r] = 0.f;
         for (int pc0 = 0; pc0 < npc; pc0 += PC) {
-            if (!loaded) q4_load_pairs<R, PC>(tile, W, row_bytes, N, npairs, row0, pc0, lane);
+            if (!loaded) q4_load_pairs<RR, PC>(tile, rowp, npairs, pc0, lane);
             loaded = false;
 #pragma unroll
             for (int pc = 0; pc < PC; pc++) {
@@ -440,7 +478,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
                 }
                 const float s0 = live ? xscale[2 * p] : 0.f, s1 = live ? xscale[2 * p + 1] : 0.f;
 #pragma unroll
-                for (int r = 0; r < R; r++) {
+                for (int r = 0; r < RR; r++) {
                     const u32x4 a = tile.a[r][pc], b = tile.b[r][pc];
                     const uint32_t c = tile.c[r][pc];
                     // block 0: scale in the low half of a[0], nibbles at bytes 2..17
@@ -462,18 +500,28 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(const uint8_t* __res
 #pragma unroll
         for (int r = 0; r < R; r++) {
             float s = wave_sum(acc[r]);
-            if (lane == 0 && row0 + r < N) yr[row0 + r] = s;
+            if (MODE == kSwiGLU) {
+                const float u = wave_sum(acc[R + r]);
+                const float e = __builtin_exp2f(s * (float)(-1.4426950408889634));
+                const float sg = 1.0f / (1.0f + e);
+                const float a = s * sg;
+                s = a * u;
+            }
+            if (lane == 0 && row0 + r < N) {
+                if (MODE == kPlain && job.resid) s = s + job.resid[(int64_t)m * N + row0 + r];
+                yr[row0 + r] = s;
+            }
         }
     }
 }
 
-template <int R, int PC>
-static hipError_t launch_q4_0_i4(const QGemvArgs& a, int waves, hipStream_t st) {
+template <int R, int PC, int MODE>
+static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
-    dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
-    size_t act_bytes = q4_0_act_bytes(a.K);
-    hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
-                       (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+    dim3 grid((unsigned)((job.total + rows_per_wg - 1) / rows_per_wg), (unsigned)M);
+    size_t act_bytes = q4_0_act_bytes(K);
+    hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, job, (const uint8_t*)act, y,
+                       (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     return hipGetLastError();
 }
 
@@ -514,26 +562,51 @@ bool q4_0_fixed_point_ok(const void* W, int64_t K) {
     return nb > 0 && nb % 2 == 0 && ((uintptr_t)W & 3) == 0 && q4_0_act_bytes(K) <= 64 * 1024;
 }
 
-// The fixed-point product from converted activations (a.act). Needs
-// q4_0_fixed_point_ok. tune: {rows, pair steps, waves}.
-hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
-    int nb = (int)(a.K / 32);
+// Launch shape of the fixed-point kernel. Many small tiles: measured on MI355X,
+// two rows per wavefront in workgroups of eight wavefronts stream best at the
+// decode shapes. tune: {rows, pair steps, waves}.
+template <int MODE>
+static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, const int* tune, hipStream_t st) {
+    int nb = (int)(K / 32);
     int npc = (nb / 2 + 63) / 64;  // steps of 64 pairs of blocks that cover a row
     int PC = npc <= 1 ? 1 : 2;
     if (tune[1] > 0) PC = tune[1];
-    // Many small tiles: measured on MI355X, two rows per wavefront in
-    // workgroups of eight wavefronts stream best at the decode shapes.
-    int R = a.N >= 4096 ? 2 : 1;
+    int R = MODE == kSwiGLU ? (job.total >= 8192 ? 2 : 1) : (job.total >= 4096 ? 2 : 1);
     if (tune[0] > 0) R = tune[0];
-    int64_t tiles = (a.N + R - 1) / R;
+    int64_t tiles = (job.total + R - 1) / R;
     int waves = 8;
     while (waves > 1 && tiles / waves < 256) waves >>= 1;
     if (tune[2] > 0) waves = tune[2];
-#define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP>(a, waves, st)
-    Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(3, 1); Q4ICASE(4, 1); Q4ICASE(7, 1); Q4ICASE(8, 1);
-    Q4ICASE(1, 2); Q4ICASE(2, 2); Q4ICASE(4, 2);
+    if (waves > 8) waves = 8;
+#define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE>(job, act, y, M, K, waves, st)
+    Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(4, 1);
+    Q4ICASE(1, 2); Q4ICASE(2, 2);
+    if constexpr (MODE != kSwiGLU) { Q4ICASE(4, 2); }
 #undef Q4ICASE
-    return launch_q4_0_i4<1, 1>(a, waves, st);
+    return launch_q4_0_i4<1, 1, MODE>(job, act, y, M, K, waves, st);
+}
+
+// The fixed-point product from converted activations (a.act), plus a.resid
+// if set. Needs q4_0_fixed_point_ok.
+hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
+    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid};
+    return dispatch_q4_0_i4<kPlain>(job, a.act, a.y, a.M, a.K, tune, st);
+}
+
+// y[m, :] = x[m, :] . [W0; W1; W2]^T for up to three matrices [n_i, K] (n_i may
+// be 0), each qualifying for the fixed-point kernel; y rows are n0 + n1 + n2 long.
+hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                const int* tune, hipStream_t st) {
+    Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
+              (int)(n[0] + n[1] + n[2]), nullptr};
+    return dispatch_q4_0_i4<kMulti>(job, act, y, M, K, tune, st);
+}
+
+// y[m, r] = SiLU(x[m, :] . gate[r]) * (x[m, :] . up[r]), gate and up [N, K].
+hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
+                                 const int* tune, hipStream_t st) {
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr};
+    return dispatch_q4_0_i4<kSwiGLU>(job, act, y, M, K, tune, st);
 }
 
 // The float32 product, any shape. tune: {rows, cols, waves, no_lds}.

@@ -108,7 +108,7 @@ def test_q4_0_gemv_random_scales_and_unaligned_start():
         check_close(got, want, 1e-4, f"q4_0 shrunk {shape}")
 
 
-@pytest.mark.parametrize("rows,cols,waves", [(1, 1, 1), (2, 1, 4), (4, 1, 8), (7, 1, 8), (8, 1, 2), (1, 2, 4), (2, 2, 8), (4, 2, 2)])
+@pytest.mark.parametrize("rows,cols,waves", [(1, 1, 1), (2, 1, 4), (4, 1, 8), (2, 1, 8), (4, 1, 2), (1, 2, 4), (2, 2, 8), (4, 2, 2)])
 def test_q4_0_fixed_point_kernel_every_launch_shape(rows, cols, waves):
     rng = np.random.default_rng(9)
     n, k = 203, 4096 + 64 * 3
@@ -211,6 +211,48 @@ def test_q4_0_gemv_linearity_at_full_size():
         assert bits_equal(gpu.qgemv(O.Q4_0, ptr, gpu.dev(e), n, k), wcol)
     finally:
         capi.check(l.mi355x_tune(b"q4_0.path", 0))
+
+
+def test_q4_0_fused_products():
+    """The fused products of a decoding step against the oracle's separate
+    ones: residual add, three matrices in one launch, SwiGLU of gate and up."""
+    rng = np.random.default_rng(31)
+    l = gpu.lib()
+    k, m = 4096, 3
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    xd = gpu.dev(x)
+    act = torch.zeros((m, l.mi355x_act_bytes(capi.Q4_0, k)), dtype=torch.uint8, device="cuda:0")
+    capi.check(l.mi355x_convert_act(capi.Q4_0, xd.data_ptr(), m, k, k, act.data_ptr(), gpu.stream()))
+    ns = (4096, 1024, 1022)
+    raws = [bench_blocks(rng, O.Q4_0, n * k) for n in ns]
+    bufs = [gpu.dev_bytes_at(r, 0) for r in raws]
+    wants = [O.qmatmul(O.Q4_0, r, x, n, k) for r, n in zip(raws, ns)]
+    gpu.say("q4_0 multi: q, k, v in one launch")
+    y = torch.full((m, sum(ns)), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(l.mi355x_qgemv_act_multi(capi.Q4_0, bufs[0][1], bufs[1][1], bufs[2][1], ns[0], ns[1], ns[2], act.data_ptr(), y.data_ptr(), m, k, gpu.stream()))
+    gpu.sync()
+    check_close(y.cpu().numpy(), np.concatenate(wants, axis=1), TOL)
+    y2 = torch.full((m, ns[0] + ns[1]), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(l.mi355x_qgemv_act_multi(capi.Q4_0, bufs[0][1], bufs[1][1], None, ns[0], ns[1], 0, act.data_ptr(), y2.data_ptr(), m, k, gpu.stream()))
+    gpu.sync()
+    assert bits_equal(y2.cpu().numpy(), y.cpu().numpy()[:, :ns[0] + ns[1]])
+    gpu.say("q4_0 add: product plus residual, in place")
+    resid = rng.normal(size=(m, ns[0])).astype(np.float32)
+    rd = gpu.dev(resid)
+    capi.check(l.mi355x_qgemv_act_add(capi.Q4_0, bufs[0][1], act.data_ptr(), rd.data_ptr(), rd.data_ptr(), m, ns[0], k, gpu.stream()))
+    gpu.sync()
+    check_close(rd.cpu().numpy(), wants[0] + resid, TOL)
+    gpu.say("q4_0 swiglu: gate and up, 14336 and a ragged 1023")
+    for n in (14336, 1023):
+        g_raw, u_raw = bench_blocks(rng, O.Q4_0, n * k), bench_blocks(rng, O.Q4_0, n * k)
+        gb, ub = gpu.dev_bytes_at(g_raw, 0), gpu.dev_bytes_at(u_raw, 0)
+        out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+        capi.check(l.mi355x_qgemv_act_swiglu(capi.Q4_0, gb[1], ub[1], act.data_ptr(), out.data_ptr(), m, n, k, gpu.stream()))
+        gpu.sync()
+        want = O.silu_mul(O.qmatmul(O.Q4_0, g_raw, x, n, k), O.qmatmul(O.Q4_0, u_raw, x, n, k))
+        got = out.cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    assert l.mi355x_qgemv_act_multi(capi.Q8_0, bufs[0][1], None, None, 4, 0, 0, act.data_ptr(), y.data_ptr(), m, k, gpu.stream()) == capi.ERR_DTYPE
 
 
 # ---- Q8_0: the int8-activation product of the CPU backend -------------------
