@@ -44,6 +44,7 @@ struct AttnParams {
     int causal;
     int64_t causal_offset;
     int chunk, nsplit;
+    const int32_t* dyn_k;  // if set, *dyn_k more keys than K (a decoding step replayed at every position)
 };
 
 // Partial results of one (query row, head, split): m, l, then o[D].
@@ -63,10 +64,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
     const int ng = G - g0 < kAttnHeads ? G - g0 : kAttnHeads;  // live query heads here
     const int b = blockIdx.z / p.Q, i = blockIdx.z % p.Q;
 
-    int64_t seen = p.K;
+    const int64_t Kt = p.K + (p.dyn_k ? *p.dyn_k : 0);
+    int64_t seen = Kt;
     if (p.causal) {
         seen = (int64_t)i + p.causal_offset + 1;
-        seen = seen < 0 ? 0 : seen > p.K ? p.K : seen;
+        seen = seen < 0 ? 0 : seen > Kt ? Kt : seen;
     }
     const int j0 = split * chunk;
     int j1 = j0 + chunk;
@@ -248,6 +250,7 @@ hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st) {
     p.causal_offset = a.causal_offset;
     p.chunk = a.chunk;
     p.nsplit = a.nsplit;
+    p.dyn_k = a.dyn_k;
     int G = a.H / a.HK, ngq = (G + kAttnHeads - 1) / kAttnHeads;
     dim3 grid((unsigned)a.nsplit, (unsigned)(a.HK * ngq), (unsigned)(a.B * a.Q));
     int redf = 4 * a.D > 32 ? 4 * a.D : 32;

@@ -57,6 +57,11 @@ struct DeviceState {
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 int g_tune_q4[5] = {0, 0, 0, 0, 0};
+}
+namespace mimir {
+void set_llama_step_mode(int mode);  // llm.hip
+}
+namespace {
 
 mi355x_status current_state(DeviceState** out) {
     int dev = 0;
@@ -470,6 +475,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
             g_tune_q4[i] = value;
             return MI355X_OK;
         }
+    if (key && strcmp(key, "llama.step") == 0 && value >= 0 && value <= 2) {
+        mimir::set_llama_step_mode(value);
+        return MI355X_OK;
+    }
     return fail(MI355X_ERR_INTERNAL, "mi355x: unknown tuning key %s", key ? key : "(null)");
 }
 

@@ -8,6 +8,7 @@
 // of RMSNorm's sum of squares, which a parallel reduction fixes differently.
 #include "device_util.h"
 #include "kernels.h"
+#include "q4_act.h"
 
 namespace mimir {
 
@@ -43,6 +44,78 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 hipError_t rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, hipStream_t st) {
     if (rows == 0 || d == 0) return hipSuccess;
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, w, y, (int)d, (float)(1.0 / (double)d), (float)eps);
+    return hipGetLastError();
+}
+
+// RMSNorm with the Q4_0 kernel's activation conversion fused in: the row is
+// held in registers between the sum of squares and the conversion, so x is
+// read once. Writes y (if not null) and the converted row. d a multiple of
+// 64 and at most 256 * 4 * 8 * kNormItems floats.
+constexpr int kNormItems = 4;
+__global__ __launch_bounds__(256) void rmsnorm_q4act_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            float* __restrict__ y, uint8_t* __restrict__ act, int d, float inv_d,
+                                                            float eps, int64_t act_row_bytes) {
+    __shared__ float part[4];
+    const float* xr = x + (int64_t)blockIdx.x * d;
+    const int nb = d >> 5, nbp = nb | 1, nq = nb * 4;
+    u32x4* plane = (u32x4*)(act + (int64_t)blockIdx.x * act_row_bytes);
+    float* xscale = (float*)(plane + kDigits * nbp);
+    // item t: block t / 4, dword t % 4: elements 4(t%4).. and 16 + 4(t%4).. of the block
+    f32x4 lo[kNormItems], hi[kNormItems];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormItems; i++) {
+        int t = threadIdx.x + i * 256;
+        if (t < nq) {
+            int b = t >> 2, q = t & 3;
+            __builtin_memcpy(&lo[i], xr + 32 * b + 4 * q, 16);
+            __builtin_memcpy(&hi[i], xr + 32 * b + 16 + 4 * q, 16);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float a = lo[i][k] * lo[i][k], c = hi[i][k] * hi[i][k];
+                ss = ss + a;
+                ss = ss + c;
+            }
+        }
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = (part[0] + part[1]) + (part[2] + part[3]);
+    float ms = total * inv_d;
+    float scale = 1.0f / __builtin_sqrtf(ms + eps);
+#pragma unroll
+    for (int i = 0; i < kNormItems; i++) {
+        int t = threadIdx.x + i * 256;
+        if (t < nq) {
+            int b = t >> 2, q = t & 3;
+            f32x4 wl, wh;
+            __builtin_memcpy(&wl, w + 32 * b + 4 * q, 16);
+            __builtin_memcpy(&wh, w + 32 * b + 16 + 4 * q, 16);
+            float l4[4], h4[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float a = lo[i][k] * scale, c = hi[i][k] * scale;
+                l4[k] = a * wl[k];
+                h4[k] = c * wh[k];
+            }
+            if (y) {
+                float* yr = y + (int64_t)blockIdx.x * d;
+                f32x4 ol = {l4[0], l4[1], l4[2], l4[3]}, oh = {h4[0], h4[1], h4[2], h4[3]};
+                __builtin_memcpy(yr + 32 * b + 4 * q, &ol, 16);
+                __builtin_memcpy(yr + 32 * b + 16 + 4 * q, &oh, 16);
+            }
+            q4_convert_item(l4, h4, plane, xscale, nbp, b, q);
+        }
+    }
+}
+
+bool rmsnorm_q4act_ok(int64_t d) { return d > 0 && d % 64 == 0 && d / 32 * 4 <= 256 * kNormItems; }
+
+hipError_t rmsnorm_q4act(const float* x, const float* w, float* y, void* act, int64_t rows, int64_t d, double eps, hipStream_t st) {
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(rmsnorm_q4act_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, w, y, (uint8_t*)act, (int)d,
+                       (float)(1.0 / (double)d), (float)eps, (int64_t)q4_0_act_row_bytes(d));
     return hipGetLastError();
 }
 
@@ -122,6 +195,102 @@ hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int 
     if (groups > 65536) groups = 65536;
     hipLaunchKernelGGL(kv_write_kernel, dim3((unsigned)groups), dim3(256), 0, st, src, cache, cache_dt, total, heads, (int)s, dim,
                        cap, pos, src_b, src_h, src_p);
+    return hipGetLastError();
+}
+
+// One position of a decoding step in one launch: qkv is [B, (H + 2 HK) * dim],
+// the rows of a fused q|k|v product. The query heads are rotated in place, the
+// key heads are rotated and written to the keys cache at the position *pos_dev
+// holds, the value heads are written to the values cache, each cast to the
+// cache's dtype. The position is read on the device so that a captured step
+// can be replayed at every position (the reference's recorded step takes the
+// position as a tensor for the same reason, llm/decode.go:27-41,166-183).
+__global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ qkv, void* __restrict__ kcache, void* __restrict__ vcache,
+                                                      int cache_dt, int B, int H, int HK, int dim, int rope_dim, int interleaved,
+                                                      int64_t cap, const float* __restrict__ cosv, const float* __restrict__ sinv,
+                                                      const int32_t* __restrict__ pos_dev) {
+    const int pos = *pos_dev;
+    const int half = rope_dim >> 1, hd2 = dim >> 1;  // work items: pairs of features
+    const int64_t row = (int64_t)(H + 2 * HK) * dim;
+    const int64_t total = (int64_t)B * (H + 2 * HK) * hd2;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        int i = (int)(t % hd2);
+        int64_t r = t / hd2;
+        int head = (int)(r % (H + 2 * HK));
+        int64_t b = r / (H + 2 * HK);
+        float* hp = qkv + b * row + (int64_t)head * dim;
+        int ia, ib;
+        float va, vb;
+        if (head < H + HK && i < half) {
+            ia = interleaved ? 2 * i : i;
+            ib = interleaved ? 2 * i + 1 : i + half;
+            float a = hp[ia], c2 = hp[ib];
+            float c = cosv[(int64_t)pos * half + i], sn = sinv[(int64_t)pos * half + i];
+            float ac = a * c, bs = c2 * sn, as = a * sn, bc = c2 * c;
+            va = ac - bs;
+            vb = interleaved ? as + bc : bc + as;
+        } else {  // values, and features past rope_dim: pass through (two at a time)
+            int j = head < H + HK ? i - half : i;
+            ia = head < H + HK ? rope_dim + 2 * j : 2 * j;
+            ib = ia + 1;
+            va = hp[ia];
+            vb = hp[ib];
+        }
+        if (head < H) {
+            hp[ia] = va;
+            hp[ib] = vb;
+        } else {
+            const bool is_k = head < H + HK;
+            const int kh = is_k ? head - H : head - H - HK;
+            void* cache = is_k ? kcache : vcache;
+            const int64_t at = ((b * HK + kh) * cap + pos) * dim;
+            if (cache_dt == kF32) {
+                ((float*)cache)[at + ia] = va;
+                ((float*)cache)[at + ib] = vb;
+            } else {
+                ((uint16_t*)cache)[at + ia] = f32_to_f16_bits(va);
+                ((uint16_t*)cache)[at + ib] = f32_to_f16_bits(vb);
+            }
+        }
+    }
+}
+
+hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
+                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
+    int64_t total = B * (H + 2 * HK) * (dim / 2);
+    if (total == 0) return hipSuccess;
+    int64_t groups = (total + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(rope_kv_kernel, dim3((unsigned)groups), dim3(256), 0, st, qkv, kcache, vcache, cache_dt, (int)B, H, HK, dim,
+                       rope_dim, interleaved, cap, cosv, sinv, pos_dev);
+    return hipGetLastError();
+}
+
+// After a step: appends the chosen tokens to the record and moves on one
+// position. state = {position, steps taken}.
+__global__ void advance_kernel(int32_t* __restrict__ state, const int32_t* __restrict__ next_tok, int32_t* __restrict__ record, int B,
+                               int pos_inc) {
+    int step = state[1];
+    if ((int)threadIdx.x < B) record[(int64_t)step * B + threadIdx.x] = next_tok[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        state[0] += pos_inc;
+        state[1] = step + 1;
+    }
+}
+
+hipError_t advance(int32_t* state, const int32_t* next_tok, int32_t* record, int B, int pos_inc, hipStream_t st) {
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(B < 64 ? 64 : ((B + 63) / 64) * 64), 0, st, state, next_tok, record, B, pos_inc);
+    return hipGetLastError();
+}
+
+__global__ void set_state_kernel(int32_t* __restrict__ state, int pos, int step) {
+    state[0] = pos;
+    state[1] = step;
+}
+
+hipError_t set_state(int32_t* state, int pos, int step, hipStream_t st) {
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, st, state, pos, step);
     return hipGetLastError();
 }
 

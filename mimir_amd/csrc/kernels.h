@@ -82,6 +82,18 @@ hipError_t rope(const float* x, float* y, int64_t rows, int64_t s, int head_dim,
                 int64_t offset, hipStream_t st);
 hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int heads, int64_t s, int dim, int64_t cap,
                     int64_t pos, int64_t src_b, int64_t src_h, int64_t src_p, hipStream_t st);
+// RMSNorm that also writes the row converted for the Q4_0 kernel (y may be
+// null); rmsnorm_q4act_ok says whether a row length qualifies.
+bool rmsnorm_q4act_ok(int64_t d);
+hipError_t rmsnorm_q4act(const float* x, const float* w, float* y, void* act, int64_t rows, int64_t d, double eps, hipStream_t st);
+// One decoding position: rotates the queries of qkv [B, (H + 2 HK) * dim] in
+// place, rotates and caches its keys, caches its values, at position *pos_dev.
+hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
+                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st);
+// state = {position, steps}: record[steps] = next_tok [B], then steps += 1 and
+// position += pos_inc.
+hipError_t advance(int32_t* state, const int32_t* next_tok, int32_t* record, int B, int pos_inc, hipStream_t st);
+hipError_t set_state(int32_t* state, int pos, int step, hipStream_t st);
 hipError_t swiglu(const float* g, const float* u, float* out, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st);
 hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, hipStream_t st);
@@ -103,6 +115,7 @@ struct AttnArgs {
     int causal;
     int64_t causal_offset;
     int chunk, nsplit;
+    const int32_t* dyn_k = nullptr;  // device int: that many more keys than K
 };
 void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, int* nsplit);
 size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit);

@@ -18,6 +18,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -84,6 +85,19 @@ struct Model {
     int64_t max_rows = 0;
     DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[4], tokens_dev, next_tok;
     hipStream_t stream = nullptr;
+
+    // The decoding step as a fixed run of launches that read the position from
+    // the device: state = {position, steps taken}; record holds the tokens
+    // chosen so far, [max_new, batch]. `fast` says the blocks qualify (Q4_0
+    // linears that the fixed-point kernel takes); step_graph replays the run.
+    bool fast = false;
+    DevBuf state, record, qkv;
+    hipGraphExec_t step_graph = nullptr;
+
+    ~Model() {
+        if (step_graph) (void)hipGraphExecDestroy(step_graph);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
 };
 
 int act_class(const Weight& w) {
@@ -221,6 +235,58 @@ static mi355x_status forward(Model& m, int64_t s) {
     return MI355X_OK;
 }
 
+// One decoding step of every sequence (llm/decode.go:188-227, stepGraph), for
+// blocks whose linears are Q4_0: the tokens come from m.next_tok and the
+// position from m.state, both on the device, so the same run of launches
+// serves every position and can be replayed as a graph. Per block: norm with
+// the activation conversion fused, q|k|v in one product, rotation and cache
+// write in one launch, split attention, conversion, output projection with the
+// residual added, norm, gate|up with SwiGLU in one product, conversion, down
+// projection with the residual added.
+static mi355x_status step_fast(Model& m) {
+    const auto& c = m.c;
+    const int64_t B = c.batch;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim, row = qd + 2 * kvd;
+    float *x = m.x.as<float>(), *qkv = m.qkv.as<float>(), *a = m.a.as<float>(), *sw = m.s.as<float>();
+    void* act = m.act[kActQ4].p;
+    const int32_t* pos = m.state.as<int32_t>();
+    if (mi355x_status st = embed_rows(m, m.next_tok.as<int32_t>(), B, x, device_error_word())) return st;
+    AttnArgs at;
+    at.q = qkv; at.kv_dtype = c.cache_dtype; at.out = a; at.lse = nullptr;
+    at.q_strides[0] = row; at.q_strides[1] = c.head_dim; at.q_strides[2] = 0;
+    at.k_strides[0] = at.v_strides[0] = (int64_t)c.kv_heads * c.context * c.head_dim;
+    at.k_strides[1] = at.v_strides[1] = (int64_t)c.context * c.head_dim;
+    at.k_strides[2] = at.v_strides[2] = c.head_dim;
+    at.o_strides[0] = qd; at.o_strides[1] = c.head_dim; at.o_strides[2] = 0;
+    at.B = B; at.Q = 1; at.K = 1; at.H = c.heads; at.HK = c.kv_heads; at.D = c.head_dim;
+    at.scale = 1.0 / std::sqrt((double)c.head_dim);
+    at.causal = 0; at.causal_offset = 0;
+    at.dyn_k = pos;  // position p holds p keys before this step's own
+    attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m.blocks[i];
+        LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
+        const void* w3[3] = {b.q.buf.p, b.k.buf.p, b.v.buf.p};
+        const int64_t n3[3] = {qd, kvd, kvd};
+        LLM_HIP(qgemv_q4_0_act_multi(w3, n3, act, qkv, B, c.embed, kNoTune, m.stream), "q|k|v");
+        LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                        c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        at.k = m.keys[i].p; at.v = m.values[i].p;
+        LLM_HIP(attention(at, m.act[0].p, m.stream), "attention");
+        LLM_HIP(q4_0_convert_act(a, B, qd, qd, act, m.stream), "convert");
+        QGemvArgs o{b.o.buf.p, nullptr, act, x, B, c.embed, qd, 0, 0};
+        o.resid = x;
+        LLM_HIP(qgemv_q4_0_act(o, kNoTune, m.stream), "attn_output");
+        LLM_HIP(rmsnorm_q4act(x, b.ffn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "ffn_norm");
+        LLM_HIP(qgemv_q4_0_act_swiglu(b.gate.buf.p, b.up.buf.p, act, sw, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
+        LLM_HIP(q4_0_convert_act(sw, B, c.hidden, c.hidden, act, m.stream), "convert");
+        QGemvArgs d{b.down.buf.p, nullptr, act, x, B, c.embed, c.hidden, 0, 0};
+        d.resid = x;
+        LLM_HIP(qgemv_q4_0_act(d, kNoTune, m.stream), "ffn_down");
+    }
+    return MI355X_OK;
+}
+
 // Norm and output projection of `rows` rows of hidden states at xin, which are
 // row_stride floats apart, into m.logits [rows, vocab].
 static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_stride) {
@@ -241,6 +307,14 @@ static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_
 }  // namespace mimir
 
 using mimir::Model;
+
+// How mi355x_llama_generate runs its decoding steps: 0 the fused launches
+// replayed as a graph where the model qualifies, 1 the same launches issued one
+// by one, 2 the general per-operator path.
+static int g_llama_step_mode = 0;
+namespace mimir {
+void set_llama_step_mode(int mode) { g_llama_step_mode = mode; }
+}
 
 extern "C" {
 
@@ -393,6 +467,20 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         attn_ws = b > attn_ws ? b : attn_ws;
     }
     LLM_HIP(m->act[0].alloc(attn_ws + 64), "hipMalloc(attention scratch)");
+    if (!m->stream) LLM_HIP(hipStreamCreate(&m->stream), "hipStreamCreate");
+    if (m->step_graph) {
+        (void)hipGraphExecDestroy(m->step_graph);
+        m->step_graph = nullptr;
+    }
+    LLM_HIP(m->state.alloc(256), "hipMalloc");
+    LLM_HIP(m->record.alloc(((size_t)c.context + 1) * c.batch * 4), "hipMalloc");  // a graph keeps its address
+    LLM_HIP(m->qkv.alloc((size_t)c.batch * (qd + 2 * kvd) * 4), "hipMalloc");
+    m->fast = rmsnorm_q4act_ok(c.embed) && c.head_dim % 2 == 0;
+    for (int i = 0; i < c.layers && m->fast; i++) {
+        Block& b = m->blocks[i];
+        for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down})
+            if (act_class(*w) != kActQ4) m->fast = false;
+    }
     m->ready = true;
     return MI355X_OK;
 }
@@ -451,6 +539,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
     if (m->cache_len + n_prompt + n_new - 1 > c.context)
         return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %lld positions for a context of %d", (long long)(m->cache_len + n_prompt + n_new - 1), c.context);
     const int64_t B = c.batch;
+    const bool use_graph = g_llama_step_mode == 0, use_fast = m->fast && g_llama_step_mode != 2;
     DevBuf picked;  // [n_new, batch]
     LLM_HIP(picked.alloc((size_t)n_new * B * 4), "hipMalloc(tokens)");
     hipEvent_t e0, e1, e2;
@@ -464,6 +553,51 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
         if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: argmax: %s", hipGetErrorName(e));
     }
     if (!st) (void)hipEventRecord(e1, m->stream);
+    if (!st && use_fast) {
+        // record[0] is the prompt's choice; each step then reads next_tok and the
+        // position from the device, and leaves its own choice in both places
+        hipError_t e = hipSuccess;  // n_new <= context: the record holds it
+        if (!st) e = hipMemcpyAsync(m->next_tok.p, picked.p, B * 4, hipMemcpyDeviceToDevice, m->stream);
+        if (!st && e == hipSuccess) e = set_state(m->state.as<int32_t>(), (int)m->cache_len, 0, m->stream);
+        if (!st && e == hipSuccess) e = advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 0, m->stream);
+        if (!st && e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: step state: %s", hipGetErrorName(e));
+        auto one_step = [&]() -> mi355x_status {
+            if (mi355x_status s2 = step_fast(*m)) return s2;
+            if (mi355x_status s2 = head(*m, m->x.as<float>(), B, c.embed)) return s2;
+            LLM_HIP(argmax(m->logits.as<float>(), B, c.vocab, m->next_tok.as<int32_t>(), m->stream), "argmax");
+            LLM_HIP(advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 1, m->stream), "advance");
+            return MI355X_OK;
+        };
+        if (!st && n_new > 1 && !m->step_graph && use_graph) {
+            hipGraph_t g = nullptr;
+            e = hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal);
+            if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: begin capture: %s", hipGetErrorName(e));
+            if (!st) {
+                mi355x_status cst = one_step();
+                e = hipStreamEndCapture(m->stream, &g);
+                if (cst) st = cst;
+                else if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: end capture: %s", hipGetErrorName(e));
+            }
+            if (!st) {
+                e = hipGraphInstantiate(&m->step_graph, g, nullptr, nullptr, 0);
+                if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: instantiate graph: %s", hipGetErrorName(e));
+            }
+            if (g) (void)hipGraphDestroy(g);
+        }
+        for (int64_t t = 1; t < n_new && !st; t++) {
+            if (m->step_graph && use_graph) {
+                e = hipGraphLaunch(m->step_graph, m->stream);
+                if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: graph launch: %s", hipGetErrorName(e));
+            } else {
+                st = one_step();
+            }
+            if (!st) m->cache_len += 1;
+        }
+        if (!st) {
+            e = hipMemcpyAsync(picked.p, m->record.p, (size_t)n_new * B * 4, hipMemcpyDeviceToDevice, m->stream);
+            if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: copy record: %s", hipGetErrorName(e));
+        }
+    } else
     for (int64_t t = 1; t < n_new && !st; t++) {
         // the step reads its tokens where the last step's argmax wrote them
         hipError_t e = hipMemcpyAsync(m->tokens_dev.p, picked.as<int32_t>() + (t - 1) * B, B * 4, hipMemcpyDeviceToDevice, m->stream);

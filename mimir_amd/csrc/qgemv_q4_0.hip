@@ -32,6 +32,7 @@
 //    binary16 subnormals.
 #include "device_util.h"
 #include "kernels.h"
+#include "q4_act.h"
 
 namespace mimir {
 
@@ -229,37 +230,7 @@ static hipError_t launch_q4_0(const QGemvArgs& a, int waves, bool xlds, hipStrea
 //   float scale[nb]      x[e] ~ scale * sum_j 16^j digit_j[e]
 // The conversion runs once per x (q4_0_convert_act), not once per workgroup
 // of the product: a decode step multiplies the same x by several matrices.
-constexpr int kDigits = 6;
-constexpr int kFixMax = 7829367;       // 7 * (16^6 - 1) / 15: the largest balanced 6-digit number
-constexpr uint32_t kFixBias = 0x888888;  // 8 in every digit
-
-size_t q4_0_act_bytes(int64_t K) {
-    int64_t nb = K / 32;
-    return (size_t)(((nb | 1) * kDigits * 16 + nb * 4 + 15) / 16 * 16);
-}
-
-// The eight values a thread holds (elements 4i..4i+3 and 16+4i..16+4i+3 of a
-// block) to kDigits dwords of digits. Z = (X + kFixBias) ^ kFixBias has the
-// two's-complement balanced digit j of X in nibble j.
-__device__ __forceinline__ void fix_digits(const float lo[4], const float hi[4], float inv, uint32_t out[kDigits]) {
-    uint32_t z[8];
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        // x * inv may round half a unit past kFixMax for the block's largest value: clamp
-        int a = (int)__builtin_rintf(lo[k] * inv), b = (int)__builtin_rintf(hi[k] * inv);
-        a = a > kFixMax ? kFixMax : a < -kFixMax ? -kFixMax : a;
-        b = b > kFixMax ? kFixMax : b < -kFixMax ? -kFixMax : b;
-        z[2 * k] = ((uint32_t)(a + (int)kFixBias)) ^ kFixBias;      // nibble position 2k
-        z[2 * k + 1] = ((uint32_t)(b + (int)kFixBias)) ^ kFixBias;  // nibble position 2k+1
-    }
-#pragma unroll
-    for (int j = 0; j < kDigits; j++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int p = 0; p < 8; p++) w |= ((z[p] >> (4 * j)) & 15u) << (4 * p);
-        out[j] = w;
-    }
-}
+size_t q4_0_act_bytes(int64_t K) { return q4_0_act_row_bytes(K); }
 
 // Thread t of a row takes item t: block t / 4, dword t % 4. The block's four
 // items sit in consecutive lanes (the item count and the stride are multiples
@@ -275,37 +246,7 @@ __global__ __launch_bounds__(256) void q4_0_convert_act_kernel(const float* __re
         int b = t >> 2, d = t & 3;
         f32x4 vlo = load_f32x4(xr + 32 * (int64_t)b + 4 * d), vhi = load_f32x4(xr + 32 * (int64_t)b + 16 + 4 * d);
         float lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
-        float amax = 0.f;
-        bool finite = true;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            float a0 = __builtin_fabsf(lo[k]), a1 = __builtin_fabsf(hi[k]);
-            finite = finite && a0 < __builtin_inff() && a1 < __builtin_inff();  // false for NaN too
-            amax = fmaxf(amax, fmaxf(a0, a1));
-        }
-        amax = fmaxf(amax, dpp_f32<0xb1>(amax));
-        amax = fmaxf(amax, dpp_f32<0x4e>(amax));
-        float bad = finite ? 0.f : 1.f;
-        bad = fmaxf(bad, dpp_f32<0xb1>(bad));
-        bad = fmaxf(bad, dpp_f32<0x4e>(bad));
-        float scale, inv;
-        if (bad != 0.f) {  // a NaN or an infinity in the block: its products are NaN
-            scale = __builtin_nanf("");
-            inv = 0.f;
-#pragma unroll
-            for (int k = 0; k < 4; k++) lo[k] = hi[k] = 0.f;
-        } else if (amax < 0x1p-100f) {  // nothing to represent (and 1/amax would overflow)
-            scale = 0.f;
-            inv = 0.f;
-        } else {
-            scale = amax / (float)kFixMax;
-            inv = (float)kFixMax / amax;
-        }
-        uint32_t dig[kDigits];
-        fix_digits(lo, hi, inv, dig);
-#pragma unroll
-        for (int j = 0; j < kDigits; j++) ((uint32_t*)(plane + j * nbp + b))[d] = dig[j];
-        if (d == 0) xscale[b] = scale;
+        q4_convert_item(lo, hi, plane, xscale, nbp, b, d);
     }
 }
 

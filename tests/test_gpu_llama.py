@@ -170,3 +170,50 @@ def test_random_init_q4_0_model_matches_oracle_and_greedy_tokens(batch):
             if a != w:
                 assert margins[i] < 0.02 * scale, (b, i, a, w, margins[i])
                 break  # the sequences part here by construction
+
+
+@pytest.mark.parametrize("batch,cache", [(1, capi.F32), (2, capi.F16)])
+def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, cache):
+    """The decoding step exists three times: per operator (what the logits tests
+    above pin against the oracle), fused launches (norm with conversion, q|k|v
+    in one product, rotation with the cache write, SwiGLU and residual
+    epilogues), and those launches replayed as a graph that reads position and
+    tokens from device memory. All three must choose the same tokens, replay
+    after replay, and again on a second call that starts from another cache
+    length with the graph the first call built."""
+    lib = gpu.lib()
+    c = _small_q4_config(batch, cache)
+    om = OL.synthetic(_oracle_config(c), seed=1, output_dt=O.Q4_0)
+    m = Llama(c)
+    _upload_synthetic(m, om)
+    m.finalize(40)
+    rng = np.random.default_rng(5)
+    runs = {}
+    try:
+        for mode in (2, 1, 0, 0):
+            gpu.say(f"generate, step mode {mode}, batch {batch}")
+            capi.check(lib.mi355x_tune(b"llama.step", mode))
+            m.reset()
+            prompts = np.random.default_rng(5).integers(0, c.vocab, (batch, 9))
+            first, _ = m.generate(prompts, 30)
+            assert m.cache_len == 9 + 29
+            # a second call continues the same caches from where the first stopped
+            more, _ = m.generate(first[:, -1:], 12)
+            assert m.cache_len == 9 + 29 + 1 + 11
+            runs.setdefault(mode, []).append(np.concatenate([first, more], 1))
+    finally:
+        capi.check(lib.mi355x_tune(b"llama.step", 0))
+    # the per-operator steps against the oracle, then the others against them
+    want, margins = om.generate(prompts[0].tolist(), 30, capacity=c.context, cache_dtype=O.F32 if cache == capi.F32 else O.F16)
+    got = runs[2][0][0, :30].tolist()
+    for i, (a, w) in enumerate(zip(got, want)):
+        if a != w:
+            assert margins[i] < 1e-3 * 170.0, (i, a, w, margins[i])
+            break
+    # attention splits the keys differently when the position comes from the
+    # device (a fixed plan for the whole context), so a sum may round another
+    # way; tokens differ only if two logits tie to that precision
+    same = [np.array_equal(runs[2][0], r) for r in (runs[1][0], runs[0][0], runs[0][1])]
+    assert np.array_equal(runs[0][0], runs[0][1])
+    assert np.array_equal(runs[1][0], runs[0][0])
+    assert all(same), (runs[2][0], runs[0][0])
