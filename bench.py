@@ -25,6 +25,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+# HBM bytes of one launch of the GEMV kernel at the benchmark shape, from
+# rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
+# reads for a copy kernel of known size (the summaries under profiles/ hold the
+# runs): FETCH_SIZE 16215.494 KiB x 1.99976, WRITE_SIZE 56.003 KiB x 1.0.
+TRAFFIC_BYTES_PER_LAUNCH = 33262752
 
 
 def gemv_bytes(n: int, k: int, block_bytes: int = 18) -> int:
@@ -42,75 +47,104 @@ def bench_blocks_q4_0(rng, n_elems):
     return b.reshape(-1)
 
 
-def time_gemv(lib, capi, torch, dt, n, k, steps, warmup, n_bufs, seed=0, check=True):
-    """Times `steps` launches after `warmup`, rotating over n_bufs copies of W.
-    Returns (ms per step by wall clock, ms per launch by HIP events)."""
-    rng = np.random.default_rng(seed)
-    raw = bench_blocks_q4_0(rng, n * k)
-    x = rng.normal(size=k).astype(np.float32)
-    w0 = torch.from_numpy(raw).to("cuda:0")
-    bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
-    xd = torch.from_numpy(x).to("cuda:0")
-    y = torch.empty(n, dtype=torch.float32, device="cuda:0")
-    st = torch.cuda.current_stream().cuda_stream
+class Gemv:
+    """One Q4_0 product y = x . W^T with n_bufs HBM-resident copies of W."""
 
-    def launch(i):
-        capi.check(lib.mi355x_qgemv(dt, bufs[i % n_bufs].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, st))
+    def __init__(self, lib, capi, torch, n, k, n_bufs, seed=0):
+        self.lib, self.capi, self.torch, self.n, self.k, self.n_bufs = lib, capi, torch, n, k, n_bufs
+        rng = np.random.default_rng(seed)
+        self.raw = bench_blocks_q4_0(rng, n * k)
+        self.x = rng.normal(size=k).astype(np.float32)
+        w0 = torch.from_numpy(self.raw).to("cuda:0")
+        self.bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
+        self.xd = torch.from_numpy(self.x).to("cuda:0")
+        self.y = torch.empty(n, dtype=torch.float32, device="cuda:0")
+        self.act = torch.empty(lib.mi355x_act_bytes(capi.Q4_0, k) + 64, dtype=torch.uint8, device="cuda:0")
+        self.stream = torch.cuda.Stream()
 
-    if check:  # the result is checked against the oracle before anything is timed
+    def step(self, i):
+        """The boundary's product: activation conversion, then the GEMV."""
+        self.capi.check(self.lib.mi355x_qgemv(self.capi.Q4_0, self.bufs[i % self.n_bufs].data_ptr(), self.xd.data_ptr(), self.y.data_ptr(),
+                                              1, self.n, self.k, self.k, self.stream.cuda_stream))
+
+    def kernel(self, i):
+        """The GEMV kernel alone, over activations converted beforehand."""
+        self.capi.check(self.lib.mi355x_qgemv_act(self.capi.Q4_0, self.bufs[i % self.n_bufs].data_ptr(), self.act.data_ptr(), self.y.data_ptr(),
+                                                  1, self.n, self.k, self.stream.cuda_stream))
+
+    def check(self):
+        """Both routes against the oracle, before anything is timed."""
         import oracle as O
-        launch(0)
-        capi.check(lib.mi355x_sync(st))
-        want = O.qmatmul(O.Q4_0, raw, x, n, k)
-        got = y.cpu().numpy()
-        err = np.abs(got - want) / np.maximum(1, np.abs(want))
-        if not np.all(err <= 1e-3):
-            raise SystemExit(f"bench: GEMV {n}x{k} differs from the oracle: worst {err.max():.3e}")
-    for i in range(warmup):
-        launch(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        launch(warmup + i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    ev_ms = e0.elapsed_time(e1) / steps
-    return wall_ms, ev_ms
+        want = O.qmatmul(O.Q4_0, self.raw, self.x, self.n, self.k)
+        self.capi.check(self.lib.mi355x_convert_act(self.capi.Q4_0, self.xd.data_ptr(), 1, self.k, self.k, self.act.data_ptr(), self.stream.cuda_stream))
+        for name, fn in (("qgemv", self.step), ("qgemv_act", self.kernel)):
+            self.y.zero_()
+            self.torch.cuda.synchronize()
+            fn(0)
+            self.stream.synchronize()
+            err = np.abs(self.y.cpu().numpy() - want) / np.maximum(1, np.abs(want))
+            if not np.all(err <= 1e-3):
+                raise SystemExit(f"bench: {name} {self.n}x{self.k} differs from the oracle: worst {err.max():.3e}")
 
+    def kernel_durations(self, steps, warmup):
+        """Mean, min and max microseconds of the GEMV kernel itself over `steps`
+        launches in a row: each launch carries its own pair of HIP events on the
+        launching stream, which read the kernel's begin and end as the
+        profiler's kernel trace does."""
+        import ctypes as C
+        with self.torch.cuda.stream(self.stream):
+            for i in range(max(warmup, 3)):
+                self.kernel(i)
+            self.stream.synchronize()
+            self.capi.check(self.lib.mi355x_timed_begin(steps))
+            for i in range(steps):
+                self.kernel(i)
+            ms = (C.c_float * steps)()
+            n = C.c_int(0)
+            self.capi.check(self.lib.mi355x_timed_end(ms, C.byref(n)))
+        if n.value != steps:
+            raise SystemExit(f"bench: {n.value} timed launches, want {steps}")
+        us = np.array(ms[:steps], np.float64) * 1e3
+        return float(us.mean()), float(us.min()), float(us.max())
 
-def time_gemv_graph(lib, capi, torch, dt, n, k, steps, warmup, n_bufs, seed=0):
-    """The same launches captured once into a HIP graph and replayed, which
-    takes the host's launch cost out of the device timeline."""
-    rng = np.random.default_rng(seed)
-    raw = bench_blocks_q4_0(rng, n * k)
-    w0 = torch.from_numpy(raw).to("cuda:0")
-    bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
-    xd = torch.from_numpy(rng.normal(size=k).astype(np.float32)).to("cuda:0")
-    y = torch.empty(n, dtype=torch.float32, device="cuda:0")
-    s = torch.cuda.Stream()
-    g = torch.cuda.CUDAGraph()
-    per_graph = n_bufs
-    with torch.cuda.stream(s):
-        for i in range(3):
-            capi.check(lib.mi355x_qgemv(dt, bufs[i % n_bufs].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, s.cuda_stream))
-        s.synchronize()
-        with torch.cuda.graph(g, stream=s):
-            for i in range(per_graph):
-                capi.check(lib.mi355x_qgemv(dt, bufs[i].data_ptr(), xd.data_ptr(), y.data_ptr(), 1, n, k, k, s.cuda_stream))
-        reps = max(1, steps // per_graph)
-        for _ in range(max(1, warmup // per_graph)):
-            g.replay()
-        s.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(s)
-        for _ in range(reps):
-            g.replay()
-        e1.record(s)
-        s.synchronize()
-    return e0.elapsed_time(e1) / (reps * per_graph)
+    def time(self, fn, steps, warmup, graph=True):
+        """Milliseconds per call of fn over exactly `steps` calls after `warmup`,
+        between HIP events on the stream that carries the launches. With graph,
+        the calls are captured n_bufs at a time (plus one graph for the
+        remainder) and replayed, as the decoder replays its step, so the host's
+        launch cost stays off the device's timeline. Also returns wall ms/call."""
+        torch, s = self.torch, self.stream
+        with torch.cuda.stream(s):
+            for i in range(max(warmup, 3)):
+                fn(i)
+            s.synchronize()
+            graphs = []
+            if graph:
+                for count in (self.n_bufs, steps % self.n_bufs):
+                    g = None
+                    if count:
+                        g = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(g, stream=s):
+                            for i in range(count):
+                                fn(i)
+                    graphs.append(g)
+                graphs[0].replay()
+                s.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record(s)
+            if graph:
+                for _ in range(steps // self.n_bufs):
+                    graphs[0].replay()
+                if graphs[1] is not None:
+                    graphs[1].replay()
+            else:
+                for i in range(steps):
+                    fn(i)
+            e1.record(s)
+            s.synchronize()
+            wall = (time.perf_counter() - t0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall
 
 
 def stream_ceiling(lib, capi, torch, nbytes, n_bufs, steps):
@@ -229,7 +263,11 @@ def main():
     ap.add_argument("--bufs", type=int, default=16, help="copies of W to rotate over (16 x 33 MB > the 256 MB last-level cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
-    ap.add_argument("--decode", action="store_true", help="also decode with the whole random-init 8B-shaped model (batch 1)")
+    ap.add_argument("--counters", type=int, default=0, metavar="N",
+                    help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
+    ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
+    ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
+    ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
     ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--decode-batch", type=int, default=1)
     args = ap.parse_args()
@@ -244,36 +282,63 @@ def main():
     capi.check(lib.mi355x_init(0))
 
     n, k = 14336, 4096
-    wall_ms, ev_ms = time_gemv(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, args.bufs)
+    g = Gemv(lib, capi, torch, n, k, args.bufs)
+    g.check()
+    if args.counters:
+        # for a counter run of the profiler: a few launches of the GEMV kernel and,
+        # to scale the counters by, of a copy of known size (256 MiB read, 256 MiB
+        # written), each from buffers the cache does not hold
+        src = [torch.empty(1 << 28, dtype=torch.uint8, device="cuda:0").random_(0, 255) for _ in range(2)]
+        dst = torch.empty(1 << 28, dtype=torch.uint8, device="cuda:0")
+        with torch.cuda.stream(g.stream):
+            for i in range(args.counters):
+                g.kernel(i)
+                dst.copy_(src[i % 2])
+            g.stream.synchronize()
+        print(json.dumps({"counters": args.counters, "gemv_bytes": gemv_bytes(n, k), "copy_read_bytes": 1 << 28, "copy_write_bytes": 1 << 28}))
+        return
+    # a step: the product as the boundary takes it (float32 activations in,
+    # conversion and GEMV), graph-replayed; the roofline: its GEMV kernel alone
+    step_ms, step_wall_ms = g.time(g.step, args.steps, args.warmup, graph=not args.eager)
+    seq_ms, _ = g.time(g.kernel, args.steps, args.warmup, graph=True)
+    kern_us, kern_min, kern_max = g.kernel_durations(args.steps, args.warmup)
     bytes_ = gemv_bytes(n, k)
-    value = bytes_ / (wall_ms * 1e-3) / 1e9
-    achieved = bytes_ / (ev_ms * 1e-3) / 1e9
+    value = bytes_ / (step_ms * 1e-3) / 1e9
+    achieved = bytes_ / (kern_us * 1e-6) / 1e9
     out = {
         "metric": "Q4_0 GEMV HBM GB/s (% of peak); decode tok/s, 8B-shape, batch 1",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "ms_per_step": round(step_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i4 x 24-bit fixed point, f32 scales and output", "data": "synthetic",
         "config": {"workload": "Q4_0 decode GEMV 4096->14336 (Llama-3-8B gate/up), batch 1, W rotated over "
-                               f"{args.bufs} HBM-resident copies", "N": n, "K": k, "M": 1},
+                               f"{args.bufs} HBM-resident copies; a step = activation conversion + GEMV, "
+                               + ("launched one by one" if args.eager else "replayed from a HIP graph"),
+                   "N": n, "K": k, "M": 1, "wall_ms_per_step": round(step_wall_ms, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "qgemv_q4_0_kernel", "bytes_per_launch": bytes_, "us_per_launch": round(ev_ms * 1e3, 3)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "qgemv_q4_0_i4_kernel<2, 1, 0>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
+                     "us_min": round(kern_min, 3), "us_max": round(kern_max, 3),
+                     # launches of the kernel alone back to back in a graph, the wait between dependent kernels included
+                     "us_per_launch_in_sequence": round(seq_ms * 1e3, 3)},
     }
     extra = {}
     if args.all_shapes:
         for name, (nn, kk) in {"down_14336->4096": (4096, 14336), "qo_4096->4096": (4096, 4096), "kv_4096->1024": (1024, 4096)}.items():
-            nb = max(args.bufs, int(600e6 // gemv_bytes(nn, kk)) + 1)
-            w, e = time_gemv(lib, capi, torch, capi.Q4_0, nn, kk, args.steps, args.warmup, min(nb, 256))
+            nb = min(256, max(args.bufs, int(600e6 // gemv_bytes(nn, kk)) + 1))
+            gg = Gemv(lib, capi, torch, nn, kk, nb)
+            gg.check()
+            e, _ = gg.time(gg.kernel, args.steps, args.warmup)
             extra[name] = {"us_per_launch": round(e * 1e3, 3), "GBps": round(gemv_bytes(nn, kk) / (e * 1e-3) / 1e9, 1)}
-        extra["gate_up_hot_1buf"] = {"us_per_launch": round(time_gemv(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, 1, check=False)[1] * 1e3, 3)}
-        extra["gate_up_graph"] = {"us_per_launch": round(time_gemv_graph(lib, capi, torch, capi.Q4_0, n, k, args.steps, args.warmup, args.bufs) * 1e3, 3)}
+            del gg
+        extra["gate_up_eager_step_us"] = round(g.time(g.step, args.steps, args.warmup, graph=False)[0] * 1e3, 3)
         extra["stream_read_33MB_GBps"] = round(stream_ceiling(lib, capi, torch, 33030144, args.bufs, args.steps), 1)
         extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
         out["extra"] = extra
-    if args.decode:
+    del g
+    if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(n, k)
+        out["cpu_baseline"] = cpu_baseline(n, k, seconds=10.0)
     print(json.dumps(out), flush=True)
 
 

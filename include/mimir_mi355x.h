@@ -214,6 +214,12 @@ MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* promp
  * (else the per-operator path), 1 the same launches without the graph, 2 the
  * per-operator path always. */
 MI355X_API mi355x_status mi355x_tune(const char* key, int value);
+/* Between timed_begin and timed_end, each launch of the fixed-point Q4_0 GEMV
+ * kernel made by the calling thread (at most max_launches of them; not under
+ * stream capture) is bracketed by its own pair of HIP events. timed_end waits
+ * for the device and writes the milliseconds of each launch, in order. */
+MI355X_API mi355x_status mi355x_timed_begin(int max_launches);
+MI355X_API mi355x_status mi355x_timed_end(float* ms_each, int* n_launches);
 /* Reads `bytes` bytes at p with 128-bit loads from `grid` workgroups of
  * `threads` threads and folds them into scratch (at least grid*threads/64
  * floats): the practical ceiling of a streaming read on this device. */

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <vector>
 #include <string>
 
 #include "kernels.h"
@@ -58,8 +59,17 @@ std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 int g_tune_q4[5] = {0, 0, 0, 0, 0};
 }
+thread_local std::vector<hipEvent_t> t_events;
+thread_local size_t t_events_used = 0;
 namespace mimir {
 void set_llama_step_mode(int mode);  // llm.hip
+bool next_timing_events(hipEvent_t* start, hipEvent_t* stop) {
+    if (t_events_used + 2 > t_events.size()) return false;
+    *start = t_events[t_events_used];
+    *stop = t_events[t_events_used + 1];
+    t_events_used += 2;
+    return true;
+}
 }
 namespace {
 
@@ -480,6 +490,29 @@ mi355x_status mi355x_tune(const char* key, int value) {
         return MI355X_OK;
     }
     return fail(MI355X_ERR_INTERNAL, "mi355x: unknown tuning key %s", key ? key : "(null)");
+}
+
+// Per-launch timing of the fixed-point Q4_0 kernel: between timed_begin and
+// timed_end every such launch of this thread carries its own pair of events.
+mi355x_status mi355x_timed_begin(int max_launches) {
+    if (max_launches <= 0 || max_launches > (1 << 20) || !t_events.empty()) return fail(MI355X_ERR_INTERNAL, "mi355x: timed_begin(%d)", max_launches);
+    t_events.resize(2 * (size_t)max_launches);
+    for (auto& e : t_events) HIP_TRY(hipEventCreate(&e), "hipEventCreate");
+    t_events_used = 0;
+    return MI355X_OK;
+}
+
+mi355x_status mi355x_timed_end(float* ms_each, int* n_launches) {
+    if (!ms_each || !n_launches) return fail(MI355X_ERR_INTERNAL, "mi355x: timed_end: null pointer");
+    hipError_t e = hipDeviceSynchronize();
+    size_t n = t_events_used / 2;
+    for (size_t i = 0; i < n && e == hipSuccess; i++) e = hipEventElapsedTime(&ms_each[i], t_events[2 * i], t_events[2 * i + 1]);
+    for (auto& ev : t_events) (void)hipEventDestroy(ev);
+    t_events.clear();
+    t_events_used = 0;
+    *n_launches = (int)n;
+    HIP_TRY(e, "timed_end");
+    return MI355X_OK;
 }
 
 mi355x_status mi355x_stream_read(const void* p, size_t bytes, float* scratch, int grid, int threads, void* stream) {

@@ -123,6 +123,9 @@ hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
 
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.
+// While a measurement is on (capi.hip), hands out the next pair of events for a
+// launch to be bracketed by; false otherwise.
+bool next_timing_events(hipEvent_t* start, hipEvent_t* stop);
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);
 int stream_read_out_len(int grid, int threads);
 

@@ -30,6 +30,7 @@
 //  qgemv_q4_0_kernel      any shape and any 2-byte aligned W: float32
 //    multiply-adds through v_fma_mix_f32 on nibbles masked in place as
 //    binary16 subnormals.
+#include <hip/hip_ext.h>
 #include "device_util.h"
 #include "kernels.h"
 #include "q4_act.h"
@@ -461,8 +462,13 @@ static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, in
     int rows_per_wg = R * waves;
     dim3 grid((unsigned)((job.total + rows_per_wg - 1) / rows_per_wg), (unsigned)M);
     size_t act_bytes = q4_0_act_bytes(K);
-    hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, job, (const uint8_t*)act, y,
-                       (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
+    hipEvent_t t0, t1;
+    if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
+        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, t0, t1, 0, job,
+                              (const uint8_t*)act, y, (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
+    else
+        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, job, (const uint8_t*)act, y,
+                           (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     return hipGetLastError();
 }
 
