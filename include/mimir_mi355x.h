@@ -209,6 +209,8 @@ MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* promp
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
+ * "attention.path" = 1 makes mi355x_attention use its general kernels also for
+ * one query position (which otherwise takes a single-launch kernel).
  * "llama.step" chooses how mi355x_llama_generate runs its decoding steps: 0 the
  * fused launches replayed as a HIP graph where every block's linears are Q4_0
  * (else the per-operator path), 1 the same launches without the graph, 2 the

@@ -1,0 +1,357 @@
+// Attention of one query position per sequence (a decoding step) on gfx950:
+// the same arithmetic as attention.hip (OpAttention, backend/op.go:117-129; the
+// CPU's decode branch forwardFew, backend/cpu/attention.go:437-535) in one
+// launch that is all latency at batch 1, so it is shaped for few, wide,
+// independent loads and no second kernel.
+//
+// A workgroup of 256 threads takes one key head, up to four of its query heads
+// and one share of the keys the step sees (the shares are equal: the number of
+// keys may come from device memory, so that a replayed graph serves every
+// position, and every workgroup of the grid has work at every position).
+// Sixteen lanes share a key row, 16 or 32 bytes each, so a wavefront's load
+// covers four whole rows; the sixteen key groups of the workgroup take
+// consecutive keys. Scores go through LDS for the softmax, values are
+// accumulated per key group and summed through LDS. Each workgroup writes its
+// share's (max, sum, weighted values) and takes a ticket; the one that draws
+// the last ticket of its heads combines the shares, so no workgroup ever waits
+// for another. It can also leave the result in the fixed-point form the Q4_0
+// product reads (q4_act.h), which saves the conversion launch before the
+// output projection.
+#include "device_util.h"
+#include "kernels.h"
+#include "q4_act.h"
+
+namespace mimir {
+
+namespace {
+
+constexpr int kHeads = 4;      // query heads per workgroup
+constexpr int kThreads = 256;
+constexpr int kKeyGroups = 16;
+constexpr int kCounterBytes = (int)kAttnTicketBytes;  // tickets at the front of the workspace
+
+struct DecParams {
+    int64_t q_b, q_h;
+    int64_t k_b, k_h, k_p;
+    int64_t v_b, v_h, v_p;
+    int64_t o_b, o_h;
+    int B, H, HK, K, kmax;
+    float scale;
+    int causal;
+    int64_t causal_offset;
+    int cmax, nsplit;
+    const int32_t* dyn_k;
+    int64_t act_row_bytes;
+};
+
+__device__ __forceinline__ float group16_sum(float v) {
+    v += dpp_f32<0xb1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4e>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    return v;
+}
+
+// FPL consecutive elements of a cache row as floats.
+template <typename KV, int FPL>
+__device__ __forceinline__ void load_row(const KV* p, float out[FPL]) {
+    if constexpr (sizeof(KV) == 4) {
+#pragma unroll
+        for (int i = 0; i < FPL; i += 4) {
+            f32x4 t;
+            __builtin_memcpy(&t, __builtin_assume_aligned(p + i, 16), 16);
+            out[i] = t[0]; out[i + 1] = t[1]; out[i + 2] = t[2]; out[i + 3] = t[3];
+        }
+    } else {
+        uint32_t w[FPL / 2];
+        __builtin_memcpy(w, __builtin_assume_aligned(p, FPL == 4 ? 8 : 16), FPL * 2);
+#pragma unroll
+        for (int i = 0; i < FPL / 2; i++) {
+            out[2 * i] = f16_bits_to_f32((uint16_t)(w[i] & 0xffffu));
+            out[2 * i + 1] = f16_bits_to_f32((uint16_t)(w[i] >> 16));
+        }
+    }
+}
+
+template <typename KV, int FPL>
+__global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __restrict__ q, const KV* __restrict__ k,
+                                                               const KV* __restrict__ v, float* __restrict__ ws,
+                                                               uint32_t* __restrict__ counters, float* __restrict__ out,
+                                                               float* __restrict__ lse, uint8_t* __restrict__ act, DecParams p) {
+    constexpr int D = 16 * FPL;
+    constexpr int OPL = D / 64;  // results a lane holds of its wavefront's head
+    extern __shared__ float smem[];
+    float* sc = smem;                  // [4][cmax] scores, then weights
+    float* osl = sc + kHeads * p.cmax; // [16][4][D] values per key group; later the combine's factors and results
+    __shared__ float red[2 * kHeads];
+    __shared__ int s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int part = tid & 15, kg = tid >> 4;
+    const int split = blockIdx.x, nsplit = p.nsplit, cmax = p.cmax;
+    const int G = p.H / p.HK, ngq = (G + kHeads - 1) / kHeads;
+    const int hk = blockIdx.y / ngq, g0 = (blockIdx.y % ngq) * kHeads;
+    const int ng = G - g0 < kHeads ? G - g0 : kHeads;
+    const int b = blockIdx.z;
+
+    int64_t seen = (int64_t)p.K + (p.dyn_k ? *p.dyn_k : 0);
+    if (p.causal) {
+        int64_t c = p.causal_offset + 1;
+        seen = c < seen ? c : seen;
+    }
+    seen = seen < 0 ? 0 : seen > p.kmax ? p.kmax : seen;
+    const int per = (int)((seen + nsplit - 1) / nsplit);  // <= cmax
+    const int j0 = split * per;
+    const int j1 = j0 + per < (int)seen ? j0 + per : (int)seen;
+    const int nj = j1 > j0 ? j1 - j0 : 0;
+
+    float qr[kHeads][FPL];
+#pragma unroll
+    for (int g = 0; g < kHeads; g++) {
+        if (g < ng) {
+            load_row<float, FPL>(q + b * p.q_b + (int64_t)(hk * G + g0 + g) * p.q_h + part * FPL, qr[g]);
+#pragma unroll
+            for (int f = 0; f < FPL; f++) qr[g][f] = qr[g][f] * p.scale;
+        } else {
+#pragma unroll
+            for (int f = 0; f < FPL; f++) qr[g][f] = 0.f;
+        }
+    }
+    const KV* kbase = k + b * p.k_b + (int64_t)hk * p.k_h + part * FPL;
+    const KV* vbase = v + b * p.v_b + (int64_t)hk * p.v_h + part * FPL;
+
+    // scores of key j0 + jj, jj = jj0 + 16 u + kg: four rows in flight per thread
+    for (int jj0 = 0; jj0 < nj; jj0 += 4 * kKeyGroups) {
+        float kf[4][FPL];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int jj = jj0 + kKeyGroups * u + kg;
+            load_row<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kf[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int jj = jj0 + kKeyGroups * u + kg;
+#pragma unroll
+            for (int g = 0; g < kHeads; g++) {
+                float s = 0.f;
+#pragma unroll
+                for (int f = 0; f < FPL; f++) s = fmaf(qr[g][f], kf[u][f], s);
+                s = group16_sum(s);
+                if (part == 0 && jj < nj) sc[g * cmax + jj] = s;
+            }
+        }
+    }
+    __syncthreads();
+
+    // per head (wavefront g takes head g): max, exp, sum over the share's scores
+    {
+        float m = -__builtin_inff();
+        for (int jj = lane; jj < nj; jj += 64) m = fmaxf(m, sc[wave * cmax + jj]);
+        m = wave_max(m);
+        float l = 0.f;
+        if (nj > 0 && m > -__builtin_inff()) {
+            for (int jj = lane; jj < nj; jj += 64) {
+                float e = __builtin_expf(sc[wave * cmax + jj] - m);
+                sc[wave * cmax + jj] = e;
+                l += e;
+            }
+        } else {
+            for (int jj = lane; jj < nj; jj += 64) sc[wave * cmax + jj] = 0.f;
+        }
+        l = wave_sum(l);
+        if (lane == 0) {
+            red[wave] = m;
+            red[kHeads + wave] = l;
+        }
+    }
+    __syncthreads();
+
+    // values: key group kg sums its keys' rows, weighted, for the four heads
+    float o[kHeads][FPL];
+#pragma unroll
+    for (int g = 0; g < kHeads; g++)
+#pragma unroll
+        for (int f = 0; f < FPL; f++) o[g][f] = 0.f;
+    for (int jj0 = 0; jj0 < nj; jj0 += 4 * kKeyGroups) {
+        float vf[4][FPL];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int jj = jj0 + kKeyGroups * u + kg;
+            load_row<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vf[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int jj = jj0 + kKeyGroups * u + kg;
+            const bool live = jj < nj;
+#pragma unroll
+            for (int g = 0; g < kHeads; g++) {
+                float pj = live ? sc[g * cmax + jj] : 0.f;
+#pragma unroll
+                for (int f = 0; f < FPL; f++) o[g][f] = fmaf(pj, live ? vf[u][f] : 0.f, o[g][f]);
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < kHeads; g++)
+#pragma unroll
+        for (int f = 0; f < FPL; f++) osl[(kg * kHeads + g) * D + part * FPL + f] = o[g][f];
+    __syncthreads();
+    // wavefront g now holds head g: lane takes features lane + 64 c
+    const int g = wave, h = hk * G + g0 + g;
+    float r[OPL];
+#pragma unroll
+    for (int c = 0; c < OPL; c++) {
+        float s = 0.f;
+#pragma unroll
+        for (int x = 0; x < kKeyGroups; x++) s += osl[(x * kHeads + g) * D + lane + 64 * c];
+        r[c] = s;
+    }
+    float M = red[g], L = red[kHeads + g];
+
+    if (nsplit > 1) {
+        if (g < ng) {
+            float* w = ws + (((int64_t)b * p.H + h) * nsplit + split) * (D + 2);
+            if (lane == 0) {
+                w[0] = M;
+                w[1] = L;
+            }
+#pragma unroll
+            for (int c = 0; c < OPL; c++) w[2 + lane + 64 * c] = r[c];
+        }
+        // the last workgroup of these heads to get here combines the shares
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t* ctr = counters + (int64_t)b * gridDim.y + blockIdx.y;
+            uint32_t ticket = atomicAdd(ctr, 1u);
+            s_last = ticket == (uint32_t)(nsplit - 1);
+            if (s_last) *ctr = 0;  // for the next launch
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();
+        float* fs = osl + g * 64;  // factor of share s of head g
+        float f = 0.f, ls = 0.f, ms = -__builtin_inff();
+        const float* w0 = ws + ((int64_t)b * p.H + h) * nsplit * (D + 2);
+        if (g < ng && lane < nsplit) {
+            ms = w0[lane * (D + 2)];
+            ls = w0[lane * (D + 2) + 1];
+        }
+        M = wave_max(ms);
+        if (ls != 0.f && M > -__builtin_inff()) f = __builtin_expf(ms - M);
+        L = wave_sum(ls * f);
+        fs[lane] = f;
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < OPL; c++) r[c] = 0.f;
+        if (g < ng) {
+            for (int s = 0; s < nsplit; s++) {
+                float fsv = fs[s];
+#pragma unroll
+                for (int c = 0; c < OPL; c++) r[c] = fmaf(w0[s * (D + 2) + 2 + lane + 64 * c], fsv, r[c]);
+            }
+        }
+        __syncthreads();  // fs is read; the results go over it
+    }
+
+    // (sum p v) * (1 / sum p); a row that sees no key gets zeros and -Inf
+    const float inv = L == 0.f ? 0.f : 1.0f / L;
+    float* fin = osl;  // [4][D]
+#pragma unroll
+    for (int c = 0; c < OPL; c++) {
+        float val = L == 0.f ? 0.f : r[c] * inv;
+        if (g < ng && out) out[b * p.o_b + (int64_t)h * p.o_h + lane + 64 * c] = val;
+        if (act) fin[g * D + lane + 64 * c] = g < ng ? val : 0.f;
+    }
+    if (g < ng && lse && lane == 0) lse[(int64_t)b * p.H + h] = L == 0.f ? -__builtin_inff() : M + __builtin_logf(L);
+    if (!act) return;
+    __syncthreads();
+    // item t: head t / (D/8), block (t % (D/8)) / 4 of the head, dword t % 4
+    const int nit = ng * (D / 8);
+    if (tid < nit) {
+        const int gi = tid / (D / 8), rr = tid % (D / 8), blk = rr >> 2, dq = rr & 3;
+        float lo[4], hi[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            lo[e] = fin[gi * D + blk * 32 + 4 * dq + e];
+            hi[e] = fin[gi * D + blk * 32 + 16 + 4 * dq + e];
+        }
+        const int nb = p.H * D / 32, nbp = nb | 1;
+        u32x4* plane = (u32x4*)(act + (int64_t)b * p.act_row_bytes);
+        float* xscale = (float*)(plane + kDigits * nbp);
+        q4_convert_item(lo, hi, plane, xscale, nbp, (hk * G + g0 + gi) * (D / 32) + blk, dq);
+    }
+}
+
+}  // namespace
+
+// Shares of the keys and the most keys a share can hold, for at most kmax keys.
+void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax) {
+    int G = H / HK, ngq = (G + kHeads - 1) / kHeads;
+    int64_t rows = B * HK * ngq;
+    int64_t ns = 512 / (rows > 0 ? rows : 1);
+    ns = ns > 64 ? 64 : ns;
+    int64_t by_keys = kmax / 32;
+    ns = ns > by_keys ? by_keys : ns;
+    ns = ns < 1 ? 1 : ns;
+    *nsplit = (int)ns;
+    int64_t c = (kmax + ns - 1) / ns;
+    *cmax = (int)(c < 1 ? 1 : c);
+}
+
+size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit) {
+    return kCounterBytes + (nsplit <= 1 ? 0 : (size_t)(B * H * nsplit * (D + 2)) * sizeof(float));
+}
+
+// Whether the decode kernel takes this call: one query position, heads of 64
+// or 128 features, rows of the caches and of q aligned for 16-byte loads.
+bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
+    if (a.Q != 1 || (a.D != 64 && a.D != 128) || a.B <= 0 || a.B > 65535) return false;
+    int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
+    if (a.B * a.HK * ngq > kCounterBytes / 4 || (int64_t)a.HK * ngq > 65535) return false;
+    const int es = a.kv_dtype == kF16 ? 2 : 4;
+    const int fpl = a.D / 16;
+    const int row_align = fpl * es >= 16 ? 16 : 8;
+    for (int i = 0; i < 3; i++)
+        if ((a.k_strides[i] * es) % row_align || (a.v_strides[i] * es) % row_align) return false;
+    if (((uintptr_t)a.k | (uintptr_t)a.v) % row_align || (uintptr_t)a.q % 16 || a.q_strides[0] % 4 || a.q_strides[1] % 4) return false;
+    int ns, cm;
+    attention_decode_plan(a.B, a.H, a.HK, kmax, &ns, &cm);
+    size_t lds = (size_t)(kHeads * cm + kKeyGroups * kHeads * a.D) * sizeof(float);
+    return lds <= 60 * 1024 && kmax <= INT32_MAX / 2;
+}
+
+// a.K keys (plus *a.dyn_k), at most kmax. workspace: attention_decode_workspace_bytes
+// bytes whose first 4096 were zero before the first launch (the tickets reset
+// themselves). act, if set, gets row b's result [H * D] in the Q4_0 product's
+// fixed-point form, act_row_bytes apart; out may then be null.
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st) {
+    DecParams p;
+    p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
+    p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];
+    p.v_b = a.v_strides[0]; p.v_h = a.v_strides[1]; p.v_p = a.v_strides[2];
+    p.o_b = a.o_strides[0]; p.o_h = a.o_strides[1];
+    p.B = (int)a.B; p.H = a.H; p.HK = a.HK; p.K = (int)a.K; p.kmax = (int)kmax;
+    p.scale = (float)a.scale;
+    p.causal = a.causal;
+    p.causal_offset = a.causal_offset;
+    attention_decode_plan(a.B, a.H, a.HK, kmax, &p.nsplit, &p.cmax);
+    p.dyn_k = a.dyn_k;
+    p.act_row_bytes = act_row_bytes;
+    int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
+    dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
+    size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);
+    uint32_t* counters = (uint32_t*)workspace;
+    float* ws = (float*)((uint8_t*)workspace + kCounterBytes);
+#define DEC_LAUNCH(KV, FPL)                                                                                                   \
+    hipLaunchKernelGGL((attn_decode_kernel<KV, FPL>), grid, dim3(kThreads), lds, st, a.q, (const KV*)a.k, (const KV*)a.v, ws, \
+                       counters, a.out, a.lse, (uint8_t*)act, p)
+    if (a.kv_dtype == kF16) {
+        if (a.D == 128) DEC_LAUNCH(uint16_t, 8); else DEC_LAUNCH(uint16_t, 4);
+    } else {
+        if (a.D == 128) DEC_LAUNCH(float, 8); else DEC_LAUNCH(float, 4);
+    }
+#undef DEC_LAUNCH
+    return hipGetLastError();
+}
+
+}  // namespace mimir

@@ -53,11 +53,15 @@ struct DeviceState {
     // Partial results of split attention, grown and shared likewise.
     void* attn = nullptr;
     size_t attn_bytes = 0;
+    // Tickets and candidates of the split argmax.
+    void* argmax = nullptr;
+    size_t argmax_bytes = 0;
 };
 
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 int g_tune_q4[5] = {0, 0, 0, 0, 0};
+int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
 thread_local std::vector<hipEvent_t> t_events;
 thread_local size_t t_events_used = 0;
@@ -118,11 +122,28 @@ mi355x_status attn_scratch(size_t bytes, void** out) {
         size_t want = bytes < (4u << 20) ? (4u << 20) : bytes;
         void* p = nullptr;
         HIP_TRY(hipMalloc(&p, want), "hipMalloc(attention scratch)");
+        HIP_TRY(hipMemset(p, 0, mimir::kAttnTicketBytes), "hipMemset(attention tickets)");  // the decode kernel's tickets
         if (s->attn) HIP_TRY(hipFree(s->attn), "hipFree(attention scratch)");
         s->attn = p;
         s->attn_bytes = want;
     }
     *out = s->attn;
+    return MI355X_OK;
+}
+
+mi355x_status argmax_scratch(size_t bytes, void** out) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (s->argmax_bytes < bytes) {
+        void* p = nullptr;
+        HIP_TRY(hipMalloc(&p, bytes), "hipMalloc(argmax scratch)");
+        HIP_TRY(hipMemset(p, 0, mimir::kArgmaxTicketBytes), "hipMemset(argmax tickets)");
+        if (s->argmax) HIP_TRY(hipFree(s->argmax), "hipFree(argmax scratch)");
+        s->argmax = p;
+        s->argmax_bytes = bytes;
+    }
+    *out = s->argmax;
     return MI355X_OK;
 }
 
@@ -446,11 +467,18 @@ mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const v
     }
     a.B = B; a.Q = Q; a.K = K; a.H = H; a.HK = HK; a.D = D;
     a.scale = scale; a.causal = causal; a.causal_offset = causal_offset;
-    mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
     void* ws = nullptr;
-    if (size_t need = mimir::attention_workspace_bytes(B, H, Q, D, a.nsplit))
-        if (mi355x_status st = attn_scratch(need, &ws)) return st;
-    HIP_TRY(mimir::attention(a, ws, (hipStream_t)stream), "launch attention");
+    if (g_tune_attn != 1 && mimir::attention_decode_ok(a, K)) {  // one query position: a single launch
+        int cmax;
+        mimir::attention_decode_plan(B, H, HK, K, &a.nsplit, &cmax);
+        if (mi355x_status st = attn_scratch(mimir::attention_decode_workspace_bytes(B, H, D, a.nsplit), &ws)) return st;
+        HIP_TRY(mimir::attention_decode(a, K, ws, nullptr, 0, (hipStream_t)stream), "launch attention_decode");
+        return MI355X_OK;
+    }
+    mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
+    // the scratch begins with the decode kernel's tickets
+    if (mi355x_status st = attn_scratch(mimir::kAttnTicketBytes + mimir::attention_workspace_bytes(B, H, Q, D, a.nsplit), &ws)) return st;
+    HIP_TRY(mimir::attention(a, (uint8_t*)ws + mimir::kAttnTicketBytes, (hipStream_t)stream), "launch attention");
     return MI355X_OK;
 }
 
@@ -474,7 +502,10 @@ mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_
     if (rows < 0 || n <= 0 || n > INT32_MAX || rows > 65535) return fail(MI355X_ERR_SHAPE, "mi355x: argmax of [%lld, %lld]", (long long)rows, (long long)n);
     if (rows == 0) return MI355X_OK;
     if (!logits || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: argmax: null pointer");
-    HIP_TRY(mimir::argmax(logits, rows, n, out, (hipStream_t)stream), "launch argmax");
+    void* ws = nullptr;
+    if (rows <= 1024)
+        if (mi355x_status st = argmax_scratch(mimir::argmax_workspace_bytes(1024), &ws)) return st;
+    HIP_TRY(mimir::argmax(logits, rows, n, out, ws, (hipStream_t)stream), "launch argmax");
     return MI355X_OK;
 }
 
@@ -485,6 +516,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
             g_tune_q4[i] = value;
             return MI355X_OK;
         }
+    if (key && strcmp(key, "attention.path") == 0) {
+        g_tune_attn = value;
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "llama.step") == 0 && value >= 0 && value <= 2) {
         mimir::set_llama_step_mode(value);
         return MI355X_OK;

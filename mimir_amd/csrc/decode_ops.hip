@@ -378,9 +378,99 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
     }
 }
 
-hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, hipStream_t st) {
+// The same over many workgroups per row: each scans a span of the row and
+// leaves its candidate; the last one of a row to finish (a ticket per row)
+// picks among the candidates. tickets: one zeroed word per row, which the last
+// workgroup zeroes again.
+constexpr int kArgmaxBlocks = 64;  // at most, per row
+
+__device__ __forceinline__ void argmax_better(float& best, int& at, float v, int i) {
+    if (v > best || (v == best && i < at)) {
+        best = v;
+        at = i;
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_split_kernel(const float* __restrict__ logits, int64_t n, int span, int32_t* __restrict__ out,
+                                                           uint32_t* __restrict__ tickets, float* __restrict__ cand_v,
+                                                           int* __restrict__ cand_i) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    __shared__ int s_last;
+    const int r = blockIdx.y, nblk = gridDim.x;
+    const float* row = logits + (int64_t)r * n;
+    const int64_t lo = (int64_t)blockIdx.x * span, hi = lo + span < n ? lo + span : n;
+    float best = -__builtin_inff();
+    int at = 0x7fffffff;
+    for (int64_t i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * 256) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = i0 + 256 * u < hi ? row[i0 + 256 * u] : -__builtin_inff();
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i0 + 256 * u < hi) argmax_better(best, at, v[u], (int)(i0 + 256 * u));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off);
+        int oi = __shfl_xor(at, off);
+        argmax_better(best, at, ov, oi);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        bv[threadIdx.x >> 6] = best;
+        bi[threadIdx.x >> 6] = at;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) argmax_better(best, at, bv[w], bi[w]);
+        cand_v[r * kArgmaxBlocks + blockIdx.x] = best;
+        cand_i[r * kArgmaxBlocks + blockIdx.x] = at;
+        __threadfence();
+        uint32_t ticket = atomicAdd(&tickets[r], 1u);
+        s_last = ticket == (uint32_t)(nblk - 1);
+        if (s_last) tickets[r] = 0;
+    }
+    __syncthreads();
+    if (!s_last || threadIdx.x >= 64) return;
+    __threadfence();
+    best = -__builtin_inff();
+    at = 0x7fffffff;
+    if ((int)threadIdx.x < nblk) {
+        best = cand_v[r * kArgmaxBlocks + threadIdx.x];
+        at = cand_i[r * kArgmaxBlocks + threadIdx.x];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off);
+        int oi = __shfl_xor(at, off);
+        argmax_better(best, at, ov, oi);
+    }
+    if (threadIdx.x == 0) {
+        float first = row[0];
+        if (first != first || at == 0x7fffffff) at = 0;  // NaN at 0, or nothing but NaNs
+        out[r] = at;
+    }
+}
+
+size_t argmax_workspace_bytes(int64_t rows) { return kArgmaxTicketBytes + (size_t)rows * kArgmaxBlocks * 8; }
+
+// workspace: argmax_workspace_bytes(rows) bytes whose first kArgmaxTicketBytes were
+// zero before the first launch, or null for the one-workgroup kernel.
+hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, void* workspace, hipStream_t st) {
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, n, out);
+    if (!workspace || rows > (int64_t)(kArgmaxTicketBytes / 4) || n < 8192) {
+        hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, n, out);
+        return hipGetLastError();
+    }
+    int64_t nblk = (n + 4095) / 4096;
+    nblk = nblk > kArgmaxBlocks ? kArgmaxBlocks : nblk;
+    int64_t span = ((n + nblk - 1) / nblk + 255) / 256 * 256;
+    nblk = (n + span - 1) / span;
+    uint32_t* tickets = (uint32_t*)workspace;
+    float* cand_v = (float*)((uint8_t*)workspace + kArgmaxTicketBytes);
+    int* cand_i = (int*)(cand_v + rows * kArgmaxBlocks);
+    hipLaunchKernelGGL(argmax_split_kernel, dim3((unsigned)nblk, (unsigned)rows), dim3(256), 0, st, logits, n, (int)span, out, tickets,
+                       cand_v, cand_i);
     return hipGetLastError();
 }
 

@@ -96,7 +96,11 @@ hipError_t advance(int32_t* state, const int32_t* next_tok, int32_t* record, int
 hipError_t set_state(int32_t* state, int pos, int step, hipStream_t st);
 hipError_t swiglu(const float* g, const float* u, float* out, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st);
-hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, hipStream_t st);
+// workspace: argmax_workspace_bytes(rows) bytes, the first kArgmaxTicketBytes zero
+// before the first launch (they restore themselves), or null for one workgroup a row.
+constexpr size_t kArgmaxTicketBytes = 4096;
+size_t argmax_workspace_bytes(int64_t rows);
+hipError_t argmax(const float* logits, int64_t rows, int64_t n, int32_t* out, void* workspace, hipStream_t st);
 
 // Attention of queries [B, H, Q, D] over keys and values [B, HK, K, D], each
 // read through strides {batch, head, position} (features contiguous). chunk
@@ -120,6 +124,17 @@ struct AttnArgs {
 void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, int* nsplit);
 size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit);
 hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
+
+// One query position per sequence in a single launch (attention_decode.hip).
+// The workspace begins with kAttnTicketBytes of tickets that must be zero before
+// the first launch and restore themselves; a.K keys plus *a.dyn_k, at most kmax.
+// act, if set, receives the result in the Q4_0 product's fixed-point form
+// (out may then be null; needs o_strides {H * D, D, .}).
+constexpr size_t kAttnTicketBytes = 4096;
+bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
+void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
+size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st);
 
 // A plain streaming read of `bytes` bytes, summed into out[0..grid): the
 // practical ceiling of HBM reads to compare the products against.

@@ -91,7 +91,7 @@ struct Model {
     // chosen so far, [max_new, batch]. `fast` says the blocks qualify (Q4_0
     // linears that the fixed-point kernel takes); step_graph replays the run.
     bool fast = false;
-    DevBuf state, record, qkv;
+    DevBuf state, record, qkv, argmax_ws;
     hipGraphExec_t step_graph = nullptr;
 
     ~Model() {
@@ -217,8 +217,8 @@ static mi355x_status forward(Model& m, int64_t s) {
         at.causal = 1; at.causal_offset = past;
         attention_plan(B, c.heads, c.kv_heads, s, at.K, &at.chunk, &at.nsplit);
         size_t need = attention_workspace_bytes(B, c.heads, s, c.head_dim, at.nsplit);
-        if (need > m.act[0].bytes) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: attention scratch of %zu bytes, need %zu", m.act[0].bytes, need);
-        LLM_HIP(attention(at, m.act[0].p, m.stream), "attention");
+        if (need + kAttnTicketBytes > m.act[0].bytes) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: attention scratch of %zu bytes, need %zu", m.act[0].bytes, need);
+        LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
         if (mi355x_status st = convert_for(m, a, rows, qd, {&b.o}, done)) return st;
         if (mi355x_status st = linear(m, b.o, a, o, rows)) return st;
         LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
@@ -262,7 +262,8 @@ static mi355x_status step_fast(Model& m) {
     at.scale = 1.0 / std::sqrt((double)c.head_dim);
     at.causal = 0; at.causal_offset = 0;
     at.dyn_k = pos;  // position p holds p keys before this step's own
-    attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
+    const bool one_launch = attention_decode_ok(at, c.context);
+    if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
         LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
@@ -272,8 +273,13 @@ static mi355x_status step_fast(Model& m) {
         LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
                         c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
         at.k = m.keys[i].p; at.v = m.values[i].p;
-        LLM_HIP(attention(at, m.act[0].p, m.stream), "attention");
-        LLM_HIP(q4_0_convert_act(a, B, qd, qd, act, m.stream), "convert");
+        if (one_launch) {  // leaves its result converted for the output projection
+            at.out = nullptr;
+            LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, (int64_t)q4_0_act_bytes(qd), m.stream), "attention");
+        } else {
+            LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
+            LLM_HIP(q4_0_convert_act(a, B, qd, qd, act, m.stream), "convert");
+        }
         QGemvArgs o{b.o.buf.p, nullptr, act, x, B, c.embed, qd, 0, 0};
         o.resid = x;
         LLM_HIP(qgemv_q4_0_act(o, kNoTune, m.stream), "attn_output");
@@ -466,13 +472,24 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         size_t b = attention_workspace_bytes(c.batch, c.heads, max_tokens, c.head_dim, (int)((c.context + cc - 1) / cc));
         attn_ws = b > attn_ws ? b : attn_ws;
     }
+    {
+        int ns, cm;
+        attention_decode_plan(c.batch, c.heads, c.kv_heads, c.context, &ns, &cm);
+        size_t b = attention_decode_workspace_bytes(c.batch, c.heads, c.head_dim, ns);
+        attn_ws = (b > attn_ws ? b : attn_ws) + kAttnTicketBytes;
+    }
     LLM_HIP(m->act[0].alloc(attn_ws + 64), "hipMalloc(attention scratch)");
+    LLM_HIP(hipMemset(m->act[0].p, 0, kAttnTicketBytes), "hipMemset(attention tickets)");
     if (!m->stream) LLM_HIP(hipStreamCreate(&m->stream), "hipStreamCreate");
     if (m->step_graph) {
         (void)hipGraphExecDestroy(m->step_graph);
         m->step_graph = nullptr;
     }
     LLM_HIP(m->state.alloc(256), "hipMalloc");
+    if (c.batch <= (int)(kArgmaxTicketBytes / 4)) {
+        LLM_HIP(m->argmax_ws.alloc(argmax_workspace_bytes(c.batch)), "hipMalloc");
+        LLM_HIP(hipMemset(m->argmax_ws.p, 0, kArgmaxTicketBytes), "hipMemset");
+    }
     LLM_HIP(m->record.alloc(((size_t)c.context + 1) * c.batch * 4), "hipMalloc");  // a graph keeps its address
     LLM_HIP(m->qkv.alloc((size_t)c.batch * (qd + 2 * kvd) * 4), "hipMalloc");
     m->fast = rmsnorm_q4act_ok(c.embed) && c.head_dim % 2 == 0;
@@ -549,7 +566,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
     mi355x_status st = forward(*m, n_prompt);
     if (!st) st = head(*m, m->x.as<float>() + (n_prompt - 1) * c.embed, B, n_prompt * c.embed);
     if (!st) {
-        hipError_t e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>(), m->stream);
+        hipError_t e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>(), m->argmax_ws.p, m->stream);
         if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: argmax: %s", hipGetErrorName(e));
     }
     if (!st) (void)hipEventRecord(e1, m->stream);
@@ -564,7 +581,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
         auto one_step = [&]() -> mi355x_status {
             if (mi355x_status s2 = step_fast(*m)) return s2;
             if (mi355x_status s2 = head(*m, m->x.as<float>(), B, c.embed)) return s2;
-            LLM_HIP(argmax(m->logits.as<float>(), B, c.vocab, m->next_tok.as<int32_t>(), m->stream), "argmax");
+            LLM_HIP(argmax(m->logits.as<float>(), B, c.vocab, m->next_tok.as<int32_t>(), m->argmax_ws.p, m->stream), "argmax");
             LLM_HIP(advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 1, m->stream), "advance");
             return MI355X_OK;
         };
@@ -605,7 +622,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
         st = forward(*m, 1);
         if (!st) st = head(*m, m->x.as<float>(), B, c.embed);
         if (!st) {
-            e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>() + t * B, m->stream);
+            e = argmax(m->logits.as<float>(), B, c.vocab, picked.as<int32_t>() + t * B, m->argmax_ws.p, m->stream);
             if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: argmax: %s", hipGetErrorName(e));
         }
     }
