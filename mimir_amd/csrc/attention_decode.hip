@@ -52,6 +52,10 @@ __device__ __forceinline__ float group16_sum(float v) {
     return v;
 }
 
+// Stores and loads that are coherent across the device on their own.
+__device__ __forceinline__ void coherent_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float coherent_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
 // FPL consecutive elements of a cache row as floats.
 template <typename KV, int FPL>
 __device__ __forceinline__ void load_row(const KV* p, float out[FPL]) {
@@ -208,33 +212,39 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     float M = red[g], L = red[kHeads + g];
 
     if (nsplit > 1) {
+        // The shares travel between workgroups (and so between the L2 caches of
+        // the chip's dies) through stores and loads that are coherent at device
+        // scope by themselves (relaxed atomics: write-through stores, loads that
+        // bypass stale lines), so no cache-wide write-back or invalidation is
+        // needed. Ordering: every thread's stores have completed (the counters
+        // are waited on, then the barrier) before thread 0 takes the ticket, and
+        // the combining loads are issued only after the last ticket is known.
         if (g < ng) {
             float* w = ws + (((int64_t)b * p.H + h) * nsplit + split) * (D + 2);
             if (lane == 0) {
-                w[0] = M;
-                w[1] = L;
+                coherent_store(w, M);
+                coherent_store(w + 1, L);
             }
 #pragma unroll
-            for (int c = 0; c < OPL; c++) w[2 + lane + 64 * c] = r[c];
+            for (int c = 0; c < OPL; c++) coherent_store(w + 2 + lane + 64 * c, r[c]);
         }
-        // the last workgroup of these heads to get here combines the shares
-        __threadfence();
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (tid == 0) {
             uint32_t* ctr = counters + (int64_t)b * gridDim.y + blockIdx.y;
-            uint32_t ticket = atomicAdd(ctr, 1u);
+            uint32_t ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = ticket == (uint32_t)(nsplit - 1);
-            if (s_last) *ctr = 0;  // for the next launch
+            if (s_last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
         }
         __syncthreads();
         if (!s_last) return;
-        __threadfence();
+        // the last workgroup of these heads to get here combines the shares
         float* fs = osl + g * 64;  // factor of share s of head g
         float f = 0.f, ls = 0.f, ms = -__builtin_inff();
         const float* w0 = ws + ((int64_t)b * p.H + h) * nsplit * (D + 2);
         if (g < ng && lane < nsplit) {
-            ms = w0[lane * (D + 2)];
-            ls = w0[lane * (D + 2) + 1];
+            ms = coherent_load(w0 + lane * (D + 2));
+            ls = coherent_load(w0 + lane * (D + 2) + 1);
         }
         M = wave_max(ms);
         if (ls != 0.f && M > -__builtin_inff()) f = __builtin_expf(ms - M);
@@ -244,10 +254,20 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 #pragma unroll
         for (int c = 0; c < OPL; c++) r[c] = 0.f;
         if (g < ng) {
-            for (int s = 0; s < nsplit; s++) {
-                float fsv = fs[s];
+            for (int s0 = 0; s0 < nsplit; s0 += 8) {  // eight shares' loads in flight
+                float t[8][OPL];
 #pragma unroll
-                for (int c = 0; c < OPL; c++) r[c] = fmaf(w0[s * (D + 2) + 2 + lane + 64 * c], fsv, r[c]);
+                for (int u = 0; u < 8; u++) {
+                    const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;
+#pragma unroll
+                    for (int c = 0; c < OPL; c++) t[u][c] = coherent_load(w0 + s * (D + 2) + 2 + lane + 64 * c);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const float fsv = s0 + u < nsplit ? fs[s0 + u] : 0.f;
+#pragma unroll
+                    for (int c = 0; c < OPL; c++) r[c] = fmaf(t[u][c], fsv, r[c]);
+                }
             }
         }
         __syncthreads();  // fs is read; the results go over it

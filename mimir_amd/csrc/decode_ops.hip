@@ -423,21 +423,23 @@ __global__ __launch_bounds__(256) void argmax_split_kernel(const float* __restri
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < 4; w++) argmax_better(best, at, bv[w], bi[w]);
-        cand_v[r * kArgmaxBlocks + blockIdx.x] = best;
-        cand_i[r * kArgmaxBlocks + blockIdx.x] = at;
-        __threadfence();
-        uint32_t ticket = atomicAdd(&tickets[r], 1u);
+        // candidates cross between workgroups through stores and loads that are
+        // coherent at device scope on their own; the stores have completed
+        // before the ticket is taken
+        __hip_atomic_store(&cand_v[r * kArgmaxBlocks + blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&cand_i[r * kArgmaxBlocks + blockIdx.x], at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);
+        uint32_t ticket = __hip_atomic_fetch_add(&tickets[r], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = ticket == (uint32_t)(nblk - 1);
-        if (s_last) tickets[r] = 0;
+        if (s_last) __hip_atomic_store(&tickets[r], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!s_last || threadIdx.x >= 64) return;
-    __threadfence();
     best = -__builtin_inff();
     at = 0x7fffffff;
     if ((int)threadIdx.x < nblk) {
-        best = cand_v[r * kArgmaxBlocks + threadIdx.x];
-        at = cand_i[r * kArgmaxBlocks + threadIdx.x];
+        best = __hip_atomic_load(&cand_v[r * kArgmaxBlocks + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        at = __hip_atomic_load(&cand_i[r * kArgmaxBlocks + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {

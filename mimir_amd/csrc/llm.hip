@@ -262,6 +262,7 @@ static mi355x_status step_fast(Model& m) {
     at.scale = 1.0 / std::sqrt((double)c.head_dim);
     at.causal = 0; at.causal_offset = 0;
     at.dyn_k = pos;  // position p holds p keys before this step's own
+    at.k = m.keys[0].p; at.v = m.values[0].p;  // every layer's caches are allocated alike
     const bool one_launch = attention_decode_ok(at, c.context);
     if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
