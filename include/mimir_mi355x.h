@@ -103,6 +103,17 @@ MI355X_API size_t mi355x_act_bytes(int dtype, int64_t K);
 MI355X_API mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
 MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The same product for prompt-sized M with bfloat16 activations, as
+ * Tensor.MatMulT computes it for a half-precision x and a block-quantized w
+ * (tensor/quant.go:45-48: x cast to float32, the product accumulated in float32,
+ * one rounding to x's dtype): X [M, K] bfloat16 with rows x_row_stride elements
+ * apart, W [N, K] Q4_0, Y [M, N] contiguous of out_dtype MI355X_BF16 (the
+ * reference's result) or MI355X_F32 (the same sums before the rounding). K a
+ * multiple of 64 runs on the matrix cores; other shapes through the decode
+ * kernels. */
+MI355X_API mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K,
+                                           int64_t x_row_stride, int out_dtype, void* stream);
+
 /* The fused products of a decoding step, over converted activations (Q4_0
  * weights that qualify for mi355x_qgemv_act). The reference fuses the same
  * products on its CPU path by concatenating the weights (fusedFor,
@@ -209,6 +220,7 @@ MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* promp
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
+ * "qgemm.path" = 1 makes mi355x_qgemm_bf16 take its general route for every shape.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).
  * "llama.step" chooses how mi355x_llama_generate runs its decoding steps: 0 the

@@ -57,6 +57,7 @@ SYMBOLS = {
     "mi355x_llama_logits": (C.c_uint32, [_vp, _vp, _i64, _int, _vp]),
     "mi355x_llama_generate": (C.c_uint32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "mi355x_tune": (C.c_uint32, [C.c_char_p, _int]),
+    "mi355x_qgemm_bf16": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "mi355x_timed_begin": (C.c_uint32, [_int]),
     "mi355x_timed_end": (C.c_uint32, [_vp, _vp]),
     "mi355x_stream_read": (C.c_uint32, [_vp, _sz, _vp, _int, _int, _vp]),

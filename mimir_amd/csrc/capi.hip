@@ -53,6 +53,9 @@ struct DeviceState {
     // Partial results of split attention, grown and shared likewise.
     void* attn = nullptr;
     size_t attn_bytes = 0;
+    // Float32 copies of activations and results for qgemm_bf16's general route.
+    void* gemm = nullptr;
+    size_t gemm_bytes = 0;
     // Tickets and candidates of the split argmax.
     void* argmax = nullptr;
     size_t argmax_bytes = 0;
@@ -61,6 +64,7 @@ struct DeviceState {
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 int g_tune_q4[5] = {0, 0, 0, 0, 0};
+int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
 thread_local std::vector<hipEvent_t> t_events;
@@ -128,6 +132,21 @@ mi355x_status attn_scratch(size_t bytes, void** out) {
         s->attn_bytes = want;
     }
     *out = s->attn;
+    return MI355X_OK;
+}
+
+mi355x_status gemm_scratch(size_t bytes, void** out) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (s->gemm_bytes < bytes) {
+        void* p = nullptr;
+        HIP_TRY(hipMalloc(&p, bytes), "hipMalloc(gemm scratch)");
+        if (s->gemm) HIP_TRY(hipFree(s->gemm), "hipFree(gemm scratch)");
+        s->gemm = p;
+        s->gemm_bytes = bytes;
+    }
+    *out = s->gemm;
     return MI355X_OK;
 }
 
@@ -237,6 +256,43 @@ mi355x_status mi355x_sync(void* stream) {
         if (bits & mimir::kErrIndex) return fail(MI355X_ERR_INDEX, "mi355x: a gather read an index out of range");
         return fail(MI355X_ERR_INTERNAL, "mi355x: device error bits %#x", bits);
     }
+    return MI355X_OK;
+}
+
+// Tensor.MatMulT with bfloat16 activations (tensor/quant.go:45-48): float32
+// product, one rounding to the output's dtype.
+mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride,
+                                int out_dtype, void* stream) {
+    if (dtype != MI355X_Q4_0) return fail(MI355X_ERR_DTYPE, "mi355x: qgemm_bf16 by weights of dtype %d (Q4_0 only)", dtype);
+    if (out_dtype != MI355X_BF16 && out_dtype != MI355X_F32) return fail(MI355X_ERR_DTYPE, "mi355x: qgemm_bf16 into dtype %d", out_dtype);
+    if (M < 0 || N < 0 || K < 0 || K % 32 != 0)
+        return fail(MI355X_ERR_INTERNAL, "mi355x: qgemm_bf16 of [%lld, %lld] by [%lld, %lld] in blocks of 32", (long long)M, (long long)K,
+                    (long long)N, (long long)K);
+    if (M == 0 || N == 0) return MI355X_OK;
+    if (!W || !X || !Y) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemm_bf16: null pointer");
+    if (M > 65535 || N > (int64_t)1 << 24 || K > (int64_t)1 << 24)
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemm_bf16 of %lld rows by [%lld, %lld]: too large", (long long)M, (long long)N, (long long)K);
+    if (M > 1 && x_row_stride < K) return fail(MI355X_ERR_SHAPE, "mi355x: qgemm_bf16: rows of x %lld apart overlap (K = %lld)", (long long)x_row_stride, (long long)K);
+    hipStream_t st = (hipStream_t)stream;
+    const bool f32 = out_dtype == MI355X_F32;
+    if (K == 0) {
+        HIP_TRY(mimir::fill_u32(Y, 0, f32 ? M * N : (M * N + 1) / 2, st), "launch fill");
+        return MI355X_OK;
+    }
+    void* ws;
+    if (g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
+        if (mi355x_status s2 = act_scratch(mimir::qgemm_q4_0_workspace_bytes(M, K), &ws)) return s2;
+        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, ws, st), "launch qgemm_q4_0");
+        return MI355X_OK;
+    }
+    // any other shape: the activations as float32 through the decode kernels, then one rounding
+    const size_t xb = ((size_t)M * K * 4 + 255) & ~(size_t)255, yb = ((size_t)M * N * 4 + 255) & ~(size_t)255;
+    if (mi355x_status s2 = gemm_scratch(xb + yb, &ws)) return s2;
+    float* xf = (float*)ws;
+    float* yf = f32 ? (float*)Y : (float*)((uint8_t*)ws + xb);
+    HIP_TRY(mimir::bf16_rows_to_f32(X, xf, M, K, x_row_stride, st), "launch cast");
+    if (mi355x_status s2 = mi355x_qgemv(dtype, W, xf, yf, M, N, K, K, stream)) return s2;
+    if (!f32) HIP_TRY(mimir::f32_to_bf16(yf, Y, M * N, st), "launch cast");
     return MI355X_OK;
 }
 
@@ -516,6 +572,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
             g_tune_q4[i] = value;
             return MI355X_OK;
         }
+    if (key && strcmp(key, "qgemm.path") == 0) {
+        g_tune_gemm = value;
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "attention.path") == 0) {
         g_tune_attn = value;
         return MI355X_OK;

@@ -1,0 +1,178 @@
+"""The prompt-sized Q4_0 product with bfloat16 activations on the matrix cores,
+through the C ABI, against the oracle's restatement of Tensor.MatMulT for a
+half x and a block-quantized w (tensor/quant.go:45-48): float32 product over
+dequantized weights, one rounding to bfloat16.
+
+The device sums in another order (one Q4_0 block at a time on the matrix cores,
+then 128 scaled block sums), so its float32 result differs from the oracle's in
+the last bits, and its bfloat16 result differs where such a difference crosses a
+rounding boundary: by one unit in the last place of bfloat16, at a small share of
+the outputs. The float32 output is held to 2e-5 of max(1, |want|) (the bound asked
+for is 1e-3)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from mimir_amd import capi
+from tests import gpu
+from tests.helpers import bench_blocks, random_blocks
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_bits(a):
+    return O.f32_to_bf16(np.ascontiguousarray(a, np.float32))
+
+
+def qgemm(w_raw, x_bits, n, k, out_dt=capi.BF16, x_stride=None, w_offset=0):
+    l = gpu.lib()
+    m = x_bits.shape[0]
+    wbuf, wp = gpu.dev_bytes_at(w_raw, w_offset)
+    xs = k if x_stride is None else x_stride
+    xbuf = torch.zeros(m * xs + 8, dtype=torch.int16, device="cuda:0")
+    xbuf[: m * xs].view(m, xs)[:, :k] = torch.from_numpy(x_bits.view(np.int16)).to("cuda:0")
+    if out_dt == capi.BF16:
+        y = torch.full((m, n), -1, dtype=torch.int16, device="cuda:0")
+    else:
+        y = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(l.mi355x_qgemm_bf16(capi.Q4_0, wp, xbuf.data_ptr(), y.data_ptr(), m, n, k, xs, out_dt, gpu.stream()))
+    gpu.sync()
+    out = y.cpu().numpy()
+    return out.view(np.uint16) if out_dt == capi.BF16 else out
+
+
+def reference_f32(w_raw, x_bits, n, k):
+    """The float32 sums before the rounding: the oracle's product of float32
+    activations with the dequantized weights."""
+    return O.qmatmul(O.Q4_0, w_raw, O.bf16_to_f32(x_bits), n, k)
+
+
+def f32_bound(w_raw, x_bits, n, k):
+    """2e-6 of sum_k |x| |w|: random scales span binary16's range, so terms of
+    very different size cancel, and the error of a float32 sum goes with the
+    size of its terms, not of its result (the reference's own sum is as far
+    from the exact one)."""
+    wf = np.abs(O.dequantize(O.Q4_0, w_raw).reshape(n, k).astype(np.float64))
+    mag = np.abs(O.bf16_to_f32(x_bits).astype(np.float64)) @ wf.T
+    return np.maximum(2e-6 * mag, 1e-30)
+
+
+def check_f32(got32, want_f32, bound, what=""):
+    err = np.abs(got32.astype(np.float64) - want_f32)
+    worst = float((err / bound).max())
+    assert worst <= 1.0, (what, worst, float(err.max()))
+
+
+def check_bf16(got, want_bits, bound):
+    """Equal, or apart by one bfloat16 step (the float32 sums differ in their
+    last bits, which now and then straddle a rounding boundary) plus what the
+    float32 sums themselves may differ by; few outputs differ at all."""
+    g = O.bf16_to_f32(got).astype(np.float64); w = O.bf16_to_f32(want_bits).astype(np.float64)
+    differ = got != want_bits
+    ulp = np.maximum(np.abs(w), 2.0 ** -126) * 2.0 ** -7
+    over = np.abs(g - w) - (ulp * 1.01 + 2 * bound)
+    assert np.all(over[differ] <= 0), float(over[differ].max())
+    assert differ.mean() <= 0.01, float(differ.mean())
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 128, 64), (32, 128, 128), (70, 200, 192), (1, 130, 4096), (200, 384, 1024), (129, 257, 320)])
+def test_small_and_ragged_shapes(m, n, k):
+    rng = np.random.default_rng(m * 7 + n)
+    w = random_blocks(rng, O.Q4_0, n * k)
+    x = bf16_bits(rng.normal(size=(m, k)))
+    gpu.say(f"qgemm_bf16 {m}x{k} by {n}x{k}")
+    want_f32 = reference_f32(w, x, n, k)
+    got32 = qgemm(w, x, n, k, capi.F32)
+    bound = f32_bound(w, x, n, k)
+    check_f32(got32, want_f32, bound)
+    got = qgemm(w, x, n, k)
+    check_bf16(got, O.q4_0_matmul_bf16(w, x, n, k), bound)
+    # strided rows of x, weights at a 2-byte aligned address
+    got2 = qgemm(w, x, n, k, x_stride=k + 24, w_offset=6)
+    assert np.array_equal(got2, got)
+
+
+def test_general_route_for_other_shapes_and_agreement():
+    """K that is no multiple of 64 goes through the decode kernels; both routes
+    agree on a shape both take."""
+    l = gpu.lib()
+    rng = np.random.default_rng(3)
+    m, n, k = 9, 70, 96
+    w = random_blocks(rng, O.Q4_0, n * k); x = bf16_bits(rng.normal(size=(m, k)))
+    gpu.say("qgemm_bf16 general route, K = 96")
+    want_f32 = reference_f32(w, x, n, k)
+    got32 = qgemm(w, x, n, k, capi.F32)
+    bound = f32_bound(w, x, n, k)
+    check_f32(got32, want_f32, bound)
+    check_bf16(qgemm(w, x, n, k), O.q4_0_matmul_bf16(w, x, n, k), bound)
+    m, n, k = 40, 256, 256
+    w = random_blocks(rng, O.Q4_0, n * k); x = bf16_bits(rng.normal(size=(m, k)))
+    fast = qgemm(w, x, n, k, capi.F32)
+    try:
+        capi.check(l.mi355x_tune(b"qgemm.path", 1))
+        slow = qgemm(w, x, n, k, capi.F32)
+    finally:
+        capi.check(l.mi355x_tune(b"qgemm.path", 0))
+    check_f32(fast, slow, f32_bound(w, x, n, k))
+
+
+def test_special_values():
+    """Zero, subnormal and negative scales; activations that span the range of
+    bfloat16; an infinity and a NaN stay in their own rows."""
+    rng = np.random.default_rng(4)
+    m, n, k = 64, 128, 128
+    w = random_blocks(rng, O.Q4_0, n * k).reshape(-1, 18)
+    for i, bits in enumerate([0x0000, 0x8000, 0x0001, 0x83ff, 0xbc00, 0x7bff]):
+        w[i::7, 0] = bits & 0xff; w[i::7, 1] = bits >> 8
+    w = w.reshape(-1)
+    xf = rng.normal(size=(m, k)).astype(np.float32)
+    xf[1] *= 1e-30; xf[2] *= 1e20; xf[3, 5] = 0.0; xf[4] = 0.0
+    x = bf16_bits(xf)
+    # keep the largest scale out of the huge row's way: its sums must stay finite for the comparison
+    gpu.say("qgemm_bf16 special values")
+    want_f32 = reference_f32(w, x, n, k)
+    got32 = qgemm(w, x, n, k, capi.F32)
+    assert np.isfinite(want_f32).all() and np.isfinite(got32).all()
+    check_f32(got32, want_f32, f32_bound(w, x, n, k))
+    xf[5, 7] = np.inf; xf[6, 9] = np.nan
+    got32 = qgemm(w, bf16_bits(xf), n, k, capi.F32)
+    assert not np.isfinite(got32[5]).any() and np.isnan(got32[6]).all()
+    assert np.array_equal(got32[:5], qgemm(w, x, n, k, capi.F32)[:5])
+
+
+@pytest.mark.parametrize("n", [4096, 14336])
+def test_prefill_shapes(n):
+    """M = 512 tokens at the 8B model's shapes, weights and activations as the
+    configurations draw them. The oracle takes a band of output columns (rows of
+    W) at N = 14336 to stay within seconds; M = 2048 is checked against the M =
+    512 result row for row, rows being independent."""
+    rng = np.random.default_rng(0)
+    m, k = 512, 4096
+    w = bench_blocks(rng, O.Q4_0, n * k)
+    x = bf16_bits(rng.normal(size=(m, k)))
+    gpu.say(f"qgemm_bf16 512x4096 by {n}x4096")
+    got = qgemm(w, x, n, k)
+    got32 = qgemm(w, x, n, k, capi.F32)
+    lo, hi = (0, n) if n == 4096 else (5000, 7048)
+    wb = w.reshape(n, -1)[lo:hi].reshape(-1)
+    want_f32 = reference_f32(wb, x, hi - lo, k)
+    err = np.abs(got32[:, lo:hi] - want_f32)
+    assert np.all(err <= 2e-5 * np.maximum(1, np.abs(want_f32))), float(err.max())  # the bound asked for is 1e-3
+    check_bf16(got[:, lo:hi], O.q4_0_matmul_bf16(wb, x, hi - lo, k), 2e-5 * np.maximum(1, np.abs(want_f32)))
+    if n == 4096:
+        gpu.say("qgemm_bf16 2048x4096 by 4096x4096")
+        x4 = np.concatenate([x, x[::-1], x, x[::-1]], axis=0)
+        got4 = qgemm(w, x4, n, k)
+        assert np.array_equal(got4[:512], got) and np.array_equal(got4[512:1024], got[::-1]) and np.array_equal(got4[1024:1536], got)
+
+
+def test_errors():
+    l = gpu.lib()
+    z = torch.zeros(4096, dtype=torch.int16, device="cuda:0")
+    p = z.data_ptr()
+    assert l.mi355x_qgemm_bf16(capi.Q8_0, p, p, p, 2, 32, 64, 64, capi.BF16, gpu.stream()) == capi.ERR_DTYPE
+    assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 64, 64, capi.F16, gpu.stream()) == capi.ERR_DTYPE
+    assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 48, 48, capi.BF16, gpu.stream()) == capi.ERR_INTERNAL
+    assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 64, 32, capi.BF16, gpu.stream()) == capi.ERR_SHAPE
+    capi.check(l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 0, 32, 64, 64, capi.BF16, gpu.stream()))
