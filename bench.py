@@ -229,6 +229,36 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256):
             "first_tokens": out[0, :8].tolist()}
 
 
+def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096), (2048, 14336)), k=4096, iters=50):
+    """The prompt-sized Q4_0 product (bfloat16 in and out) on the matrix cores:
+    TFLOP/s (2 M N K) of the whole call, between HIP events on its stream,
+    against the dense bfloat16 peak."""
+    out = {}
+    rng = np.random.default_rng(0)
+    st = torch.cuda.Stream()
+    for m, n in shapes:
+        w = torch.from_numpy(bench_blocks_q4_0(rng, n * k)).to("cuda:0")
+        x = torch.randn(m, k, device="cuda:0").to(torch.bfloat16)
+        y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+        torch.cuda.synchronize()
+        with torch.cuda.stream(st):
+            call = lambda: capi.check(lib.mi355x_qgemm_bf16(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, capi.BF16, st.cuda_stream))
+            for _ in range(5):
+                call()
+            st.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for _ in range(iters):
+                call()
+            e1.record(st)
+            st.synchronize()
+        us = e0.elapsed_time(e1) / iters * 1e3
+        tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+        out[f"M{m}_N{n}_K{k}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_peak": round(tf / 2500.0, 4)}
+        del w, x, y
+    return out
+
+
 def cpu_baseline(n, k, seconds=2.0):
     """The reference's CPU route for a Q4_0 linear, restated by the oracle:
     weights decoded to float32 once (untimed), then the float32 GEMV over all
@@ -265,6 +295,7 @@ def main():
     ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
     ap.add_argument("--counters", type=int, default=0, metavar="N",
                     help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
+    ap.add_argument("--gemm", action="store_true", help="also time the prompt-sized Q4_0 product on the matrix cores (M = 512, 2048)")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
@@ -335,6 +366,8 @@ def main():
         extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
         out["extra"] = extra
     del g
+    if args.gemm:
+        out["prefill_gemm"] = gemm_bench(lib, capi, torch)
     if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch)
     if not args.no_cpu:

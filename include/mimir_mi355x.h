@@ -108,9 +108,9 @@ MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* 
  * (tensor/quant.go:45-48: x cast to float32, the product accumulated in float32,
  * one rounding to x's dtype): X [M, K] bfloat16 with rows x_row_stride elements
  * apart, W [N, K] Q4_0, Y [M, N] contiguous of out_dtype MI355X_BF16 (the
- * reference's result) or MI355X_F32 (the same sums before the rounding). K a
- * multiple of 64 runs on the matrix cores; other shapes through the decode
- * kernels. */
+ * reference's result) or MI355X_F32 (the same sums before the rounding). Runs
+ * on the matrix cores when X is 16-byte aligned with rows a multiple of 8
+ * elements apart; otherwise through the decode kernels. */
 MI355X_API mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K,
                                            int64_t x_row_stride, int out_dtype, void* stream);
 

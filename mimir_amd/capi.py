@@ -83,9 +83,10 @@ def load() -> C.CDLL:
     """Loads the library and declares every symbol; raises if it is not built."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise FileNotFoundError(f"{LIB_PATH} is not built: run `python -m mimir_amd.build`")
-        lib = C.CDLL(LIB_PATH)
+        path = os.environ.get("MIMIR_MI355X_LIB") or LIB_PATH  # as the reference's loaders take a path from the environment
+        if not os.path.exists(path):
+            raise FileNotFoundError(f"{path} is not built: run `python -m mimir_amd.build`")
+        lib = C.CDLL(path)
         for name, (res, args) in SYMBOLS.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is missing
             fn.restype, fn.argtypes = res, args

@@ -281,8 +281,7 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     }
     void* ws;
     if (g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
-        if (mi355x_status s2 = act_scratch(mimir::qgemm_q4_0_workspace_bytes(M, K), &ws)) return s2;
-        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, ws, st), "launch qgemm_q4_0");
+        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
     // any other shape: the activations as float32 through the decode kernels, then one rounding

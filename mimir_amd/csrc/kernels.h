@@ -137,11 +137,10 @@ size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st);
 
 // Prompt-sized Q4_0 product on the matrix cores (qgemm_q4_0.hip): X [M, K]
-// bfloat16, Y [M, N] bfloat16 or float32. workspace: qgemm_q4_0_workspace_bytes.
+// bfloat16, Y [M, N] bfloat16 or float32.
 bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K, int64_t x_row_stride);
-size_t qgemm_q4_0_workspace_bytes(int64_t M, int64_t K);
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
-                           void* workspace, hipStream_t st);
+                           hipStream_t st);
 hipError_t bf16_rows_to_f32(const void* x, float* y, int64_t M, int64_t K, int64_t x_row_stride, hipStream_t st);
 hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 

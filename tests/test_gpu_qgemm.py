@@ -3,12 +3,11 @@ through the C ABI, against the oracle's restatement of Tensor.MatMulT for a
 half x and a block-quantized w (tensor/quant.go:45-48): float32 product over
 dequantized weights, one rounding to bfloat16.
 
-The device sums in another order (one Q4_0 block at a time on the matrix cores,
-then 128 scaled block sums), so its float32 result differs from the oracle's in
-the last bits, and its bfloat16 result differs where such a difference crosses a
+The device sums in another order (each weight as two bfloat16 halves on the
+matrix cores), so its float32 result differs from the oracle's in the last bits, and its bfloat16 result differs where such a difference crosses a
 rounding boundary: by one unit in the last place of bfloat16, at a small share of
-the outputs. The float32 output is held to 2e-5 of max(1, |want|) (the bound asked
-for is 1e-3)."""
+the outputs. The float32 output is held to 1e-4 of max(1, |want|) at K = 4096 (the
+bound asked for is 1e-3)."""
 import numpy as np
 import pytest
 import torch
@@ -76,7 +75,7 @@ def check_bf16(got, want_bits, bound):
     assert differ.mean() <= 0.01, float(differ.mean())
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 64), (32, 128, 128), (70, 200, 192), (1, 130, 4096), (200, 384, 1024), (129, 257, 320)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 64), (32, 128, 128), (70, 200, 192), (1, 130, 4096), (200, 384, 1024), (129, 257, 320), (33, 65, 96)])
 def test_small_and_ragged_shapes(m, n, k):
     rng = np.random.default_rng(m * 7 + n)
     w = random_blocks(rng, O.Q4_0, n * k)
@@ -94,18 +93,18 @@ def test_small_and_ragged_shapes(m, n, k):
 
 
 def test_general_route_for_other_shapes_and_agreement():
-    """K that is no multiple of 64 goes through the decode kernels; both routes
-    agree on a shape both take."""
+    """Rows of x that are not 16-byte aligned go through the decode kernels; both
+    routes agree on a shape both take."""
     l = gpu.lib()
     rng = np.random.default_rng(3)
     m, n, k = 9, 70, 96
     w = random_blocks(rng, O.Q4_0, n * k); x = bf16_bits(rng.normal(size=(m, k)))
-    gpu.say("qgemm_bf16 general route, K = 96")
+    gpu.say("qgemm_bf16 general route, rows of x 99 apart")
     want_f32 = reference_f32(w, x, n, k)
-    got32 = qgemm(w, x, n, k, capi.F32)
+    got32 = qgemm(w, x, n, k, capi.F32, x_stride=k + 3)
     bound = f32_bound(w, x, n, k)
     check_f32(got32, want_f32, bound)
-    check_bf16(qgemm(w, x, n, k), O.q4_0_matmul_bf16(w, x, n, k), bound)
+    check_bf16(qgemm(w, x, n, k, x_stride=k + 3), O.q4_0_matmul_bf16(w, x, n, k), bound)
     m, n, k = 40, 256, 256
     w = random_blocks(rng, O.Q4_0, n * k); x = bf16_bits(rng.normal(size=(m, k)))
     fast = qgemm(w, x, n, k, capi.F32)
@@ -158,8 +157,9 @@ def test_prefill_shapes(n):
     wb = w.reshape(n, -1)[lo:hi].reshape(-1)
     want_f32 = reference_f32(wb, x, hi - lo, k)
     err = np.abs(got32[:, lo:hi] - want_f32)
-    assert np.all(err <= 2e-5 * np.maximum(1, np.abs(want_f32))), float(err.max())  # the bound asked for is 1e-3
-    check_bf16(got[:, lo:hi], O.q4_0_matmul_bf16(wb, x, hi - lo, k), 2e-5 * np.maximum(1, np.abs(want_f32)))
+    # two float32 sums of 4096 terms in different orders; the bound asked for is 1e-3
+    assert np.all(err <= 1e-4 * np.maximum(1, np.abs(want_f32))), float(err.max())
+    check_bf16(got[:, lo:hi], O.q4_0_matmul_bf16(wb, x, hi - lo, k), 1e-4 * np.maximum(1, np.abs(want_f32)))
     if n == 4096:
         gpu.say("qgemm_bf16 2048x4096 by 4096x4096")
         x4 = np.concatenate([x, x[::-1], x, x[::-1]], axis=0)
