@@ -216,6 +216,56 @@ MI355X_API mi355x_status mi355x_llama_logits(void* model, const int32_t* tokens,
  * prompt pass (with the first token) and of the n_new - 1 decoding steps. */
 MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t n_prompt, int64_t n_new, int32_t* out_tokens, double* seconds);
 
+/* ---- the reference's operator interface for this path ---------------------------
+ * backend.Backend and backend.Batcher (backend/backend.go:141-171,
+ * backend/batch.go:46-52) over this library: buffers that belong to their
+ * backend, kernels described by an operation, the output's dtype and shape, and
+ * one view per input (backend.Kernel and backend.View, backend.go:174-180,
+ * view.go:23-27), checked by CheckRun (check.go:29-74) before they run.
+ * Operations: MI355X_OP_QMATMUL (In[0] float32 [..., K] through any view, In[1]
+ * block-quantized [N, K] read contiguously from a block boundary),
+ * MI355X_OP_CAST and MI355X_OP_GATHER of a block-quantized In[0] through any
+ * view, MI355X_OP_ATTENTION (q, k, v; the output holds the result [B..., H, Q, D]
+ * followed by the logsumexp [B..., H, Q]). Anything else fails with
+ * MI355X_ERR_INTERNAL. Errors: a foreign or freed buffer is MI355X_ERR_DTYPE, a
+ * size that does not match MI355X_ERR_SHAPE, a gather index out of range
+ * MI355X_ERR_INDEX at the next sync (rocm_linux.go:275-375).
+ * mi355x_backend_last_error has the message. A batch that is run again with the
+ * same kernels and buffers is recorded into a HIP graph on its second run and
+ * replayed from its third (rocm/batch_linux.go:115-203). */
+#define MI355X_MAX_RANK 8
+#define MI355X_MAX_INPUTS 4
+enum { MI355X_OP_CAST = 1, MI355X_OP_GATHER = 2, MI355X_OP_QMATMUL = 3, MI355X_OP_ATTENTION = 4 };
+typedef struct mi355x_view {
+    int32_t rank;
+    int64_t shape[MI355X_MAX_RANK], strides[MI355X_MAX_RANK]; /* in elements */
+    int64_t offset;
+} mi355x_view;
+typedef struct mi355x_kernel {
+    int32_t op, dtype, rank;
+    int64_t shape[MI355X_MAX_RANK];
+    int32_t n_in;
+    mi355x_view in[MI355X_MAX_INPUTS];
+    int32_t axis;          /* Attrs.Axis */
+    double scale;          /* Attrs.Scale */
+    int32_t causal;        /* Attrs.Causal */
+    int64_t causal_offset; /* Attrs.CausalOffset */
+} mi355x_kernel;
+MI355X_API size_t mi355x_backend_last_error(char* buf, size_t n);
+MI355X_API mi355x_status mi355x_backend_open(int device, void** backend);
+MI355X_API mi355x_status mi355x_backend_close(void* backend);
+MI355X_API mi355x_status mi355x_backend_alloc(void* backend, int dtype, int64_t n, void** buffer);
+MI355X_API mi355x_status mi355x_backend_free(void* backend, void* buffer);
+MI355X_API mi355x_status mi355x_backend_upload(void* backend, void* dst, const void* src, size_t bytes);
+MI355X_API mi355x_status mi355x_backend_download(void* backend, void* dst, size_t bytes, void* src);
+MI355X_API mi355x_status mi355x_backend_sync(void* backend);
+MI355X_API mi355x_status mi355x_backend_run(void* backend, const mi355x_kernel* k, void* const* outs, int n_outs, void* const* ins, int n_ins);
+MI355X_API mi355x_status mi355x_batch_new(const mi355x_kernel* kernels, int n, void* const* const* outs, const int* n_outs,
+                                          void* const* const* ins, const int* n_ins, void** batch);
+MI355X_API mi355x_status mi355x_batch_free(void* batch);
+MI355X_API mi355x_status mi355x_backend_run_batch(void* backend, void* batch);
+MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
+
 /* ---- measurement aids (no counterpart in the reference) ---------------------
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces

@@ -57,6 +57,19 @@ SYMBOLS = {
     "mi355x_llama_logits": (C.c_uint32, [_vp, _vp, _i64, _int, _vp]),
     "mi355x_llama_generate": (C.c_uint32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "mi355x_tune": (C.c_uint32, [C.c_char_p, _int]),
+    "mi355x_backend_last_error": (_sz, [C.c_char_p, _sz]),
+    "mi355x_backend_open": (C.c_uint32, [_int, _vp]),
+    "mi355x_backend_close": (C.c_uint32, [_vp]),
+    "mi355x_backend_alloc": (C.c_uint32, [_vp, _int, _i64, _vp]),
+    "mi355x_backend_free": (C.c_uint32, [_vp, _vp]),
+    "mi355x_backend_upload": (C.c_uint32, [_vp, _vp, _vp, _sz]),
+    "mi355x_backend_download": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "mi355x_backend_sync": (C.c_uint32, [_vp]),
+    "mi355x_backend_run": (C.c_uint32, [_vp, _vp, _vp, _int, _vp, _int]),
+    "mi355x_batch_new": (C.c_uint32, [_vp, _int, _vp, _vp, _vp, _vp, _vp]),
+    "mi355x_batch_free": (C.c_uint32, [_vp]),
+    "mi355x_backend_run_batch": (C.c_uint32, [_vp, _vp]),
+    "mi355x_backend_graph_replays": (_i64, [_vp]),
     "mi355x_qgemm_bf16": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "mi355x_timed_begin": (C.c_uint32, [_int]),
     "mi355x_timed_end": (C.c_uint32, [_vp, _vp]),

@@ -121,6 +121,81 @@ hipError_t gather_rows(int dt, const void* table, int64_t rows, int64_t k, const
     return hipGetLastError();
 }
 
+// ---- reads through views (backend/view.go): element i of the contiguous
+// output is element offset + sum_d coord_d * stride_d of the buffer ---------------
+__device__ __forceinline__ int64_t view_element(const ViewArg& v, int64_t i) {
+    int64_t at = v.offset;
+    for (int d = v.rank - 1; d >= 0; d--) {
+        at += (i % v.shape[d]) * v.strides[d];
+        i /= v.shape[d];
+    }
+    return at;
+}
+
+// OpCast of a block-quantized input read through any view (dequantAt,
+// backend/cpu/quant.go:236-256).
+template <typename T>
+__global__ __launch_bounds__(256) void dequant_view_kernel(int dt, const uint8_t* __restrict__ data, ViewArg v, int64_t n,
+                                                           T* __restrict__ out, int out_dt) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        store_as<T>(out, i, dequant_at(dt, data, view_element(v, i)), out_dt);
+}
+
+hipError_t dequantize_view(int dt, const void* data, const ViewArg& v, int64_t n, void* out, int out_dt, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    int64_t groups = (n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    if (out_dt == kF32)
+        hipLaunchKernelGGL(dequant_view_kernel<float>, dim3((unsigned)groups), dim3(256), 0, st, dt, (const uint8_t*)data, v, n, (float*)out,
+                           out_dt);
+    else
+        hipLaunchKernelGGL(dequant_view_kernel<uint16_t>, dim3((unsigned)groups), dim3(256), 0, st, dt, (const uint8_t*)data, v, n,
+                           (uint16_t*)out, out_dt);
+    return hipGetLastError();
+}
+
+// OpGather of a block-quantized table through views (gatherQuant,
+// backend/cpu/quant.go:296-327): out[m] = table[m with m[axis] = idx[m]]; an
+// index outside the axis sets bit kErrIndex of *err and writes zero.
+__global__ __launch_bounds__(256) void gather_view_kernel(int dt, const uint8_t* __restrict__ table, ViewArg tv, const int32_t* __restrict__ idx,
+                                                          ViewArg iv, int axis, int64_t n, float* __restrict__ out, uint32_t* err) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        // coordinates of i in the output, whose shape is the index view's
+        int64_t rem = i, at = tv.offset;
+        const int64_t j = idx[view_element(iv, i)];
+        bool bad = j < 0 || j >= tv.shape[axis];
+        for (int d = iv.rank - 1; d >= 0; d--) {
+            int64_t c = rem % iv.shape[d];
+            rem /= iv.shape[d];
+            at += (d == axis ? (bad ? 0 : j) : c) * tv.strides[d];
+        }
+        if (bad && err) atomicOr(err, kErrIndex);
+        out[i] = bad ? 0.f : dequant_at(dt, table, at);
+    }
+}
+
+hipError_t gather_view(int dt, const void* table, const ViewArg& tv, const int32_t* idx, const ViewArg& iv, int axis, int64_t n, float* out,
+                       uint32_t* err, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    int64_t groups = (n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(gather_view_kernel, dim3((unsigned)groups), dim3(256), 0, st, dt, (const uint8_t*)table, tv, idx, iv, axis, n, out, err);
+    return hipGetLastError();
+}
+
+// A view of 32-bit elements copied into a contiguous buffer (OpContiguous).
+__global__ __launch_bounds__(256) void copy_view32_kernel(const uint32_t* __restrict__ src, ViewArg v, int64_t n, uint32_t* __restrict__ out) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) out[i] = src[view_element(v, i)];
+}
+
+hipError_t copy_view32(const void* src, const ViewArg& v, int64_t n, void* out, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    int64_t groups = (n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(copy_view32_kernel, dim3((unsigned)groups), dim3(256), 0, st, (const uint32_t*)src, v, n, (uint32_t*)out);
+    return hipGetLastError();
+}
+
 // ---- fill (a kernel, not a memset node, so callers may capture it) ---------
 __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t v, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;

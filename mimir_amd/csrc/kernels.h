@@ -163,6 +163,18 @@ enum : uint32_t { kErrIndex = 1u, kErrInternal = 2u };
 // (kF32, kBF16 or kF16): OpCast of a contiguous view.
 hipError_t dequantize(int dt, const void* data, int64_t first, int64_t n, void* out, int out_dt, hipStream_t st);
 
+// How a kernel reads a buffer (backend.View, backend/view.go:23-27), by value.
+constexpr int kMaxRank = 8;
+struct ViewArg {
+    int rank;
+    int64_t shape[kMaxRank], strides[kMaxRank];
+    int64_t offset;
+};
+hipError_t dequantize_view(int dt, const void* data, const ViewArg& v, int64_t n, void* out, int out_dt, hipStream_t st);
+hipError_t gather_view(int dt, const void* table, const ViewArg& tv, const int32_t* idx, const ViewArg& iv, int axis, int64_t n, float* out,
+                       uint32_t* err, hipStream_t st);
+hipError_t copy_view32(const void* src, const ViewArg& v, int64_t n, void* out, hipStream_t st);
+
 // out[r, :] = dequantized row idx[r] of a [rows, k] table: OpGather on axis 0.
 hipError_t gather_rows(int dt, const void* table, int64_t rows, int64_t k, const int32_t* idx, int64_t n, float* out,
                        uint32_t* err, hipStream_t st);
