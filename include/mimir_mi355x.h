@@ -207,6 +207,10 @@ MI355X_API mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens);
 /* Empties the caches (KVCache.Reset). */
 MI355X_API mi355x_status mi355x_llama_reset(void* model);
 MI355X_API int64_t mi355x_llama_cache_len(void* model);
+/* Loads positions [0, n) of block `layer`'s caches from host arrays [batch,
+ * kv_heads, n, head_dim] of the cache's dtype and makes n the caches' length
+ * (what KVCache.Append would have left, nn/transformer.go:397-423). */
+MI355X_API mi355x_status mi355x_llama_set_cache(void* model, int32_t layer, const void* keys, const void* values, int64_t n);
 /* Model.Logits: runs tokens [batch, n], which follow the positions the caches
  * hold, appends their keys and values, and copies to the host the logits of the
  * last token [batch, vocab], or of every token [batch, n, vocab] if all. */

@@ -53,6 +53,7 @@ SYMBOLS = {
     "mi355x_llama_set_rope_factors": (C.c_uint32, [_vp, _vp, C.c_int32]),
     "mi355x_llama_finalize": (C.c_uint32, [_vp, _i64]),
     "mi355x_llama_reset": (C.c_uint32, [_vp]),
+    "mi355x_llama_set_cache": (C.c_uint32, [_vp, C.c_int32, _vp, _vp, _i64]),
     "mi355x_llama_cache_len": (_i64, [_vp]),
     "mi355x_llama_logits": (C.c_uint32, [_vp, _vp, _i64, _int, _vp]),
     "mi355x_llama_generate": (C.c_uint32, [_vp, _vp, _i64, _i64, _vp, _vp]),

@@ -510,6 +510,29 @@ mi355x_status mi355x_llama_reset(void* model) {
     return MI355X_OK;
 }
 
+// Loads positions [0, n) of one block's caches from the host (keys and values
+// [batch, kv_heads, n, head_dim] in the cache's dtype) and makes n the length
+// of every cache: KVCache contents as a prompt would have left them
+// (nn/transformer.go:348-423), for callers that keep caches of their own.
+mi355x_status mi355x_llama_set_cache(void* model, int32_t layer, const void* keys, const void* values, int64_t n) {
+    using namespace mimir;
+    Model* m = (Model*)model;
+    if (!m || !keys || !values) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama_set_cache: null pointer");
+    const auto& c = m->c;
+    if (!m->ready) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: model is not finalized");
+    if (layer < 0 || layer >= c.layers || n < 0 || n > c.context)
+        return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %lld positions of block %d into caches of %d blocks and %d positions", (long long)n, layer,
+                         c.layers, c.context);
+    const size_t esz = c.cache_dtype == kF32 ? 4 : 2;
+    const size_t row = (size_t)n * c.head_dim * esz, pitch = (size_t)c.context * c.head_dim * esz;
+    if (n > 0) {
+        LLM_HIP(hipMemcpy2D(m->keys[layer].p, pitch, keys, row, row, (size_t)c.batch * c.kv_heads, hipMemcpyHostToDevice), "hipMemcpy2D(keys)");
+        LLM_HIP(hipMemcpy2D(m->values[layer].p, pitch, values, row, row, (size_t)c.batch * c.kv_heads, hipMemcpyHostToDevice), "hipMemcpy2D(values)");
+    }
+    m->cache_len = n;
+    return MI355X_OK;
+}
+
 int64_t mi355x_llama_cache_len(void* model) { return model ? ((Model*)model)->cache_len : -1; }
 
 static mi355x_status check_tokens(Model* m, const int32_t* tokens, int64_t n) {

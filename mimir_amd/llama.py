@@ -51,6 +51,12 @@ class Llama:
     def reset(self):
         capi.check(self.lib.mi355x_llama_reset(self._h))
 
+    def set_cache(self, layer: int, keys, values):
+        """keys, values [batch, kv_heads, n, head_dim] in the cache's dtype
+        (float32, or binary16 bits as uint16)."""
+        k = np.ascontiguousarray(keys); v = np.ascontiguousarray(values)
+        capi.check(self.lib.mi355x_llama_set_cache(self._h, layer, k.ctypes.data, v.ctypes.data, k.shape[2]))
+
     @property
     def cache_len(self) -> int:
         return self.lib.mi355x_llama_cache_len(self._h)
