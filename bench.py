@@ -214,16 +214,31 @@ def build_llama(capi, layers=32, batch=1, context=1024, max_tokens=512, seed=0, 
     return m
 
 
-def decode_bench(capi, layers=32, batch=1, prompt=512, new=256):
+def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0):
     """Whole-model greedy decoding: a prompt of uniform-random token ids, then
-    `new` tokens a sequence. Returns tokens/s of the decoding steps."""
+    `new` tokens a sequence. Returns tokens/s of the decoding steps. With
+    check, the first `check` tokens of sequence 0 are compared with the CPU
+    oracle's greedy decoding of the same model and prompt."""
     t0 = time.perf_counter()
     m = build_llama(capi, layers=layers, batch=batch, context=prompt + new, max_tokens=prompt)
     build_s = time.perf_counter() - t0
     toks = np.random.default_rng(0).integers(0, m.config.vocab, (batch, prompt))
     out, (t_prompt, t_decode) = m.generate(toks, new)
     per_tok_bytes = layers * 218103808 * 0.5625 + 128256 * 4096 * 1.0625
-    return {"layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
+    verdict = {}
+    if check:
+        import oracle as O
+        from oracle import llama as OL
+        c = m.config
+        om = OL.synthetic(OL.Config(arch="llama", embed=c.embed, hidden=c.hidden, layers=c.layers, heads=c.heads, kv_heads=c.kv_heads,
+                                    head_dim=c.head_dim, rope_dim=c.rope_dim, rope_base=c.rope_base, rope_scale=1.0, eps=c.eps,
+                                    vocab=c.vocab, context=c.context), seed=0)
+        want, margins = om.generate(toks[0].tolist(), check, capacity=c.context, cache_dtype=O.F16)
+        got = out[0, :check].tolist()
+        first = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), None)
+        verdict = {"greedy_checked": check, "greedy_identical": sum(a == b for a, b in zip(got, want)), "first_mismatch": first,
+                   "oracle_min_margin": round(min(margins), 4)}
+    return {**verdict,"layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
             "decode_tok_per_s": round(batch * (new - 1) / t_decode, 1), "ms_per_step": round(t_decode / (new - 1) * 1e3, 4),
             "weight_GBps": round(per_tok_bytes / (t_decode / (new - 1)) / 1e9, 1), "build_s": round(build_s, 1),
             "first_tokens": out[0, :8].tolist()}
@@ -299,6 +314,8 @@ def main():
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
+    ap.add_argument("--decode-check", type=int, default=0, metavar="N",
+                    help="compare the first N greedy tokens with the CPU oracle's (minutes of CPU time for the 512-token prompt)")
     ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--decode-batch", type=int, default=1)
     args = ap.parse_args()
@@ -369,7 +386,7 @@ def main():
     if args.gemm:
         out["prefill_gemm"] = gemm_bench(lib, capi, torch)
     if not args.no_decode:
-        out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch)
+        out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n, k, seconds=10.0)
     print(json.dumps(out), flush=True)

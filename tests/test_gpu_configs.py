@@ -1,8 +1,7 @@
 """The benchmark configurations that name a decoder: one random-init layer at
 the 8B model's shape stepping once against a binary16 cache prefilled with
-2048 positions of N(0, 1) values, batch 1 and 8; and the model at its full
-width and vocabulary (fewer layers, so that the CPU oracle finishes in about a
-minute) decoding 64 greedy tokens, which must be the oracle's."""
+2048 positions of N(0, 1) values, batch 1 and 8; and the whole
+32-layer model decoding 64 greedy tokens, which must be the oracle's."""
 import numpy as np
 import pytest
 
@@ -61,25 +60,35 @@ def test_one_layer_step_against_a_prefilled_cache(batch):
     assert toks[:, 0].tolist() == [int(np.argmax(got[b])) for b in range(batch)]
 
 
-def test_full_width_model_64_greedy_tokens():
-    """Embeddings and output Q8_0 over the 128256-token vocabulary, Q4_0 linears,
-    binary16 cache, two layers. The tokens must be the oracle's, except from a
-    step on where the oracle's own two best logits are closer than its float32
-    sums can tell apart (none in this run; the check allows it as the
-    reference's tests do for quantized activations)."""
+def test_whole_model_64_greedy_tokens():
+    """The whole random-init model of the last configuration: 32 layers at full
+    width, embeddings and output Q8_0 over the 128256-token vocabulary, Q4_0
+    linears, binary16 cache, seed 0 with per-tensor seeds. A 128-token prompt
+    (the configuration's 512 takes the CPU oracle minutes) and 64 greedy
+    tokens, which must be the oracle's one for one. Were two of the oracle's
+    logits ever closer than its own float32 sums can tell apart, the
+    comparison would stop there, as the reference's tests allow for quantized
+    activations; in this run the smallest margin is 21."""
     gpu.lib()
-    c = _config(2, 128256, 160, 1, capi.F16)
+    c = _config(32, 128256, 200, 1, capi.F16)
     om = OL.synthetic(_oracle_config(c), seed=0)
     m = Llama(c)
     _upload_synthetic(m, om)
-    m.finalize(64)
-    prompt = np.random.default_rng(0).integers(0, c.vocab, (1, 48))
-    gpu.say("full-width model, 48-token prompt, 64 greedy tokens")
+    m.finalize(128)
+    prompt = np.random.default_rng(0).integers(0, c.vocab, (1, 128))
+    gpu.say("whole model, 128-token prompt, 64 greedy tokens")
     toks, _ = m.generate(prompt, 64)
-    want, margins = om.generate(prompt[0].tolist(), 64, capacity=c.context, cache_dtype=O.F16)
+    caches = om.new_caches(c.context, O.F16)
+    logits = om.logits(prompt[0].tolist(), caches)
     got = toks[0].tolist()
-    for i, (a, w) in enumerate(zip(got, want)):
-        if a != w:
-            assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
+    for i in range(64):
+        if i % 16 == 0:
+            gpu.say(f"oracle step {i}")
+        want = O.argmax(logits)
+        if got[i] != want:
+            top2 = np.partition(logits, -2)[-2:]
+            assert float(top2[1] - top2[0]) < 0.02 * 170.0, (i, got[i], want)
+            assert i >= 8, (i, got[:8])
             break
-    assert got[:8] == want[:8]
+        if i + 1 < 64:
+            logits = om.logits([want], caches)
