@@ -77,6 +77,31 @@ __device__ __forceinline__ void load_row(const KV* p, float out[FPL]) {
     }
 }
 
+// The same, in two steps: the bytes as loaded (so that many rows can be in
+// flight in few registers), and their values.
+template <typename KV, int FPL>
+struct RawRow {
+    uint32_t w[FPL * sizeof(KV) / 4];
+};
+template <typename KV, int FPL>
+__device__ __forceinline__ void load_raw(const KV* p, RawRow<KV, FPL>& r) {
+    constexpr int kBytes = FPL * sizeof(KV);
+    __builtin_memcpy(r.w, __builtin_assume_aligned(p, kBytes >= 16 ? 16 : 8), kBytes);
+}
+template <typename KV, int FPL>
+__device__ __forceinline__ void raw_values(const RawRow<KV, FPL>& r, float out[FPL]) {
+    if constexpr (sizeof(KV) == 4) {
+#pragma unroll
+        for (int i = 0; i < FPL; i++) out[i] = __uint_as_float(r.w[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < FPL / 2; i++) {
+            out[2 * i] = f16_bits_to_f32((uint16_t)(r.w[i] & 0xffffu));
+            out[2 * i + 1] = f16_bits_to_f32((uint16_t)(r.w[i] >> 16));
+        }
+    }
+}
+
 template <typename KV, int FPL>
 __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __restrict__ q, const KV* __restrict__ k,
                                                                const KV* __restrict__ v, float* __restrict__ ws,
@@ -123,22 +148,39 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     const KV* kbase = k + b * p.k_b + (int64_t)hk * p.k_h + part * FPL;
     const KV* vbase = v + b * p.v_b + (int64_t)hk * p.v_h + part * FPL;
 
-    // scores of key j0 + jj, jj = jj0 + 16 u + kg: four rows in flight per thread
-    for (int jj0 = 0; jj0 < nj; jj0 += 4 * kKeyGroups) {
-        float kf[4][FPL];
+    // Rows in flight per thread: key j0 + jj with jj = jj0 + 16 u + kg. The first
+    // batch of keys and of values is requested before anything is computed, so
+    // that a share of up to 16 U keys costs one trip to memory for both.
+    constexpr int U = sizeof(KV) == 2 ? 8 : 4;
+    RawRow<KV, FPL> kraw[U], vraw[U];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            int jj = jj0 + kKeyGroups * u + kg;
-            load_row<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kf[u]);
+    for (int u = 0; u < U; u++) {
+        const int jj = kKeyGroups * u + kg;
+        load_raw<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kraw[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int jj = kKeyGroups * u + kg;
+        load_raw<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vraw[u]);
+    }
+    for (int jj0 = 0; jj0 < nj; jj0 += U * kKeyGroups) {
+        if (jj0 > 0) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int jj = jj0 + kKeyGroups * u + kg;
+                load_raw<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kraw[u]);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            int jj = jj0 + kKeyGroups * u + kg;
+        for (int u = 0; u < U; u++) {
+            const int jj = jj0 + kKeyGroups * u + kg;
+            float kf[FPL];
+            raw_values<KV, FPL>(kraw[u], kf);
 #pragma unroll
             for (int g = 0; g < kHeads; g++) {
                 float s = 0.f;
 #pragma unroll
-                for (int f = 0; f < FPL; f++) s = fmaf(qr[g][f], kf[u][f], s);
+                for (int f = 0; f < FPL; f++) s = fmaf(qr[g][f], kf[f], s);
                 s = group16_sum(s);
                 if (part == 0 && jj < nj) sc[g * cmax + jj] = s;
             }
@@ -175,22 +217,25 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     for (int g = 0; g < kHeads; g++)
 #pragma unroll
         for (int f = 0; f < FPL; f++) o[g][f] = 0.f;
-    for (int jj0 = 0; jj0 < nj; jj0 += 4 * kKeyGroups) {
-        float vf[4][FPL];
+    for (int jj0 = 0; jj0 < nj; jj0 += U * kKeyGroups) {
+        if (jj0 > 0) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            int jj = jj0 + kKeyGroups * u + kg;
-            load_row<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vf[u]);
+            for (int u = 0; u < U; u++) {
+                const int jj = jj0 + kKeyGroups * u + kg;
+                load_raw<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vraw[u]);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            int jj = jj0 + kKeyGroups * u + kg;
+        for (int u = 0; u < U; u++) {
+            const int jj = jj0 + kKeyGroups * u + kg;
             const bool live = jj < nj;
+            float vf[FPL];
+            raw_values<KV, FPL>(vraw[u], vf);
 #pragma unroll
             for (int g = 0; g < kHeads; g++) {
                 float pj = live ? sc[g * cmax + jj] : 0.f;
 #pragma unroll
-                for (int f = 0; f < FPL; f++) o[g][f] = fmaf(pj, live ? vf[u][f] : 0.f, o[g][f]);
+                for (int f = 0; f < FPL; f++) o[g][f] = fmaf(pj, live ? vf[f] : 0.f, o[g][f]);
             }
         }
     }
@@ -310,7 +355,7 @@ void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, 
     int64_t rows = B * HK * ngq;
     int64_t ns = 512 / (rows > 0 ? rows : 1);
     ns = ns > 64 ? 64 : ns;
-    int64_t by_keys = kmax / 32;
+    int64_t by_keys = kmax / 128;  // a share of 128 keys is one batch of loads per thread
     ns = ns > by_keys ? by_keys : ns;
     ns = ns < 1 ? 1 : ns;
     *nsplit = (int)ns;

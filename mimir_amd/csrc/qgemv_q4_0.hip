@@ -519,6 +519,7 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     int PC = npc <= 1 ? 1 : 2;
     if (tune[1] > 0) PC = tune[1];
     int R = MODE == kSwiGLU ? (job.total >= 8192 ? 2 : 1) : (job.total >= 4096 ? 2 : 1);
+    if (MODE == kPlain && job.total >= 8192 && npc <= 1) R = 4;  // many short rows: fewer, longer-lived wavefronts stream a little better
     if (tune[0] > 0) R = tune[0];
     int64_t tiles = (job.total + R - 1) / R;
     int waves = 8;
