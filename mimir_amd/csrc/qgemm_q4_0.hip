@@ -7,9 +7,9 @@
 // The arithmetic is exact up to the order of the float32 sums, not a product
 // with weights rounded to 16 bits. A weight is (n - 8) * d with a 4-bit n and a
 // binary16 d: up to 15 significant bits, more than bfloat16's 8. So each weight
-// goes to the matrix cores as two bfloat16 numbers, hi = bfloat16(w) and
-// lo = w - hi, which together are w exactly (lo has at most 7 significant
-// bits), and Y = X . hi^T + X . lo^T with every product exact in float32
+// goes to the matrix cores as two bfloat16 numbers, hi = the upper 16 bits of
+// w and lo = w - hi, which together are w exactly (lo has at most 7
+// significant bits), and Y = X . hi^T + X . lo^T with every product exact in float32
 // (8 x 8 bits). That doubles the MFMA count and leaves nothing per output to do
 // on the vector unit inside the loop; the split itself is done once per weight
 // while the tile is staged (convert, one FMA by the scale, round, subtract,
@@ -21,9 +21,14 @@
 // fragment reads conflict-free). The loads that feed a step are what bounds
 // this kernel if they are not coalesced (a wavefront load that touches 64
 // cache lines costs 64 cycles of the L1's time), so eight lanes share the 128
-// bytes a row of X contributes to a step. One LDS buffer, the next step's data
-// waiting in registers: two workgroups fit a compute unit and fill each
-// other's barriers.
+// bytes a row of X contributes to a step. Loading, splitting and multiplying
+// must overlap, and wavefronts that all do the same thing between the same
+// barriers do not overlap anything (two workgroups on a compute unit fall into
+// step with each other too). So the workgroup's eight wavefronts have two
+// roles: four multiply (fragment reads and MFMAs only), four feed them (loads
+// two steps ahead, the split on the vector unit, LDS stores into the other of
+// two buffers). Each SIMD holds one of each, and the hardware interleaves
+// them; one barrier a step hands a buffer over.
 // v_mfma_f32_32x32x16_bf16 takes, per lane, eight consecutive k of row
 // (lane % 32), the lane's half (lane / 32) choosing which eight of the sixteen;
 // its result holds column (lane % 32) and rows 8 (i / 4) + 4 (lane / 32) + i % 4
@@ -55,23 +60,28 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return u;
 }
 
-template <int MT, bool OUT_F32>  // MT 32-row tiles per wavefront: the workgroup's tile is (64 MT) x 128
-__global__ __launch_bounds__(256, 2) void qgemm_q4_0_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W,
+template <int MT, bool OUT_F32>  // MT 32-row tiles per multiplying wavefront: the workgroup's tile is (64 MT) x 128
+__global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W,
                                                             void* __restrict__ Yv, int M, int N, int K, int64_t x_row_stride,
                                                             int tiles_m, int ntiles) {
     constexpr int BM = 64 * MT;
     constexpr int AV = BM * 8 / 256;      // 16-byte pieces of the X tile per thread (4 or 2): piece p is row p / 8, bytes 16 (p % 8)..
     extern __shared__ __align__(16) uint8_t smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const bool feeder = wave >= 4;          // wavefronts 4..7 stage, 0..3 multiply
+    const int tid = threadIdx.x & 255;      // index within the role
+    const int wm = (wave & 3) >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
 
-    // consecutive workgroup ids go round the chip's eight dies; give each die a
-    // run of tiles that share their columns of W (tiles of one column strip are
-    // consecutive), so that a strip is fetched into one L2
+    // Consecutive workgroup ids go round the chip's eight dies; give each die a
+    // run of consecutive tiles, ordered so that the tiles a die works on at one
+    // time share their rows of X: a row tile of X (BM x K bfloat16, 1 or 2 MB)
+    // stays in the die's 4 MB L2 while the strips of W (0.3 MB each) stream
+    // through, instead of all of X streaming in again for every strip.
     const int per = (ntiles + 7) >> 3;
     const int tile = ((int)blockIdx.x & 7) * per + ((int)blockIdx.x >> 3);
     if (tile >= ntiles) return;
-    const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * kBN;
+    const int tiles_n = ntiles / tiles_m;
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * kBN;
     const int nb = K >> 5;
     const int64_t w_row_bytes = (int64_t)nb * 18;
 
@@ -91,41 +101,53 @@ __global__ __launch_bounds__(256, 2) void qgemm_q4_0_kernel(const uint16_t* __re
     const int w_n = n0 + w_col < N ? n0 + w_col : N - 1;
     const uint8_t* w_src = W + (int64_t)w_n * w_row_bytes + w_blk * 18;
 
-    u32x4 ra[AV], rq;
-    uint16_t rd;
-    auto fetch = [&](int kb) {
-#pragma unroll
-        for (int i = 0; i < AV; i++) __builtin_memcpy(&ra[i], __builtin_assume_aligned(a_src[i] + (int64_t)kb * kKS, 16), 16);
-        const uint8_t* wp = w_src + (int64_t)kb * 36;
-        rd = *(const uint16_t*)wp;
-        rq = load_u32x4_unaligned(wp + 2);
+    const int nk = K / kKS;
+    struct Fetched {  // what one step needs from memory; two sets alternate
+        u32x4 ra[AV], rq;
+        uint16_t rd;
     };
-    uint16_t* As = (uint16_t*)smem;
-    uint16_t* Bh = As + BM * kLd;
-    uint16_t* Bl = Bh + kBN * kLd;
-    auto stage = [&]() {
+    auto fetch = [&](int kb, Fetched& f) {
+        kb = kb < nk ? kb : nk - 1;  // past the end: a valid step again, unused (no branch in the loop body)
+#pragma unroll
+        for (int i = 0; i < AV; i++) __builtin_memcpy(&f.ra[i], __builtin_assume_aligned(a_src[i] + (int64_t)kb * kKS, 16), 16);
+        const uint8_t* wp = w_src + (int64_t)kb * 36;
+        f.rd = *(const uint16_t*)wp;
+        f.rq = load_u32x4_unaligned(wp + 2);
+    };
+    auto stage = [&](int buf, const Fetched& f) {
+        uint16_t* As = (uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
+        uint16_t* Bh = As + BM * kLd;
+        uint16_t* Bl = Bh + kBN * kLd;
+        const u32x4* ra = f.ra;
+        const u32x4 rq = f.rq;
+        const uint16_t rd = f.rd;
 #pragma unroll
         for (int i = 0; i < AV; i++) *(u32x4*)(As + a_dst[i]) = ra[i];
-        // byte j of the block's 16 holds element j (low nibble) and 16 + j (high nibble)
-        const float d = f16_bits_to_f32(rd), d8 = -8.0f * d;
+        // byte j of the block's 16 holds element j (low nibble) and 16 + j (high
+        // nibble). All of it in full-rate integer and float instructions: the
+        // nibble goes into the mantissa of 2^23 (v_perm), minus 2^23 + 8 is n - 8,
+        // times d is the weight, exactly; its upper 16 bits are a bfloat16 (hi,
+        // truncated, not rounded: w - hi then has at most 7 significant bits and
+        // its upper 16 bits are lo, exactly).
+        const float d = f16_bits_to_f32(rd);
         u32x4 hi[4], lo[4];  // elements 0..7, 8..15 (low nibbles), 16..23, 24..31 (high nibbles)
 #pragma unroll
         for (int half = 0; half < 2; half++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t nib = (rq[i] >> (4 * half)) & 0x0f0f0f0fu;
-                float w[4], r[4];
+                uint32_t wb[4], rb[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) w[j] = fmaf((float)((nib >> (8 * j)) & 0xffu), d, d8);  // (n - 8) * d, exact
-                const uint32_t h01 = pack_bf16(w[0], w[1]), h23 = pack_bf16(w[2], w[3]);
-                r[0] = w[0] - __uint_as_float(h01 << 16);
-                r[1] = w[1] - __uint_as_float(h01 & 0xffff0000u);
-                r[2] = w[2] - __uint_as_float(h23 << 16);
-                r[3] = w[3] - __uint_as_float(h23 & 0xffff0000u);
-                hi[2 * half + (i >> 1)][2 * (i & 1)] = h01;
-                hi[2 * half + (i >> 1)][2 * (i & 1) + 1] = h23;
-                lo[2 * half + (i >> 1)][2 * (i & 1)] = pack_bf16(r[0], r[1]);
-                lo[2 * half + (i >> 1)][2 * (i & 1) + 1] = pack_bf16(r[2], r[3]);
+                for (int j = 0; j < 4; j++) {
+                    const float t = __uint_as_float(__builtin_amdgcn_perm(0x4b000000u, nib, 0x070c0c00u | (uint32_t)j)) - 8388616.0f;
+                    const float w = t * d;
+                    wb[j] = __float_as_uint(w);
+                    rb[j] = __float_as_uint(w - __uint_as_float(wb[j] & 0xffff0000u));
+                }
+                hi[2 * half + (i >> 1)][2 * (i & 1)] = __builtin_amdgcn_perm(wb[1], wb[0], 0x07060302u);
+                hi[2 * half + (i >> 1)][2 * (i & 1) + 1] = __builtin_amdgcn_perm(wb[3], wb[2], 0x07060302u);
+                lo[2 * half + (i >> 1)][2 * (i & 1)] = __builtin_amdgcn_perm(rb[1], rb[0], 0x07060302u);
+                lo[2 * half + (i >> 1)][2 * (i & 1) + 1] = __builtin_amdgcn_perm(rb[3], rb[2], 0x07060302u);
             }
         uint16_t* hrow = Bh + w_col * kLd + w_blk * 32;
         uint16_t* lrow = Bl + w_col * kLd + w_blk * 32;
@@ -144,42 +166,92 @@ __global__ __launch_bounds__(256, 2) void qgemm_q4_0_kernel(const uint16_t* __re
 #pragma unroll
             for (int i = 0; i < 16; i++) total[mt][nt][i] = 0.f;
 
-    const int nk = K / kKS;
-    fetch(0);
-    for (int kb = 0; kb < nk; kb++) {
-        stage();
-        __syncthreads();
-        fetch(kb + 1 < nk ? kb + 1 : kb);  // the last step fetches itself again: no branch in the loop body
+    auto compute = [&](int buf) {
+        const uint16_t* As = (const uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
+        const uint16_t* Bh = As + BM * kLd;
+        const uint16_t* Bl = Bh + kBN * kLd;
+        // The fragments of a block of K (of both blocks, where the registers allow)
+        // are requested before its first MFMA, so that LDS latency is paid once,
+        // not once a fragment.
+        constexpr int NB = MT <= 2 ? 2 : 1;  // blocks whose fragments are held at once
+        bf16x8 a[NB][MT][2], bh[NB][2][2], bl[NB][2][2];
 #pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-            bf16x8 a[MT][2], bh[2][2], bl[2][2];
+        for (int b0 = 0; b0 < 2; b0 += NB) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
+            for (int bi = 0; bi < NB; bi++) {
+                const int blk = b0 + bi;
 #pragma unroll
-                for (int s = 0; s < 2; s++) a[mt][s] = *(const bf16x8*)(As + (wm * (32 * MT) + mt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
+                for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
+                    for (int s = 0; s < 2; s++)
+                        a[bi][mt][s] = *(const bf16x8*)(As + (wm * (32 * MT) + mt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
-                    bh[nt][s] = *(const bf16x8*)(Bh + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
-                    bl[nt][s] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
-                }
+                for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        bh[bi][nt][s] = *(const bf16x8*)(Bh + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
+                        bl[bi][nt][s] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
+                    }
+            }
+            __builtin_amdgcn_sched_barrier(0);
             // the tiles in turn for each operand pair, so that consecutive MFMAs are independent
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
+            for (int bi = 0; bi < NB; bi++)
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int s = 0; s < 2; s++) {
 #pragma unroll
-                    for (int nt = 0; nt < 2; nt++)
-                        total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mt][s], bl[nt][s], total[mt][nt], 0, 0, 0);
+                    for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                        for (int nt = 0; nt < 2; nt++)
+                            total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi][mt][s], bl[bi][nt][s], total[mt][nt], 0, 0, 0);
 #pragma unroll
-                    for (int nt = 0; nt < 2; nt++)
-                        total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mt][s], bh[nt][s], total[mt][nt], 0, 0, 0);
-            }
+                    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                        for (int nt = 0; nt < 2; nt++)
+                            total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi][mt][s], bh[bi][nt][s], total[mt][nt], 0, 0, 0);
+                }
+            if (NB == 1) __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();  // every wavefront is done with the buffer before the next step overwrites it
+    };
+
+    // Buffer kb & 1 holds step kb. Within step kb the feeders fill the other
+    // buffer with step kb + 1 while the multipliers read this one; the barrier
+    // that ends the step says both are done.
+    if (feeder) {
+        // Loads run four steps ahead of their use (four sets of registers):
+        // under load a request takes longer than a step, and what is in flight
+        // per compute unit bounds what arrives per unit of time.
+        Fetched f0, f1, f2, f3;
+        fetch(0, f0);
+        fetch(1, f1);
+        fetch(2, f2);
+        fetch(3, f3);
+        stage(0, f0);
+        fetch(4, f0);
+        __syncthreads();
+        for (int kb = 0; kb < nk; kb += 4) {
+            stage(1, f1);  // step kb + 1 while step kb is multiplied
+            fetch(kb + 5, f1);
+            __syncthreads();
+            if (kb + 1 >= nk) break;
+            stage(0, f2);
+            fetch(kb + 6, f2);
+            __syncthreads();
+            if (kb + 2 >= nk) break;
+            stage(1, f3);
+            fetch(kb + 7, f3);
+            __syncthreads();
+            if (kb + 3 >= nk) break;
+            stage(0, f0);
+            fetch(kb + 8, f0);
+            __syncthreads();
+        }
+        return;
+    }
+    __syncthreads();
+    for (int kb = 0; kb < nk; kb++) {  // one body: the accumulators stay where they are from step to step
+        compute(kb & 1);
+        __syncthreads();
     }
 
     // one rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51)
@@ -235,18 +307,34 @@ bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K
 // finite scales, Y [M, N] bfloat16, or float32 if out_f32.
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
                            hipStream_t st) {
-    // 128-row tiles unless they would leave compute units idle
+    // the tallest tiles that still give every compute unit work: a taller tile
+    // reads less from LDS per MFMA (a wavefront multiplies 32 MT x 64 of it)
     const int64_t tiles_n = (N + kBN - 1) / kBN;
-    const bool tall = ((M + 127) / 128) * tiles_n >= 384;
-    const int BM = tall ? 128 : 64;
+    const int MT = ((M + 255) / 256) * tiles_n >= 384 ? 4 : ((M + 127) / 128) * tiles_n >= 384 ? 2 : 1;
+    const int BM = 64 * MT;
     const int tiles_m = (int)((M + BM - 1) / BM);
     const int ntiles = (int)(tiles_m * tiles_n);
     dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
-    const size_t lds = stage_bytes(BM);
-#define QGEMM_LAUNCH(MT, F32)                                                                                                      \
-    hipLaunchKernelGGL((qgemm_q4_0_kernel<MT, F32>), grid, dim3(256), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y, (int)M,   \
+    const size_t lds = 2 * stage_bytes(BM);
+    {  // more dynamic LDS than a kernel gets by default
+        static bool raised = false;
+        if (!raised) {
+            const int most = (int)(2 * stage_bytes(256));
+            hipError_t e = hipSuccess;
+#define QGEMM_RAISE(MT_, F32_) \
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_kernel<MT_, F32_>, hipFuncAttributeMaxDynamicSharedMemorySize, most)
+            QGEMM_RAISE(1, true); QGEMM_RAISE(1, false); QGEMM_RAISE(2, true); QGEMM_RAISE(2, false); QGEMM_RAISE(4, true); QGEMM_RAISE(4, false);
+#undef QGEMM_RAISE
+            if (e != hipSuccess) return e;
+            raised = true;
+        }
+    }
+#define QGEMM_LAUNCH(MT_, F32_)                                                                                                     \
+    hipLaunchKernelGGL((qgemm_q4_0_kernel<MT_, F32_>), grid, dim3(512), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y, (int)M, \
                        (int)N, (int)K, x_row_stride, tiles_m, ntiles)
-    if (tall) {
+    if (MT == 4) {
+        if (out_f32) QGEMM_LAUNCH(4, true); else QGEMM_LAUNCH(4, false);
+    } else if (MT == 2) {
         if (out_f32) QGEMM_LAUNCH(2, true); else QGEMM_LAUNCH(2, false);
     } else {
         if (out_f32) QGEMM_LAUNCH(1, true); else QGEMM_LAUNCH(1, false);

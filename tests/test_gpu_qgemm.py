@@ -167,6 +167,28 @@ def test_prefill_shapes(n):
         assert np.array_equal(got4[:512], got) and np.array_equal(got4[512:1024], got[::-1]) and np.array_equal(got4[1024:1536], got)
 
 
+def test_tall_tiles():
+    """M = 2048 by N = 6144 takes the 256-row tiles: a band of columns against
+    the oracle, and ragged edges (M = 2000, N = 6100) against the same rows and
+    columns of the whole product."""
+    rng = np.random.default_rng(21)
+    m, n, k = 2048, 6144, 1024
+    w = bench_blocks(rng, O.Q4_0, n * k)
+    x = bf16_bits(rng.normal(size=(m, k)))
+    gpu.say("qgemm_bf16 2048x1024 by 6144x1024")
+    got32 = qgemm(w, x, n, k, capi.F32)
+    lo, hi = 3000, 3512
+    wb = w.reshape(n, -1)[lo:hi].reshape(-1)
+    want_f32 = reference_f32(wb, x, hi - lo, k)
+    err = np.abs(got32[:, lo:hi] - want_f32)
+    assert np.all(err <= 1e-4 * np.maximum(1, np.abs(want_f32))), float(err.max())
+    got = qgemm(w, x, n, k)
+    check_bf16(got[:, lo:hi], O.q4_0_matmul_bf16(wb, x, hi - lo, k), 1e-4 * np.maximum(1, np.abs(want_f32)))
+    gpu.say("qgemm_bf16 2000x1024 by 6100x1024")
+    part = qgemm(w.reshape(n, -1)[:6100].reshape(-1), x[:2000], 6100, k)
+    assert np.array_equal(part, got[:2000, :6100])
+
+
 def test_errors():
     l = gpu.lib()
     z = torch.zeros(4096, dtype=torch.int16, device="cuda:0")
