@@ -51,6 +51,12 @@ constexpr int kLd = kKS + 8;    // bfloat16 elements per LDS row
 
 constexpr size_t stage_bytes(int BM) { return (size_t)(BM + 2 * kBN) * kLd * 2; }  // X, hi, lo
 
+// The barrier of the main loop. __syncthreads() also waits for every global load
+// in flight (its fence covers all memory), which would stall each step for a
+// full trip to memory and undo the prefetching; the loop only hands LDS
+// buffers over, so it waits for LDS traffic alone.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Two floats to a packed pair of bfloat16, rounded to nearest even.
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     f32x2 f = {a, b};
@@ -102,7 +108,15 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
     const uint8_t* w_src = W + (int64_t)w_n * w_row_bytes + w_blk * 18;
 
     const int nk = K / kKS;
-    struct Fetched {  // what one step needs from memory; two sets alternate
+    // W reaches the feeders in one of two ways. With 64- and 128-row tiles there
+    // is room in LDS for a raw panel of four steps of W (144 bytes a row, two
+    // buffers): nine lanes share a row's 144 bytes, so a wavefront load touches
+    // about ten cache lines instead of 64, and each feeder then picks its block
+    // out of LDS. With 256-row tiles every feeder loads its own 18 bytes.
+    constexpr bool PANEL = MT <= 2;
+    constexpr int kPanelBytes = kBN * 144, kPanelPieces = kBN * 9;
+    uint8_t* raw = smem + 2 * stage_bytes(BM);
+    struct Fetched {  // what one step needs from memory
         u32x4 ra[AV], rq;
         uint16_t rd;
     };
@@ -110,17 +124,45 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         kb = kb < nk ? kb : nk - 1;  // past the end: a valid step again, unused (no branch in the loop body)
 #pragma unroll
         for (int i = 0; i < AV; i++) __builtin_memcpy(&f.ra[i], __builtin_assume_aligned(a_src[i] + (int64_t)kb * kKS, 16), 16);
-        const uint8_t* wp = w_src + (int64_t)kb * 36;
-        f.rd = *(const uint16_t*)wp;
-        f.rq = load_u32x4_unaligned(wp + 2);
+        if (!PANEL) {
+            const uint8_t* wp = w_src + (int64_t)kb * 36;
+            f.rd = *(const uint16_t*)wp;
+            f.rq = load_u32x4_unaligned(wp + 2);
+        }
     };
-    auto stage = [&](int buf, const Fetched& f) {
+    u32x4 pw[5];
+    auto panel_fetch = [&](int q) {
+        const int np = nk >> 2;
+        q = q < np ? q : np - 1;
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            const int pid = tid + 256 * i;
+            if (pid < kPanelPieces) {
+                const int row = pid / 9, pc = pid % 9;
+                const int n = n0 + row < N ? n0 + row : N - 1;
+                __builtin_memcpy(&pw[i], __builtin_assume_aligned(W + (int64_t)n * w_row_bytes + (int64_t)q * 144 + pc * 16, 16), 16);
+            }
+        }
+    };
+    auto panel_store = [&](int q) {
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            const int pid = tid + 256 * i;
+            if (pid < kPanelPieces) *(u32x4*)(raw + (q & 1) * kPanelBytes + (pid / 9) * 144 + (pid % 9) * 16) = pw[i];
+        }
+    };
+    auto stage = [&](int buf, const Fetched& f, int step) {
         uint16_t* As = (uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
         uint16_t* Bh = As + BM * kLd;
         uint16_t* Bl = Bh + kBN * kLd;
         const u32x4* ra = f.ra;
-        const u32x4 rq = f.rq;
-        const uint16_t rd = f.rd;
+        u32x4 rq = f.rq;
+        uint16_t rd = f.rd;
+        if (PANEL) {  // this thread's block of the step, out of the raw panel
+            const uint8_t* pb = raw + ((step >> 2) & 1) * kPanelBytes + w_col * 144 + ((step & 3) * 2 + w_blk) * 18;
+            rd = *(const uint16_t*)pb;
+            __builtin_memcpy(&rq, __builtin_assume_aligned(pb + 2, 2), 16);
+        }
 #pragma unroll
         for (int i = 0; i < AV; i++) *(u32x4*)(As + a_dst[i]) = ra[i];
         // byte j of the block's 16 holds element j (low nibble) and 16 + j (high
@@ -166,92 +208,98 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
 #pragma unroll
             for (int i = 0; i < 16; i++) total[mt][nt][i] = 0.f;
 
+    // A step is four slices of 16 of K. The fragments of slice i + 1 are read from
+    // LDS while the MFMAs of slice i run (two sets of fragment registers), so
+    // that only the first slice's reads are waited for.
     auto compute = [&](int buf) {
         const uint16_t* As = (const uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
         const uint16_t* Bh = As + BM * kLd;
         const uint16_t* Bl = Bh + kBN * kLd;
-        // The fragments of a block of K (of both blocks, where the registers allow)
-        // are requested before its first MFMA, so that LDS latency is paid once,
-        // not once a fragment.
-        constexpr int NB = MT <= 2 ? 2 : 1;  // blocks whose fragments are held at once
-        bf16x8 a[NB][MT][2], bh[NB][2][2], bl[NB][2][2];
+        bf16x8 a[2][MT], bh[2][2], bl[2][2];
+        auto read_slice = [&](int set, int sl) {  // slice sl: block sl / 2, half sl % 2
+            const int koff = (sl >> 1) * 32 + (sl & 1) * 16 + lh * 8;
 #pragma unroll
-        for (int b0 = 0; b0 < 2; b0 += NB) {
+            for (int nt = 0; nt < 2; nt++) bl[set][nt] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + koff);
 #pragma unroll
-            for (int bi = 0; bi < NB; bi++) {
-                const int blk = b0 + bi;
+            for (int mt = 0; mt < MT; mt++) a[set][mt] = *(const bf16x8*)(As + (wm * (32 * MT) + mt * 32 + l32) * kLd + koff);
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+            for (int nt = 0; nt < 2; nt++) bh[set][nt] = *(const bf16x8*)(Bh + (wn * 64 + nt * 32 + l32) * kLd + koff);
+        };
+        read_slice(0, 0);
 #pragma unroll
-                    for (int s = 0; s < 2; s++)
-                        a[bi][mt][s] = *(const bf16x8*)(As + (wm * (32 * MT) + mt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
-#pragma unroll
-                for (int nt = 0; nt < 2; nt++)
-#pragma unroll
-                    for (int s = 0; s < 2; s++) {
-                        bh[bi][nt][s] = *(const bf16x8*)(Bh + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
-                        bl[bi][nt][s] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + blk * 32 + s * 16 + lh * 8);
-                    }
-            }
-            __builtin_amdgcn_sched_barrier(0);
+        for (int sl = 0; sl < 4; sl++) {
+            if (sl < 3) read_slice((sl + 1) & 1, sl + 1);
             // the tiles in turn for each operand pair, so that consecutive MFMAs are independent
 #pragma unroll
-            for (int bi = 0; bi < NB; bi++)
+            for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
+                for (int nt = 0; nt < 2; nt++)
+                    total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[sl & 1][mt], bl[sl & 1][nt], total[mt][nt], 0, 0, 0);
 #pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
+            for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                        for (int nt = 0; nt < 2; nt++)
-                            total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi][mt][s], bl[bi][nt][s], total[mt][nt], 0, 0, 0);
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                        for (int nt = 0; nt < 2; nt++)
-                            total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi][mt][s], bh[bi][nt][s], total[mt][nt], 0, 0, 0);
-                }
-            if (NB == 1) __builtin_amdgcn_sched_barrier(0);
+                for (int nt = 0; nt < 2; nt++)
+                    total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[sl & 1][mt], bh[sl & 1][nt], total[mt][nt], 0, 0, 0);
         }
+        // the order asked of the scheduler: slice 0's reads, then slice by slice the
+        // next slice's reads ahead of this slice's MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, MT + 4, 0);
+#pragma unroll
+        for (int sl = 0; sl < 3; sl++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, MT + 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4 * MT, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4 * MT, 0);
     };
 
     // Buffer kb & 1 holds step kb. Within step kb the feeders fill the other
     // buffer with step kb + 1 while the multipliers read this one; the barrier
     // that ends the step says both are done.
     if (feeder) {
-        // Loads run four steps ahead of their use (four sets of registers):
-        // under load a request takes longer than a step, and what is in flight
-        // per compute unit bounds what arrives per unit of time.
+        // Loads run four steps ahead of their use (four sets of registers, and the
+        // raw panel a panel ahead): under load a request takes longer than a step.
         Fetched f0, f1, f2, f3;
+        if (PANEL) {
+            panel_fetch(0);
+            panel_store(0);
+            panel_fetch(1);
+        }
         fetch(0, f0);
         fetch(1, f1);
         fetch(2, f2);
         fetch(3, f3);
-        stage(0, f0);
+        lds_barrier();  // raw panel 0 is in place
+        stage(0, f0, 0);
         fetch(4, f0);
-        __syncthreads();
+        lds_barrier();
         for (int kb = 0; kb < nk; kb += 4) {
-            stage(1, f1);  // step kb + 1 while step kb is multiplied
+            stage(1, f1, kb + 1);  // step kb + 1 while step kb is multiplied
             fetch(kb + 5, f1);
-            __syncthreads();
+            lds_barrier();
             if (kb + 1 >= nk) break;
-            stage(0, f2);
+            stage(0, f2, kb + 2);
             fetch(kb + 6, f2);
-            __syncthreads();
+            lds_barrier();
             if (kb + 2 >= nk) break;
-            stage(1, f3);
+            stage(1, f3, kb + 3);
             fetch(kb + 7, f3);
-            __syncthreads();
+            if (PANEL) {  // the next panel goes into the other raw buffer, a step before its first use
+                panel_store((kb >> 2) + 1);
+                panel_fetch((kb >> 2) + 2);
+            }
+            lds_barrier();
             if (kb + 3 >= nk) break;
-            stage(0, f0);
+            stage(0, f0, kb + 4);
             fetch(kb + 8, f0);
-            __syncthreads();
+            lds_barrier();
         }
         return;
     }
-    __syncthreads();
+    lds_barrier();
+    lds_barrier();
     for (int kb = 0; kb < nk; kb++) {  // one body: the accumulators stay where they are from step to step
         compute(kb & 1);
-        __syncthreads();
+        lds_barrier();
     }
 
     // one rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51)
@@ -296,10 +344,10 @@ hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st) {
     return hipGetLastError();
 }
 
-// Whether the matrix-core kernel takes this product: rows of X aligned for
-// 16-byte loads, W at least 2-byte aligned.
+// Whether the matrix-core kernel takes this product: K in panels of 256, rows
+// of X and of W aligned for 16-byte loads.
 bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K, int64_t x_row_stride) {
-    return M > 0 && N > 0 && K > 0 && K % kKS == 0 && ((uintptr_t)X & 15) == 0 && x_row_stride % 8 == 0 && ((uintptr_t)W & 1) == 0 &&
+    return M > 0 && N > 0 && K > 0 && K % 256 == 0 && ((uintptr_t)X & 15) == 0 && x_row_stride % 8 == 0 && ((uintptr_t)W & 15) == 0 &&
            M <= (1 << 24) && N <= (1 << 24) && K <= (1 << 24);
 }
 
@@ -315,11 +363,11 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
     const int tiles_m = (int)((M + BM - 1) / BM);
     const int ntiles = (int)(tiles_m * tiles_n);
     dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
-    const size_t lds = 2 * stage_bytes(BM);
+    const size_t lds = 2 * stage_bytes(BM) + (MT <= 2 ? 2 * kBN * 144 : 0);
     {  // more dynamic LDS than a kernel gets by default
         static bool raised = false;
         if (!raised) {
-            const int most = (int)(2 * stage_bytes(256));
+            const int most = 160 * 1024;
             hipError_t e = hipSuccess;
 #define QGEMM_RAISE(MT_, F32_) \
     if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_kernel<MT_, F32_>, hipFuncAttributeMaxDynamicSharedMemorySize, most)

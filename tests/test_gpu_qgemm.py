@@ -75,7 +75,7 @@ def check_bf16(got, want_bits, bound):
     assert differ.mean() <= 0.01, float(differ.mean())
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 64), (32, 128, 128), (70, 200, 192), (1, 130, 4096), (200, 384, 1024), (129, 257, 320), (33, 65, 96)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (32, 128, 512), (70, 200, 768), (1, 130, 4096), (200, 384, 1024), (129, 257, 1280), (33, 65, 96), (40, 130, 192)])
 def test_small_and_ragged_shapes(m, n, k):
     rng = np.random.default_rng(m * 7 + n)
     w = random_blocks(rng, O.Q4_0, n * k)
@@ -87,8 +87,8 @@ def test_small_and_ragged_shapes(m, n, k):
     check_f32(got32, want_f32, bound)
     got = qgemm(w, x, n, k)
     check_bf16(got, O.q4_0_matmul_bf16(w, x, n, k), bound)
-    # strided rows of x, weights at a 2-byte aligned address
-    got2 = qgemm(w, x, n, k, x_stride=k + 24, w_offset=6)
+    # strided rows of x, weights at another address (K = 96 and 192 take the general route: K must be whole panels of 256)
+    got2 = qgemm(w, x, n, k, x_stride=k + 24, w_offset=32)
     assert np.array_equal(got2, got)
 
 
