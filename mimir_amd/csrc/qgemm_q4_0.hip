@@ -270,27 +270,27 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         fetch(3, f3);
         lds_barrier();  // raw panel 0 is in place
         stage(0, f0, 0);
-        fetch(4, f0);
         lds_barrier();
+        // each turn first requests the loads of three steps ahead (into the set of
+        // registers the turn before consumed), so that the load unit works through
+        // them while this wavefront does the arithmetic of the step it stages
         for (int kb = 0; kb < nk; kb += 4) {
+            fetch(kb + 4, f0);
             stage(1, f1, kb + 1);  // step kb + 1 while step kb is multiplied
-            fetch(kb + 5, f1);
             lds_barrier();
             if (kb + 1 >= nk) break;
+            fetch(kb + 5, f1);
             stage(0, f2, kb + 2);
-            fetch(kb + 6, f2);
             lds_barrier();
             if (kb + 2 >= nk) break;
+            fetch(kb + 6, f2);
+            if (PANEL) panel_store((kb >> 2) + 1);  // the next panel into the other raw buffer, a step before its first use
+            if (PANEL) panel_fetch((kb >> 2) + 2);
             stage(1, f3, kb + 3);
-            fetch(kb + 7, f3);
-            if (PANEL) {  // the next panel goes into the other raw buffer, a step before its first use
-                panel_store((kb >> 2) + 1);
-                panel_fetch((kb >> 2) + 2);
-            }
             lds_barrier();
             if (kb + 3 >= nk) break;
+            fetch(kb + 7, f3);
             stage(0, f0, kb + 4);
-            fetch(kb + 8, f0);
             lds_barrier();
         }
         return;
