@@ -274,6 +274,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
+ * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
+ * kernels takes; "kquant.path" = 1 forces their variant that reads x from
+ * global memory (otherwise used only for rows of x too long for the LDS).
  * "qgemm.path" = 1 makes mi355x_qgemm_bf16 take its general route for every shape.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).

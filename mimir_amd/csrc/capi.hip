@@ -571,6 +571,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
             g_tune_q4[i] = value;
             return MI355X_OK;
         }
+    if (key && (strcmp(key, "kquant.rows") == 0 || strcmp(key, "kquant.path") == 0)) {
+        mimir::set_kquant_tune(key[7] == 'p', value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "qgemm.path") == 0) {
         g_tune_gemm = value;
         return MI355X_OK;

@@ -70,6 +70,8 @@ hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
+// which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in global memory.
+void set_kquant_tune(int which, int value);
 
 // y = x . W^T for a float32, binary16 or bfloat16 W [N, K].
 hipError_t gemv_float(int dt, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride,

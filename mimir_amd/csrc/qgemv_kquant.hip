@@ -8,11 +8,16 @@
 // The integers are exact; only the order in which a row's super-blocks are
 // added differs from the CPU's.
 //
-// One wavefront per row of W, read in place in ggml's layout; the lanes split
-// each super-block (4 lanes of 64 weights for Q4_K, 8 lanes of 32 for Q6_K)
-// and walk the row 16 or 8 super-blocks at a time. These are the formats real
-// Llama files use for a minority of tensors; they are written for
-// correctness first.
+// W is read in place in ggml's layout. The kernels that serve ordinary shapes
+// stage the converted row of x in LDS once per workgroup; a wavefront owns R
+// rows of W and walks them 16 (Q4_K) or 8 (Q6_K) super-blocks at a time, a
+// lane taking 16 bytes of nibbles per load so that a super-block is fetched
+// with a few 128-bit loads per lane (the texture addresser issues one
+// wavefront load in the same time whatever its width, and it, not HBM, bounds
+// a kernel built from dword loads). The loads of the next pass are requested
+// before the current pass is multiplied. A second pair of kernels, one
+// wavefront per row with x read from global memory, serves rows of x too long
+// for the LDS.
 #include "device_util.h"
 #include "kernels.h"
 
@@ -106,7 +111,7 @@ __device__ __forceinline__ int i16_at(const uint16_t* p, int i) { return (int)(i
 
 // qdotQ4KGo (backend/cpu/qmatmul.go:148-172): lane (sb, j) takes the 64
 // weights of nibble group j of super-block sb.
-__global__ __launch_bounds__(256) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+__global__ __launch_bounds__(256) void qgemv_q4k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
                                                         float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
@@ -159,7 +164,7 @@ __global__ __launch_bounds__(256) void qgemv_q4k_kernel(const uint8_t* __restric
 
 // qdotQ6KGo (backend/cpu/qmatmul.go:180-200): lane (sb, n, k) takes the 32
 // weights of quarter k of half n of super-block sb, groups 8n+2k and 8n+2k+1.
-__global__ __launch_bounds__(256) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+__global__ __launch_bounds__(256) void qgemv_q6k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
                                                         float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
@@ -201,16 +206,273 @@ __global__ __launch_bounds__(256) void qgemv_q6k_kernel(const uint8_t* __restric
     if (lane == 0) y[(int64_t)blockIdx.y * N + row] = acc;
 }
 
+// ---- the LDS kernels ----------------------------------------------------------
+//
+// LDS copy of one converted row: the quants of super-block sb at sb * kKqStride
+// (16 bytes of padding keep the lanes of neighbouring super-blocks off one
+// bank), then the sums and the scales as in global memory.
+constexpr int kKqStride = 256 + 16;
+constexpr int kKqThreads = 256;
+constexpr size_t kKqMaxLds = 160 * 1024;
+static size_t kq_lds_bytes(int nsb) { return (size_t)nsb * (kKqStride + 32 + 4); }
+
+__device__ __forceinline__ void kq_stage_act(const uint8_t* __restrict__ arow, int nsb, uint8_t* lds, int tid) {
+    const u32x4* src = (const u32x4*)arow;
+    for (int c = tid; c < nsb * 16; c += kKqThreads) *(u32x4*)(lds + (c >> 4) * kKqStride + (c & 15) * 16) = src[c];
+    const uint32_t* tail = (const uint32_t*)(arow + (int64_t)nsb * 256);
+    uint32_t* dst = (uint32_t*)(lds + nsb * kKqStride);
+    for (int c = tid; c < nsb * 9; c += kKqThreads) dst[c] = tail[c];
+}
+
+__device__ __forceinline__ u32x4 lds_u32x4(const uint8_t* p) { return *(const u32x4*)p; }
+
+struct Q4KTile {
+    u32x4 hdr, q0, q1;  // d, dmin and the 12 scale bytes; bytes 16j.. and 64+16j.. of the nibbles
+};
+
+// qdotQ4KGo (backend/cpu/qmatmul.go:148-172). Lane (sb, j): nibble bytes
+// 16j..16j+15 and 64+16j..64+16j+15 of super-block sb, which are 16 weights
+// each of sub-blocks 2g, 2g+1, 2g+4 and 2g+5 (g = j/2), the 16-weight chunks
+// 4g+h, 4g+2+h, 4g+8+h, 4g+10+h of the super-block (h = j%2); the sums kept
+// with x are per chunk.
+template <int R>
+__global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+                                                               float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+    extern __shared__ __align__(16) uint8_t kq_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
+    const int j = lane & 3, g = j >> 1, h = j & 1, sbl = lane >> 2;
+    const int64_t row_bytes = (int64_t)nsb * 144;
+    Q4KTile next[R];
+    auto fetch = [&](int sb0) {
+        int sb = sb0 + sbl;
+        sb = sb < nsb ? sb : nsb - 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = row0 + r;
+            row = row < N ? row : N - 1;
+            const uint8_t* wb = W + (int64_t)row * row_bytes + (int64_t)sb * 144;
+            next[r].hdr = *(const u32x4*)wb;
+            next[r].q0 = *(const u32x4*)(wb + 16 + 16 * j);
+            next[r].q1 = *(const u32x4*)(wb + 80 + 16 * j);
+        }
+    };
+    fetch(0);
+    kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
+    __syncthreads();
+    const int16_t* sums = (const int16_t*)(kq_lds + nsb * kKqStride);
+    const float* xd = (const float*)(kq_lds + nsb * (kKqStride + 32));
+    const int ca = 4 * g + h, sh = 16 * g;
+    float acc[R], accm[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = accm[r] = 0.f;
+    for (int sb0 = 0; sb0 < nsb; sb0 += 16) {
+        int sb = sb0 + sbl;
+        const bool live = sb < nsb;
+        sb = live ? sb : nsb - 1;
+        Q4KTile cur[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) cur[r] = next[r];
+        if (sb0 + 16 < nsb) fetch(sb0 + 16);
+        const uint8_t* xq = kq_lds + sb * kKqStride + 16 * ca;
+        const u32x4 xa = lds_u32x4(xq), xb = lds_u32x4(xq + 32), xc = lds_u32x4(xq + 128), xe = lds_u32x4(xq + 160);
+        const int16_t* s16 = sums + sb * 16 + ca;
+        const int sa = s16[0], sb_ = s16[2], sc_ = s16[8], se = s16[10];
+        const float xscale = xd[sb];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t s0 = cur[r].hdr[1], s1 = cur[r].hdr[2], s2 = cur[r].hdr[3];
+            // scale_min_k4 (backend/cpu/quant.go:129-134) for sub-blocks 2g, 2g+1 (< 4) and 2g+4, 2g+5
+            const int sc_a = (s0 >> sh) & 63, sc_b = (s0 >> (sh + 8)) & 63;
+            const int m_a = (s1 >> sh) & 63, m_b = (s1 >> (sh + 8)) & 63;
+            const int sc_c = ((s2 >> sh) & 0xf) | (((s0 >> (sh + 6)) & 3) << 4);
+            const int sc_e = ((s2 >> (sh + 8)) & 0xf) | (((s0 >> (sh + 14)) & 3) << 4);
+            const int m_c = ((s2 >> (sh + 4)) & 0xf) | (((s1 >> (sh + 6)) & 3) << 4);
+            const int m_e = ((s2 >> (sh + 12)) & 0xf) | (((s1 >> (sh + 14)) & 3) << 4);
+            int lo0 = 0, hi0 = 0, lo1 = 0, hi1 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t w0 = cur[r].q0[i], w1 = cur[r].q1[i];
+                lo0 = __builtin_amdgcn_sdot4((int)(w0 & 0x0F0F0F0Fu), (int)xa[i], lo0, false);
+                hi0 = __builtin_amdgcn_sdot4((int)((w0 >> 4) & 0x0F0F0F0Fu), (int)xb[i], hi0, false);
+                lo1 = __builtin_amdgcn_sdot4((int)(w1 & 0x0F0F0F0Fu), (int)xc[i], lo1, false);
+                hi1 = __builtin_amdgcn_sdot4((int)((w1 >> 4) & 0x0F0F0F0Fu), (int)xe[i], hi1, false);
+            }
+            int sumi = sc_a * lo0 + sc_b * hi0 + sc_c * lo1 + sc_e * hi1;
+            int summ = m_a * sa + m_b * sb_ + m_c * sc_ + m_e * se;
+            sumi = dpp_i32_quad_sum(live ? sumi : 0);
+            summ = dpp_i32_quad_sum(live ? summ : 0);
+            if (j == 0 && live) {
+                const uint32_t dw = cur[r].hdr[0];
+                float dd = f16_bits_to_f32((uint16_t)dw) * xscale, dm = f16_bits_to_f32((uint16_t)(dw >> 16)) * xscale;
+                float t = dd * (float)sumi;
+                acc[r] = acc[r] + t;
+                float u = dm * (float)summ;
+                accm[r] = accm[r] + u;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float a = wave_sum(acc[r]), am = wave_sum(accm[r]);
+        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = a - am;
+    }
+}
+
+// Sixteen bytes at a 2-byte aligned address as five aligned dwords; take(i)
+// shifts dword i of the sixteen out of them.
+struct Bytes16 {
+    u32x4 lo;
+    uint32_t top;
+    __device__ __forceinline__ uint32_t take(int i, uint32_t mis) const {
+        return __builtin_amdgcn_alignbyte(i == 3 ? top : lo[i + 1 > 3 ? 3 : i + 1], lo[i], mis);
+    }
+};
+// The dword after the sixteen bytes is read only where the address is off by
+// two; `last` says that nothing readable follows an aligned sixteen.
+__device__ __forceinline__ Bytes16 load_bytes16(const uint8_t* p, uint32_t mis) {
+    Bytes16 b;
+    const uint8_t* base = p - mis;
+    __builtin_memcpy(&b.lo, __builtin_assume_aligned(base, 4), 16);
+    __builtin_memcpy(&b.top, __builtin_assume_aligned(base + (mis ? 16 : 12), 4), 4);
+    return b;
+}
+
+struct Q6KTile {
+    Bytes16 ql, qh, sc;  // 16 bytes of low nibbles, the 16 bytes of high bits that go with them, the 16 scales
+    uint16_t d;
+};
+
+// qdotQ6KGo (backend/cpu/qmatmul.go:180-200). Lane (sb, n, c): bytes
+// 64n+16c..64n+16c+15 of ql, whose low nibbles are chunk 8n+c of the
+// super-block and whose high nibbles are chunk 8n+c+4, with bytes
+// 32n+16(c%2).. of qh holding their upper two bits at bit 2(c/2) and
+// 2(c/2)+4; Q6_K's scales are per chunk.
+template <int R>
+__global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
+                                                               float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+    extern __shared__ __align__(16) uint8_t kq_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
+    const int part = lane & 7, n = part >> 2, c = part & 3, sbl = lane >> 3;
+    const int64_t row_bytes = (int64_t)nsb * 210;
+    Q6KTile next[R];
+    auto fetch = [&](int sb0) {
+        int sb = sb0 + sbl;
+        sb = sb < nsb ? sb : nsb - 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = row0 + r;
+            row = row < N ? row : N - 1;
+            const uint8_t* wb = W + (int64_t)row * row_bytes + (int64_t)sb * 210;
+            const uint32_t mis = (uint32_t)(uintptr_t)wb & 3;  // 0 or 2, the same for every part of a block
+            next[r].ql = load_bytes16(wb + 64 * n + 16 * c, mis);
+            next[r].qh = load_bytes16(wb + 128 + 32 * n + 16 * (c & 1), mis);
+            next[r].sc = load_bytes16(wb + 192, mis);
+            next[r].d = load_u16(wb + 208);
+        }
+    };
+    fetch(0);
+    kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
+    __syncthreads();
+    const int16_t* sums = (const int16_t*)(kq_lds + nsb * kKqStride);
+    const float* xd = (const float*)(kq_lds + nsb * (kKqStride + 32));
+    const int chunk = 8 * n + c, shl = c & 2;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    for (int sb0 = 0; sb0 < nsb; sb0 += 8) {
+        int sb = sb0 + sbl;
+        const bool live = sb < nsb;
+        sb = live ? sb : nsb - 1;
+        Q6KTile cur[R];
+        uint32_t mis[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            cur[r] = next[r];
+            int row = row0 + r;
+            row = row < N ? row : N - 1;
+            mis[r] = (uint32_t)(uintptr_t)(W + (int64_t)row * row_bytes + (int64_t)sb * 210) & 3;
+        }
+        if (sb0 + 8 < nsb) fetch(sb0 + 8);
+        const uint8_t* xq = kq_lds + sb * kKqStride + 16 * chunk;
+        const u32x4 xl = lds_u32x4(xq), xh = lds_u32x4(xq + 64);
+        const int sl = sums[sb * 16 + chunk], sh_ = sums[sb * 16 + chunk + 4];
+        const float xscale = xd[sb];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int dl = 0, dh = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t a = cur[r].ql.take(i, mis[r]), b = cur[r].qh.take(i, mis[r]) >> shl;
+                const uint32_t vl = (a & 0x0F0F0F0Fu) | ((b & 0x03030303u) << 4);  // 0..63 per byte
+                const uint32_t vh = ((a >> 4) & 0x0F0F0F0Fu) | (((b >> 4) & 0x03030303u) << 4);
+                dl = __builtin_amdgcn_sdot4((int)vl, (int)xl[i], dl, false);
+                dh = __builtin_amdgcn_sdot4((int)vh, (int)xh[i], dh, false);
+            }
+            const uint32_t pair = n ? cur[r].sc.take(2, mis[r]) : cur[r].sc.take(0, mis[r]);
+            const uint32_t pair4 = n ? cur[r].sc.take(3, mis[r]) : cur[r].sc.take(1, mis[r]);
+            const int sc_l = (int)(int8_t)(pair >> (8 * c)), sc_h = (int)(int8_t)(pair4 >> (8 * c));
+            int sumi = sc_l * (dl - 32 * sl) + sc_h * (dh - 32 * sh_);
+            sumi = dpp_i32_group8_sum(live ? sumi : 0);
+            if (part == 0 && live) {
+                float dd = f16_bits_to_f32(cur[r].d) * xscale;
+                float t = dd * (float)sumi;
+                acc[r] = acc[r] + t;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float a = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = a;
+    }
+}
+
+static int g_kq_tune[2] = {0, 0};  // rows per wavefront (0: by shape); 1: always the kernels without LDS
+void set_kquant_tune(int which, int value) {
+    if (which >= 0 && which < 2) g_kq_tune[which] = value;
+}
+
+template <int R>
+static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st) {
+    static bool raised[2] = {false, false};
+    const size_t lds = kq_lds_bytes(nsb);
+    const int rows_per_wg = kKqThreads / 64 * R;
+    dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
+    const void* fn = dt == kQ4_K ? (const void*)qgemv_q4k_kernel<R> : (const void*)qgemv_q6k_kernel<R>;
+    if (lds > 48 * 1024 && !raised[dt == kQ4_K]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kKqMaxLds);
+        if (e != hipSuccess) return e;
+        raised[dt == kQ4_K] = true;
+    }
+    if (dt == kQ4_K)
+        hipLaunchKernelGGL(qgemv_q4k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
+                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+    else
+        hipLaunchKernelGGL(qgemv_q6k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
+                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+    return hipGetLastError();
+}
+
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     int nsb = (int)(a.K / 256);
+    // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.
+    // Q6_K's 210-byte blocks are read as aligned dwords around a 2-byte aligned start.
+    const bool lds_ok = kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;
+    if (g_kq_tune[1] != 1 && lds_ok) {
+        int R = g_kq_tune[0];
+        if (R != 1 && R != 2 && R != 4) R = (dt == kQ4_K && a.N * a.M >= 65536) ? 4 : a.N * a.M >= 2048 ? 2 : 1;  // measured: see the sweep keys of mi355x_tune
+        return R == 4 ? launch_kq<4>(dt, a, nsb, st) : R == 2 ? launch_kq<2>(dt, a, nsb, st) : launch_kq<1>(dt, a, nsb, st);
+    }
     const int waves = 4;
     dim3 grid((unsigned)((a.N + waves - 1) / waves), (unsigned)a.M);
     if (dt == kQ4_K)
-        hipLaunchKernelGGL(qgemv_q4k_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y,
-                           (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+        hipLaunchKernelGGL(qgemv_q4k_plain_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
+                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     else
-        hipLaunchKernelGGL(qgemv_q6k_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y,
-                           (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+        hipLaunchKernelGGL(qgemv_q6k_plain_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
+                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     return hipGetLastError();
 }
 

@@ -421,6 +421,32 @@ def test_kquant_gemv_matches_oracle(dt, n, k, offset):
         assert np.array_equal(got, gpu.qgemv_act(dt, ptr, gpu.dev(x), n, k))
 
 
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+def test_kquant_gemv_every_launch_shape(dt):
+    """The kernels that stage x in LDS, at every count of rows per wavefront, and the ones that
+    read it from global memory add the same integers in the same order: identical results."""
+    l = gpu.lib()
+    rng = np.random.default_rng(77 + dt)
+    for n, k in ((37, 256 * 56), (130, 256 * 9), (16, 256)):
+        raw = random_blocks(rng, dt, n * k)
+        x = rng.normal(size=(3, k)).astype(np.float32)
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        want = O.qmatmul(dt, raw, x, n, k)
+        mag = np.abs(x).astype(np.float64) @ np.abs(O.dequantize(dt, raw).reshape(n, k)).astype(np.float64).T
+        results = []
+        try:
+            for key, v in ((b"kquant.rows", 1), (b"kquant.rows", 2), (b"kquant.rows", 4), (b"kquant.path", 1)):
+                gpu.say(f"kquant gemv dt={dt} N={n} K={k} {key.decode()}={v}")
+                capi.check(l.mi355x_tune(key, v))
+                results.append(gpu.qgemv(dt, ptr, gpu.dev(x), n, k))
+        finally:
+            capi.check(l.mi355x_tune(b"kquant.rows", 0))
+            capi.check(l.mi355x_tune(b"kquant.path", 0))
+        assert np.all(np.abs(results[0] - want) <= 4e-6 * mag + 1e-30)
+        for r in results[1:]:
+            assert np.array_equal(r, results[0])
+
+
 def test_kquant_gemv_golden_and_exact_rows(golden_dir):
     cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
     for kind, dt in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
