@@ -70,7 +70,13 @@ hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
-// which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in global memory.
+// The same products for many rows of x on the matrix cores (qgemm_kquant.hip); qgemv_kquant_act
+// hands over to it from kQGemmMinRows rows of x.
+constexpr int64_t kQGemmMinRows = 8;
+bool qgemm_kquant_ok(int dt, const QGemvArgs& a);
+hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st);
+// which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in
+// global memory, 2 = never the matrix-core kernel, 3 = always the matrix-core kernel.
 void set_kquant_tune(int which, int value);
 
 // y = x . W^T for a float32, binary16 or bfloat16 W [N, K].

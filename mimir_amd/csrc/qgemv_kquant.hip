@@ -429,7 +429,9 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
     }
 }
 
-static int g_kq_tune[2] = {0, 0};  // rows per wavefront (0: by shape); 1: always the kernels without LDS
+// [0] rows per wavefront (0: by shape). [1] 1: always the kernels without LDS, 2: never the
+// matrix-core kernel, 3: the matrix-core kernel for any number of rows.
+static int g_kq_tune[2] = {0, 0};
 void set_kquant_tune(int which, int value) {
     if (which >= 0 && which < 2) g_kq_tune[which] = value;
 }
@@ -457,6 +459,8 @@ static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st)
 
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     int nsb = (int)(a.K / 256);
+    // From a few rows of x on, the matrix cores (whose results are the CPU's bit for bit).
+    if ((g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && a.M >= kQGemmMinRows)) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
     // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.
     // Q6_K's 210-byte blocks are read as aligned dwords around a 2-byte aligned start.
     const bool lds_ok = kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;
