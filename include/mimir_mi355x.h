@@ -107,10 +107,14 @@ MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* 
  * Tensor.MatMulT computes it for a half-precision x and a block-quantized w
  * (tensor/quant.go:45-48: x cast to float32, the product accumulated in float32,
  * one rounding to x's dtype): X [M, K] bfloat16 with rows x_row_stride elements
- * apart, W [N, K] Q4_0, Y [M, N] contiguous of out_dtype MI355X_BF16 (the
- * reference's result) or MI355X_F32 (the same sums before the rounding). Runs
- * on the matrix cores when X is 16-byte aligned with rows a multiple of 8
- * elements apart; otherwise through the decode kernels. */
+ * apart, W [N, K] of any block dtype, Y [M, N] contiguous of out_dtype
+ * MI355X_BF16 (the reference's result) or MI355X_F32 (the same sums before the
+ * rounding). Q4_0 runs on the bfloat16 matrix cores, exactly (each weight as two
+ * bfloat16 halves), when K is a multiple of 256, X and W are 16-byte aligned
+ * and rows of X are a multiple of 8 elements apart; otherwise, and for the other
+ * dtypes, X goes through mi355x_qgemv as float32. Q4_K and Q6_K then run on
+ * the int8 matrix cores from a few rows of X on, with the CPU's results bit for
+ * bit (backend/cpu/qtile.go:51-54 claims the same of the reference's tiles). */
 MI355X_API mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K,
                                            int64_t x_row_stride, int out_dtype, void* stream);
 
@@ -276,7 +280,8 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
  * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
  * kernels takes; "kquant.path" = 1 forces their variant that reads x from
- * global memory (otherwise used only for rows of x too long for the LDS).
+ * global memory (otherwise used only for rows of x too long for the LDS), 2
+ * keeps them off the matrix cores whatever M is, 3 puts them there for any M.
  * "qgemm.path" = 1 makes mi355x_qgemm_bf16 take its general route for every shape.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).

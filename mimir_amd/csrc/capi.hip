@@ -263,11 +263,11 @@ mi355x_status mi355x_sync(void* stream) {
 // product, one rounding to the output's dtype.
 mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride,
                                 int out_dtype, void* stream) {
-    if (dtype != MI355X_Q4_0) return fail(MI355X_ERR_DTYPE, "mi355x: qgemm_bf16 by weights of dtype %d (Q4_0 only)", dtype);
+    if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: qgemm_bf16 by weights of dtype %d", dtype);
     if (out_dtype != MI355X_BF16 && out_dtype != MI355X_F32) return fail(MI355X_ERR_DTYPE, "mi355x: qgemm_bf16 into dtype %d", out_dtype);
-    if (M < 0 || N < 0 || K < 0 || K % 32 != 0)
-        return fail(MI355X_ERR_INTERNAL, "mi355x: qgemm_bf16 of [%lld, %lld] by [%lld, %lld] in blocks of 32", (long long)M, (long long)K,
-                    (long long)N, (long long)K);
+    if (M < 0 || N < 0 || K < 0 || K % mimir::block_size(dtype) != 0)
+        return fail(MI355X_ERR_INTERNAL, "mi355x: qgemm_bf16 of [%lld, %lld] by [%lld, %lld] in blocks of %d", (long long)M, (long long)K,
+                    (long long)N, (long long)K, mimir::block_size(dtype));
     if (M == 0 || N == 0) return MI355X_OK;
     if (!W || !X || !Y) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemm_bf16: null pointer");
     if (M > 65535 || N > (int64_t)1 << 24 || K > (int64_t)1 << 24)
@@ -280,11 +280,13 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
         return MI355X_OK;
     }
     void* ws;
-    if (g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
+    if (dtype == MI355X_Q4_0 && g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
         HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
-    // any other shape: the activations as float32 through the decode kernels, then one rounding
+    // Any other shape or dtype: the activations as float32 through mi355x_qgemv, then one rounding. For
+    // Q8_0, Q4_K and Q6_K that is the reference's own sequence (cast, int8 rounding of x, integer dot
+    // products, cast), and the K-quants take their matrix-core kernel from a few rows on.
     const size_t xb = ((size_t)M * K * 4 + 255) & ~(size_t)255, yb = ((size_t)M * N * 4 + 255) & ~(size_t)255;
     if (mi355x_status s2 = gemm_scratch(xb + yb, &ws)) return s2;
     float* xf = (float*)ws;

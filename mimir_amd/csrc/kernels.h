@@ -71,8 +71,8 @@ size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
 // The same products for many rows of x on the matrix cores (qgemm_kquant.hip); qgemv_kquant_act
-// hands over to it from kQGemmMinRows rows of x.
-constexpr int64_t kQGemmMinRows = 8;
+// hands over to it where qgemm_kquant_pays says it is the faster of the two.
+bool qgemm_kquant_pays(int dt, const QGemvArgs& a);
 bool qgemm_kquant_ok(int dt, const QGemvArgs& a);
 hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st);
 // which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in

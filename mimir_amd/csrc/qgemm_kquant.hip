@@ -51,8 +51,10 @@ constexpr int kHalf = 128;       // K per step
 constexpr int kRow = kHalf + 16; // bytes per LDS row of int8
 constexpr int kSumRow = 48;      // bytes per LDS row of sixteen binary16 (32 used)
 
-// LDS: two step buffers (x rows, plane A, plane B) and two buffers of what the
-// end of a super-block needs (scales of x, sums of x, scales and mins of W).
+// LDS: two step buffers (x rows, plane A, plane B) and what the end of a
+// super-block needs (scales of x, sums of x, scales and mins of W), stored with
+// the second half's step: the barrier that ends the super-block's last step
+// also separates its readers from the next writers.
 template <int TM>
 struct Layout {
     static constexpr int x = 0;
@@ -65,7 +67,7 @@ struct Layout {
     static constexpr int dw = xsum + TM * kSumRow;     // float[kTN][2]: d, dmin
     static constexpr int mins = dw + kTN * 8;          // binary16[kTN][16], rows of kSumRow bytes
     static constexpr int side = mins + kTN * kSumRow;
-    static constexpr int total = side0 + 2 * side;
+    static constexpr int total = side0 + side;
 };
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -110,18 +112,31 @@ __device__ __forceinline__ uint32_t q4k_min(uint32_t s1, uint32_t s2, int j) {
     return j < 4 ? (s1 >> sh) & 63 : ((s2 >> (sh + 4)) & 0xf) | (((s1 >> (sh + 6)) & 3) << 4);
 }
 
-// What a thread holds between the loads of a step and its LDS stores.
-template <int XV>
-struct Fetched {
-    u32x4 x[XV];    // 16-byte pieces of the x tile
-    u32x4 hdr;      // Q4_K: d, dmin and the scales. Q6_K: x = the 8 scales of the half, y = unused, z = d
+// What a thread holds between the loads of a step and its LDS stores: its
+// piece of W, requested two steps ahead (it comes from HBM), and its pieces of
+// the x tile, requested one step ahead (they come from the L2, every tile of
+// the same rows reads them).
+struct FetchedW {
+    u32x4 hdr;      // Q4_K: d, dmin and the scales. Q6_K: x, y = the 8 scales of the half, z = d
     u32x2 q;        // 8 bytes of nibbles
     u32x2 qh;       // Q6_K: the 8 bytes of upper bits that go with them
-    u32x4 sums;     // first half only: eight int16 sums of x
-    float dx;       // first half only: the scale of one row of x
+};
+template <int XV>
+struct FetchedX {
+    u32x4 x[XV];    // 16-byte pieces of the x tile
+    u32x4 sums;     // second half only: eight int16 sums of x
+    float dx;       // second half only: the scale of one row of x
 };
 
-template <int DT, int MT>  // MT 32-row tiles per wavefront: the workgroup's tile is (128 MT) x 64
+template <int H>
+struct Half {
+    static constexpr int value = H;
+};
+
+// MT 32-row tiles per wavefront: the workgroup's tile is (128 MT) x 64. DEPTH says how far ahead of
+// its LDS stores a step's global loads are requested: 0 one step for W and x, 1 two steps for W, 2 two
+// steps for both; each step further costs the registers of one more set of loads.
+template <int DT, int MT, int DEPTH>
 __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
                                                             float* __restrict__ y, int M, int N, int nsb,
                                                             int64_t act_row_bytes, int tiles_m, int ntiles) {
@@ -142,32 +157,30 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
     if (slot >= per_xcd * tiles_m || t >= ntiles) return;
     const int m0 = tm * TM, n0 = t * kTN;
 
-    // this thread's part of the W tile: 8 bytes of nibbles of row wn_, piece c8 of the half
+    // This thread's part of the W tile: 8 bytes of nibbles of row wrow_i, piece c8 of the half. Its
+    // addresses, and those of its pieces of x, are a base the workgroup shares plus 32 bits of its own.
     const int wrow_i = tid >> 3, c8 = tid & 7;
-    int wrow_g = n0 + wrow_i;
-    wrow_g = wrow_g < N ? wrow_g : N - 1;
-    const uint8_t* wrow = W + (int64_t)wrow_g * nsb * BB;
-    // and of the x tile
-    const uint8_t* xrow[XV];
+    const int last_n = N - 1 - n0, last_m = M - 1 - m0;
+    const uint8_t* w_t = W + (int64_t)n0 * nsb * BB;
+    const uint32_t woff = (uint32_t)(wrow_i < last_n ? wrow_i : last_n) * (uint32_t)(nsb * BB);
+    const uint8_t* act_t = act + (int64_t)m0 * act_row_bytes;
+    uint32_t xoff[XV];
 #pragma unroll
     for (int i = 0; i < XV; i++) {
-        int r = m0 + ((tid + 512 * i) >> 3);
-        r = r < M ? r : M - 1;
-        xrow[i] = act + (int64_t)r * act_row_bytes + 16 * (tid & 7);
+        const int r = (tid + 512 * i) >> 3;
+        xoff[i] = (uint32_t)(r < last_m ? r : last_m) * (uint32_t)act_row_bytes + 16 * (tid & 7);
     }
-    int srow = m0 + (tid >> 1);  // sums: two threads a row (TM = 256), or the first 256 threads (TM = 128)
-    srow = srow < M ? srow : M - 1;
-    const uint8_t* sums_src = act + (int64_t)srow * act_row_bytes + (int64_t)nsb * 256 + 16 * (tid & 1);
-    int drow = m0 + tid;
-    drow = drow < M ? drow : M - 1;
-    const uint8_t* dx_src = act + (int64_t)drow * act_row_bytes + (int64_t)nsb * 288;
+    // sums: two threads a row (TM = 256), or the first 256 threads (TM = 128); scales: a thread a row
+    const uint32_t soff = (uint32_t)((tid >> 1) < last_m ? (tid >> 1) : last_m) * (uint32_t)act_row_bytes + 16 * (tid & 1);
+    const uint32_t doff = (uint32_t)(tid < last_m ? tid : last_m) * (uint32_t)act_row_bytes;
+    const uint8_t* sums_t = act_t + (int64_t)nsb * 256;
+    const uint8_t* dx_t = act_t + (int64_t)nsb * 288;
 
-    Fetched<XV> f;
-    auto fetch = [&](int step) {
-        const int sb = step >> 1, h = step & 1;
-#pragma unroll
-        for (int i = 0; i < XV; i++) f.x[i] = *(const u32x4*)(xrow[i] + (int64_t)sb * 256 + kHalf * h);
-        const uint8_t* wb = wrow + (int64_t)sb * BB;
+    FetchedW fw0, fw1;
+    FetchedX<XV> fx0, fx1;
+    auto fetch_w = [&](FetchedW& f, int sb, auto half) {
+        constexpr int h = decltype(half)::value;
+        const uint8_t* wb = w_t + (int64_t)sb * BB + woff;
         if (DT == kQ4_K) {
             f.hdr = *(const u32x4*)wb;
             f.q = *(const u32x2*)(wb + 16 + 64 * h + 8 * c8);
@@ -179,19 +192,24 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             f.hdr[1] = sc[1];
             f.hdr[2] = load_u16(wb + 208);
         }
-        if (h == 0) {
-            if (DT == kQ4_K && (TM == 256 || tid < 256)) f.sums = *(const u32x4*)(sums_src + (int64_t)sb * 32);
-            if (tid < TM) f.dx = *(const float*)(dx_src + (int64_t)sb * 4);
+    };
+    auto fetch_x = [&](FetchedX<XV>& fx, int sb, auto half) {
+        constexpr int h = decltype(half)::value;
+#pragma unroll
+        for (int i = 0; i < XV; i++) fx.x[i] = *(const u32x4*)(act_t + ((int64_t)sb * 256 + kHalf * h) + xoff[i]);
+        if (h == 1) {
+            if (DT == kQ4_K && (TM == 256 || tid < 256)) fx.sums = *(const u32x4*)(sums_t + (int64_t)sb * 32 + soff);
+            if (tid < TM) fx.dx = *(const float*)(dx_t + (int64_t)sb * 4 + doff);
         }
     };
-    auto stage = [&](int step) {
-        const int sb = step >> 1, h = step & 1;
-        uint8_t* buf = smem + (step & 1) * L::step;
-        uint8_t* side = smem + L::side0 + (sb & 1) * L::side;
+    auto stage = [&](const FetchedW& f, const FetchedX<XV>& fx, int sb, auto half) {
+        constexpr int h = decltype(half)::value;
+        uint8_t* buf = smem + h * L::step;
+        uint8_t* side = smem + L::side0;
 #pragma unroll
         for (int i = 0; i < XV; i++) {
             const int p = tid + 512 * i;
-            *(u32x4*)(buf + L::x + (p >> 3) * kRow + 16 * (p & 7)) = f.x[i];
+            *(u32x4*)(buf + L::x + (p >> 3) * kRow + 16 * (p & 7)) = fx.x[i];
         }
         u32x2 alo, blo, ahi, bhi;
         int klo, khi;
@@ -208,7 +226,7 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             }
             klo = 64 * (c8 >> 2) + 8 * (c8 & 3);
             khi = klo + 32;
-            if (h == 0) {
+            if (h == 1) {
                 if (c8 == 0) {
                     float* dw = (float*)(side + L::dw) + 2 * wrow_i;
                     dw[0] = f16_bits_to_f32((uint16_t)f.hdr[0]);
@@ -233,7 +251,7 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             }
             klo = 8 * c8;
             khi = klo + 64;
-            if (h == 0 && c8 == 0) {
+            if (h == 1 && c8 == 0) {
                 float* dw = (float*)(side + L::dw) + 2 * wrow_i;
                 dw[0] = f16_bits_to_f32((uint16_t)f.hdr[2]);
             }
@@ -244,13 +262,13 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
         *(u32x2*)(wa + khi) = ahi;
         *(u32x2*)(wbp + klo) = blo;
         *(u32x2*)(wbp + khi) = bhi;
-        if (h == 0) {
+        if (h == 1) {
             if (DT == kQ4_K && (TM == 256 || tid < 256)) {
-                const s16x8 s = __builtin_bit_cast(s16x8, f.sums);
+                const s16x8 s = __builtin_bit_cast(s16x8, fx.sums);
                 const f16x8 hsum = __builtin_convertvector(s, f16x8);
                 *(f16x8*)(side + L::xsum + (tid >> 1) * kSumRow + 16 * (tid & 1)) = hsum;
             }
-            if (tid < TM) ((float*)(side + L::dx))[tid] = f.dx;
+            if (tid < TM) ((float*)(side + L::dx))[tid] = fx.dx;
         }
     };
 
@@ -264,13 +282,9 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             acc[mt][i] = accm[mt][i] = 0.f;
         }
 
-    const int steps = 2 * nsb;
-    fetch(0);
-    stage(0);
-    lds_barrier();
-    for (int step = 0; step < steps; step++) {
-        if (step + 1 < steps) fetch(step + 1);
-        const uint8_t* buf = smem + (step & 1) * L::step;
+    auto compute = [&](int sb, auto half) {
+        constexpr int h = decltype(half)::value;
+        const uint8_t* buf = smem + h * L::step;
         const uint8_t* xa = buf + L::x + (wm * 32 * MT + l32) * kRow + 16 * lh;
         const uint8_t* pa = buf + L::wa + (wn * 32 + l32) * kRow + 16 * lh;
         const uint8_t* pb = buf + L::wb + (wn * 32 + l32) * kRow + 16 * lh;
@@ -284,8 +298,9 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
                 acc_b[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wb, acc_b[mt], 0, 0, 0);
             }
         }
-        if (step & 1) {  // the super-block is complete
-            const uint8_t* side = smem + L::side0 + ((step >> 1) & 1) * L::side;
+        if (h == 1) {  // the super-block is complete
+            __builtin_amdgcn_sched_barrier(0);
+            const uint8_t* side = smem + L::side0;
             const float* dwp = (const float*)(side + L::dw) + 2 * (wn * 32 + l32);
             const float dw = dwp[0], dmin = DT == kQ4_K ? dwp[1] : 0.f;
 #pragma unroll
@@ -319,9 +334,44 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
                         acc_b[mt][i] = 0;
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);  // one tile at a time: interleaving them costs registers the kernel lacks
             }
         }
-        if (step + 1 < steps) stage(step + 1);
+    };
+
+    const Half<0> h0;
+    const Half<1> h1;
+    // Sets of loads: with two steps of lead, the steps of a first half use fw0 / fx0 and those of a
+    // second half fw1 / fx1; with one step of lead there is one set.
+    FetchedW& fwb = DEPTH >= 1 ? fw1 : fw0;
+    FetchedX<XV>& fxb = DEPTH >= 2 ? fx1 : fx0;
+    fetch_w(fw0, 0, h0);
+    fetch_x(fx0, 0, h0);
+    if (DEPTH >= 1) fetch_w(fw1, 0, h1);
+    if (DEPTH >= 2) fetch_x(fx1, 0, h1);
+    stage(fw0, fx0, 0, h0);
+    lds_barrier();
+    for (int sb = 0; sb < nsb; sb++) {
+        const bool more = sb + 1 < nsb;
+        if (DEPTH >= 1) {
+            if (more) fetch_w(fw0, sb + 1, h0);
+        } else {
+            fetch_w(fw0, sb, h1);
+        }
+        if (DEPTH >= 2) {
+            if (more) fetch_x(fx0, sb + 1, h0);
+        } else {
+            fetch_x(fx0, sb, h1);
+        }
+        compute(sb, h0);
+        stage(fwb, fxb, sb, h1);
+        lds_barrier();
+        if (more) {
+            if (DEPTH >= 1) fetch_w(fw1, sb + 1, h1); else fetch_w(fw0, sb + 1, h0);
+            if (DEPTH >= 2) fetch_x(fx1, sb + 1, h1); else fetch_x(fx0, sb + 1, h0);
+        }
+        compute(sb, h1);
+        if (more) stage(fw0, fx0, sb + 1, h0);
         lds_barrier();
     }
 
@@ -337,16 +387,18 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 
 template <int DT, int MT>
 hipError_t launch(const QGemvArgs& a, int nsb, hipStream_t st) {
+    // What the registers allow: 256 a lane at two wavefronts a SIMD.
+    constexpr int DEPTH = MT == 1 ? 2 : DT == kQ6_K ? 1 : 0;
     typedef Layout<128 * MT> L;
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemm_kquant_kernel<DT, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, L::total);
+        hipError_t e = hipFuncSetAttribute((const void*)qgemm_kquant_kernel<DT, MT, DEPTH>, hipFuncAttributeMaxDynamicSharedMemorySize, L::total);
         if (e != hipSuccess) return e;
         raised = true;
     }
     const int tiles_m = (int)((a.M + 128 * MT - 1) / (128 * MT)), ntiles = (int)((a.N + kTN - 1) / kTN);
     const int per_xcd = (ntiles + 7) / 8;
-    hipLaunchKernelGGL((qgemm_kquant_kernel<DT, MT>), dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), L::total, st,
+    hipLaunchKernelGGL((qgemm_kquant_kernel<DT, MT, DEPTH>), dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), L::total, st,
                        (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, (int)a.M, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K),
                        tiles_m, ntiles);
     return hipGetLastError();
@@ -357,14 +409,28 @@ hipError_t launch(const QGemvArgs& a, int nsb, hipStream_t st) {
 bool qgemm_kquant_ok(int dt, const QGemvArgs& a) {
     // Q4_K's blocks are read with aligned loads (144 bytes keep a 16-byte aligned W aligned); Q6_K's 2-byte aligned.
     return (dt == kQ4_K || dt == kQ6_K) && a.K % 256 == 0 && a.K > 0 && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0 &&
-           ((uintptr_t)a.act & 15) == 0 && a.M * ((a.N + kTN - 1) / kTN) < ((int64_t)1 << 30);
+           ((uintptr_t)a.act & 15) == 0 && a.M * ((a.N + kTN - 1) / kTN) < ((int64_t)1 << 30) && a.K <= (1 << 20);
+}
+
+static bool tall_tiles(const QGemvArgs& a) {
+    // 256-row tiles halve the work of splitting W; 128-row tiles where those would leave compute units idle.
+    return a.M > 128 && ((a.M + 255) / 256) * ((a.N + kTN - 1) / kTN) >= 256;
+}
+
+// The row-by-row kernels read W once per row of x, at about 8 TB/s once it sits in the caches; a
+// workgroup here spends about 2.1 us (5.5 with 256-row tiles) per super-block of K, 256 workgroups
+// at a time. Measured on 4096 x 4096 to 14336 x 4096 weights, 2 to 64 rows.
+bool qgemm_kquant_pays(int dt, const QGemvArgs& a) {
+    if (a.M < 8) return false;
+    const double nsb = (double)(a.K / 256), rows_us = (double)a.M * (double)a.N * nsb * (dt == kQ4_K ? 144 : 210) / 8.0e6;
+    const bool tall = tall_tiles(a);
+    const int64_t tiles = ((a.M + (tall ? 255 : 127)) / (tall ? 256 : 128)) * ((a.N + kTN - 1) / kTN);
+    return (double)((tiles + 255) / 256) * nsb * (tall ? 5.5 : 2.1) < rows_us;
 }
 
 hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st) {
     const int nsb = (int)(a.K / 256);
-    const int64_t ntiles = (a.N + kTN - 1) / kTN;
-    // 256-row tiles halve the work of splitting W; 128-row tiles where those would leave compute units idle.
-    const bool tall = a.M > 128 && ((a.M + 255) / 256) * ntiles >= 256;
+    const bool tall = tall_tiles(a);
     if (dt == kQ4_K) return tall ? launch<kQ4_K, 2>(a, nsb, st) : launch<kQ4_K, 1>(a, nsb, st);
     return tall ? launch<kQ6_K, 2>(a, nsb, st) : launch<kQ6_K, 1>(a, nsb, st);
 }

@@ -460,7 +460,7 @@ static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st)
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     int nsb = (int)(a.K / 256);
     // From a few rows of x on, the matrix cores (whose results are the CPU's bit for bit).
-    if ((g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && a.M >= kQGemmMinRows)) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
+    if ((g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && qgemm_kquant_pays(dt, a))) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
     // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.
     // Q6_K's 210-byte blocks are read as aligned dwords around a 2-byte aligned start.
     const bool lds_ok = kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;

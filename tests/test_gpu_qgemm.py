@@ -193,7 +193,8 @@ def test_errors():
     l = gpu.lib()
     z = torch.zeros(4096, dtype=torch.int16, device="cuda:0")
     p = z.data_ptr()
-    assert l.mi355x_qgemm_bf16(capi.Q8_0, p, p, p, 2, 32, 64, 64, capi.BF16, gpu.stream()) == capi.ERR_DTYPE
+    assert l.mi355x_qgemm_bf16(capi.F16, p, p, p, 2, 32, 64, 64, capi.BF16, gpu.stream()) == capi.ERR_DTYPE
+    assert l.mi355x_qgemm_bf16(capi.Q4_K, p, p, p, 2, 32, 64, 64, capi.BF16, gpu.stream()) == capi.ERR_INTERNAL  # K not in blocks of 256
     assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 64, 64, capi.F16, gpu.stream()) == capi.ERR_DTYPE
     assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 48, 48, capi.BF16, gpu.stream()) == capi.ERR_INTERNAL
     assert l.mi355x_qgemm_bf16(capi.Q4_0, p, p, p, 2, 32, 64, 32, capi.BF16, gpu.stream()) == capi.ERR_SHAPE

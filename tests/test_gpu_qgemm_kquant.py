@@ -13,6 +13,15 @@ from tests.helpers import bits_equal, exact_rows, random_blocks
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture
+def matrix_cores():
+    """The library picks the faster kernel by shape; these tests are about one of them."""
+    l = gpu.lib()
+    capi.check(l.mi355x_tune(b"kquant.path", 3))
+    yield
+    capi.check(l.mi355x_tune(b"kquant.path", 0))
+
+
 def product(dt, raw, x, n, k, offset=0):
     buf, ptr = gpu.dev_bytes_at(raw, offset)
     return gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
@@ -21,7 +30,7 @@ def product(dt, raw, x, n, k, offset=0):
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
 @pytest.mark.parametrize("m,n,k", [(8, 5, 256), (33, 64, 1280), (130, 100, 512), (256, 64, 256), (300, 200, 768),
                                    (129, 65, 256 * 17), (512, 2048, 1024)])
-def test_matches_the_cpu_bit_for_bit(dt, m, n, k):
+def test_matches_the_cpu_bit_for_bit(dt, m, n, k, matrix_cores):
     rng = np.random.default_rng(m + n + k + dt)
     raw = random_blocks(rng, dt, n * k)
     x = rng.normal(size=(m, k)).astype(np.float32)
@@ -33,7 +42,7 @@ def test_matches_the_cpu_bit_for_bit(dt, m, n, k):
 
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
-def test_extreme_quants_and_scales(dt):
+def test_extreme_quants_and_scales(dt, matrix_cores):
     """Every quant and scale at its largest magnitude with x at +-127 per super-block: the largest integer sums
     the planes and the sums of x can reach (backend/cpu/quant_test.go:164-204)."""
     m, n, k = 40, 64, 512
@@ -59,7 +68,7 @@ def test_extreme_quants_and_scales(dt):
 
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
-def test_rows_with_nan_and_inf(dt):
+def test_rows_with_nan_and_inf(dt, matrix_cores):
     m, n, k = 16, 70, 768
     rng = np.random.default_rng(5)
     raw = random_blocks(rng, dt, n * k)
@@ -73,7 +82,7 @@ def test_rows_with_nan_and_inf(dt):
     assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
 
 
-def test_q6_k_from_a_2_byte_aligned_start_and_q4_k_from_a_misaligned_one():
+def test_q6_k_from_a_2_byte_aligned_start_and_q4_k_from_a_misaligned_one(matrix_cores):
     m, n, k = 64, 96, 1024
     rng = np.random.default_rng(6)
     x = rng.normal(size=(m, k)).astype(np.float32)
@@ -110,3 +119,32 @@ def test_one_row_and_the_row_by_row_kernels_agree_within_rounding(dt):
         assert np.all(np.abs(got - want2) <= 4e-6 * mag + 1e-30)
     finally:
         capi.check(l.mi355x_tune(b"kquant.path", 0))
+
+
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+def test_prompt_sized_products_take_the_matrix_cores_and_bf16_rounds_once(dt):
+    """Left to itself the library sends a prompt-sized product to the matrix cores (the CPU's bits), and
+    mi355x_qgemm_bf16 is the reference's sequence for a half x: cast to float32, product, one rounding
+    (tensor/quant.go:45-48)."""
+    import torch
+    m, n, k = 512, 1024, 2048
+    rng = np.random.default_rng(31 + dt)
+    raw = random_blocks(rng, dt, n * k)
+    xb = O.f32_to_bf16(rng.normal(size=(m, k)).astype(np.float32))
+    xf = O.bf16_to_f32(xb)
+    want = O.qmatmul(dt, raw, xf, n, k)
+    gpu.say(f"kquant gemm dt={dt} default dispatch")
+    assert bits_equal(product(dt, raw, xf, n, k), want)
+    l = gpu.lib()
+    wbuf, wp = gpu.dev_bytes_at(raw, 0)
+    xd = torch.from_numpy(xb.view(np.int16)).to("cuda:0")
+    for out_dt in (capi.BF16, capi.F32):
+        y = torch.zeros((m, n), dtype=torch.int16 if out_dt == capi.BF16 else torch.float32, device="cuda:0")
+        gpu.say(f"qgemm_bf16 dt={dt} out={out_dt}")
+        capi.check(l.mi355x_qgemm_bf16(dt, wp, xd.data_ptr(), y.data_ptr(), m, n, k, k, out_dt, gpu.stream()))
+        gpu.sync()
+        got = y.cpu().numpy()
+        if out_dt == capi.BF16:
+            assert np.array_equal(got.view(np.uint16), O.f32_to_bf16(want))
+        else:
+            assert bits_equal(got, want)
