@@ -170,9 +170,11 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
         const int r = (tid + 512 * i) >> 3;
         xoff[i] = (uint32_t)(r < last_m ? r : last_m) * (uint32_t)act_row_bytes + 16 * (tid & 7);
     }
-    // sums: two threads a row (TM = 256), or the first 256 threads (TM = 128); scales: a thread a row
-    const uint32_t soff = (uint32_t)((tid >> 1) < last_m ? (tid >> 1) : last_m) * (uint32_t)act_row_bytes + 16 * (tid & 1);
-    const uint32_t doff = (uint32_t)(tid < last_m ? tid : last_m) * (uint32_t)act_row_bytes;
+    // sums: two threads a row; scales: a thread a row
+    // (with 128-row tiles two threads do the same row's part: branch-free, and the same bytes to the same place)
+    const int srow = (tid >> 1) & (TM - 1), drow = tid & (TM - 1);
+    const uint32_t soff = (uint32_t)(srow < last_m ? srow : last_m) * (uint32_t)act_row_bytes + 16 * (tid & 1);
+    const uint32_t doff = (uint32_t)(drow < last_m ? drow : last_m) * (uint32_t)act_row_bytes;
     const uint8_t* sums_t = act_t + (int64_t)nsb * 256;
     const uint8_t* dx_t = act_t + (int64_t)nsb * 288;
 
@@ -198,8 +200,8 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 #pragma unroll
         for (int i = 0; i < XV; i++) fx.x[i] = *(const u32x4*)(act_t + ((int64_t)sb * 256 + kHalf * h) + xoff[i]);
         if (h == 1) {
-            if (DT == kQ4_K && (TM == 256 || tid < 256)) fx.sums = *(const u32x4*)(sums_t + (int64_t)sb * 32 + soff);
-            if (tid < TM) fx.dx = *(const float*)(dx_t + (int64_t)sb * 4 + doff);
+            if (DT == kQ4_K) fx.sums = *(const u32x4*)(sums_t + (int64_t)sb * 32 + soff);
+            fx.dx = *(const float*)(dx_t + (int64_t)sb * 4 + doff);
         }
     };
     auto stage = [&](const FetchedW& f, const FetchedX<XV>& fx, int sb, auto half) {
@@ -227,11 +229,9 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             klo = 64 * (c8 >> 2) + 8 * (c8 & 3);
             khi = klo + 32;
             if (h == 1) {
-                if (c8 == 0) {
-                    float* dw = (float*)(side + L::dw) + 2 * wrow_i;
-                    dw[0] = f16_bits_to_f32((uint16_t)f.hdr[0]);
-                    dw[1] = f16_bits_to_f32((uint16_t)(f.hdr[0] >> 16));
-                }
+                float* dw = (float*)(side + L::dw) + 2 * wrow_i;  // the row's eight threads store the same two values
+                dw[0] = f16_bits_to_f32((uint16_t)f.hdr[0]);
+                dw[1] = f16_bits_to_f32((uint16_t)(f.hdr[0] >> 16));
                 // sub-block c8's min, once for each of its two groups of 16
                 const _Float16 mn = (_Float16)(float)q4k_min(f.hdr[2], f.hdr[3], c8);
                 const uint32_t pair = (uint32_t)__builtin_bit_cast(uint16_t, mn) * 0x00010001u;
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
             }
             klo = 8 * c8;
             khi = klo + 64;
-            if (h == 1 && c8 == 0) {
+            if (h == 1) {
                 float* dw = (float*)(side + L::dw) + 2 * wrow_i;
                 dw[0] = f16_bits_to_f32((uint16_t)f.hdr[2]);
             }
@@ -263,12 +263,12 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
         *(u32x2*)(wbp + klo) = blo;
         *(u32x2*)(wbp + khi) = bhi;
         if (h == 1) {
-            if (DT == kQ4_K && (TM == 256 || tid < 256)) {
+            if (DT == kQ4_K) {
                 const s16x8 s = __builtin_bit_cast(s16x8, fx.sums);
                 const f16x8 hsum = __builtin_convertvector(s, f16x8);
-                *(f16x8*)(side + L::xsum + (tid >> 1) * kSumRow + 16 * (tid & 1)) = hsum;
+                *(f16x8*)(side + L::xsum + srow * kSumRow + 16 * (tid & 1)) = hsum;
             }
-            if (tid < TM) ((float*)(side + L::dx))[tid] = fx.dx;
+            ((float*)(side + L::dx))[drow] = fx.dx;
         }
     };
 
@@ -277,10 +277,7 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            acc_a[mt][i] = acc_b[mt][i] = 0;
-            acc[mt][i] = accm[mt][i] = 0.f;
-        }
+        for (int i = 0; i < 16; i++) acc[mt][i] = accm[mt][i] = 0.f;
 
     auto compute = [&](int sb, auto half) {
         constexpr int h = decltype(half)::value;
@@ -294,12 +291,22 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
                 const i32x4 x = *(const i32x4*)(xa + mt * 32 * kRow + 32 * s);
-                acc_a[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wa, acc_a[mt], 0, 0, 0);
-                acc_b[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wb, acc_b[mt], 0, 0, 0);
+                if (h == 0 && s == 0) {  // a super-block's first products start its sums from the constant zero
+                    i32x16 zero;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) zero[i] = 0;
+                    acc_a[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wa, zero, 0, 0, 0);
+                    acc_b[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wb, zero, 0, 0, 0);
+                } else {
+                    acc_a[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wa, acc_a[mt], 0, 0, 0);
+                    acc_b[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, wb, acc_b[mt], 0, 0, 0);
+                }
             }
         }
-        if (h == 1) {  // the super-block is complete
-            __builtin_amdgcn_sched_barrier(0);
+    };
+    // The end of a super-block: its integer sums into the float32 sums, as the CPU does it.
+    auto finish = [&]() {
+        {
             const uint8_t* side = smem + L::side0;
             const float* dwp = (const float*)(side + L::dw) + 2 * (wn * 32 + l32);
             const float dw = dwp[0], dmin = DT == kQ4_K ? dwp[1] : 0.f;
@@ -330,8 +337,6 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
                             const float u = dm * summ[i];
                             accm[mt][i] = accm[mt][i] + u;
                         }
-                        acc_a[mt][i] = 0;
-                        acc_b[mt][i] = 0;
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);  // one tile at a time: interleaving them costs registers the kernel lacks
@@ -351,27 +356,20 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
     if (DEPTH >= 2) fetch_x(fx1, 0, h1);
     stage(fw0, fx0, 0, h0);
     lds_barrier();
+    // No branches inside: the last super-block requests and stages itself again, into buffers nobody reads.
     for (int sb = 0; sb < nsb; sb++) {
-        const bool more = sb + 1 < nsb;
-        if (DEPTH >= 1) {
-            if (more) fetch_w(fw0, sb + 1, h0);
-        } else {
-            fetch_w(fw0, sb, h1);
-        }
-        if (DEPTH >= 2) {
-            if (more) fetch_x(fx0, sb + 1, h0);
-        } else {
-            fetch_x(fx0, sb, h1);
-        }
+        const int nx = sb + 1 < nsb ? sb + 1 : sb;
+        if (DEPTH >= 1) fetch_w(fw0, nx, h0); else fetch_w(fw0, sb, h1);
+        if (DEPTH >= 2) fetch_x(fx0, nx, h0); else fetch_x(fx0, sb, h1);
         compute(sb, h0);
         stage(fwb, fxb, sb, h1);
         lds_barrier();
-        if (more) {
-            if (DEPTH >= 1) fetch_w(fw1, sb + 1, h1); else fetch_w(fw0, sb + 1, h0);
-            if (DEPTH >= 2) fetch_x(fx1, sb + 1, h1); else fetch_x(fx0, sb + 1, h0);
-        }
+        if (DEPTH >= 1) fetch_w(fw1, nx, h1); else fetch_w(fw0, nx, h0);
+        if (DEPTH >= 2) fetch_x(fx1, nx, h1); else fetch_x(fx0, nx, h0);
         compute(sb, h1);
-        if (more) stage(fw0, fx0, sb + 1, h0);
+        __builtin_amdgcn_sched_barrier(0);
+        finish();
+        stage(fw0, fx0, nx, h0);
         lds_barrier();
     }
 
@@ -388,7 +386,7 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 template <int DT, int MT>
 hipError_t launch(const QGemvArgs& a, int nsb, hipStream_t st) {
     // What the registers allow: 256 a lane at two wavefronts a SIMD.
-    constexpr int DEPTH = MT == 1 ? 2 : DT == kQ6_K ? 1 : 0;
+    constexpr int DEPTH = MT == 1 ? 2 : 1;
     typedef Layout<128 * MT> L;
     static bool raised = false;
     if (!raised) {
