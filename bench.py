@@ -244,33 +244,54 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0):
             "first_tokens": out[0, :8].tolist()}
 
 
+def bench_blocks_kquant(rng, dtype_bytes, n_elems):
+    """Random Q4_K (144-byte) or Q6_K (210-byte) super-blocks: every field uniform, the binary16 scales |N(0, 0.02)|."""
+    raw = rng.integers(0, 256, size=(n_elems // 256, dtype_bytes), dtype=np.uint8)
+    scales = np.abs(rng.normal(0, 0.02, size=(raw.shape[0], 2))).astype(np.float16).view(np.uint8).reshape(-1, 4)
+    if dtype_bytes == 144:
+        raw[:, 0:4] = scales
+    else:
+        raw[:, 208:210] = scales[:, 0:2]
+    return raw.reshape(-1)
+
+
 def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096), (2048, 14336)), k=4096, iters=50):
-    """The prompt-sized Q4_0 product (bfloat16 in and out) on the matrix cores:
-    TFLOP/s (2 M N K) of the whole call, between HIP events on its stream,
-    against the dense bfloat16 peak."""
+    """The prompt-sized products with bfloat16 activations and results, mi355x_qgemm_bf16 as a whole
+    (for Q4_K and Q6_K that includes the casts and the int8 rounding of x): TFLOP/s (2 M N K) between
+    HIP events on its stream, against the dense peak of the matrix instruction used (bfloat16 2.5 PFLOP/s
+    for Q4_0, int8 5.0 POP/s for the K-quants; each weight takes two multiplications in both)."""
     out = {}
     rng = np.random.default_rng(0)
     st = torch.cuda.Stream()
-    for m, n in shapes:
-        w = torch.from_numpy(bench_blocks_q4_0(rng, n * k)).to("cuda:0")
-        x = torch.randn(m, k, device="cuda:0").to(torch.bfloat16)
-        y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
-        torch.cuda.synchronize()
-        with torch.cuda.stream(st):
-            call = lambda: capi.check(lib.mi355x_qgemm_bf16(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, capi.BF16, st.cuda_stream))
-            for _ in range(5):
-                call()
-            st.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(st)
-            for _ in range(iters):
-                call()
-            e1.record(st)
-            st.synchronize()
-        us = e0.elapsed_time(e1) / iters * 1e3
-        tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
-        out[f"M{m}_N{n}_K{k}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_bf16_peak": round(tf / 2500.0, 4)}
-        del w, x, y
+    kinds = (("q4_0", capi.Q4_0, 2500.0, "frac_of_bf16_peak"), ("q4_K", capi.Q4_K, 5000.0, "frac_of_int8_peak"),
+             ("q6_K", capi.Q6_K, 5000.0, "frac_of_int8_peak"))
+    for name, dt, peak, frac_key in kinds:
+        res = {}
+        for m, n in shapes:
+            if dt == capi.Q4_0:
+                raw = bench_blocks_q4_0(rng, n * k)
+            else:
+                raw = bench_blocks_kquant(rng, 144 if dt == capi.Q4_K else 210, n * k)
+            w = torch.from_numpy(raw).to("cuda:0")
+            x = torch.randn(m, k, device="cuda:0").to(torch.bfloat16)
+            y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+            torch.cuda.synchronize()
+            with torch.cuda.stream(st):
+                call = lambda: capi.check(lib.mi355x_qgemm_bf16(dt, w.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, capi.BF16, st.cuda_stream))
+                for _ in range(5):
+                    call()
+                st.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(st)
+                for _ in range(iters):
+                    call()
+                e1.record(st)
+                st.synchronize()
+            us = e0.elapsed_time(e1) / iters * 1e3
+            tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+            res[f"M{m}_N{n}_K{k}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1), frac_key: round(tf / peak, 4)}
+            del w, x, y
+        out[name] = res
     return out
 
 

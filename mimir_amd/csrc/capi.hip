@@ -284,6 +284,17 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
         HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
+    if ((dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) && g_tune_gemm != 1 && ((uintptr_t)X & 7) == 0 && x_row_stride % 4 == 0) {
+        // the int8 rounding reads the bfloat16 rows directly and the matrix-core kernel rounds its results
+        void* act;
+        if (mi355x_status s2 = act_scratch(mimir::kq_act_bytes(K) * (size_t)M, &act)) return s2;
+        mimir::QGemvArgs a{W, nullptr, act, (float*)Y, M, N, K, 0, 0};
+        if (mimir::qgemm_kquant_ok(dtype, a) && mimir::qgemm_kquant_pays(dtype, a)) {
+            HIP_TRY(mimir::kq_convert_act_bf16(X, M, K, x_row_stride, act, st), "launch kq_convert_act");
+            HIP_TRY(mimir::qgemm_kquant(dtype, a, st, !f32), "launch qgemm_kquant");
+            return MI355X_OK;
+        }
+    }
     // Any other shape or dtype: the activations as float32 through mi355x_qgemv, then one rounding. For
     // Q8_0, Q4_K and Q6_K that is the reference's own sequence (cast, int8 rounding of x, integer dot
     // products, cast), and the K-quants take their matrix-core kernel from a few rows on.

@@ -69,12 +69,15 @@ hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // (kq_convert_act, kq_act_bytes(K) bytes per row), integer dot products.
 size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+// The same from bfloat16 rows (8-byte aligned, a multiple of 4 elements apart).
+hipError_t kq_convert_act_bf16(const void* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
 // The same products for many rows of x on the matrix cores (qgemm_kquant.hip); qgemv_kquant_act
 // hands over to it where qgemm_kquant_pays says it is the faster of the two.
 bool qgemm_kquant_pays(int dt, const QGemvArgs& a);
 bool qgemm_kquant_ok(int dt, const QGemvArgs& a);
-hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st);
+// y float32, or with out_bf16 each result rounded once to bfloat16 into y taken as uint16_t*.
+hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st, bool out_bf16 = false);
 // which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in
 // global memory, 2 = never the matrix-core kernel, 3 = always the matrix-core kernel.
 void set_kquant_tune(int which, int value);

@@ -136,9 +136,9 @@ struct Half {
 // MT 32-row tiles per wavefront: the workgroup's tile is (128 MT) x 64. DEPTH says how far ahead of
 // its LDS stores a step's global loads are requested: 0 one step for W and x, 1 two steps for W, 2 two
 // steps for both; each step further costs the registers of one more set of loads.
-template <int DT, int MT, int DEPTH>
+template <int DT, int MT, int DEPTH, bool OUT_BF16>
 __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                            float* __restrict__ y, int M, int N, int nsb,
+                                                            void* __restrict__ yv, int M, int N, int nsb,
                                                             int64_t act_row_bytes, int tiles_m, int ntiles) {
     constexpr int TM = 128 * MT;
     constexpr int XV = TM * 8 / 512;  // 16-byte pieces of x per thread and step: piece p is row p / 8, bytes 16 (p % 8)..
@@ -379,25 +379,29 @@ __global__ __launch_bounds__(512) void qgemm_kquant_kernel(const uint8_t* __rest
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int m = m0 + wm * 32 * MT + 32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3);
-            if (m < M && n < N) y[(int64_t)m * N + n] = DT == kQ4_K ? acc[mt][i] - accm[mt][i] : acc[mt][i];
+            if (m < M && n < N) {
+                const float v = DT == kQ4_K ? acc[mt][i] - accm[mt][i] : acc[mt][i];
+                if (OUT_BF16) ((uint16_t*)yv)[(int64_t)m * N + n] = f32_to_bf16_bits(v);
+                else ((float*)yv)[(int64_t)m * N + n] = v;
+            }
         }
 }
 
-template <int DT, int MT>
+template <int DT, int MT, bool OUT_BF16>
 hipError_t launch(const QGemvArgs& a, int nsb, hipStream_t st) {
     // What the registers allow: 256 a lane at two wavefronts a SIMD.
     constexpr int DEPTH = MT == 1 ? 2 : 1;
     typedef Layout<128 * MT> L;
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemm_kquant_kernel<DT, MT, DEPTH>, hipFuncAttributeMaxDynamicSharedMemorySize, L::total);
+        hipError_t e = hipFuncSetAttribute((const void*)qgemm_kquant_kernel<DT, MT, DEPTH, OUT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, L::total);
         if (e != hipSuccess) return e;
         raised = true;
     }
     const int tiles_m = (int)((a.M + 128 * MT - 1) / (128 * MT)), ntiles = (int)((a.N + kTN - 1) / kTN);
     const int per_xcd = (ntiles + 7) / 8;
-    hipLaunchKernelGGL((qgemm_kquant_kernel<DT, MT, DEPTH>), dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), L::total, st,
-                       (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, (int)a.M, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K),
+    hipLaunchKernelGGL((qgemm_kquant_kernel<DT, MT, DEPTH, OUT_BF16>), dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), L::total, st,
+                       (const uint8_t*)a.W, (const uint8_t*)a.act, (void*)a.y, (int)a.M, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K),
                        tiles_m, ntiles);
     return hipGetLastError();
 }
@@ -426,11 +430,16 @@ bool qgemm_kquant_pays(int dt, const QGemvArgs& a) {
     return (double)((tiles + 255) / 256) * nsb * (tall ? 5.5 : 2.1) < rows_us;
 }
 
-hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st) {
+template <bool OUT_BF16>
+static hipError_t pick(int dt, const QGemvArgs& a, hipStream_t st) {
     const int nsb = (int)(a.K / 256);
     const bool tall = tall_tiles(a);
-    if (dt == kQ4_K) return tall ? launch<kQ4_K, 2>(a, nsb, st) : launch<kQ4_K, 1>(a, nsb, st);
-    return tall ? launch<kQ6_K, 2>(a, nsb, st) : launch<kQ6_K, 1>(a, nsb, st);
+    if (dt == kQ4_K) return tall ? launch<kQ4_K, 2, OUT_BF16>(a, nsb, st) : launch<kQ4_K, 1, OUT_BF16>(a, nsb, st);
+    return tall ? launch<kQ6_K, 2, OUT_BF16>(a, nsb, st) : launch<kQ6_K, 1, OUT_BF16>(a, nsb, st);
+}
+
+hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st, bool out_bf16) {
+    return out_bf16 ? pick<true>(dt, a, st) : pick<false>(dt, a, st);
 }
 
 }  // namespace mimir

@@ -47,16 +47,26 @@ __device__ __forceinline__ int dpp_i32_group8_sum(int v) {
 
 // quantizeRow for super-blocks of 256 with sums: one wavefront per
 // super-block, lane i taking values 4i..4i+3.
-__global__ __launch_bounds__(64) void kq_convert_act_kernel(const float* __restrict__ x, int64_t x_row_stride, int nsb,
+template <bool BF16>  // x float32, or bfloat16 (widened exactly, as the cast in front of the product does: tensor/quant.go:45-48)
+__global__ __launch_bounds__(64) void kq_convert_act_kernel(const void* __restrict__ xv, int64_t x_row_stride, int nsb,
                                                             uint8_t* __restrict__ act, int64_t act_row_bytes) {
     const int sb = blockIdx.x, lane = threadIdx.x;
-    const float* xr = x + (int64_t)blockIdx.y * x_row_stride + 256 * (int64_t)sb;
+    const int64_t at = (int64_t)blockIdx.y * x_row_stride + 256 * (int64_t)sb + 4 * lane;
     uint8_t* row = act + (int64_t)blockIdx.y * act_row_bytes;
     uint32_t* q = (uint32_t*)row + (int64_t)sb * 64;
     uint16_t* sums = (uint16_t*)(row + (int64_t)nsb * 256) + sb * 16;
     float* dscale = (float*)(row + (int64_t)nsb * 288);
     f32x4 v;
-    __builtin_memcpy(&v, xr + 4 * lane, 16);
+    if (BF16) {
+        u32x2 h;
+        __builtin_memcpy(&h, (const uint16_t*)xv + at, 8);
+        v[0] = __builtin_bit_cast(float, h[0] << 16);
+        v[1] = __builtin_bit_cast(float, h[0] & 0xffff0000u);
+        v[2] = __builtin_bit_cast(float, h[1] << 16);
+        v[3] = __builtin_bit_cast(float, h[1] & 0xffff0000u);
+    } else {
+        __builtin_memcpy(&v, (const float*)xv + at, 16);
+    }
     float amax = 0.f;
     bool finite = true;
 #pragma unroll
@@ -91,7 +101,14 @@ __global__ __launch_bounds__(64) void kq_convert_act_kernel(const float* __restr
 
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
     int nsb = (int)(K / 256);
-    hipLaunchKernelGGL(kq_convert_act_kernel, dim3((unsigned)nsb, (unsigned)M), dim3(64), 0, st, x, x_row_stride, nsb,
+    hipLaunchKernelGGL(kq_convert_act_kernel<false>, dim3((unsigned)nsb, (unsigned)M), dim3(64), 0, st, (const void*)x, x_row_stride,
+                       nsb, (uint8_t*)act, (int64_t)kq_act_bytes(K));
+    return hipGetLastError();
+}
+
+hipError_t kq_convert_act_bf16(const void* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
+    int nsb = (int)(K / 256);
+    hipLaunchKernelGGL(kq_convert_act_kernel<true>, dim3((unsigned)nsb, (unsigned)M), dim3(64), 0, st, x, x_row_stride, nsb,
                        (uint8_t*)act, (int64_t)kq_act_bytes(K));
     return hipGetLastError();
 }
