@@ -5,8 +5,8 @@
 // qmatmul.go:208-254), integer dot products weighted by the 6-bit (Q4_K) or
 // int8 (Q6_K) sub-block scales, one float32 multiply-add pair per super-block
 // (multiply, then add: never fused), Q4_K's mins applied through the sums.
-// The integers are exact; only the order in which a row's super-blocks are
-// added differs from the CPU's.
+// The integers are exact and a row's super-blocks are added in the CPU's
+// order: the results are the CPU's bit for bit.
 //
 // W is read in place in ggml's layout. The kernels that serve ordinary shapes
 // stage the converted row of x in LDS once per workgroup; a wavefront owns R
@@ -43,6 +43,18 @@ __device__ __forceinline__ int dpp_i32_group8_sum(int v) {
     v = dpp_i32_quad_sum(v);
     v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true);
     return v;
+}
+
+// Every STRIDE-th lane holds the term of one super-block, in the order of the
+// super-blocks; they are added to acc one after the other, the order in which the
+// CPU adds its super-blocks (qmatmul.go:148-200), so the float32 sum is the CPU's
+// bit for bit. A lane without a term holds +0, which changes no sum that began at +0.
+template <int STRIDE>
+__device__ __forceinline__ float add_in_order(float acc, float term) {
+#pragma unroll
+    for (int q = 0; q < 64 / STRIDE; q++)
+        acc = acc + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, term), q * STRIDE));
+    return acc;
 }
 
 // quantizeRow for super-blocks of 256 with sums: one wavefront per
@@ -165,17 +177,16 @@ __global__ __launch_bounds__(256) void qgemv_q4k_plain_kernel(const uint8_t* __r
         int summ = m0 * (i16_at(s, 0) + i16_at(s, 1)) + m1 * (i16_at(s, 2) + i16_at(s, 3));
         sumi = dpp_i32_quad_sum(live ? sumi : 0);
         summ = dpp_i32_quad_sum(live ? summ : 0);
+        float t = 0.f, u = 0.f;
         if (j == 0 && live) {
             float xdv = xd[sb];
             float dd = f16_bits_to_f32(load_u16(wb)) * xdv, dm = f16_bits_to_f32(load_u16(wb + 2)) * xdv;
-            float t = dd * (float)sumi;
-            acc = acc + t;
-            float u = dm * (float)summ;
-            accm = accm + u;
+            t = dd * (float)sumi;
+            u = dm * (float)summ;
         }
+        acc = add_in_order<4>(acc, t);
+        accm = add_in_order<4>(accm, u);
     }
-    acc = wave_sum(acc);
-    accm = wave_sum(accm);
     if (lane == 0) y[(int64_t)blockIdx.y * N + row] = acc - accm;
 }
 
@@ -213,13 +224,13 @@ __global__ __launch_bounds__(256) void qgemv_q6k_plain_kernel(const uint8_t* __r
         const uint16_t* xs = xsums + sb * 16 + g0;
         int sumi = sc0 * s[0] - 32 * sc0 * i16_at(xs, 0) + sc1 * s[1] - 32 * sc1 * i16_at(xs, 1);
         sumi = dpp_i32_group8_sum(live ? sumi : 0);
+        float t = 0.f;
         if (part == 0 && live) {
             float dd = f16_bits_to_f32(load_u16(wb + 208)) * xd[sb];
-            float t = dd * (float)sumi;
-            acc = acc + t;
+            t = dd * (float)sumi;
         }
+        acc = add_in_order<8>(acc, t);
     }
-    acc = wave_sum(acc);
     if (lane == 0) y[(int64_t)blockIdx.y * N + row] = acc;
 }
 
@@ -319,21 +330,20 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __
             int summ = m_a * sa + m_b * sb_ + m_c * sc_ + m_e * se;
             sumi = dpp_i32_quad_sum(live ? sumi : 0);
             summ = dpp_i32_quad_sum(live ? summ : 0);
+            float t = 0.f, u = 0.f;
             if (j == 0 && live) {
                 const uint32_t dw = cur[r].hdr[0];
                 float dd = f16_bits_to_f32((uint16_t)dw) * xscale, dm = f16_bits_to_f32((uint16_t)(dw >> 16)) * xscale;
-                float t = dd * (float)sumi;
-                acc[r] = acc[r] + t;
-                float u = dm * (float)summ;
-                accm[r] = accm[r] + u;
+                t = dd * (float)sumi;
+                u = dm * (float)summ;
             }
+            acc[r] = add_in_order<4>(acc[r], t);
+            accm[r] = add_in_order<4>(accm[r], u);
         }
     }
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        float a = wave_sum(acc[r]), am = wave_sum(accm[r]);
-        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = a - am;
-    }
+    for (int r = 0; r < R; r++)
+        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = acc[r] - accm[r];
 }
 
 // Sixteen bytes at a 2-byte aligned address as five aligned dwords; take(i)
@@ -432,18 +442,17 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
             const int sc_l = (int)(int8_t)(pair >> (8 * c)), sc_h = (int)(int8_t)(pair4 >> (8 * c));
             int sumi = sc_l * (dl - 32 * sl) + sc_h * (dh - 32 * sh_);
             sumi = dpp_i32_group8_sum(live ? sumi : 0);
+            float t = 0.f;
             if (part == 0 && live) {
                 float dd = f16_bits_to_f32(cur[r].d) * xscale;
-                float t = dd * (float)sumi;
-                acc[r] = acc[r] + t;
+                t = dd * (float)sumi;
             }
+            acc[r] = add_in_order<8>(acc[r], t);
         }
     }
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        float a = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = a;
-    }
+    for (int r = 0; r < R; r++)
+        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = acc[r];
 }
 
 // [0] rows per wavefront (0: by shape). [1] 1: always the kernels without LDS, 2: never the
@@ -483,7 +492,7 @@ hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     const bool lds_ok = kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;
     if (g_kq_tune[1] != 1 && lds_ok) {
         int R = g_kq_tune[0];
-        if (R != 1 && R != 2 && R != 4) R = (dt == kQ4_K && a.N * a.M >= 65536) ? 4 : a.N * a.M >= 2048 ? 2 : 1;  // measured: see the sweep keys of mi355x_tune
+        if (R != 1 && R != 2 && R != 4) R = a.N * a.M >= 2048 ? 2 : 1;  // measured: see the sweep keys of mi355x_tune
         return R == 4 ? launch_kq<4>(dt, a, nsb, st) : R == 2 ? launch_kq<2>(dt, a, nsb, st) : launch_kq<1>(dt, a, nsb, st);
     }
     const int waves = 4;

@@ -409,22 +409,20 @@ def test_kquant_activation_rounding_is_bit_exact(dt):
 def test_kquant_gemv_matches_oracle(dt, n, k, offset):
     rng = np.random.default_rng(n + k + dt)
     raw = random_blocks(rng, dt, n * k)
-    wabs = np.abs(O.dequantize(dt, raw).reshape(n, k)).astype(np.float64)
     for shape in ((k,), (2, 3, k)):
         x = rng.normal(size=shape).astype(np.float32)
         gpu.say(f"kquant gemv dt={dt} N={n} K={k} offset={offset} x{shape}")
         buf, ptr = gpu.dev_bytes_at(raw, offset)
         got = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
         want = O.qmatmul(dt, raw, x, n, k)
-        mag = np.abs(x.reshape(-1, k)).astype(np.float64) @ wabs.T
-        assert np.all(np.abs(got.reshape(-1, n) - want.reshape(-1, n)) <= 4e-6 * mag + 1e-30)
+        assert bits_equal(got, want)  # integer sums, and the float32 operations of qdotQ4KGo / qdotQ6KGo in their order
         assert np.array_equal(got, gpu.qgemv_act(dt, ptr, gpu.dev(x), n, k))
 
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
 def test_kquant_gemv_every_launch_shape(dt):
     """The kernels that stage x in LDS, at every count of rows per wavefront, and the ones that
-    read it from global memory add the same integers in the same order: identical results."""
+    read it from global memory all give the CPU's bits."""
     l = gpu.lib()
     rng = np.random.default_rng(77 + dt)
     for n, k in ((37, 256 * 56), (130, 256 * 9), (16, 256)):
@@ -432,7 +430,6 @@ def test_kquant_gemv_every_launch_shape(dt):
         x = rng.normal(size=(3, k)).astype(np.float32)
         buf, ptr = gpu.dev_bytes_at(raw, 0)
         want = O.qmatmul(dt, raw, x, n, k)
-        mag = np.abs(x).astype(np.float64) @ np.abs(O.dequantize(dt, raw).reshape(n, k)).astype(np.float64).T
         results = []
         try:
             for key, v in ((b"kquant.rows", 1), (b"kquant.rows", 2), (b"kquant.rows", 4), (b"kquant.path", 1)):
@@ -442,9 +439,8 @@ def test_kquant_gemv_every_launch_shape(dt):
         finally:
             capi.check(l.mi355x_tune(b"kquant.rows", 0))
             capi.check(l.mi355x_tune(b"kquant.path", 0))
-        assert np.all(np.abs(results[0] - want) <= 4e-6 * mag + 1e-30)
-        for r in results[1:]:
-            assert np.array_equal(r, results[0])
+        for r in results:
+            assert bits_equal(r, want)
 
 
 def test_kquant_gemv_golden_and_exact_rows(golden_dir):
