@@ -349,6 +349,9 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 
 }  // namespace
 
+static int g_force_splits = 0;  // measurement aid: a fixed number of shares
+void set_attention_decode_splits(int n) { g_force_splits = n; }
+
 // Shares of the keys and the most keys a share can hold, for at most kmax keys.
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax) {
     int G = H / HK, ngq = (G + kHeads - 1) / kHeads;
@@ -358,6 +361,7 @@ void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, 
     int64_t by_keys = kmax / 128;  // a share of 128 keys is one batch of loads per thread
     ns = ns > by_keys ? by_keys : ns;
     ns = ns < 1 ? 1 : ns;
+    if (g_force_splits > 0 && g_force_splits <= 64) ns = g_force_splits;
     *nsplit = (int)ns;
     int64_t c = (kmax + ns - 1) / ns;
     *cmax = (int)(c < 1 ? 1 : c);

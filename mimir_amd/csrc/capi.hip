@@ -592,6 +592,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
         g_tune_gemm = value;
         return MI355X_OK;
     }
+    if (key && strcmp(key, "attention.splits") == 0) {
+        mimir::set_attention_decode_splits(value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "attention.path") == 0) {
         g_tune_attn = value;
         return MI355X_OK;

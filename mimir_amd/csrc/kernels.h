@@ -53,6 +53,18 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // concatenated in y; and a SwiGLU pair: y = SiLU(x . gate^T) * (x . up^T).
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st);
+// What follows the q, k, v projections in a decoding step (rope_kv), as the tail of their fused product.
+struct Q4RopeTail {
+    const float* cosv = nullptr;   // [position][rope_dim / 2]
+    const float* sinv = nullptr;
+    const int32_t* pos = nullptr;  // the position, read on the device
+    void* kcache = nullptr;        // [M, HK, cap, dim]
+    void* vcache = nullptr;
+    int cache_dt = 0, H = 0, HK = 0, dim = 0, rope_dim = 0;
+    int64_t cap = 0;
+};
+hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                   const Q4RopeTail& rope, const int* tune, hipStream_t st);
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st);
 
@@ -143,6 +155,7 @@ hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
 // (out may then be null; needs o_strides {H * D, D, .}).
 constexpr size_t kAttnTicketBytes = 4096;
 bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
+void set_attention_decode_splits(int n);
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st);

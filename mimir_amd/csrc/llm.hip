@@ -270,9 +270,18 @@ static mi355x_status step_fast(Model& m) {
         LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
         const void* w3[3] = {b.q.buf.p, b.k.buf.p, b.v.buf.p};
         const int64_t n3[3] = {qd, kvd, kvd};
-        LLM_HIP(qgemv_q4_0_act_multi(w3, n3, act, qkv, B, c.embed, kNoTune, m.stream), "q|k|v");
-        LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
-                        c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        if (c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0) {  // the rotation and the cache writes ride on the product
+            Q4RopeTail tail;
+            tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
+            tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
+            tail.cache_dt = c.cache_dtype; tail.H = c.heads; tail.HK = c.kv_heads; tail.dim = c.head_dim; tail.rope_dim = c.rope_dim;
+            tail.cap = c.context;
+            LLM_HIP(qgemv_q4_0_act_qkv_rope(w3, n3, act, qkv, B, c.embed, tail, kNoTune, m.stream), "q|k|v, rope and cache");
+        } else {
+            LLM_HIP(qgemv_q4_0_act_multi(w3, n3, act, qkv, B, c.embed, kNoTune, m.stream), "q|k|v");
+            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        }
         at.k = m.keys[i].p; at.v = m.values[i].p;
         if (one_launch) {  // leaves its result converted for the output projection
             at.out = nullptr;

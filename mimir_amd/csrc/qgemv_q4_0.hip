@@ -322,14 +322,50 @@ __device__ __forceinline__ void q4_pair_dot(const uint32_t q0[4], const uint32_t
 //   kSwiGLU   y[m, r] = SiLU(x[m, :] . W0[r]) * (x[m, :] . W1[r]): gate and up
 //             of a SwiGLU feed-forward (llm/model.go:446-448), the activation
 //             applied as tensor/elementwise.go:520-525,583-585 computes it
-enum Q4Mode { kPlain = 0, kMulti = 1, kSwiGLU = 2 };
+//   kRope     kMulti for the q, k, v projections of a decoding step, then what
+//             rope_kv does with the result: pairs of features (2i, 2i+1) of the
+//             query and key heads rotated by the angle of the position read on
+//             the device (nn/transformer.go:146-257, interleaved layout), queries
+//             left in y, keys and values cast into their caches at that position
+//             (KVCache.Write, nn/transformer.go:464). Rows per wavefront even.
+enum Q4Mode { kPlain = 0, kMulti = 1, kSwiGLU = 2, kRope = 3 };
 
 struct Q4Job {
     const uint8_t* W[3];
     int n[3];
     int total;           // rows of y
     const float* resid;  // [M, total] or null
+    Q4RopeTail rope;     // kRope only
 };
+
+// Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
+__device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int m, int row, float a, float b, float* yr) {
+    const int head = row / t.dim, f = row - head * t.dim;
+    float va = a, vb = b;
+    if (head < t.H + t.HK && f < t.rope_dim) {
+        const int half = t.rope_dim >> 1, i = f >> 1;
+        const float c = t.cosv[(int64_t)pos * half + i], sn = t.sinv[(int64_t)pos * half + i];
+        const float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;  // four products, then one subtraction and one addition
+        va = ac - bs;
+        vb = as + bc;
+    }
+    if (head < t.H) {
+        yr[row] = va;
+        yr[row + 1] = vb;
+        return;
+    }
+    const bool is_k = head < t.H + t.HK;
+    const int kh = is_k ? head - t.H : head - t.H - t.HK;
+    void* cache = is_k ? t.kcache : t.vcache;
+    const int64_t at = (((int64_t)m * t.HK + kh) * t.cap + pos) * t.dim + f;
+    if (t.cache_dt == kF32) {
+        ((float*)cache)[at] = va;
+        ((float*)cache)[at + 1] = vb;
+    } else {
+        ((uint16_t*)cache)[at] = f32_to_f16_bits(va);
+        ((uint16_t*)cache)[at + 1] = f32_to_f16_bits(vb);
+    }
+}
 
 template <int R, int PC, int MODE>
 __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y,
@@ -347,6 +383,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     const int wg_row0 = blockIdx.x * rows_per_wg;
     const int npairs = nb >> 1;
     const int npc = (npairs + 63) >> 6;
+    const int rope_pos = MODE == kRope ? *job.rope.pos : 0;
 
     // The address of the weights behind row t of the tile at row0; rows past
     // the end are clamped into the matrix (their sums are never stored).
@@ -358,7 +395,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
         }
         int g = row0 + t;
         g = g < N ? g : N - 1;
-        if (MODE == kMulti) {
+        if (MODE == kMulti || MODE == kRope) {
             if (g >= job.n[0] + job.n[1]) return job.W[2] + (int64_t)(g - job.n[0] - job.n[1]) * row_bytes;
             if (g >= job.n[0]) return job.W[1] + (int64_t)(g - job.n[0]) * row_bytes;
         }
@@ -438,6 +475,14 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
                     acc[r] = fmaf(w1, f1, acc[r]);
                 }
             }
+        }
+        if (MODE == kRope) {
+#pragma unroll
+            for (int r = 0; r + 1 < R; r += 2) {
+                const float a = wave_sum(acc[r]), b = wave_sum(acc[r + 1]);
+                if (lane == 0 && row0 + r < N) q4_rope_store(job.rope, rope_pos, m, row0 + r, a, b, yr);
+            }
+            continue;
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -521,23 +566,29 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     int R = MODE == kSwiGLU ? (job.total >= 8192 ? 2 : 1) : (job.total >= 4096 ? 2 : 1);
     if (MODE == kPlain && job.total >= 8192 && npc <= 1) R = 4;  // many short rows: fewer, longer-lived wavefronts stream a little better
     if (tune[0] > 0) R = tune[0];
+    if (MODE == kRope) R = 2;  // a wavefront's two rows are the pair of features a rotation takes
     int64_t tiles = (job.total + R - 1) / R;
     int waves = 8;
     while (waves > 1 && tiles / waves < 256) waves >>= 1;
     if (tune[2] > 0) waves = tune[2];
     if (waves > 8) waves = 8;
 #define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE>(job, act, y, M, K, waves, st)
-    Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(4, 1);
-    Q4ICASE(1, 2); Q4ICASE(2, 2);
-    if constexpr (MODE != kSwiGLU) { Q4ICASE(4, 2); }
+    if constexpr (MODE == kRope) {
+        Q4ICASE(2, 1);
+        return launch_q4_0_i4<2, 2, MODE>(job, act, y, M, K, waves, st);
+    } else {
+        Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(4, 1);
+        Q4ICASE(1, 2); Q4ICASE(2, 2);
+        if constexpr (MODE != kSwiGLU) { Q4ICASE(4, 2); }
+        return launch_q4_0_i4<1, 1, MODE>(job, act, y, M, K, waves, st);
+    }
 #undef Q4ICASE
-    return launch_q4_0_i4<1, 1, MODE>(job, act, y, M, K, waves, st);
 }
 
 // The fixed-point product from converted activations (a.act), plus a.resid
 // if set. Needs q4_0_fixed_point_ok.
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid};
+    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}};
     return dispatch_q4_0_i4<kPlain>(job, a.act, a.y, a.M, a.K, tune, st);
 }
 
@@ -546,14 +597,24 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr};
+              (int)(n[0] + n[1] + n[2]), nullptr, {}};
     return dispatch_q4_0_i4<kMulti>(job, act, y, M, K, tune, st);
+}
+
+// The q, k, v projections of a decoding step with the rotation and the cache
+// writes behind them (see kRope): y [M, n0 + n1 + n2] receives the rotated
+// queries only. Needs the interleaved layout, even head and rotation widths.
+hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                   const Q4RopeTail& rope, const int* tune, hipStream_t st) {
+    Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
+              (int)(n[0] + n[1] + n[2]), nullptr, rope};
+    return dispatch_q4_0_i4<kRope>(job, act, y, M, K, tune, st);
 }
 
 // y[m, r] = SiLU(x[m, :] . gate[r]) * (x[m, :] . up[r]), gate and up [N, K].
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr};
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, y, M, K, tune, st);
 }
 
