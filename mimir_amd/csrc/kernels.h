@@ -53,6 +53,9 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // concatenated in y; and a SwiGLU pair: y = SiLU(x . gate^T) * (x . up^T).
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st);
+bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
+hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
+                                         int64_t K, const int* tune, hipStream_t st);
 // What follows the q, k, v projections in a decoding step (rope_kv), as the tail of their fused product.
 struct Q4RopeTail {
     const float* cosv = nullptr;   // [position][rope_dim / 2]

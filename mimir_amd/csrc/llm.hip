@@ -83,7 +83,7 @@ struct Model {
 
     // activations of up to max_rows rows (batch x tokens of one call)
     int64_t max_rows = 0;
-    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[4], tokens_dev, next_tok;
+    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[4], act2, tokens_dev, next_tok;
     hipStream_t stream = nullptr;
 
     // The decoding step as a fixed run of launches that read the position from
@@ -294,9 +294,15 @@ static mi355x_status step_fast(Model& m) {
         o.resid = x;
         LLM_HIP(qgemv_q4_0_act(o, kNoTune, m.stream), "attn_output");
         LLM_HIP(rmsnorm_q4act(x, b.ffn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "ffn_norm");
-        LLM_HIP(qgemv_q4_0_act_swiglu(b.gate.buf.p, b.up.buf.p, act, sw, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
-        LLM_HIP(q4_0_convert_act(sw, B, c.hidden, c.hidden, act, m.stream), "convert");
-        QGemvArgs d{b.down.buf.p, nullptr, act, x, B, c.embed, c.hidden, 0, 0};
+        void* act_down = act;
+        if (q4_0_swiglu_convert_ok(c.hidden, c.embed)) {  // the conversion rides on the product, into a buffer of its own
+            act_down = m.act2.p;
+            LLM_HIP(qgemv_q4_0_act_swiglu_convert(b.gate.buf.p, b.up.buf.p, act, act_down, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
+        } else {
+            LLM_HIP(qgemv_q4_0_act_swiglu(b.gate.buf.p, b.up.buf.p, act, sw, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
+            LLM_HIP(q4_0_convert_act(sw, B, c.hidden, c.hidden, act, m.stream), "convert");
+        }
+        QGemvArgs d{b.down.buf.p, nullptr, act_down, x, B, c.embed, c.hidden, 0, 0};
         d.resid = x;
         LLM_HIP(qgemv_q4_0_act(d, kNoTune, m.stream), "ffn_down");
     }
@@ -475,6 +481,7 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : (kmax + 63) / 64 * 64;
         LLM_HIP(m->act[cls].alloc(act_row_bytes(cls, kk) * rows + 64), "hipMalloc(activations)");
     }
+    LLM_HIP(m->act2.alloc(q4_0_act_bytes((c.hidden + 63) / 64 * 64) * c.batch + 64), "hipMalloc(activations)");
     int chunk, nsplit;
     attention_plan(c.batch, c.heads, c.kv_heads, max_tokens, c.context, &chunk, &nsplit);
     size_t attn_ws = 0;  // the most splits come from the smallest chunk

@@ -336,6 +336,11 @@ struct Q4Job {
     int total;           // rows of y
     const float* resid;  // [M, total] or null
     Q4RopeTail rope;     // kRope only
+    // kSwiGLU only: if set, the results go to act_out in the fixed-point form the next product
+    // reads (row m at act_out + m * act_out_row_bytes) instead of y. A workgroup then owns exactly
+    // the 32 results of one block, so rows_per_wg is 32 and total a multiple of 32.
+    uint8_t* act_out;
+    int64_t act_out_row_bytes;
 };
 
 // Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
@@ -494,10 +499,23 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
                 const float a = s * sg;
                 s = a * u;
             }
-            if (lane == 0 && row0 + r < N) {
+            if (MODE == kSwiGLU && job.act_out) {
+                if (lane == 0) ((float*)(lds_i4 + n16))[r0 + r] = s;  // behind the staged activations
+            } else if (lane == 0 && row0 + r < N) {
                 if (MODE == kPlain && job.resid) s = s + job.resid[(int64_t)m * N + row0 + r];
                 yr[row0 + r] = s;
             }
+        }
+    }
+    if (MODE == kSwiGLU && job.act_out) {  // the workgroup's 32 results are block blockIdx.x of the next product's x
+        __syncthreads();
+        if (tid < 4) {
+            const f32x4* v = (const f32x4*)(lds_i4 + n16);
+            const f32x4 vlo = v[tid], vhi = v[4 + tid];
+            float lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
+            u32x4* plane = (u32x4*)(job.act_out + (int64_t)m * job.act_out_row_bytes);
+            const int nbp_out = (N >> 5) | 1;
+            q4_convert_item(lo, hi, plane, (float*)(plane + kDigits * nbp_out), nbp_out, blockIdx.x, tid);
         }
     }
 }
@@ -505,14 +523,16 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
 template <int R, int PC, int MODE>
 static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
+    if (MODE == kSwiGLU && job.act_out) rows_per_wg = 32;  // a block of results a workgroup, in one or two turns of its wavefronts
     dim3 grid((unsigned)((job.total + rows_per_wg - 1) / rows_per_wg), (unsigned)M);
     size_t act_bytes = q4_0_act_bytes(K);
+    const size_t lds_bytes = act_bytes + (MODE == kSwiGLU ? 128 : 0);  // kSwiGLU: room for a block of results
     hipEvent_t t0, t1;
     if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
-        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, t0, t1, 0, job,
+        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,
                               (const uint8_t*)act, y, (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     else
-        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), act_bytes, st, job, (const uint8_t*)act, y,
+        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), lds_bytes, st, job, (const uint8_t*)act, y,
                            (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     return hipGetLastError();
 }
@@ -567,11 +587,13 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     if (MODE == kPlain && job.total >= 8192 && npc <= 1) R = 4;  // many short rows: fewer, longer-lived wavefronts stream a little better
     if (tune[0] > 0) R = tune[0];
     if (MODE == kRope) R = 2;  // a wavefront's two rows are the pair of features a rotation takes
+    if (MODE == kSwiGLU && job.act_out) R = tune[0] == 4 ? 4 : 2, PC = 1;  // eight wavefronts, two turns of two rows (or one of four)
     int64_t tiles = (job.total + R - 1) / R;
     int waves = 8;
     while (waves > 1 && tiles / waves < 256) waves >>= 1;
     if (tune[2] > 0) waves = tune[2];
     if (waves > 8) waves = 8;
+    if (MODE == kSwiGLU && job.act_out) waves = 8;
 #define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE>(job, act, y, M, K, waves, st)
     if constexpr (MODE == kRope) {
         Q4ICASE(2, 1);
@@ -588,7 +610,7 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
 // The fixed-point product from converted activations (a.act), plus a.resid
 // if set. Needs q4_0_fixed_point_ok.
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}};
+    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}, nullptr, 0};
     return dispatch_q4_0_i4<kPlain>(job, a.act, a.y, a.M, a.K, tune, st);
 }
 
@@ -597,7 +619,7 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, {}};
+              (int)(n[0] + n[1] + n[2]), nullptr, {}, nullptr, 0};
     return dispatch_q4_0_i4<kMulti>(job, act, y, M, K, tune, st);
 }
 
@@ -607,15 +629,29 @@ hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], cons
 hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                    const Q4RopeTail& rope, const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, rope};
+              (int)(n[0] + n[1] + n[2]), nullptr, rope, nullptr, 0};
     return dispatch_q4_0_i4<kRope>(job, act, y, M, K, tune, st);
 }
 
 // y[m, r] = SiLU(x[m, :] . gate[r]) * (x[m, :] . up[r]), gate and up [N, K].
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}};
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, nullptr, 0};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, y, M, K, tune, st);
+}
+
+// Whether qgemv_q4_0_act_swiglu_convert takes the shape: rows of x that one
+// step of the wavefront covers, and whole blocks of results.
+bool q4_0_swiglu_convert_ok(int64_t N, int64_t K) { return K / 64 <= 64 && N % 64 == 0; }
+
+// The same, with the results left in the fixed-point form of activations in
+// act_out (q4_0_act_bytes(N) bytes a row, not the buffer act points into)
+// instead of float32: the conversion that would follow as a launch of its own.
+hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
+                                         int64_t K, const int* tune, hipStream_t st) {
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, (uint8_t*)act_out,
+              (int64_t)q4_0_act_bytes(N)};
+    return dispatch_q4_0_i4<kSwiGLU>(job, act, nullptr, M, K, tune, st);
 }
 
 // The float32 product, any shape. tune: {rows, cols, waves, no_lds}.
