@@ -51,7 +51,6 @@ hipError_t rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64
 // held in registers between the sum of squares and the conversion, so x is
 // read once. Writes y (if not null) and the converted row. d a multiple of
 // 64 and at most 256 * 4 * 8 * kNormItems floats.
-constexpr int kNormItems = 4;
 __global__ __launch_bounds__(256) void rmsnorm_q4act_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             float* __restrict__ y, uint8_t* __restrict__ act, int d, float inv_d,
                                                             float eps, int64_t act_row_bytes) {
@@ -59,55 +58,12 @@ __global__ __launch_bounds__(256) void rmsnorm_q4act_kernel(const float* __restr
     const float* xr = x + (int64_t)blockIdx.x * d;
     const int nb = d >> 5, nbp = nb | 1, nq = nb * 4;
     u32x4* plane = (u32x4*)(act + (int64_t)blockIdx.x * act_row_bytes);
-    float* xscale = (float*)(plane + kDigits * nbp);
-    // item t: block t / 4, dword t % 4: elements 4(t%4).. and 16 + 4(t%4).. of the block
-    f32x4 lo[kNormItems], hi[kNormItems];
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < kNormItems; i++) {
-        int t = threadIdx.x + i * 256;
-        if (t < nq) {
-            int b = t >> 2, q = t & 3;
-            __builtin_memcpy(&lo[i], xr + 32 * b + 4 * q, 16);
-            __builtin_memcpy(&hi[i], xr + 32 * b + 16 + 4 * q, 16);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float a = lo[i][k] * lo[i][k], c = hi[i][k] * hi[i][k];
-                ss = ss + a;
-                ss = ss + c;
-            }
-        }
-    }
-    ss = wave_sum(ss);
+    NormRow row;
+    float ss = wave_sum(norm_load(row, xr, nq, threadIdx.x));
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
-    float total = (part[0] + part[1]) + (part[2] + part[3]);
-    float ms = total * inv_d;
-    float scale = 1.0f / __builtin_sqrtf(ms + eps);
-#pragma unroll
-    for (int i = 0; i < kNormItems; i++) {
-        int t = threadIdx.x + i * 256;
-        if (t < nq) {
-            int b = t >> 2, q = t & 3;
-            f32x4 wl, wh;
-            __builtin_memcpy(&wl, w + 32 * b + 4 * q, 16);
-            __builtin_memcpy(&wh, w + 32 * b + 16 + 4 * q, 16);
-            float l4[4], h4[4];
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float a = lo[i][k] * scale, c = hi[i][k] * scale;
-                l4[k] = a * wl[k];
-                h4[k] = c * wh[k];
-            }
-            if (y) {
-                float* yr = y + (int64_t)blockIdx.x * d;
-                f32x4 ol = {l4[0], l4[1], l4[2], l4[3]}, oh = {h4[0], h4[1], h4[2], h4[3]};
-                __builtin_memcpy(yr + 32 * b + 4 * q, &ol, 16);
-                __builtin_memcpy(yr + 32 * b + 16 + 4 * q, &oh, 16);
-            }
-            q4_convert_item(l4, h4, plane, xscale, nbp, b, q);
-        }
-    }
+    norm_convert(row, part, w, y ? y + (int64_t)blockIdx.x * d : nullptr, plane, (float*)(plane + kDigits * nbp), nbp, nq, threadIdx.x,
+                 inv_d, eps);
 }
 
 bool rmsnorm_q4act_ok(int64_t d) { return d > 0 && d % 64 == 0 && d / 32 * 4 <= 256 * kNormItems; }

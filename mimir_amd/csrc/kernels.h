@@ -53,9 +53,18 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // concatenated in y; and a SwiGLU pair: y = SiLU(x . gate^T) * (x . up^T).
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st);
+// The RMSNorm in front of a product as that product's first phase: with x and w set, every
+// workgroup normalizes and converts row m of x [M, K] for itself and `act` is not read
+// (q4_0_norm_head_ok(K) must hold); with w null the product reads `act` as usual.
+struct Q4NormHead {
+    const float* x = nullptr;
+    const float* w = nullptr;
+    double eps = 0;
+};
+bool q4_0_norm_head_ok(int64_t K);
 bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
-                                         int64_t K, const int* tune, hipStream_t st);
+                                         int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st);
 // What follows the q, k, v projections in a decoding step (rope_kv), as the tail of their fused product.
 struct Q4RopeTail {
     const float* cosv = nullptr;   // [position][rope_dim / 2]
@@ -67,7 +76,7 @@ struct Q4RopeTail {
     int64_t cap = 0;
 };
 hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
-                                   const Q4RopeTail& rope, const int* tune, hipStream_t st);
+                                   const Q4RopeTail& rope, const Q4NormHead& norm, const int* tune, hipStream_t st);
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st);
 

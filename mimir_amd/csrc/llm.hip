@@ -264,10 +264,10 @@ static mi355x_status step_fast(Model& m) {
     at.dyn_k = pos;  // position p holds p keys before this step's own
     at.k = m.keys[0].p; at.v = m.values[0].p;  // every layer's caches are allocated alike
     const bool one_launch = attention_decode_ok(at, c.context);
+    const bool norm_head = q4_0_norm_head_ok(c.embed);
     if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
-        LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
         const void* w3[3] = {b.q.buf.p, b.k.buf.p, b.v.buf.p};
         const int64_t n3[3] = {qd, kvd, kvd};
         if (c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0) {  // the rotation and the cache writes ride on the product
@@ -276,8 +276,15 @@ static mi355x_status step_fast(Model& m) {
             tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
             tail.cache_dt = c.cache_dtype; tail.H = c.heads; tail.HK = c.kv_heads; tail.dim = c.head_dim; tail.rope_dim = c.rope_dim;
             tail.cap = c.context;
-            LLM_HIP(qgemv_q4_0_act_qkv_rope(w3, n3, act, qkv, B, c.embed, tail, kNoTune, m.stream), "q|k|v, rope and cache");
+            Q4NormHead head;  // and the norm in front of it is its first phase
+            if (norm_head) {
+                head.x = x; head.w = b.attn_norm.buf.as<float>(); head.eps = c.eps;
+            } else {
+                LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
+            }
+            LLM_HIP(qgemv_q4_0_act_qkv_rope(w3, n3, act, qkv, B, c.embed, tail, head, kNoTune, m.stream), "norm, q|k|v, rope and cache");
         } else {
+            LLM_HIP(rmsnorm_q4act(x, b.attn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "attn_norm");
             LLM_HIP(qgemv_q4_0_act_multi(w3, n3, act, qkv, B, c.embed, kNoTune, m.stream), "q|k|v");
             LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
                             c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
@@ -293,12 +300,19 @@ static mi355x_status step_fast(Model& m) {
         QGemvArgs o{b.o.buf.p, nullptr, act, x, B, c.embed, qd, 0, 0};
         o.resid = x;
         LLM_HIP(qgemv_q4_0_act(o, kNoTune, m.stream), "attn_output");
-        LLM_HIP(rmsnorm_q4act(x, b.ffn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "ffn_norm");
         void* act_down = act;
         if (q4_0_swiglu_convert_ok(c.hidden, c.embed)) {  // the conversion rides on the product, into a buffer of its own
             act_down = m.act2.p;
-            LLM_HIP(qgemv_q4_0_act_swiglu_convert(b.gate.buf.p, b.up.buf.p, act, act_down, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
+            Q4NormHead head;
+            if (norm_head) {
+                head.x = x; head.w = b.ffn_norm.buf.as<float>(); head.eps = c.eps;
+            } else {
+                LLM_HIP(rmsnorm_q4act(x, b.ffn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "ffn_norm");
+            }
+            LLM_HIP(qgemv_q4_0_act_swiglu_convert(b.gate.buf.p, b.up.buf.p, act, act_down, B, c.hidden, c.embed, head, kNoTune, m.stream),
+                    "norm, gate|up, conversion");
         } else {
+            LLM_HIP(rmsnorm_q4act(x, b.ffn_norm.buf.as<float>(), nullptr, act, B, c.embed, c.eps, m.stream), "ffn_norm");
             LLM_HIP(qgemv_q4_0_act_swiglu(b.gate.buf.p, b.up.buf.p, act, sw, B, c.hidden, c.embed, kNoTune, m.stream), "gate|up");
             LLM_HIP(q4_0_convert_act(sw, B, c.hidden, c.hidden, act, m.stream), "convert");
         }

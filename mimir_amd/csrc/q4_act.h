@@ -85,4 +85,69 @@ __device__ __forceinline__ void q4_convert_item(float lo[4], float hi[4], u32x4*
     if (d == 0) xscale[b] = scale;
 }
 
+// RMSNorm of one row (RMSNorm.Forward, nn/transformer.go:50-61) with the
+// conversion behind it, for the first 256 threads of a workgroup: thread t < 256
+// holds items t, t + 256, ... (an item is block t / 4, dword t % 4: elements
+// 4(t%4).. and 16 + 4(t%4).. of the block), at most kNormItems of them, so the
+// row is read once. The stand-alone kernel and the products that take the norm as
+// their first phase share these two functions, hence the same sums in the same order.
+constexpr int kNormItems = 4;
+
+struct NormRow {
+    f32x4 lo[kNormItems], hi[kNormItems];
+};
+
+// Loads the thread's items of the row and returns its share of the sum of squares.
+__device__ __forceinline__ float norm_load(NormRow& r, const float* __restrict__ xr, int nq, int t0) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormItems; i++) {
+        int t = t0 + i * 256;
+        if (t < nq) {
+            int b = t >> 2, q = t & 3;
+            __builtin_memcpy(&r.lo[i], xr + 32 * b + 4 * q, 16);
+            __builtin_memcpy(&r.hi[i], xr + 32 * b + 16 + 4 * q, 16);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float a = r.lo[i][k] * r.lo[i][k], c = r.hi[i][k] * r.hi[i][k];
+                ss = ss + a;
+                ss = ss + c;
+            }
+        }
+    }
+    return ss;
+}
+
+// part: the four wavefronts' sums. Scales, multiplies by the norm's weights,
+// writes y (if not null) and the converted items.
+__device__ __forceinline__ void norm_convert(const NormRow& r, const float* part, const float* __restrict__ w, float* yr, u32x4* plane,
+                                             float* xscale, int nbp, int nq, int t0, float inv_d, float eps) {
+    float total = (part[0] + part[1]) + (part[2] + part[3]);
+    float ms = total * inv_d;
+    float scale = 1.0f / __builtin_sqrtf(ms + eps);
+#pragma unroll
+    for (int i = 0; i < kNormItems; i++) {
+        int t = t0 + i * 256;
+        if (t < nq) {
+            int b = t >> 2, q = t & 3;
+            f32x4 wl, wh;
+            __builtin_memcpy(&wl, w + 32 * b + 4 * q, 16);
+            __builtin_memcpy(&wh, w + 32 * b + 16 + 4 * q, 16);
+            float l4[4], h4[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float a = r.lo[i][k] * scale, c = r.hi[i][k] * scale;
+                l4[k] = a * wl[k];
+                h4[k] = c * wh[k];
+            }
+            if (yr) {
+                f32x4 ol = {l4[0], l4[1], l4[2], l4[3]}, oh = {h4[0], h4[1], h4[2], h4[3]};
+                __builtin_memcpy(yr + 32 * b + 4 * q, &ol, 16);
+                __builtin_memcpy(yr + 32 * b + 16 + 4 * q, &oh, 16);
+            }
+            q4_convert_item(l4, h4, plane, xscale, nbp, b, q);
+        }
+    }
+}
+
 }  // namespace mimir

@@ -341,6 +341,11 @@ struct Q4Job {
     // the 32 results of one block, so rows_per_wg is 32 and total a multiple of 32.
     uint8_t* act_out;
     int64_t act_out_row_bytes;
+    // NORM kernels only: the product's x is RMSNorm(norm_x[m, :]) * norm_w, normalized and
+    // converted by every workgroup for itself as its first phase instead of read from act.
+    const float* norm_x;
+    const float* norm_w;
+    float norm_inv_d, norm_eps;
 };
 
 // Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
@@ -372,7 +377,7 @@ __device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int 
     }
 }
 
-template <int R, int PC, int MODE>
+template <int R, int PC, int MODE, bool NORM = false>
 __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y,
                                                              int nb, int64_t act_row_bytes, int rows_per_wg) {
     constexpr int RR = MODE == kSwiGLU ? 2 * R : R;  // rows of weights a tile reads
@@ -414,10 +419,17 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
     const int n16 = (int)(act_row_bytes >> 4);
     u32x4 park[kPark];
+    __shared__ float norm_part[4];
+    NormRow norm_row;
+    float norm_ss = 0.f;
+    if (NORM) {  // eight wavefronts; the first four hold the row between its sum of squares and its conversion
+        if (tid < 256) norm_ss = norm_load(norm_row, job.norm_x + (int64_t)m * nb * 32, nb * 4, tid);
+    } else {
 #pragma unroll
-    for (int i = 0; i < kPark; i++) {
-        int idx = tid + i * (int)blockDim.x;
-        if (idx < n16) park[i] = act_row[idx];
+        for (int i = 0; i < kPark; i++) {
+            int idx = tid + i * (int)blockDim.x;
+            if (idx < n16) park[i] = act_row[idx];
+        }
     }
     Q4PairTile<RR, PC> tile;
     int r0 = wave * R;
@@ -427,12 +439,23 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     // Unconditional (rows are clamped into W): a branch here would make the
     // wait before the LDS stores below cover the weights' loads as well.
     q4_load_pairs<RR, PC>(tile, rowp, npairs, 0, lane);
+    if (NORM) {
+        if (tid < 256) {
+            norm_ss = wave_sum(norm_ss);
+            if (lane == 0) norm_part[wave] = norm_ss;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weights' loads stay in flight
+        if (tid < 256)
+            norm_convert(norm_row, norm_part, job.norm_w, nullptr, (u32x4*)lds_i4, (float*)(lds_i4 + kDigits * nbp), nbp, nb * 4, tid,
+                         job.norm_inv_d, job.norm_eps);
+    } else {
 #pragma unroll
-    for (int i = 0; i < kPark; i++) {
-        int idx = tid + i * (int)blockDim.x;
-        if (idx < n16) lds_i4[idx] = park[i];
+        for (int i = 0; i < kPark; i++) {
+            int idx = tid + i * (int)blockDim.x;
+            if (idx < n16) lds_i4[idx] = park[i];
+        }
+        for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_i4[idx] = act_row[idx];
     }
-    for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_i4[idx] = act_row[idx];
     __syncthreads();
 
     bool loaded = true;
@@ -520,7 +543,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     }
 }
 
-template <int R, int PC, int MODE>
+template <int R, int PC, int MODE, bool NORM = false>
 static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
     if (MODE == kSwiGLU && job.act_out) rows_per_wg = 32;  // a block of results a workgroup, in one or two turns of its wavefronts
@@ -529,10 +552,10 @@ static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, in
     const size_t lds_bytes = act_bytes + (MODE == kSwiGLU ? 128 : 0);  // kSwiGLU: room for a block of results
     hipEvent_t t0, t1;
     if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
-        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,
+        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, NORM>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,
                               (const uint8_t*)act, y, (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     else
-        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE>), grid, dim3(64 * waves), lds_bytes, st, job, (const uint8_t*)act, y,
+        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, NORM>), grid, dim3(64 * waves), lds_bytes, st, job, (const uint8_t*)act, y,
                            (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     return hipGetLastError();
 }
@@ -595,6 +618,10 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     if (waves > 8) waves = 8;
     if (MODE == kSwiGLU && job.act_out) waves = 8;
 #define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE>(job, act, y, M, K, waves, st)
+    if (job.norm_w) {  // kRope, and kSwiGLU with converted results: two rows, eight wavefronts, rows one step long
+        if constexpr (MODE == kRope || MODE == kSwiGLU) return launch_q4_0_i4<2, 1, MODE, true>(job, act, y, M, K, 8, st);
+        return hipErrorInvalidValue;
+    }
     if constexpr (MODE == kRope) {
         Q4ICASE(2, 1);
         return launch_q4_0_i4<2, 2, MODE>(job, act, y, M, K, waves, st);
@@ -610,7 +637,7 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
 // The fixed-point product from converted activations (a.act), plus a.resid
 // if set. Needs q4_0_fixed_point_ok.
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}, nullptr, 0};
+    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
     return dispatch_q4_0_i4<kPlain>(job, a.act, a.y, a.M, a.K, tune, st);
 }
 
@@ -619,7 +646,7 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, {}, nullptr, 0};
+              (int)(n[0] + n[1] + n[2]), nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
     return dispatch_q4_0_i4<kMulti>(job, act, y, M, K, tune, st);
 }
 
@@ -627,16 +654,20 @@ hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], cons
 // writes behind them (see kRope): y [M, n0 + n1 + n2] receives the rotated
 // queries only. Needs the interleaved layout, even head and rotation widths.
 hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
-                                   const Q4RopeTail& rope, const int* tune, hipStream_t st) {
+                                   const Q4RopeTail& rope, const Q4NormHead& norm, const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, rope, nullptr, 0};
+              (int)(n[0] + n[1] + n[2]), nullptr, rope, nullptr, 0, norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps};
     return dispatch_q4_0_i4<kRope>(job, act, y, M, K, tune, st);
 }
+
+// Whether a product can take the norm of its x as its first phase (Q4NormHead): x short enough for
+// the norm's 256 threads and for one step of a wavefront.
+bool q4_0_norm_head_ok(int64_t K) { return K % 64 == 0 && K / 8 <= 256 * kNormItems && K / 64 <= 64; }
 
 // y[m, r] = SiLU(x[m, :] . gate[r]) * (x[m, :] . up[r]), gate and up [N, K].
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, nullptr, 0};
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, y, M, K, tune, st);
 }
 
@@ -648,9 +679,9 @@ bool q4_0_swiglu_convert_ok(int64_t N, int64_t K) { return K / 64 <= 64 && N % 6
 // act_out (q4_0_act_bytes(N) bytes a row, not the buffer act points into)
 // instead of float32: the conversion that would follow as a launch of its own.
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
-                                         int64_t K, const int* tune, hipStream_t st) {
+                                         int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, (uint8_t*)act_out,
-              (int64_t)q4_0_act_bytes(N)};
+              (int64_t)q4_0_act_bytes(N), norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, nullptr, M, K, tune, st);
 }
 
