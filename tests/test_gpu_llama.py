@@ -217,3 +217,37 @@ def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, ca
     assert np.array_equal(runs[0][0], runs[0][1])
     assert np.array_equal(runs[1][0], runs[0][0])
     assert all(same), (runs[2][0], runs[0][0])
+
+
+def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
+    """The fused step lets the rotation, the norms and the conversion of SwiGLU's results ride on the products
+    only where their shapes allow: interleaved pairs, rows of x one step of a wavefront long. A model with
+    half-split pairs (qwen2's layout) and 4160 features takes the separate launches instead, and must choose the
+    same tokens as the per-operator path."""
+    lib = gpu.lib()
+    c = capi.LlamaConfig()
+    c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = 4160, 320, 2, 2, 1, 64, 64, 301
+    c.context, c.interleaved, c.cache_dtype, c.batch = 48, 0, capi.F16, 2
+    c.rope_base, c.rope_scale, c.eps = 10000.0, 1.0, 1e-5
+    oc = OL.Config(arch="qwen2", embed=c.embed, hidden=c.hidden, layers=c.layers, heads=c.heads, kv_heads=c.kv_heads, head_dim=c.head_dim,
+                   rope_dim=c.rope_dim, rope_base=c.rope_base, rope_scale=1.0, eps=c.eps, vocab=c.vocab, context=c.context)
+    om = OL.synthetic(oc, seed=3, output_dt=O.Q4_0)
+    m = Llama(c)
+    _upload_synthetic(m, om)
+    m.finalize(16)
+    prompts = np.random.default_rng(9).integers(0, c.vocab, (2, 7))
+    runs = {}
+    try:
+        for mode in (2, 1, 0):
+            gpu.say(f"generate without riders, step mode {mode}")
+            capi.check(lib.mi355x_tune(b"llama.step", mode))
+            m.reset()
+            runs[mode], _ = m.generate(prompts, 20)
+    finally:
+        capi.check(lib.mi355x_tune(b"llama.step", 0))
+    want, margins = om.generate(prompts[0].tolist(), 20, capacity=c.context, cache_dtype=O.F16)
+    for i, (a, w) in enumerate(zip(runs[2][0].tolist(), want)):
+        if a != w:
+            assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
+            break
+    assert np.array_equal(runs[1], runs[2]) and np.array_equal(runs[0], runs[2])
