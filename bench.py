@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
 # reads for a copy kernel of known size (the summaries under profiles/ hold the
 # runs): FETCH_SIZE and WRITE_SIZE in KiB x 1024, scaled by 1.99976 and 1.0.
-TRAFFIC_BYTES_PER_LAUNCH = 33274522
+TRAFFIC_BYTES_PER_LAUNCH = 33281810
 
 
 def gemv_bytes(n: int, k: int, block_bytes: int = 18) -> int:
@@ -385,7 +385,7 @@ def main():
                    "N": n, "K": k, "M": 1, "wall_ms_per_step": round(step_wall_ms, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "qgemv_q4_0_i4_kernel<4, 1, 0>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
+                     "kernel": "qgemv_q4_0_i4_kernel<4, 1, 0, false>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
                      "us_min": round(kern_min, 3), "us_max": round(kern_max, 3),
                      # launches of the kernel alone back to back in a graph, the wait between dependent kernels included
                      "us_per_launch_in_sequence": round(seq_ms * 1e3, 3)},

@@ -59,10 +59,10 @@ __global__ __launch_bounds__(256) void rmsnorm_q4act_kernel(const float* __restr
     const int nb = d >> 5, nbp = nb | 1, nq = nb * 4;
     u32x4* plane = (u32x4*)(act + (int64_t)blockIdx.x * act_row_bytes);
     NormRow row;
-    float ss = wave_sum(norm_load(row, xr, nq, threadIdx.x));
+    float ss = wave_sum(norm_load(row, xr, w, nq, threadIdx.x));
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
-    norm_convert(row, part, w, y ? y + (int64_t)blockIdx.x * d : nullptr, plane, (float*)(plane + kDigits * nbp), nbp, nq, threadIdx.x,
+    norm_convert(row, part, y ? y + (int64_t)blockIdx.x * d : nullptr, plane, (float*)(plane + kDigits * nbp), nbp, nq, threadIdx.x,
                  inv_d, eps);
 }
 

@@ -94,11 +94,12 @@ __device__ __forceinline__ void q4_convert_item(float lo[4], float hi[4], u32x4*
 constexpr int kNormItems = 4;
 
 struct NormRow {
-    f32x4 lo[kNormItems], hi[kNormItems];
+    f32x4 lo[kNormItems], hi[kNormItems];  // x
+    f32x4 wl[kNormItems], wh[kNormItems];  // the norm's weights, requested with x so that they are there when the sum is
 };
 
-// Loads the thread's items of the row and returns its share of the sum of squares.
-__device__ __forceinline__ float norm_load(NormRow& r, const float* __restrict__ xr, int nq, int t0) {
+// Loads the thread's items of the row (and of the weights) and returns its share of the sum of squares.
+__device__ __forceinline__ float norm_load(NormRow& r, const float* __restrict__ xr, const float* __restrict__ w, int nq, int t0) {
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < kNormItems; i++) {
@@ -107,6 +108,8 @@ __device__ __forceinline__ float norm_load(NormRow& r, const float* __restrict__
             int b = t >> 2, q = t & 3;
             __builtin_memcpy(&r.lo[i], xr + 32 * b + 4 * q, 16);
             __builtin_memcpy(&r.hi[i], xr + 32 * b + 16 + 4 * q, 16);
+            __builtin_memcpy(&r.wl[i], w + 32 * b + 4 * q, 16);
+            __builtin_memcpy(&r.wh[i], w + 32 * b + 16 + 4 * q, 16);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 float a = r.lo[i][k] * r.lo[i][k], c = r.hi[i][k] * r.hi[i][k];
@@ -120,8 +123,8 @@ __device__ __forceinline__ float norm_load(NormRow& r, const float* __restrict__
 
 // part: the four wavefronts' sums. Scales, multiplies by the norm's weights,
 // writes y (if not null) and the converted items.
-__device__ __forceinline__ void norm_convert(const NormRow& r, const float* part, const float* __restrict__ w, float* yr, u32x4* plane,
-                                             float* xscale, int nbp, int nq, int t0, float inv_d, float eps) {
+__device__ __forceinline__ void norm_convert(const NormRow& r, const float* part, float* yr, u32x4* plane, float* xscale, int nbp, int nq,
+                                             int t0, float inv_d, float eps) {
     float total = (part[0] + part[1]) + (part[2] + part[3]);
     float ms = total * inv_d;
     float scale = 1.0f / __builtin_sqrtf(ms + eps);
@@ -130,15 +133,12 @@ __device__ __forceinline__ void norm_convert(const NormRow& r, const float* part
         int t = t0 + i * 256;
         if (t < nq) {
             int b = t >> 2, q = t & 3;
-            f32x4 wl, wh;
-            __builtin_memcpy(&wl, w + 32 * b + 4 * q, 16);
-            __builtin_memcpy(&wh, w + 32 * b + 16 + 4 * q, 16);
             float l4[4], h4[4];
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 float a = r.lo[i][k] * scale, c = r.hi[i][k] * scale;
-                l4[k] = a * wl[k];
-                h4[k] = c * wh[k];
+                l4[k] = a * r.wl[i][k];
+                h4[k] = c * r.wh[i][k];
             }
             if (yr) {
                 f32x4 ol = {l4[0], l4[1], l4[2], l4[3]}, oh = {h4[0], h4[1], h4[2], h4[3]};

@@ -423,7 +423,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     NormRow norm_row;
     float norm_ss = 0.f;
     if (NORM) {  // eight wavefronts; the first four hold the row between its sum of squares and its conversion
-        if (tid < 256) norm_ss = norm_load(norm_row, job.norm_x + (int64_t)m * nb * 32, nb * 4, tid);
+        if (tid < 256) norm_ss = norm_load(norm_row, job.norm_x + (int64_t)m * nb * 32, job.norm_w, nb * 4, tid);
     } else {
 #pragma unroll
         for (int i = 0; i < kPark; i++) {
@@ -446,7 +446,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weights' loads stay in flight
         if (tid < 256)
-            norm_convert(norm_row, norm_part, job.norm_w, nullptr, (u32x4*)lds_i4, (float*)(lds_i4 + kDigits * nbp), nbp, nb * 4, tid,
+            norm_convert(norm_row, norm_part, nullptr, (u32x4*)lds_i4, (float*)(lds_i4 + kDigits * nbp), nbp, nb * 4, tid,
                          job.norm_inv_d, job.norm_eps);
     } else {
 #pragma unroll
