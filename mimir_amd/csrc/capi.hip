@@ -64,6 +64,9 @@ struct DeviceState {
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 int g_tune_q4[5] = {0, 0, 0, 0, 0};
+// Up to this many rows of x the Q4_0 product converts x inside its own launch (each workgroup
+// for itself); beyond, one conversion launch serves all workgroups.
+constexpr int64_t kConvertInProductRows = 8;
 int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
@@ -330,6 +333,11 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
     switch (dtype) {
     case MI355X_Q4_0:
         if (g_tune_q4[4] != 1 && mimir::q4_0_fixed_point_ok(W, K)) {
+            if (M <= kConvertInProductRows && ((uintptr_t)x & 15) == 0 && (M == 1 || x_row_stride % 4 == 0)) {
+                // few rows: one launch, every workgroup converts x for itself
+                HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
+                return MI355X_OK;
+            }
             void* act;
             if (mi355x_status st = act_scratch(mimir::q4_0_act_bytes(K) * (size_t)M, &act)) return st;
             HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");

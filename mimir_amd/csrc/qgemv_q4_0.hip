@@ -341,11 +341,13 @@ struct Q4Job {
     // the 32 results of one block, so rows_per_wg is 32 and total a multiple of 32.
     uint8_t* act_out;
     int64_t act_out_row_bytes;
-    // NORM kernels only: the product's x is RMSNorm(norm_x[m, :]) * norm_w, normalized and
-    // converted by every workgroup for itself as its first phase instead of read from act.
+    // HEAD 1: the product's x is RMSNorm(norm_x[m, :]) * norm_w, normalized and converted by
+    // every workgroup for itself as its first phase instead of read from act. HEAD 2: x is
+    // norm_x[m, :] itself (rows x_row_stride floats apart), converted likewise.
     const float* norm_x;
     const float* norm_w;
     float norm_inv_d, norm_eps;
+    int64_t x_row_stride;
 };
 
 // Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
@@ -377,7 +379,9 @@ __device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int 
     }
 }
 
-template <int R, int PC, int MODE, bool NORM = false>
+constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
+
+template <int R, int PC, int MODE, int HEAD = kHeadAct>
 __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y,
                                                              int nb, int64_t act_row_bytes, int rows_per_wg) {
     constexpr int RR = MODE == kSwiGLU ? 2 * R : R;  // rows of weights a tile reads
@@ -422,8 +426,20 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     __shared__ float norm_part[4];
     NormRow norm_row;
     float norm_ss = 0.f;
-    if (NORM) {  // eight wavefronts; the first four hold the row between its sum of squares and its conversion
-        if (tid < 256) norm_ss = norm_load(norm_row, job.norm_x + (int64_t)m * nb * 32, job.norm_w, nb * 4, tid);
+    constexpr int kCv = 2;  // items of x a thread requests ahead of the weights when it converts x itself
+    f32x4 cv_lo[kCv], cv_hi[kCv];
+    const int nq = nb * 4;
+    if (HEAD == kHeadNorm) {  // eight wavefronts; the first four hold the row between its sum of squares and its conversion
+        if (tid < 256) norm_ss = norm_load(norm_row, job.norm_x + (int64_t)m * nb * 32, job.norm_w, nq, tid);
+    } else if (HEAD == kHeadConvert) {
+        const float* xr = job.norm_x + (int64_t)m * job.x_row_stride;
+#pragma unroll
+        for (int i = 0; i < kCv; i++) {
+            int t = tid + i * (int)blockDim.x;
+            t = t < nq ? t : nq - 1;
+            cv_lo[i] = load_f32x4(xr + 32 * (t >> 2) + 4 * (t & 3));
+            cv_hi[i] = load_f32x4(xr + 32 * (t >> 2) + 16 + 4 * (t & 3));
+        }
     } else {
 #pragma unroll
         for (int i = 0; i < kPark; i++) {
@@ -439,15 +455,34 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     // Unconditional (rows are clamped into W): a branch here would make the
     // wait before the LDS stores below cover the weights' loads as well.
     q4_load_pairs<RR, PC>(tile, rowp, npairs, 0, lane);
-    if (NORM) {
+    if (HEAD != kHeadAct) __builtin_amdgcn_sched_barrier(0);  // the weights' loads stay ahead of the arithmetic on x below
+    if (HEAD == kHeadNorm) {
         if (tid < 256) {
             norm_ss = wave_sum(norm_ss);
             if (lane == 0) norm_part[wave] = norm_ss;
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weights' loads stay in flight
         if (tid < 256)
-            norm_convert(norm_row, norm_part, nullptr, (u32x4*)lds_i4, (float*)(lds_i4 + kDigits * nbp), nbp, nb * 4, tid,
+            norm_convert(norm_row, norm_part, nullptr, (u32x4*)lds_i4, (float*)(lds_i4 + kDigits * nbp), nbp, nq, tid,
                          job.norm_inv_d, job.norm_eps);
+    } else if (HEAD == kHeadConvert) {
+        // items t = tid, tid + blockDim, ...: the four items of a block sit in four consecutive lanes
+        const float* xr = job.norm_x + (int64_t)m * job.x_row_stride;
+        u32x4* plane = (u32x4*)lds_i4;
+        float* xs = (float*)(lds_i4 + kDigits * nbp);
+#pragma unroll
+        for (int i = 0; i < kCv; i++) {
+            const int t = tid + i * (int)blockDim.x;
+            if (t < nq) {
+                float lo[4] = {cv_lo[i][0], cv_lo[i][1], cv_lo[i][2], cv_lo[i][3]}, hi[4] = {cv_hi[i][0], cv_hi[i][1], cv_hi[i][2], cv_hi[i][3]};
+                q4_convert_item(lo, hi, plane, xs, nbp, t >> 2, t & 3);
+            }
+        }
+        for (int t = tid + kCv * (int)blockDim.x; t < nq; t += (int)blockDim.x) {
+            const f32x4 vlo = load_f32x4(xr + 32 * (t >> 2) + 4 * (t & 3)), vhi = load_f32x4(xr + 32 * (t >> 2) + 16 + 4 * (t & 3));
+            float lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
+            q4_convert_item(lo, hi, plane, xs, nbp, t >> 2, t & 3);
+        }
     } else {
 #pragma unroll
         for (int i = 0; i < kPark; i++) {
@@ -543,7 +578,7 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     }
 }
 
-template <int R, int PC, int MODE, bool NORM = false>
+template <int R, int PC, int MODE, int HEAD = kHeadAct>
 static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
     if (MODE == kSwiGLU && job.act_out) rows_per_wg = 32;  // a block of results a workgroup, in one or two turns of its wavefronts
@@ -552,10 +587,10 @@ static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, in
     const size_t lds_bytes = act_bytes + (MODE == kSwiGLU ? 128 : 0);  // kSwiGLU: room for a block of results
     hipEvent_t t0, t1;
     if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
-        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, NORM>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,
+        hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, HEAD>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,
                               (const uint8_t*)act, y, (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     else
-        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, NORM>), grid, dim3(64 * waves), lds_bytes, st, job, (const uint8_t*)act, y,
+        hipLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, HEAD>), grid, dim3(64 * waves), lds_bytes, st, job, (const uint8_t*)act, y,
                            (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
     return hipGetLastError();
 }
@@ -619,13 +654,22 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     if (MODE == kSwiGLU && job.act_out) waves = 8;
 #define Q4ICASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE>(job, act, y, M, K, waves, st)
     if (job.norm_w) {  // kRope, and kSwiGLU with converted results: two rows, eight wavefronts, rows one step long
-        if constexpr (MODE == kRope || MODE == kSwiGLU) return launch_q4_0_i4<2, 1, MODE, true>(job, act, y, M, K, 8, st);
+        if constexpr (MODE == kRope || MODE == kSwiGLU) return launch_q4_0_i4<2, 1, MODE, kHeadNorm>(job, act, y, M, K, 8, st);
         return hipErrorInvalidValue;
     }
     if constexpr (MODE == kRope) {
         Q4ICASE(2, 1);
         return launch_q4_0_i4<2, 2, MODE>(job, act, y, M, K, waves, st);
     } else {
+        if constexpr (MODE == kPlain) {
+            if (job.norm_x) {  // x itself, converted by every workgroup
+#define Q4CCASE(RR, PP) if (R == RR && PC == PP) return launch_q4_0_i4<RR, PP, MODE, kHeadConvert>(job, act, y, M, K, waves, st)
+                Q4CCASE(1, 1); Q4CCASE(2, 1); Q4CCASE(4, 1);
+                Q4CCASE(1, 2); Q4CCASE(2, 2); Q4CCASE(4, 2);
+#undef Q4CCASE
+                return launch_q4_0_i4<1, 1, MODE, kHeadConvert>(job, act, y, M, K, waves, st);
+            }
+        }
         Q4ICASE(1, 1); Q4ICASE(2, 1); Q4ICASE(4, 1);
         Q4ICASE(1, 2); Q4ICASE(2, 2);
         if constexpr (MODE != kSwiGLU) { Q4ICASE(4, 2); }
@@ -637,7 +681,9 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
 // The fixed-point product from converted activations (a.act), plus a.resid
 // if set. Needs q4_0_fixed_point_ok.
 hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
+    // without converted activations every workgroup converts its row of a.x for itself (few rows of x: a launch saved)
+    Q4Job job{{(const uint8_t*)a.W, nullptr, nullptr}, {(int)a.N, 0, 0}, (int)a.N, a.resid, {}, nullptr, 0, a.act ? nullptr : a.x, nullptr, 0.f, 0.f,
+              a.x_row_stride};
     return dispatch_q4_0_i4<kPlain>(job, a.act, a.y, a.M, a.K, tune, st);
 }
 
@@ -646,7 +692,7 @@ hipError_t qgemv_q4_0_act(const QGemvArgs& a, const int* tune, hipStream_t st) {
 hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                 const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
+              (int)(n[0] + n[1] + n[2]), nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f, 0};
     return dispatch_q4_0_i4<kMulti>(job, act, y, M, K, tune, st);
 }
 
@@ -656,7 +702,7 @@ hipError_t qgemv_q4_0_act_multi(const void* const W[3], const int64_t n[3], cons
 hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                    const Q4RopeTail& rope, const Q4NormHead& norm, const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)W[0], (const uint8_t*)W[1], (const uint8_t*)W[2]}, {(int)n[0], (int)n[1], (int)n[2]},
-              (int)(n[0] + n[1] + n[2]), nullptr, rope, nullptr, 0, norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps};
+              (int)(n[0] + n[1] + n[2]), nullptr, rope, nullptr, 0, norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps, K};
     return dispatch_q4_0_i4<kRope>(job, act, y, M, K, tune, st);
 }
 
@@ -667,7 +713,7 @@ bool q4_0_norm_head_ok(int64_t K) { return K % 64 == 0 && K / 8 <= 256 * kNormIt
 // y[m, r] = SiLU(x[m, :] . gate[r]) * (x[m, :] . up[r]), gate and up [N, K].
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st) {
-    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f};
+    Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, nullptr, 0, nullptr, nullptr, 0.f, 0.f, 0};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, y, M, K, tune, st);
 }
 
@@ -681,7 +727,7 @@ bool q4_0_swiglu_convert_ok(int64_t N, int64_t K) { return K / 64 <= 64 && N % 6
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
                                          int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st) {
     Q4Job job{{(const uint8_t*)gate, (const uint8_t*)up, nullptr}, {(int)N, (int)N, 0}, (int)N, nullptr, {}, (uint8_t*)act_out,
-              (int64_t)q4_0_act_bytes(N), norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps};
+              (int64_t)q4_0_act_bytes(N), norm.x, norm.w, (float)(1.0 / (double)K), (float)norm.eps, K};
     return dispatch_q4_0_i4<kSwiGLU>(job, act, nullptr, M, K, tune, st);
 }
 
