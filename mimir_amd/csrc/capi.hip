@@ -349,6 +349,12 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         return MI355X_OK;
     case MI355X_Q8_0: {
         if (!mimir::q8_act_fits(K)) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv by q8_0 with K = %lld: rows longer than 57344 are not supported", (long long)K);
+        // Small products in one launch (a.act stays null: every workgroup rounds x for itself); this kernel does not
+        // request its weights ahead of that, so on large ones a conversion launch of its own is the faster (measured).
+        if (M <= kConvertInProductRows && N * K <= (int64_t)24 << 20 && ((uintptr_t)x & 15) == 0 && (M == 1 || x_row_stride % 4 == 0)) {
+            HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0");
+            return MI355X_OK;
+        }
         void* act;
         if (mi355x_status st = act_scratch(mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
         HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");

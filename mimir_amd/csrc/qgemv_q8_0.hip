@@ -33,6 +33,38 @@ size_t q8_act_bytes(int64_t K) {
 // quantizeRow (backend/cpu/qmatmul.go:208-254) for blocks of 32. Thread t takes
 // four values: block t / 8, dword t % 8; a block's eight threads are
 // consecutive lanes.
+// Item t of a row (block t / 8, dword t % 8; a block's eight items in eight consecutive lanes,
+// all active) from its four values: the dword of quants into q, the block's scale from its first item.
+__device__ __forceinline__ void q8_convert_item(const f32x4 v, uint32_t* q, float* dscale, int nbp, int t) {
+    const int b = t >> 3, i = t & 7;
+    float amax = 0.f;
+    bool finite = true;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float a = __builtin_fabsf(v[k]);
+        finite = finite && a < __builtin_inff();  // false for NaN too
+        if (a > amax) amax = a;
+    }
+    amax = group8_max(amax);
+    float bad = group8_max(finite ? 0.f : 1.f);
+    float d = 0.f;
+    uint32_t packed = 0;
+    if (bad != 0.f) {
+        d = __builtin_nanf("");
+    } else if (amax != 0.f) {
+        d = amax / 127.0f;
+        float id = 127.0f / amax;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            int r = (int)__builtin_rintf(v[k] * id);  // nearest, ties to even
+            r = r > 127 ? 127 : r < -127 ? -127 : r;
+            packed |= (uint32_t)(r & 0xff) << (8 * k);
+        }
+    }
+    q[((i >> 2) * nbp + b) * 4 + (i & 3)] = packed;
+    if (i == 0) dscale[b] = d;
+}
+
 __global__ __launch_bounds__(256) void q8_convert_act_kernel(const float* __restrict__ x, int64_t x_row_stride, int nb,
                                                              uint8_t* __restrict__ act, int64_t act_row_bytes) {
     const float* xr = x + (int64_t)blockIdx.y * x_row_stride;
@@ -41,35 +73,9 @@ __global__ __launch_bounds__(256) void q8_convert_act_kernel(const float* __rest
     float* dscale = (float*)(q + 2 * nbp * 4);
     const int nq = nb * 8;
     for (int t = blockIdx.x * blockDim.x + threadIdx.x; t < nq; t += gridDim.x * blockDim.x) {
-        int b = t >> 3, i = t & 7;
         f32x4 v;
-        __builtin_memcpy(&v, xr + 32 * (int64_t)b + 4 * i, 16);
-        float amax = 0.f;
-        bool finite = true;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            float a = __builtin_fabsf(v[k]);
-            finite = finite && a < __builtin_inff();  // false for NaN too
-            if (a > amax) amax = a;
-        }
-        amax = group8_max(amax);
-        float bad = group8_max(finite ? 0.f : 1.f);
-        float d = 0.f;
-        uint32_t packed = 0;
-        if (bad != 0.f) {
-            d = __builtin_nanf("");
-        } else if (amax != 0.f) {
-            d = amax / 127.0f;
-            float id = 127.0f / amax;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                int r = (int)__builtin_rintf(v[k] * id);  // nearest, ties to even
-                r = r > 127 ? 127 : r < -127 ? -127 : r;
-                packed |= (uint32_t)(r & 0xff) << (8 * k);
-            }
-        }
-        q[((i >> 2) * nbp + b) * 4 + (i & 3)] = packed;
-        if (i == 0) dscale[b] = d;
+        __builtin_memcpy(&v, xr + 4 * (int64_t)t, 16);
+        q8_convert_item(v, q, dscale, nbp, t);
     }
 }
 
@@ -105,7 +111,9 @@ __device__ __forceinline__ void q8_block(const uint32_t w[8], const u32x4 xa, co
     }
 }
 
-template <int R, bool ALIGNED>
+// CONVERT: act is float32 x (rows act_row_bytes bytes apart) and every workgroup rounds its row to
+// int8 for itself (few rows of x: a launch saved); otherwise act holds rows converted beforehand.
+template <int R, bool ALIGNED, bool CONVERT>
 __global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
                                                          float* __restrict__ y, int N, int nb, int64_t act_row_bytes,
                                                          int rows_per_wg) {
@@ -123,21 +131,31 @@ __global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restri
     const int nsteps = (nunits + 63) >> 6;
 
     // Stage the converted activations (see qgemv_q4_0_i4_kernel for the order).
-    constexpr int kPark = 2;
-    const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
-    const int n16 = (int)(act_row_bytes >> 4);
-    u32x4 park[kPark];
+    if (CONVERT) {
+        const float* xr = (const float*)(act + (int64_t)m * act_row_bytes);
+        const int nq = nb * 8;
+        for (int t = tid; t < nq; t += (int)blockDim.x) {
+            f32x4 v;
+            __builtin_memcpy(&v, xr + 4 * (int64_t)t, 16);
+            q8_convert_item(v, (uint32_t*)lds_q8, (float*)(lds_q8 + 2 * nbp), nbp, t);
+        }
+    } else {
+        constexpr int kPark = 2;
+        const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
+        const int n16 = (int)(act_row_bytes >> 4);
+        u32x4 park[kPark];
 #pragma unroll
-    for (int i = 0; i < kPark; i++) {
-        int idx = tid + i * (int)blockDim.x;
-        if (idx < n16) park[i] = act_row[idx];
-    }
+        for (int i = 0; i < kPark; i++) {
+            int idx = tid + i * (int)blockDim.x;
+            if (idx < n16) park[i] = act_row[idx];
+        }
 #pragma unroll
-    for (int i = 0; i < kPark; i++) {
-        int idx = tid + i * (int)blockDim.x;
-        if (idx < n16) lds_q8[idx] = park[i];
+        for (int i = 0; i < kPark; i++) {
+            int idx = tid + i * (int)blockDim.x;
+            if (idx < n16) lds_q8[idx] = park[i];
+        }
+        for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_q8[idx] = act_row[idx];
     }
-    for (int idx = tid + kPark * (int)blockDim.x; idx < n16; idx += (int)blockDim.x) lds_q8[idx] = act_row[idx];
     __syncthreads();
 
     for (int r0 = wave * R; r0 < rows_per_wg; r0 += waves * R) {
@@ -220,8 +238,12 @@ static hipError_t launch_q8(const QGemvArgs& a, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
     dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);
     size_t act_bytes = q8_act_bytes(a.K);
-    hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
-                       (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+    if (a.act)
+        hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED, false>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
+                           (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+    else  // float32 x, converted by every workgroup
+        hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED, true>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
+                           (const uint8_t*)a.x, a.y, (int)a.N, (int)(a.K / 32), a.x_row_stride * 4, rows_per_wg);
     return hipGetLastError();
 }
 
