@@ -278,6 +278,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
+ * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
+ * kernel, 2 puts them all on the kernel that shares W among rows of x.
+ * "attention.splits" = n fixes the shares of the keys in decode attention.
  * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
  * kernels takes; "kquant.path" = 1 forces their variant that reads x from
  * global memory (otherwise used only for rows of x too long for the LDS), 2

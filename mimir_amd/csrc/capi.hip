@@ -333,8 +333,8 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
     switch (dtype) {
     case MI355X_Q4_0:
         if (g_tune_q4[4] != 1 && mimir::q4_0_fixed_point_ok(W, K)) {
-            if (M <= kConvertInProductRows && ((uintptr_t)x & 15) == 0 && (M == 1 || x_row_stride % 4 == 0)) {
-                // few rows: one launch, every workgroup converts x for itself
+            if (M == 1 && ((uintptr_t)x & 15) == 0) {
+                // one row: one launch, every workgroup converts x for itself (several rows: converted once, multiplied together)
                 HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
                 return MI355X_OK;
             }
@@ -604,6 +604,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "qgemm.path") == 0) {
         g_tune_gemm = value;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.batch_off") == 0) {
+        mimir::set_q4_batch_off(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "attention.splits") == 0) {

@@ -62,6 +62,7 @@ struct Q4NormHead {
     double eps = 0;
 };
 bool q4_0_norm_head_ok(int64_t K);
+void set_q4_batch_off(int v);  // 1: products of several rows of x stay on the one-row kernel
 bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
                                          int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st);

@@ -264,7 +264,8 @@ static mi355x_status step_fast(Model& m) {
     at.dyn_k = pos;  // position p holds p keys before this step's own
     at.k = m.keys[0].p; at.v = m.values[0].p;  // every layer's caches are allocated alike
     const bool one_launch = attention_decode_ok(at, c.context);
-    const bool norm_head = q4_0_norm_head_ok(c.embed);
+    // one sequence: the norms ride on the products; with several, norms of their own are the faster (measured at 8)
+    const bool norm_head = q4_0_norm_head_ok(c.embed) && B == 1;
     if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];

@@ -380,6 +380,8 @@ __device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int 
 }
 
 constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
+static int g_q4_batch_off = 0;  // measurement aid: 1 keeps products of several rows of x on the one-row kernel, 2 puts all on the batch kernel
+void set_q4_batch_off(int v) { g_q4_batch_off = v; }
 
 template <int R, int PC, int MODE, int HEAD = kHeadAct>
 __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y,
@@ -578,6 +580,201 @@ __global__ __launch_bounds__(512) void qgemv_q4_0_i4_kernel(Q4Job job, const uin
     }
 }
 
+// The same product for several rows of x at once: a workgroup stages MB converted rows in LDS, a
+// wavefront unpacks its rows of W once per step and multiplies them with one row of x after the
+// other, so W is read from memory once for MB rows of x instead of once for each. Every row of x
+// meets the same lanes, steps and reductions as in the kernel above, so its results are the same
+// bits. Over converted activations only; tails as above (the block of SwiGLU results per row of x).
+template <int R, int MODE, int MB>
+__global__ __launch_bounds__(512) void qgemv_q4_0_i4_batch_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y, int M,
+                                                                   int nb, int64_t act_row_bytes, int rows_per_wg) {
+    constexpr int RR = MODE == kSwiGLU ? 2 * R : R;
+    extern __shared__ u32x4 lds_i4[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+    const int m0 = blockIdx.y * MB;
+    const int mc = M - m0 < MB ? M - m0 : MB;  // rows of x this workgroup has
+    const int N = job.total;
+    const int nbp = nb | 1;
+    const int n16 = (int)(act_row_bytes >> 4);
+    const int64_t row_bytes = (int64_t)nb * 18;
+    const int wg_row0 = blockIdx.x * rows_per_wg;
+    const int npairs = nb >> 1;
+    const int npc = (npairs + 63) >> 6;
+    const int rope_pos = MODE == kRope ? *job.rope.pos : 0;
+    float* outv = (float*)(lds_i4 + MB * n16);  // kSwiGLU with act_out: 32 results per row of x
+
+    auto row_ptr = [&](int row0, int t) -> const uint8_t* {
+        if (MODE == kSwiGLU) {
+            int r = row0 + (t < R ? t : t - R);
+            r = r < N ? r : N - 1;
+            return job.W[t < R ? 0 : 1] + (int64_t)r * row_bytes;
+        }
+        int g = row0 + t;
+        g = g < N ? g : N - 1;
+        if (MODE == kMulti || MODE == kRope) {
+            if (g >= job.n[0] + job.n[1]) return job.W[2] + (int64_t)(g - job.n[0] - job.n[1]) * row_bytes;
+            if (g >= job.n[0]) return job.W[1] + (int64_t)(g - job.n[0]) * row_bytes;
+        }
+        return job.W[0] + (int64_t)g * row_bytes;
+    };
+
+    Q4PairTile<RR, 1> tile;
+    int r0 = wave * R;
+    const uint8_t* rowp[RR];
+#pragma unroll
+    for (int t = 0; t < RR; t++) rowp[t] = row_ptr(wg_row0 + r0, t);
+    q4_load_pairs<RR, 1>(tile, rowp, npairs, 0, lane);  // in flight while the rows of x are staged
+    const u32x4* src = (const u32x4*)(act + (int64_t)m0 * act_row_bytes);
+    for (int idx = tid; idx < mc * n16; idx += (int)blockDim.x) lds_i4[idx] = src[idx];
+    __syncthreads();
+
+    bool loaded = true;
+    for (; r0 < rows_per_wg; r0 += waves * R) {
+        const int row0 = wg_row0 + r0;
+        if (row0 >= N) break;
+        if (!loaded) {
+#pragma unroll
+            for (int t = 0; t < RR; t++) rowp[t] = row_ptr(row0, t);
+        }
+        float acc[MB][RR];
+#pragma unroll
+        for (int mi = 0; mi < MB; mi++)
+#pragma unroll
+            for (int r = 0; r < RR; r++) acc[mi][r] = 0.f;
+        for (int pc = 0; pc < npc; pc++) {
+            if (!loaded) q4_load_pairs<RR, 1>(tile, rowp, npairs, pc, lane);
+            loaded = false;
+            int p = lane + 64 * pc;
+            const bool live = p < npairs;
+            p = live ? p : npairs - 1;
+            // the rows of W of this step, unpacked once for all rows of x
+            uint32_t q0[RR][4], q1[RR][4];
+            float dw0[RR], dw1[RR];
+#pragma unroll
+            for (int r = 0; r < RR; r++) {
+                const u32x4 a = tile.a[r][0], b = tile.b[r][0];
+                q0[r][0] = __builtin_amdgcn_alignbyte(a[1], a[0], 2);
+                q0[r][1] = __builtin_amdgcn_alignbyte(a[2], a[1], 2);
+                q0[r][2] = __builtin_amdgcn_alignbyte(a[3], a[2], 2);
+                q0[r][3] = __builtin_amdgcn_alignbyte(b[0], a[3], 2);
+                q1[r][0] = b[1], q1[r][1] = b[2], q1[r][2] = b[3], q1[r][3] = tile.c[r][0];
+                dw0[r] = f16_bits_to_f32((uint16_t)(a[0] & 0xffffu));
+                dw1[r] = f16_bits_to_f32((uint16_t)(b[0] >> 16));
+            }
+#pragma unroll
+            for (int mi = 0; mi < MB; mi++) {
+                if (mi < mc) {
+                    const u32x4* xrow = lds_i4 + mi * n16;
+                    const float* xscale = (const float*)(xrow + kDigits * nbp);
+                    u32x4 d0[kDigits], d1[kDigits];
+#pragma unroll
+                    for (int j = 0; j < kDigits; j++) {
+                        d0[j] = xrow[j * nbp + 2 * p];
+                        d1[j] = xrow[j * nbp + 2 * p + 1];
+                    }
+                    const float s0 = live ? xscale[2 * p] : 0.f, s1 = live ? xscale[2 * p + 1] : 0.f;
+#pragma unroll
+                    for (int r = 0; r < RR; r++) {
+                        int i0, i1;
+                        q4_pair_dot(q0[r], q1[r], d0, d1, i0, i1);
+                        const float f0 = (float)i0, f1 = (float)i1;
+                        // a lane past the row's end re-reads the last pair: it must add exactly zero
+                        const float w0 = live ? dw0[r] * s0 : 0.f;
+                        const float w1 = live ? dw1[r] * s1 : 0.f;
+                        acc[mi][r] = fmaf(w0, f0, acc[mi][r]);
+                        acc[mi][r] = fmaf(w1, f1, acc[mi][r]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int mi = 0; mi < MB; mi++) {
+            if (mi >= mc) break;
+            const int m = m0 + mi;
+            float* yr = y + (int64_t)m * N;
+            if (MODE == kRope) {
+#pragma unroll
+                for (int r = 0; r + 1 < R; r += 2) {
+                    const float a = wave_sum(acc[mi][r]), b = wave_sum(acc[mi][r + 1]);
+                    if (lane == 0 && row0 + r < N) q4_rope_store(job.rope, rope_pos, m, row0 + r, a, b, yr);
+                }
+                continue;
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float s = wave_sum(acc[mi][r]);
+                if (MODE == kSwiGLU) {
+                    const float u = wave_sum(acc[mi][R + r]);
+                    const float e = __builtin_exp2f(s * (float)(-1.4426950408889634));
+                    const float sg = 1.0f / (1.0f + e);
+                    const float a = s * sg;
+                    s = a * u;
+                }
+                if (MODE == kSwiGLU && job.act_out) {
+                    if (lane == 0) outv[32 * mi + r0 + r] = s;
+                } else if (lane == 0 && row0 + r < N) {
+                    if (MODE == kPlain && job.resid) s = s + job.resid[(int64_t)m * N + row0 + r];
+                    yr[row0 + r] = s;
+                }
+            }
+        }
+    }
+    if (MODE == kSwiGLU && job.act_out) {  // per row of x, the workgroup's 32 results are block blockIdx.x of the next product's x
+        __syncthreads();
+        if (tid < 4 * mc) {
+            const int mi = tid >> 2, d = tid & 3;
+            const f32x4* v = (const f32x4*)(outv + 32 * mi);
+            const f32x4 vlo = v[d], vhi = v[4 + d];
+            float lo[4] = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi[4] = {vhi[0], vhi[1], vhi[2], vhi[3]};
+            u32x4* plane = (u32x4*)(job.act_out + (int64_t)(m0 + mi) * job.act_out_row_bytes);
+            const int nbp_out = (N >> 5) | 1;
+            q4_convert_item(lo, hi, plane, (float*)(plane + kDigits * nbp_out), nbp_out, blockIdx.x, d);
+        }
+    }
+}
+
+// Rows of x a workgroup of the batch kernel can stage (8, 4, 2; 0: none fits).
+static int q4_batch_rows(int64_t M, int64_t K) {
+    const size_t row = q4_0_act_bytes(K);
+    for (int mb = 8; mb >= 2; mb >>= 1)
+        if (M >= mb && (size_t)mb * row + 1024 <= 144 * 1024) return mb;
+    return M >= 2 && 2 * row + 1024 <= 144 * 1024 ? 2 : 0;
+}
+
+template <int R, int MODE, int MB>
+static hipError_t launch_q4_0_i4_batch(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st) {
+    static bool raised = false;
+    const size_t act_bytes = q4_0_act_bytes(K), lds_bytes = MB * act_bytes + MB * 128;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)qgemv_q4_0_i4_batch_kernel<R, MODE, MB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           160 * 1024);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    const int rows_per_wg = MODE == kSwiGLU && job.act_out ? 32 : R * 8;
+    dim3 grid((unsigned)((job.total + rows_per_wg - 1) / rows_per_wg), (unsigned)((M + MB - 1) / MB));
+    hipLaunchKernelGGL((qgemv_q4_0_i4_batch_kernel<R, MODE, MB>), grid, dim3(512), lds_bytes, st, job, (const uint8_t*)act, y, (int)M,
+                       (int)(K / 32), (int64_t)act_bytes, rows_per_wg);
+    return hipGetLastError();
+}
+
+// From two rows of x on the batch kernel, where it is the faster: both kernels are bound by the
+// vector arithmetic of the six digit planes, not by reading W, so sharing W gains only where staging
+// x per workgroup is what costs (rows of x from 8192 on: 20 % faster at 4096 x 14336, 15 to 60 %
+// slower at K = 4096; measured for 2 to 512 rows of x).
+template <int MODE>
+static bool dispatch_q4_0_i4_batch(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st, hipError_t* err) {
+    if (job.norm_x || g_q4_batch_off == 1 || (K < 8192 && g_q4_batch_off != 2)) return false;
+    const int mb = q4_batch_rows(M, K);
+    if (mb == 0) return false;
+    constexpr int R = MODE == kSwiGLU ? 2 : 4;
+    *err = mb == 8 ? launch_q4_0_i4_batch<R, MODE, 8>(job, act, y, M, K, st)
+           : mb == 4 ? launch_q4_0_i4_batch<R, MODE, 4>(job, act, y, M, K, st)
+                     : launch_q4_0_i4_batch<R, MODE, 2>(job, act, y, M, K, st);
+    return true;
+}
+
 template <int R, int PC, int MODE, int HEAD = kHeadAct>
 static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, int waves, hipStream_t st) {
     int rows_per_wg = R * waves;
@@ -637,6 +834,10 @@ bool q4_0_fixed_point_ok(const void* W, int64_t K) {
 // decode shapes. tune: {rows, pair steps, waves}.
 template <int MODE>
 static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, const int* tune, hipStream_t st) {
+    if constexpr (MODE != kMulti) {
+        hipError_t e;
+        if (M >= 2 && tune[0] == 0 && tune[1] == 0 && tune[2] == 0 && dispatch_q4_0_i4_batch<MODE>(job, act, y, M, K, st, &e)) return e;
+    }
     int nb = (int)(K / 32);
     int npc = (nb / 2 + 63) / 64;  // steps of 64 pairs of blocks that cover a row
     int PC = npc <= 1 ? 1 : 2;

@@ -213,6 +213,30 @@ def test_q4_0_gemv_linearity_at_full_size():
         capi.check(l.mi355x_tune(b"q4_0.path", 0))
 
 
+@pytest.mark.parametrize("m,n,k", [(2, 100, 4096), (5, 257, 1280), (8, 4096, 4096), (11, 64, 14336), (37, 130, 256)])
+def test_q4_0_gemv_of_several_rows_reads_w_once_and_gives_each_row_its_own_bits(m, n, k):
+    """The batch kernel multiplies a workgroup's rows of W with up to eight rows of x (as many as fit the
+    LDS); every row of x meets the same lanes and reductions as alone, so the results equal the one-row
+    kernel's bit for bit, whatever M leaves for the last group. (The library picks it for long rows of x.)"""
+    l = gpu.lib()
+    rng = np.random.default_rng(m * n + k)
+    raw = random_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    gpu.say(f"q4_0 gemv batch M={m} N={n} K={k}")
+    try:
+        capi.check(l.mi355x_tune(b"q4_0.batch_off", 2))  # the batch kernel whatever the shape
+        got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+        capi.check(l.mi355x_tune(b"q4_0.batch_off", 1))  # the one-row kernel
+        rows = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    finally:
+        capi.check(l.mi355x_tune(b"q4_0.batch_off", 0))
+    assert np.array_equal(got, rows)
+    # random scales span binary16's range: the bound goes with the size of the terms, not of the result
+    mag = np.abs(x).astype(np.float64) @ np.abs(O.dequantize(O.Q4_0, raw).reshape(n, k)).astype(np.float64).T
+    assert np.all(np.abs(got - O.qmatmul(O.Q4_0, raw, x, n, k)) <= 2e-6 * mag + 1e-30)
+
+
 def test_q4_0_fused_products():
     """The fused products of a decoding step against the oracle's separate
     ones: residual add, three matrices in one launch, SwiGLU of gate and up."""
