@@ -268,6 +268,30 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
     st = torch.cuda.Stream()
     kinds = (("q4_0", capi.Q4_0, 2500.0, "frac_of_bf16_peak"), ("q4_K", capi.Q4_K, 5000.0, "frac_of_int8_peak"),
              ("q6_K", capi.Q6_K, 5000.0, "frac_of_int8_peak"))
+    # float32 activations by Q4_0 (what the decoder's prompt pass multiplies): mi355x_qgemv, whose 24-bit
+    # fixed-point x takes three int8 multiplications a weight
+    res = {}
+    for m, n in shapes:
+        w = torch.from_numpy(bench_blocks_q4_0(rng, n * k)).to("cuda:0")
+        x = torch.randn(m, k, device="cuda:0")
+        y = torch.empty(m, n, dtype=torch.float32, device="cuda:0")
+        torch.cuda.synchronize()
+        with torch.cuda.stream(st):
+            call = lambda: capi.check(lib.mi355x_qgemv(capi.Q4_0, w.data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, st.cuda_stream))
+            for _ in range(5):
+                call()
+            st.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for _ in range(iters):
+                call()
+            e1.record(st)
+            st.synchronize()
+        us = e0.elapsed_time(e1) / iters * 1e3
+        tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+        res[f"M{m}_N{n}_K{k}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1), "frac_of_int8_peak": round(tf / 5000.0, 4)}
+        del w, x, y
+    out["q4_0_f32_x"] = res
     for name, dt, peak, frac_key in kinds:
         res = {}
         for m, n in shapes:

@@ -67,6 +67,9 @@ int g_tune_q4[5] = {0, 0, 0, 0, 0};
 // Up to this many rows of x the Q4_0 product converts x inside its own launch (each workgroup
 // for itself); beyond, one conversion launch serves all workgroups.
 constexpr int64_t kConvertInProductRows = 8;
+// Rows of x from which the Q4_0 product of float32 x goes to the int8 matrix cores: 16 means wherever its
+// cost model says it pays; "q4_0.fx_rows" sets another threshold, which then holds for every shape.
+int g_fx_min_rows = 16;
 int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
@@ -333,6 +336,15 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
     switch (dtype) {
     case MI355X_Q4_0:
         if (g_tune_q4[4] != 1 && mimir::q4_0_fixed_point_ok(W, K)) {
+            if (g_tune_q4[4] != 2 && M >= g_fx_min_rows && (g_fx_min_rows != 16 ? mimir::qgemm_q4_0_fx_ok(W, M, N, K) : mimir::qgemm_q4_0_fx_pays(W, M, N, K)) &&
+                ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0) {
+                // many rows: the same fixed-point arithmetic on the int8 matrix cores
+                void* act;
+                if (mi355x_status st = act_scratch(mimir::q4_0_fx_act_bytes(K) * (size_t)M, &act)) return st;
+                HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_fx_convert_act");
+                HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, (hipStream_t)stream), "launch qgemm_q4_0_fx");
+                return MI355X_OK;
+            }
             if (M == 1 && ((uintptr_t)x & 15) == 0) {
                 // one row: one launch, every workgroup converts x for itself (several rows: converted once, multiplied together)
                 HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
@@ -604,6 +616,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "qgemm.path") == 0) {
         g_tune_gemm = value;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.fx_rows") == 0) {
+        g_fx_min_rows = value > 0 ? value : 16;
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.batch_off") == 0) {

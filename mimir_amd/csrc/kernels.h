@@ -173,6 +173,14 @@ void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, 
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st);
 
+// The fixed-point Q4_0 product for many rows of float32 x on the int8 matrix cores (qgemm_q4_0_fx.hip):
+// x converted by q4_0_fx_convert_act (q4_0_fx_act_bytes(K) bytes a row), K a multiple of 128.
+size_t q4_0_fx_act_bytes(int64_t K);
+hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+bool qgemm_q4_0_fx_ok(const void* W, int64_t M, int64_t N, int64_t K);
+bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K);  // and is the faster choice
+hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, hipStream_t st);
+
 // Prompt-sized Q4_0 product on the matrix cores (qgemm_q4_0.hip): X [M, K]
 // bfloat16, Y [M, N] bfloat16 or float32.
 bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K, int64_t x_row_stride);

@@ -63,7 +63,7 @@ struct Weight {
 };
 
 // The form of converted activations a weight's product reads.
-enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3 };
+enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4 };  // kActFx: Q4_0 by many rows of x, on the matrix cores
 
 struct Block {
     Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down;
@@ -83,7 +83,7 @@ struct Model {
 
     // activations of up to max_rows rows (batch x tokens of one call)
     int64_t max_rows = 0;
-    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[4], act2, tokens_dev, next_tok;
+    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[5], act2, tokens_dev, next_tok;
     hipStream_t stream = nullptr;
 
     // The decoding step as a fixed run of launches that read the position from
@@ -100,9 +100,11 @@ struct Model {
     }
 };
 
-int act_class(const Weight& w) {
+int act_class(const Weight& w, int64_t rows = 1) {
     switch (w.dtype) {
-    case kQ4_0: return q4_0_fixed_point_ok(w.buf.p, w.k) ? kActQ4 : kActNone;
+    case kQ4_0:
+        if (qgemm_q4_0_fx_pays(w.buf.p, rows, w.n, w.k)) return kActFx;
+        return q4_0_fixed_point_ok(w.buf.p, w.k) ? kActQ4 : kActNone;
     case kQ8_0: return q8_act_fits(w.k) ? kActQ8 : kActNone;
     case kQ4_K: case kQ6_K: return kActKQ;
     default: return kActNone;
@@ -114,6 +116,7 @@ size_t act_row_bytes(int cls, int64_t K) {
     case kActQ4: return q4_0_act_bytes(K);
     case kActQ8: return q8_act_bytes(K);
     case kActKQ: return kq_act_bytes(K);
+    case kActFx: return q4_0_fx_act_bytes(K);
     default: return 0;
     }
 }
@@ -121,15 +124,16 @@ size_t act_row_bytes(int cls, int64_t K) {
 const int kNoTune[5] = {0, 0, 0, 0, 0};
 
 // Converts rows of x once for every activation form that `ws` need.
-mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[4]) {
-    for (int i = 0; i < 4; i++) done[i] = false;
+mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[5]) {
+    for (int i = 0; i < 5; i++) done[i] = false;
     for (const Weight* w : ws) {
-        int cls = act_class(*w);
+        int cls = act_class(*w, rows);
         if (cls == kActNone || done[cls]) continue;
         size_t need = act_row_bytes(cls, K) * (size_t)rows;
         if (m.act[cls].bytes < need) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: activation scratch of %zu bytes, need %zu", m.act[cls].bytes, need);
         hipError_t e = cls == kActQ4   ? q4_0_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
                        : cls == kActQ8 ? q8_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
+                       : cls == kActFx ? q4_0_fx_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
                                        : kq_convert_act(x, rows, K, K, m.act[cls].p, m.stream);
         LLM_HIP(e, "convert activations");
         done[cls] = true;
@@ -139,11 +143,15 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
 
 // y[rows, n] = x[rows, k] . W^T (nn/layers.go:49-55 -> tensor/quant.go:35-56).
 mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows) {
-    int cls = act_class(w);
+    int cls = act_class(w, rows);
     QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
     hipError_t e;
     switch (w.dtype) {
-    case kQ4_0: e = cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream) : qgemv_q4_0(a, kNoTune, m.stream); break;
+    case kQ4_0:
+        e = cls == kActFx   ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, m.stream)
+            : cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream)
+                            : qgemv_q4_0(a, kNoTune, m.stream);
+        break;
     case kQ8_0:
         if (cls != kActQ8) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: q8_0 rows of %lld are too long", (long long)w.k);
         e = qgemv_q8_0_act(a, kNoTune, m.stream);
@@ -178,7 +186,7 @@ static mi355x_status forward(Model& m, int64_t s) {
     const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
     float *x = m.x.as<float>(), *h = m.h.as<float>(), *q = m.q.as<float>(), *k = m.k.as<float>(), *v = m.v.as<float>();
     float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
-    bool done[4];
+    bool done[5];
     if (mi355x_status st = embed_rows(m, m.tokens_dev.as<int32_t>(), rows, x, device_error_word())) return st;
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
@@ -336,7 +344,7 @@ static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_
             LLM_HIP(rmsnorm(xin + r * row_stride, m.norm.buf.as<float>(), hl + r * c.embed, 1, c.embed, c.eps, m.stream), "output_norm");
     }
     const Weight& w = m.tied ? m.embed : m.output;
-    bool done[4];
+    bool done[5];
     if (mi355x_status st = convert_for(m, hl, rows, c.embed, {&w}, done)) return st;
     return linear(m, w, hl, m.logits.as<float>(), rows);
 }
@@ -492,8 +500,8 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     LLM_HIP(m->logits.alloc((size_t)rows * c.vocab * 4), "hipMalloc(logits)");
     LLM_HIP(m->tokens_dev.alloc(rows * 4), "hipMalloc"); LLM_HIP(m->next_tok.alloc(c.batch * 4), "hipMalloc");
     const int64_t kmax = c.hidden > qd ? (c.hidden > c.embed ? c.hidden : c.embed) : (qd > c.embed ? qd : c.embed);
-    for (int cls = 1; cls < 4; cls++) {
-        int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : (kmax + 63) / 64 * 64;
+    for (int cls = 1; cls < 5; cls++) {
+        int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : cls == kActFx ? (kmax + 127) / 128 * 128 : (kmax + 63) / 64 * 64;
         LLM_HIP(m->act[cls].alloc(act_row_bytes(cls, kk) * rows + 64), "hipMalloc(activations)");
     }
     LLM_HIP(m->act2.alloc(q4_0_act_bytes((c.hidden + 63) / 64 * 64) * c.batch + 64), "hipMalloc(activations)");
