@@ -84,7 +84,12 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * (backend/cpu/qmatmul.go:310-405): for Q8_0, Q4_K and Q6_K each block of a
  * row of x is rounded to int8 first and the dot products are integer; for
  * Q4_0 it is the float32 product with the dequantized weights, the route the
- * reference takes for that file dtype (io/mim/dtype.go:118-123). */
+ * reference takes for that file dtype (io/mim/dtype.go:118-123).
+ * One entry point for every M, as OpQMatMul is one operation: by dtype and
+ * shape the library runs row kernels (few rows of x; one launch for one row of
+ * x by Q4_0 or a small Q8_0 matrix) or, from enough rows on, kernels on the
+ * int8 matrix cores (Q4_0, Q4_K, Q6_K); which one ran changes the results only
+ * by the order of float32 additions (Q4_0, Q8_0) or not at all (Q4_K, Q6_K). */
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
 
@@ -281,6 +286,8 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
  * kernel, 2 puts them all on the kernel that shares W among rows of x.
  * "attention.splits" = n fixes the shares of the keys in decode attention.
+ * "q4_0.fx_rows" = n sends Q4_0 products of at least n rows of float32 x to the
+ * int8 matrix cores whatever the shape (0: the built-in cost model).
  * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
  * kernels takes; "kquant.path" = 1 forces their variant that reads x from
  * global memory (otherwise used only for rows of x too long for the LDS), 2
