@@ -161,20 +161,22 @@ hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int 
 // cache's dtype. The position is read on the device so that a captured step
 // can be replayed at every position (the reference's recorded step takes the
 // position as a tensor for the same reason, llm/decode.go:27-41,166-183).
-__global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ qkv, void* __restrict__ kcache, void* __restrict__ vcache,
-                                                      int cache_dt, int B, int H, int HK, int dim, int rope_dim, int interleaved,
-                                                      int64_t cap, const float* __restrict__ cosv, const float* __restrict__ sinv,
-                                                      const int32_t* __restrict__ pos_dev) {
+__global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                      int64_t q_row, int64_t k_row, int64_t v_row, void* __restrict__ kcache,
+                                                      void* __restrict__ vcache, int cache_dt, int B, int H, int HK, int dim, int rope_dim,
+                                                      int interleaved, int64_t cap, const float* __restrict__ cosv,
+                                                      const float* __restrict__ sinv, const int32_t* __restrict__ pos_dev) {
     const int pos = *pos_dev;
     const int half = rope_dim >> 1, hd2 = dim >> 1;  // work items: pairs of features
-    const int64_t row = (int64_t)(H + 2 * HK) * dim;
     const int64_t total = (int64_t)B * (H + 2 * HK) * hd2;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
         int i = (int)(t % hd2);
         int64_t r = t / hd2;
         int head = (int)(r % (H + 2 * HK));
         int64_t b = r / (H + 2 * HK);
-        float* hp = qkv + b * row + (int64_t)head * dim;
+        // sequence b's heads: H of queries at q, HK of keys at k, HK of values at v, rows q_row, k_row, v_row floats apart
+        const float* hp = head < H ? q + b * q_row + (int64_t)head * dim
+                                   : head < H + HK ? k + b * k_row + (int64_t)(head - H) * dim : v + b * v_row + (int64_t)(head - H - HK) * dim;
         int ia, ib;
         float va, vb;
         if (head < H + HK && i < half) {
@@ -193,8 +195,9 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ qkv, v
             vb = hp[ib];
         }
         if (head < H) {
-            hp[ia] = va;
-            hp[ib] = vb;
+            float* qp = q + b * q_row + (int64_t)head * dim;
+            qp[ia] = va;
+            qp[ib] = vb;
         } else {
             const bool is_k = head < H + HK;
             const int kh = is_k ? head - H : head - H - HK;
@@ -211,15 +214,32 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ qkv, v
     }
 }
 
-hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
-                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
+static hipError_t rope_kv_launch(float* q, const float* k, const float* v, int64_t q_row, int64_t k_row, int64_t v_row, void* kcache,
+                                 void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim, int interleaved, int64_t cap,
+                                 const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
     int64_t total = B * (H + 2 * HK) * (dim / 2);
     if (total == 0) return hipSuccess;
     int64_t groups = (total + 255) / 256;
     if (groups > 65536) groups = 65536;
-    hipLaunchKernelGGL(rope_kv_kernel, dim3((unsigned)groups), dim3(256), 0, st, qkv, kcache, vcache, cache_dt, (int)B, H, HK, dim,
-                       rope_dim, interleaved, cap, cosv, sinv, pos_dev);
+    hipLaunchKernelGGL(rope_kv_kernel, dim3((unsigned)groups), dim3(256), 0, st, q, k, v, q_row, k_row, v_row, kcache, vcache, cache_dt,
+                       (int)B, H, HK, dim, rope_dim, interleaved, cap, cosv, sinv, pos_dev);
     return hipGetLastError();
+}
+
+// qkv [B, (H + 2 HK) dim]: each sequence's query, key and value heads in one row.
+hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
+                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
+    const int64_t row = (int64_t)(H + 2 * HK) * dim;
+    return rope_kv_launch(qkv, qkv + (int64_t)H * dim, qkv + (int64_t)(H + HK) * dim, row, row, row, kcache, vcache, cache_dt, B, H, HK, dim,
+                          rope_dim, interleaved, cap, cosv, sinv, pos_dev, st);
+}
+
+// q [B, H dim], k and v [B, HK dim], each contiguous.
+hipError_t rope_kv_split(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim,
+                         int rope_dim, int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev,
+                         hipStream_t st) {
+    return rope_kv_launch(q, k, v, (int64_t)H * dim, (int64_t)HK * dim, (int64_t)HK * dim, kcache, vcache, cache_dt, B, H, HK, dim, rope_dim,
+                          interleaved, cap, cosv, sinv, pos_dev, st);
 }
 
 // After a step: appends the chosen tokens to the record and moves on one

@@ -332,6 +332,60 @@ static mi355x_status step_fast(Model& m) {
     return MI355X_OK;
 }
 
+// One decoding step of every sequence for blocks of any supported dtypes: the per-operator launches of
+// forward() for one position, but with the position read from m.state on the device (rotation, cache
+// write, number of keys), so that the step can be captured once and replayed as a graph like step_fast
+// (the reference records its decoding step for the same reason, llm/decode.go:79-160).
+static mi355x_status step_any(Model& m) {
+    const auto& c = m.c;
+    const int64_t B = c.batch;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
+    float *x = m.x.as<float>(), *h = m.h.as<float>(), *q = m.q.as<float>(), *k = m.k.as<float>(), *v = m.v.as<float>();
+    float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
+    const int32_t* pos = m.state.as<int32_t>();
+    bool done[5];
+    if (mi355x_status st = embed_rows(m, m.next_tok.as<int32_t>(), B, x, device_error_word())) return st;
+    AttnArgs at;
+    at.q = q; at.kv_dtype = c.cache_dtype; at.out = a; at.lse = nullptr;
+    at.q_strides[0] = qd; at.q_strides[1] = c.head_dim; at.q_strides[2] = 0;
+    at.k_strides[0] = at.v_strides[0] = (int64_t)c.kv_heads * c.context * c.head_dim;
+    at.k_strides[1] = at.v_strides[1] = (int64_t)c.context * c.head_dim;
+    at.k_strides[2] = at.v_strides[2] = c.head_dim;
+    at.o_strides[0] = qd; at.o_strides[1] = c.head_dim; at.o_strides[2] = 0;
+    at.B = B; at.Q = 1; at.K = 1; at.H = c.heads; at.HK = c.kv_heads; at.D = c.head_dim;
+    at.scale = 1.0 / std::sqrt((double)c.head_dim);
+    at.causal = 0; at.causal_offset = 0;
+    at.dyn_k = pos;  // position p holds p keys before this step's own
+    at.k = m.keys[0].p; at.v = m.values[0].p;
+    const bool one_launch = attention_decode_ok(at, c.context);
+    if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m.blocks[i];
+        LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "attn_norm");
+        if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.q, &b.k, &b.v}, done)) return st;
+        if (mi355x_status st = linear(m, b.q, h, q, B)) return st;
+        if (mi355x_status st = linear(m, b.k, h, k, B)) return st;
+        if (mi355x_status st = linear(m, b.v, h, v, B)) return st;
+        LLM_HIP(rope_kv_split(q, k, v, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim,
+                              c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        at.k = m.keys[i].p; at.v = m.values[i].p;
+        if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream), "attention");
+        else LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
+        if (mi355x_status st = convert_for(m, a, B, qd, {&b.o}, done)) return st;
+        if (mi355x_status st = linear(m, b.o, a, o, B)) return st;
+        LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+        LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "ffn_norm");
+        if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate, &b.up}, done)) return st;
+        if (mi355x_status st = linear(m, b.gate, h, gate, B)) return st;
+        if (mi355x_status st = linear(m, b.up, h, up, B)) return st;
+        LLM_HIP(swiglu(gate, up, sw, B, c.hidden, c.hidden, m.stream), "swiglu");
+        if (mi355x_status st = convert_for(m, sw, B, c.hidden, {&b.down}, done)) return st;
+        if (mi355x_status st = linear(m, b.down, sw, o, B)) return st;
+        LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+    }
+    return MI355X_OK;
+}
+
 // Norm and output projection of `rows` rows of hidden states at xin, which are
 // row_stride floats apart, into m.logits [rows, vocab].
 static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_stride) {
@@ -619,7 +673,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
     if (m->cache_len + n_prompt + n_new - 1 > c.context)
         return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %lld positions for a context of %d", (long long)(m->cache_len + n_prompt + n_new - 1), c.context);
     const int64_t B = c.batch;
-    const bool use_graph = g_llama_step_mode == 0, use_fast = m->fast && g_llama_step_mode != 2;
+    const bool use_graph = g_llama_step_mode == 0, use_fast = g_llama_step_mode != 2;  // 2: forward() with the position from the host
     DevBuf picked;  // [n_new, batch]
     LLM_HIP(picked.alloc((size_t)n_new * B * 4), "hipMalloc(tokens)");
     hipEvent_t e0, e1, e2;
@@ -642,7 +696,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
         if (!st && e == hipSuccess) e = advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 0, m->stream);
         if (!st && e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: step state: %s", hipGetErrorName(e));
         auto one_step = [&]() -> mi355x_status {
-            if (mi355x_status s2 = step_fast(*m)) return s2;
+            if (mi355x_status s2 = m->fast ? step_fast(*m) : step_any(*m)) return s2;
             if (mi355x_status s2 = head(*m, m->x.as<float>(), B, c.embed)) return s2;
             LLM_HIP(argmax(m->logits.as<float>(), B, c.vocab, m->next_tok.as<int32_t>(), m->argmax_ws.p, m->stream), "argmax");
             LLM_HIP(advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 1, m->stream), "advance");
