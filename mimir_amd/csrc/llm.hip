@@ -42,14 +42,23 @@ namespace {
 struct DevBuf {
     void* p = nullptr;
     size_t bytes = 0;
-    ~DevBuf() {
-        if (p) (void)hipFree(p);
+    bool view = false;  // p points into another buffer's memory
+    ~DevBuf() { release(); }
+    void release() {
+        if (p && !view) (void)hipFree(p);
+        p = nullptr;
+        view = false;
     }
     hipError_t alloc(size_t n) {
-        if (p) (void)hipFree(p);
-        p = nullptr;
+        release();
         bytes = n;
         return hipMalloc(&p, n < 4 ? 4 : n);
+    }
+    void point_at(void* q, size_t n) {
+        release();
+        p = q;
+        bytes = n;
+        view = true;
     }
     template <typename T>
     T* as() const { return (T*)p; }
@@ -65,8 +74,12 @@ struct Weight {
 // The form of converted activations a weight's product reads.
 enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4 };  // kActFx: Q4_0 by many rows of x, on the matrix cores
 
+// qkv and gate_up: where q, k, v (gate, up) share a block dtype, finalize also keeps their rows in one
+// buffer, which a decoding step multiplies in one product (the reference concatenates the same
+// weights for its recorded step, fusedFor, llm/decode.go:240-266). Models that take step_fast do
+// not need them (its kernels read the three matrices where they are).
 struct Block {
-    Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down;
+    Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down, qkv, gate_up;
 };
 
 struct Model {
@@ -91,7 +104,7 @@ struct Model {
     // chosen so far, [max_new, batch]. `fast` says the blocks qualify (Q4_0
     // linears that the fixed-point kernel takes); step_graph replays the run.
     bool fast = false;
-    DevBuf state, record, qkv, argmax_ws;
+    DevBuf state, record, qkv, gu, argmax_ws;  // gu: gate|up of a step, [batch, 2 hidden]
     hipGraphExec_t step_graph = nullptr;
 
     ~Model() {
@@ -142,9 +155,12 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
 }
 
 // y[rows, n] = x[rows, k] . W^T (nn/layers.go:49-55 -> tensor/quant.go:35-56).
-mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows) {
+// With resid, y = product + resid (which may be y); only the row kernels of the quantized dtypes add it.
+mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows, const float* resid = nullptr) {
     int cls = act_class(w, rows);
+    if (resid && (cls == kActFx || cls == kActNone)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
     QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
+    a.resid = resid;
     hipError_t e;
     switch (w.dtype) {
     case kQ4_0:
@@ -342,6 +358,7 @@ static mi355x_status step_any(Model& m) {
     const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
     float *x = m.x.as<float>(), *h = m.h.as<float>(), *q = m.q.as<float>(), *k = m.k.as<float>(), *v = m.v.as<float>();
     float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
+    float *qkv = m.qkv.as<float>(), *gu = m.gu.as<float>();
     const int32_t* pos = m.state.as<int32_t>();
     bool done[5];
     if (mi355x_status st = embed_rows(m, m.next_tok.as<int32_t>(), B, x, device_error_word())) return st;
@@ -362,26 +379,49 @@ static mi355x_status step_any(Model& m) {
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
         LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "attn_norm");
-        if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.q, &b.k, &b.v}, done)) return st;
-        if (mi355x_status st = linear(m, b.q, h, q, B)) return st;
-        if (mi355x_status st = linear(m, b.k, h, k, B)) return st;
-        if (mi355x_status st = linear(m, b.v, h, v, B)) return st;
-        LLM_HIP(rope_kv_split(q, k, v, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim,
-                              c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        if (b.qkv.set()) {  // one product into [B, q | k | v]
+            if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.qkv}, done)) return st;
+            if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
+            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+            at.q = qkv; at.q_strides[0] = qd + 2 * kvd;
+        } else {
+            if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.q, &b.k, &b.v}, done)) return st;
+            if (mi355x_status st = linear(m, b.q, h, q, B)) return st;
+            if (mi355x_status st = linear(m, b.k, h, k, B)) return st;
+            if (mi355x_status st = linear(m, b.v, h, v, B)) return st;
+            LLM_HIP(rope_kv_split(q, k, v, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim,
+                                  c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+            at.q = q; at.q_strides[0] = qd;
+        }
         at.k = m.keys[i].p; at.v = m.values[i].p;
         if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream), "attention");
         else LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
         if (mi355x_status st = convert_for(m, a, B, qd, {&b.o}, done)) return st;
-        if (mi355x_status st = linear(m, b.o, a, o, B)) return st;
-        LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+        if (act_class(b.o, B) != kActNone) {  // the residual rides on the product
+            if (mi355x_status st = linear(m, b.o, a, x, B, x)) return st;
+        } else {
+            if (mi355x_status st = linear(m, b.o, a, o, B)) return st;
+            LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+        }
         LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "ffn_norm");
-        if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate, &b.up}, done)) return st;
-        if (mi355x_status st = linear(m, b.gate, h, gate, B)) return st;
-        if (mi355x_status st = linear(m, b.up, h, up, B)) return st;
-        LLM_HIP(swiglu(gate, up, sw, B, c.hidden, c.hidden, m.stream), "swiglu");
+        if (b.gate_up.set()) {  // one product into [B, gate | up]
+            if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate_up}, done)) return st;
+            if (mi355x_status st = linear(m, b.gate_up, h, gu, B)) return st;
+            LLM_HIP(swiglu(gu, gu + c.hidden, sw, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+        } else {
+            if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate, &b.up}, done)) return st;
+            if (mi355x_status st = linear(m, b.gate, h, gate, B)) return st;
+            if (mi355x_status st = linear(m, b.up, h, up, B)) return st;
+            LLM_HIP(swiglu(gate, up, sw, B, c.hidden, c.hidden, m.stream), "swiglu");
+        }
         if (mi355x_status st = convert_for(m, sw, B, c.hidden, {&b.down}, done)) return st;
-        if (mi355x_status st = linear(m, b.down, sw, o, B)) return st;
-        LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+        if (act_class(b.down, B) != kActNone) {
+            if (mi355x_status st = linear(m, b.down, sw, x, B, x)) return st;
+        } else {
+            if (mi355x_status st = linear(m, b.down, sw, o, B)) return st;
+            LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
+        }
     }
     return MI355X_OK;
 }
@@ -592,6 +632,34 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down})
             if (act_class(*w) != kActQ4) m->fast = false;
     }
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m->blocks[i];
+        b.qkv.buf.release();
+        b.gate_up.buf.release();
+        if (m->fast) continue;
+        auto fuse = [&](std::initializer_list<const Weight*> parts, Weight& into) -> mi355x_status {
+            const Weight* first = *parts.begin();
+            size_t total = 0;
+            int64_t n = 0;
+            for (const Weight* p : parts) {
+                // a part that is not a multiple of 16 bytes long would leave the next one misaligned for the kernels' wide loads
+                if (!is_quantized(p->dtype) || p->dtype != first->dtype || p->k != first->k || p->buf.bytes % 16) return MI355X_OK;
+                total += p->buf.bytes;
+                n += p->n;
+            }
+            LLM_HIP(into.buf.alloc(total), "hipMalloc(fused weights)");
+            size_t off = 0;
+            for (const Weight* p : parts) {
+                LLM_HIP(hipMemcpy((uint8_t*)into.buf.p + off, p->buf.p, p->buf.bytes, hipMemcpyDeviceToDevice), "hipMemcpy(fused weights)");
+                off += p->buf.bytes;
+            }
+            into.dtype = first->dtype; into.n = n; into.k = first->k;
+            return MI355X_OK;
+        };
+        if (mi355x_status st = fuse({&b.q, &b.k, &b.v}, b.qkv)) return st;
+        if (mi355x_status st = fuse({&b.gate, &b.up}, b.gate_up)) return st;
+    }
+    LLM_HIP(m->gu.alloc((size_t)c.batch * 2 * c.hidden * 4), "hipMalloc");
     m->ready = true;
     return MI355X_OK;
 }

@@ -140,8 +140,8 @@ __device__ __forceinline__ int i16_at(const uint16_t* p, int i) { return (int)(i
 
 // qdotQ4KGo (backend/cpu/qmatmul.go:148-172): lane (sb, j) takes the 64
 // weights of nibble group j of super-block sb.
-__global__ __launch_bounds__(256) void qgemv_q4k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                        float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+__global__ __launch_bounds__(256) void qgemv_q4k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
+                                                              const float* resid, int N, int nsb, int64_t act_row_bytes) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
     const uint8_t* arow = act + (int64_t)blockIdx.y * act_row_bytes;
@@ -187,13 +187,17 @@ __global__ __launch_bounds__(256) void qgemv_q4k_plain_kernel(const uint8_t* __r
         acc = add_in_order<4>(acc, t);
         accm = add_in_order<4>(accm, u);
     }
-    if (lane == 0) y[(int64_t)blockIdx.y * N + row] = acc - accm;
+    if (lane == 0) {
+        const int64_t at = (int64_t)blockIdx.y * N + row;
+        const float v = acc - accm;
+        y[at] = resid ? v + resid[at] : v;
+    }
 }
 
 // qdotQ6KGo (backend/cpu/qmatmul.go:180-200): lane (sb, n, k) takes the 32
 // weights of quarter k of half n of super-block sb, groups 8n+2k and 8n+2k+1.
-__global__ __launch_bounds__(256) void qgemv_q6k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                        float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+__global__ __launch_bounds__(256) void qgemv_q6k_plain_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
+                                                              const float* resid, int N, int nsb, int64_t act_row_bytes) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= N) return;
     const uint8_t* arow = act + (int64_t)blockIdx.y * act_row_bytes;
@@ -231,7 +235,10 @@ __global__ __launch_bounds__(256) void qgemv_q6k_plain_kernel(const uint8_t* __r
         }
         acc = add_in_order<8>(acc, t);
     }
-    if (lane == 0) y[(int64_t)blockIdx.y * N + row] = acc;
+    if (lane == 0) {
+        const int64_t at = (int64_t)blockIdx.y * N + row;
+        y[at] = resid ? acc + resid[at] : acc;
+    }
 }
 
 // ---- the LDS kernels ----------------------------------------------------------
@@ -264,8 +271,8 @@ struct Q4KTile {
 // 4g+h, 4g+2+h, 4g+8+h, 4g+10+h of the super-block (h = j%2); the sums kept
 // with x are per chunk.
 template <int R>
-__global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                               float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+__global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
+                                                               const float* resid, int N, int nsb, int64_t act_row_bytes) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -343,7 +350,11 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __
     }
 #pragma unroll
     for (int r = 0; r < R; r++)
-        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = acc[r] - accm[r];
+        if (lane == 0 && row0 + r < N) {
+            const int64_t at = (int64_t)blockIdx.y * N + row0 + r;
+            const float v = acc[r] - accm[r];
+            y[at] = resid ? v + resid[at] : v;
+        }
 }
 
 // Sixteen bytes at a 2-byte aligned address as five aligned dwords; take(i)
@@ -376,8 +387,8 @@ struct Q6KTile {
 // 32n+16(c%2).. of qh holding their upper two bits at bit 2(c/2) and
 // 2(c/2)+4; Q6_K's scales are per chunk.
 template <int R>
-__global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                               float* __restrict__ y, int N, int nsb, int64_t act_row_bytes) {
+__global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
+                                                               const float* resid, int N, int nsb, int64_t act_row_bytes) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -452,7 +463,10 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
     }
 #pragma unroll
     for (int r = 0; r < R; r++)
-        if (lane == 0 && row0 + r < N) y[(int64_t)blockIdx.y * N + row0 + r] = acc[r];
+        if (lane == 0 && row0 + r < N) {
+            const int64_t at = (int64_t)blockIdx.y * N + row0 + r;
+            y[at] = resid ? acc[r] + resid[at] : acc[r];
+        }
 }
 
 // [0] rows per wavefront (0: by shape). [1] 1: always the kernels without LDS, 2: never the
@@ -476,17 +490,17 @@ static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st)
     }
     if (dt == kQ4_K)
         hipLaunchKernelGGL(qgemv_q4k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     else
         hipLaunchKernelGGL(qgemv_q6k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     return hipGetLastError();
 }
 
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     int nsb = (int)(a.K / 256);
     // From a few rows of x on, the matrix cores (whose results are the CPU's bit for bit).
-    if ((g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && qgemm_kquant_pays(dt, a))) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
+    if (!a.resid && (g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && qgemm_kquant_pays(dt, a))) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
     // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.
     // Q6_K's 210-byte blocks are read as aligned dwords around a 2-byte aligned start.
     const bool lds_ok = kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;
@@ -499,10 +513,10 @@ hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     dim3 grid((unsigned)((a.N + waves - 1) / waves), (unsigned)a.M);
     if (dt == kQ4_K)
         hipLaunchKernelGGL(qgemv_q4k_plain_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     else
         hipLaunchKernelGGL(qgemv_q6k_plain_kernel, grid, dim3(64 * waves), 0, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     return hipGetLastError();
 }
 

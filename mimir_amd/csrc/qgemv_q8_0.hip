@@ -114,9 +114,8 @@ __device__ __forceinline__ void q8_block(const uint32_t w[8], const u32x4 xa, co
 // CONVERT: act is float32 x (rows act_row_bytes bytes apart) and every workgroup rounds its row to
 // int8 for itself (few rows of x: a launch saved); otherwise act holds rows converted beforehand.
 template <int R, bool ALIGNED, bool CONVERT>
-__global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                         float* __restrict__ y, int N, int nb, int64_t act_row_bytes,
-                                                         int rows_per_wg) {
+__global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
+                                                         const float* resid, int N, int nb, int64_t act_row_bytes, int rows_per_wg) {
     extern __shared__ u32x4 lds_q8[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
@@ -226,7 +225,10 @@ __global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restri
         for (int r = 0; r < R; r++) {
             float a0 = wave_sum(acc[r][0]), a1 = wave_sum(acc[r][1]), a2 = wave_sum(acc[r][2]), a3 = wave_sum(acc[r][3]);
             float s02 = a0 + a2, s13 = a1 + a3;
-            if (lane == 0 && row0 + r < N) yr[row0 + r] = s02 + s13;
+            if (lane == 0 && row0 + r < N) {
+                const float v = s02 + s13;
+                yr[row0 + r] = resid ? v + resid[(int64_t)m * N + row0 + r] : v;
+            }
         }
     }
 }
@@ -240,10 +242,10 @@ static hipError_t launch_q8(const QGemvArgs& a, int waves, hipStream_t st) {
     size_t act_bytes = q8_act_bytes(a.K);
     if (a.act)
         hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED, false>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
-                           (const uint8_t*)a.act, a.y, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
+                           (const uint8_t*)a.act, a.y, a.resid, (int)a.N, (int)(a.K / 32), (int64_t)act_bytes, rows_per_wg);
     else  // float32 x, converted by every workgroup
         hipLaunchKernelGGL((qgemv_q8_0_kernel<R, ALIGNED, true>), grid, dim3(64 * waves), act_bytes, st, (const uint8_t*)a.W,
-                           (const uint8_t*)a.x, a.y, (int)a.N, (int)(a.K / 32), a.x_row_stride * 4, rows_per_wg);
+                           (const uint8_t*)a.x, a.y, a.resid, (int)a.N, (int)(a.K / 32), a.x_row_stride * 4, rows_per_wg);
     return hipGetLastError();
 }
 
