@@ -94,6 +94,10 @@ hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // (kq_convert_act, kq_act_bytes(K) bytes per row), integer dot products.
 size_t kq_act_bytes(int64_t K);
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+// RMSNorm then conversion, and SiLU(g) * u then conversion, each in one launch and with the separate
+// kernels' arithmetic (d and n multiples of 256; x, w, g, u 16-byte aligned).
+hipError_t rmsnorm_kq_act(const float* x, const float* w, void* act, int64_t rows, int64_t d, double eps, hipStream_t st);
+hipError_t swiglu_kq_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 // The same from bfloat16 rows (8-byte aligned, a multiple of 4 elements apart).
 hipError_t kq_convert_act_bf16(const void* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);

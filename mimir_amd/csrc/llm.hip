@@ -378,8 +378,17 @@ static mi355x_status step_any(Model& m) {
     if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
-        LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "attn_norm");
-        if (b.qkv.set()) {  // one product into [B, q | k | v]
+        if (b.qkv.set() && act_class(b.qkv, B) == kActKQ) {  // norm and conversion in one launch, one product into [B, q | k | v]
+            LLM_HIP(rmsnorm_kq_act(x, b.attn_norm.buf.as<float>(), m.act[kActKQ].p, B, c.embed, c.eps, m.stream), "attn_norm");
+            if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
+        } else {
+            LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "attn_norm");
+        }
+        if (b.qkv.set() && act_class(b.qkv, B) == kActKQ) {
+            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+            at.q = qkv; at.q_strides[0] = qd + 2 * kvd;
+        } else if (b.qkv.set()) {  // one product into [B, q | k | v]
             if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.qkv}, done)) return st;
             if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
             LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
@@ -404,18 +413,28 @@ static mi355x_status step_any(Model& m) {
             if (mi355x_status st = linear(m, b.o, a, o, B)) return st;
             LLM_HIP(add(x, o, x, B * c.embed, m.stream), "residual");
         }
-        LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "ffn_norm");
-        if (b.gate_up.set()) {  // one product into [B, gate | up]
+        const bool down_kq = act_class(b.down, B) == kActKQ;  // then SwiGLU leaves its result converted
+        if (b.gate_up.set() && act_class(b.gate_up, B) == kActKQ) {
+            LLM_HIP(rmsnorm_kq_act(x, b.ffn_norm.buf.as<float>(), m.act[kActKQ].p, B, c.embed, c.eps, m.stream), "ffn_norm");
+            if (mi355x_status st = linear(m, b.gate_up, h, gu, B)) return st;
+            if (down_kq) LLM_HIP(swiglu_kq_act(gu, gu + c.hidden, m.act[kActKQ].p, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+            else LLM_HIP(swiglu(gu, gu + c.hidden, sw, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+        } else if (b.gate_up.set()) {  // one product into [B, gate | up]
+            LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "ffn_norm");
             if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate_up}, done)) return st;
             if (mi355x_status st = linear(m, b.gate_up, h, gu, B)) return st;
-            LLM_HIP(swiglu(gu, gu + c.hidden, sw, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+            if (down_kq) LLM_HIP(swiglu_kq_act(gu, gu + c.hidden, m.act[kActKQ].p, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+            else LLM_HIP(swiglu(gu, gu + c.hidden, sw, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
         } else {
+            LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "ffn_norm");
             if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.gate, &b.up}, done)) return st;
             if (mi355x_status st = linear(m, b.gate, h, gate, B)) return st;
             if (mi355x_status st = linear(m, b.up, h, up, B)) return st;
-            LLM_HIP(swiglu(gate, up, sw, B, c.hidden, c.hidden, m.stream), "swiglu");
+            if (down_kq) LLM_HIP(swiglu_kq_act(gate, up, m.act[kActKQ].p, B, c.hidden, c.hidden, m.stream), "swiglu");
+            else LLM_HIP(swiglu(gate, up, sw, B, c.hidden, c.hidden, m.stream), "swiglu");
         }
-        if (mi355x_status st = convert_for(m, sw, B, c.hidden, {&b.down}, done)) return st;
+        if (!down_kq)
+            if (mi355x_status st = convert_for(m, sw, B, c.hidden, {&b.down}, done)) return st;
         if (act_class(b.down, B) != kActNone) {
             if (mi355x_status st = linear(m, b.down, sw, x, B, x)) return st;
         } else {

@@ -57,28 +57,11 @@ __device__ __forceinline__ float add_in_order(float acc, float term) {
     return acc;
 }
 
-// quantizeRow for super-blocks of 256 with sums: one wavefront per
-// super-block, lane i taking values 4i..4i+3.
-template <bool BF16>  // x float32, or bfloat16 (widened exactly, as the cast in front of the product does: tensor/quant.go:45-48)
-__global__ __launch_bounds__(64) void kq_convert_act_kernel(const void* __restrict__ xv, int64_t x_row_stride, int nsb,
-                                                            uint8_t* __restrict__ act, int64_t act_row_bytes) {
-    const int sb = blockIdx.x, lane = threadIdx.x;
-    const int64_t at = (int64_t)blockIdx.y * x_row_stride + 256 * (int64_t)sb + 4 * lane;
-    uint8_t* row = act + (int64_t)blockIdx.y * act_row_bytes;
+// quantizeRow for one super-block of 256 with its sums: one wavefront, lane i holding values 4i..4i+3.
+__device__ __forceinline__ void kq_convert_superblock(const f32x4 v, int sb, int lane, int nsb, uint8_t* __restrict__ row) {
     uint32_t* q = (uint32_t*)row + (int64_t)sb * 64;
     uint16_t* sums = (uint16_t*)(row + (int64_t)nsb * 256) + sb * 16;
     float* dscale = (float*)(row + (int64_t)nsb * 288);
-    f32x4 v;
-    if (BF16) {
-        u32x2 h;
-        __builtin_memcpy(&h, (const uint16_t*)xv + at, 8);
-        v[0] = __builtin_bit_cast(float, h[0] << 16);
-        v[1] = __builtin_bit_cast(float, h[0] & 0xffff0000u);
-        v[2] = __builtin_bit_cast(float, h[1] << 16);
-        v[3] = __builtin_bit_cast(float, h[1] & 0xffff0000u);
-    } else {
-        __builtin_memcpy(&v, (const float*)xv + at, 16);
-    }
     float amax = 0.f;
     bool finite = true;
 #pragma unroll
@@ -109,6 +92,94 @@ __global__ __launch_bounds__(64) void kq_convert_act_kernel(const void* __restri
     int s16 = dpp_i32_quad_sum(local);  // 16 quants = 4 consecutive lanes
     if ((lane & 3) == 0) sums[lane >> 2] = (uint16_t)(int16_t)s16;
     if (lane == 0) dscale[sb] = d;
+}
+
+// One wavefront per super-block.
+template <bool BF16>  // x float32, or bfloat16 (widened exactly, as the cast in front of the product does: tensor/quant.go:45-48)
+__global__ __launch_bounds__(64) void kq_convert_act_kernel(const void* __restrict__ xv, int64_t x_row_stride, int nsb,
+                                                            uint8_t* __restrict__ act, int64_t act_row_bytes) {
+    const int sb = blockIdx.x, lane = threadIdx.x;
+    const int64_t at = (int64_t)blockIdx.y * x_row_stride + 256 * (int64_t)sb + 4 * lane;
+    f32x4 v;
+    if (BF16) {
+        u32x2 h;
+        __builtin_memcpy(&h, (const uint16_t*)xv + at, 8);
+        v[0] = __builtin_bit_cast(float, h[0] << 16);
+        v[1] = __builtin_bit_cast(float, h[0] & 0xffff0000u);
+        v[2] = __builtin_bit_cast(float, h[1] << 16);
+        v[3] = __builtin_bit_cast(float, h[1] & 0xffff0000u);
+    } else {
+        __builtin_memcpy(&v, (const float*)xv + at, 16);
+    }
+    kq_convert_superblock(v, sb, lane, nsb, act + (int64_t)blockIdx.y * act_row_bytes);
+}
+
+// RMSNorm (rmsnorm_kernel's arithmetic, operation for operation: nn/transformer.go:50-61) and the
+// conversion of its result in one launch: a workgroup of four wavefronts per row sums the squares as
+// rmsnorm_kernel does, then each wavefront converts every fourth super-block.
+__global__ __launch_bounds__(256) void rmsnorm_kq_act_kernel(const float* __restrict__ x, const float* __restrict__ w, int d, float inv_d,
+                                                             float eps, uint8_t* __restrict__ act, int64_t act_row_bytes) {
+    __shared__ float part[4];
+    const float* xr = x + (int64_t)blockIdx.x * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = xr[i];
+        float sq = v * v;
+        ss = ss + sq;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = (part[0] + part[1]) + (part[2] + part[3]);
+    float ms = total * inv_d;
+    float scale = 1.0f / __builtin_sqrtf(ms + eps);
+    const int lane = threadIdx.x & 63, nsb = d >> 8;
+    for (int sb = threadIdx.x >> 6; sb < nsb; sb += 4) {
+        f32x4 v, wv;
+        __builtin_memcpy(&v, xr + 256 * sb + 4 * lane, 16);
+        __builtin_memcpy(&wv, w + 256 * sb + 4 * lane, 16);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float t = v[k] * scale;
+            v[k] = t * wv[k];
+        }
+        kq_convert_superblock(v, sb, lane, nsb, act + (int64_t)blockIdx.x * act_row_bytes);
+    }
+}
+
+hipError_t rmsnorm_kq_act(const float* x, const float* w, void* act, int64_t rows, int64_t d, double eps, hipStream_t st) {
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(rmsnorm_kq_act_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, w, (int)d, (float)(1.0 / (double)d), (float)eps,
+                       (uint8_t*)act, (int64_t)kq_act_bytes(d));
+    return hipGetLastError();
+}
+
+// SiLU(g) * u (swiglu_kernel's arithmetic: llm/model.go:446-448) and the conversion of the result in one
+// launch, one wavefront per super-block; rows of g and u are `stride` floats apart.
+__global__ __launch_bounds__(64) void swiglu_kq_act_kernel(const float* __restrict__ g, const float* __restrict__ u, int64_t stride, int nsb,
+                                                           uint8_t* __restrict__ act, int64_t act_row_bytes) {
+    const int sb = blockIdx.x, lane = threadIdx.x;
+    const int64_t at = (int64_t)blockIdx.y * stride + 256 * (int64_t)sb + 4 * lane;
+    const float nl2e = (float)(-1.4426950408889634);
+    f32x4 gv, uv, v;
+    __builtin_memcpy(&gv, g + at, 16);
+    __builtin_memcpy(&uv, u + at, 16);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float e = __builtin_exp2f(gv[k] * nl2e);
+        float sg = 1.0f / (1.0f + e);
+        float a = gv[k] * sg;
+        v[k] = a * uv[k];
+    }
+    kq_convert_superblock(v, sb, lane, nsb, act + (int64_t)blockIdx.y * act_row_bytes);
+}
+
+hipError_t swiglu_kq_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st) {
+    if (rows == 0) return hipSuccess;
+    int nsb = (int)(n / 256);
+    hipLaunchKernelGGL(swiglu_kq_act_kernel, dim3((unsigned)nsb, (unsigned)rows), dim3(64), 0, st, g, u, stride, nsb, (uint8_t*)act,
+                       (int64_t)kq_act_bytes(n));
+    return hipGetLastError();
 }
 
 hipError_t kq_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {

@@ -235,11 +235,25 @@ class Model:
 # ---- synthetic models in the shapes the benchmark configurations name -----
 
 def _q_blocks(rng, dt, n, k):
+    """Random blocks of dtype dt for an [n, k] weight: quants uniform over their range, binary16 scales
+    |N(0, 0.02)| (divided by 32 for the K-quants, whose sub-block scales multiply them)."""
+    def half(count, scale):
+        d = np.abs(rng.normal(0, scale, count)).astype(np.float32).astype(np.float16).view(np.uint16)
+        return np.stack([d & 0xff, d >> 8], 1).astype(np.uint8)
+
+    if dt in (O.Q4_K, O.Q6_K):
+        nb = n * k // 256
+        bb = 144 if dt == O.Q4_K else 210
+        b = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
+        if dt == O.Q4_K:
+            b[:, 0:2], b[:, 2:4] = half(nb, 0.02 / 32), half(nb, 0.02 / 32)
+        else:
+            b[:, 208:210] = half(nb, 0.02 / 32)
+        return Weight(dt, n, k, b.reshape(-1))
     nb = n * k // 32
     bb = 18 if dt == O.Q4_0 else 34
     b = np.empty((nb, bb), np.uint8)
-    d = np.abs(rng.normal(0, 0.02, nb)).astype(np.float32).astype(np.float16).view(np.uint16)
-    b[:, 0], b[:, 1] = d & 0xff, d >> 8
+    b[:, 0:2] = half(nb, 0.02)
     if dt == O.Q4_0:
         b[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
     else:

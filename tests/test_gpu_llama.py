@@ -96,7 +96,7 @@ def _small_q4_config(batch, cache):
 
 
 def _upload_synthetic(m: Llama, om: OL.Model):
-    dt = {O.Q4_0: capi.Q4_0, O.Q8_0: capi.Q8_0}
+    dt = {O.Q4_0: capi.Q4_0, O.Q8_0: capi.Q8_0, O.Q4_K: capi.Q4_K, O.Q6_K: capi.Q6_K}
     m.set_tensor("token_embd.weight", dt[om.embed.dtype], om.embed.data, om.embed.n * om.embed.k)
     m.set_tensor("output.weight", dt[om.output.dtype], om.output.data, om.output.n * om.output.k)
     m.set_tensor("output_norm.weight", capi.F32, om.norm, om.norm.size)
@@ -251,3 +251,38 @@ def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
             assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
             break
     assert np.array_equal(runs[1], runs[2]) and np.array_equal(runs[0], runs[2])
+
+
+@pytest.mark.parametrize("linear_dt,batch", [(O.Q4_K, 1), (O.Q6_K, 2), (O.Q8_0, 1)])
+def test_k_quant_and_q8_0_models_decode_from_a_graph(linear_dt, batch):
+    """Models whose linears are not Q4_0 take the generic decoding step: q|k|v and gate|up as one product
+    each over weights kept together, norm and SwiGLU with the int8 conversion in the same launch (K-quants),
+    residuals in the products' epilogues, the position on the device, the whole step replayed as a graph. It
+    must choose the tokens of the per-operator path (position from the host) and of the oracle."""
+    lib = gpu.lib()
+    c = capi.LlamaConfig()
+    c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = 512, 1024, 2, 4, 2, 64, 64, 301
+    c.context, c.interleaved, c.cache_dtype, c.batch = 64, 1, capi.F16, batch
+    c.rope_base, c.rope_scale, c.eps = 10000.0, 1.0, 1e-5
+    om = OL.synthetic(_oracle_config(c), seed=7, linear_dt=linear_dt)
+    m = Llama(c)
+    _upload_synthetic(m, om)
+    m.finalize(16)
+    prompts = np.random.default_rng(11).integers(0, c.vocab, (batch, 6))
+    runs = {}
+    try:
+        for mode in (2, 1, 0, 0):
+            gpu.say(f"generate dtype {linear_dt}, step mode {mode}, batch {batch}")
+            capi.check(lib.mi355x_tune(b"llama.step", mode))
+            m.reset()
+            first, _ = m.generate(prompts, 20)
+            more, _ = m.generate(first[:, -1:], 9)  # a second call continues the caches (and replays the graph)
+            runs.setdefault(mode, []).append(np.concatenate([first, more], 1))
+    finally:
+        capi.check(lib.mi355x_tune(b"llama.step", 0))
+    want, margins = om.generate(prompts[0].tolist(), 20, capacity=c.context, cache_dtype=O.F16)
+    for i, (a, w) in enumerate(zip(runs[2][0][0, :20].tolist(), want)):
+        if a != w:
+            assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
+            break
+    assert np.array_equal(runs[1][0], runs[2][0]) and np.array_equal(runs[0][0], runs[2][0]) and np.array_equal(runs[0][1], runs[2][0])
