@@ -191,10 +191,10 @@ def q_blocks(rng, kind, n_elems):
 
 
 def build_llama(capi, layers=32, batch=1, context=1024, max_tokens=512, seed=0, embed=4096, hidden=14336, heads=32, kv_heads=8,
-                head_dim=128, vocab=128256):
-    """A random-init Llama-3-8B-shaped decoder on the device: Q4_0 linears, Q8_0
-    embeddings and output, norm weights N(1, 0.02), binary16 KV cache. Each
-    tensor's generator is seeded from its name."""
+                head_dim=128, vocab=128256, linear="q4_0"):
+    """A random-init Llama-3-8B-shaped decoder on the device: Q4_0 linears (or
+    Q4_K, Q6_K with `linear`), Q8_0 embeddings and output, norm weights
+    N(1, 0.02), binary16 KV cache. Each tensor's generator is seeded from its name."""
     from mimir_amd.llama import Llama
     c = capi.LlamaConfig()
     c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = embed, hidden, layers, heads, kv_heads, head_dim, head_dim, vocab
@@ -212,22 +212,26 @@ def build_llama(capi, layers=32, batch=1, context=1024, max_tokens=512, seed=0, 
             m.set_tensor(p + leaf + ".weight", capi.F32, rng(p + leaf + ".weight").normal(1, 0.02, embed).astype(np.float32), embed)
         for leaf, n, k in (("attn_q", qd, embed), ("attn_k", kvd, embed), ("attn_v", kvd, embed), ("attn_output", embed, qd),
                            ("ffn_gate", hidden, embed), ("ffn_up", hidden, embed), ("ffn_down", embed, hidden)):
-            m.set_tensor(p + leaf + ".weight", capi.Q4_0, q_blocks(rng(p + leaf + ".weight"), "q4_0", n * k), n * k)
+            if linear == "q4_0":
+                m.set_tensor(p + leaf + ".weight", capi.Q4_0, q_blocks(rng(p + leaf + ".weight"), "q4_0", n * k), n * k)
+            else:
+                dt, bb = (capi.Q4_K, 144) if linear == "q4_K" else (capi.Q6_K, 210)
+                m.set_tensor(p + leaf + ".weight", dt, bench_blocks_kquant(rng(p + leaf + ".weight"), bb, n * k), n * k)
     m.finalize(max_tokens)
     return m
 
 
-def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0):
+def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear="q4_0"):
     """Whole-model greedy decoding: a prompt of uniform-random token ids, then
     `new` tokens a sequence. Returns tokens/s of the decoding steps. With
     check, the first `check` tokens of sequence 0 are compared with the CPU
     oracle's greedy decoding of the same model and prompt."""
     t0 = time.perf_counter()
-    m = build_llama(capi, layers=layers, batch=batch, context=prompt + new, max_tokens=prompt)
+    m = build_llama(capi, layers=layers, batch=batch, context=prompt + new, max_tokens=prompt, linear=linear)
     build_s = time.perf_counter() - t0
     toks = np.random.default_rng(0).integers(0, m.config.vocab, (batch, prompt))
     out, (t_prompt, t_decode) = m.generate(toks, new)
-    per_tok_bytes = layers * 218103808 * 0.5625 + 128256 * 4096 * 1.0625
+    per_tok_bytes = layers * 218103808 * {"q4_0": 0.5625, "q4_K": 0.5625, "q6_K": 0.8203125}[linear] + 128256 * 4096 * 1.0625
     verdict = {}
     if check:
         import oracle as O
@@ -241,7 +245,7 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0):
         first = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), None)
         verdict = {"greedy_checked": check, "greedy_identical": sum(a == b for a, b in zip(got, want)), "first_mismatch": first,
                    "oracle_min_margin": round(min(margins), 4)}
-    return {**verdict,"layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
+    return {**verdict, "linear_dtype": linear, "layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
             "decode_tok_per_s": round(batch * (new - 1) / t_decode, 1), "ms_per_step": round(t_decode / (new - 1) * 1e3, 4),
             "weight_GBps": round(per_tok_bytes / (t_decode / (new - 1)) / 1e9, 1), "build_s": round(build_s, 1),
             "first_tokens": out[0, :8].tolist()}
@@ -372,6 +376,8 @@ def main():
                     help="compare the first N greedy tokens with the CPU oracle's (minutes of CPU time for the 512-token prompt)")
     ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--decode-batch", type=int, default=1)
+    ap.add_argument("--decode-linear", choices=("q4_0", "q4_K", "q6_K"), default="q4_0",
+                    help="block dtype of the decoder's linear weights (the oracle check is for q4_0)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives or sharding are built)")
@@ -445,7 +451,8 @@ def main():
     if args.gemm:
         out["prefill_gemm"] = gemm_bench(lib, capi, torch)
     if not args.no_decode:
-        out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check)
+        out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check if args.decode_linear == "q4_0" else 0,
+                                     linear=args.decode_linear)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n, k, seconds=10.0)
     print(json.dumps(out), flush=True)

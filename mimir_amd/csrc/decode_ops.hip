@@ -23,21 +23,26 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     __shared__ float part[4];
     const float* xr = x + (int64_t)blockIdx.x * d;
     float* yr = y + (int64_t)blockIdx.x * d;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = xr[i];
-        float sq = v * v;
-        ss = ss + sq;
-    }
-    ss = wave_sum(ss);
+    float ss = wave_sum(strided_sum_squares(xr, d, threadIdx.x));
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     float total = (part[0] + part[1]) + (part[2] + part[3]);
     float ms = total * inv_d;
     float scale = 1.0f / __builtin_sqrtf(ms + eps);
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = xr[i] * scale;
-        yr[i] = w ? v * w[i] : v;
+    for (int i0 = threadIdx.x; i0 < d; i0 += 8 * 256) {  // loads in batches, as above
+        float xv[8], wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int i = i0 + 256 * u;
+            xv[u] = i < d ? xr[i] : 0.f;
+            wv[u] = w && i < d ? w[i] : 1.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int i = i0 + 256 * u;
+            float v = xv[u] * scale;
+            if (i < d) yr[i] = w ? v * wv[u] : v;
+        }
     }
 }
 

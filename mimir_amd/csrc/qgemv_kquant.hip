@@ -115,42 +115,39 @@ __global__ __launch_bounds__(64) void kq_convert_act_kernel(const void* __restri
 }
 
 // RMSNorm (rmsnorm_kernel's arithmetic, operation for operation: nn/transformer.go:50-61) and the
-// conversion of its result in one launch: a workgroup of four wavefronts per row sums the squares as
-// rmsnorm_kernel does, then each wavefront converts every fourth super-block.
+// conversion of its result in one launch: a workgroup of four wavefronts sums the row's squares as
+// rmsnorm_kernel does (each workgroup of a row for itself), then each wavefront converts one super-block.
 __global__ __launch_bounds__(256) void rmsnorm_kq_act_kernel(const float* __restrict__ x, const float* __restrict__ w, int d, float inv_d,
                                                              float eps, uint8_t* __restrict__ act, int64_t act_row_bytes) {
     __shared__ float part[4];
-    const float* xr = x + (int64_t)blockIdx.x * d;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = xr[i];
-        float sq = v * v;
-        ss = ss + sq;
+    const float* xr = x + (int64_t)blockIdx.y * d;
+    const int lane = threadIdx.x & 63, nsb = d >> 8;
+    const int sb = blockIdx.x * 4 + (threadIdx.x >> 6);
+    f32x4 v = {0.f, 0.f, 0.f, 0.f}, wv = {0.f, 0.f, 0.f, 0.f};
+    if (sb < nsb) {  // requested with the loads of the sum
+        __builtin_memcpy(&v, xr + 256 * sb + 4 * lane, 16);
+        __builtin_memcpy(&wv, w + 256 * sb + 4 * lane, 16);
     }
-    ss = wave_sum(ss);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    float ss = wave_sum(strided_sum_squares(xr, d, threadIdx.x));
+    if (lane == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     float total = (part[0] + part[1]) + (part[2] + part[3]);
     float ms = total * inv_d;
     float scale = 1.0f / __builtin_sqrtf(ms + eps);
-    const int lane = threadIdx.x & 63, nsb = d >> 8;
-    for (int sb = threadIdx.x >> 6; sb < nsb; sb += 4) {
-        f32x4 v, wv;
-        __builtin_memcpy(&v, xr + 256 * sb + 4 * lane, 16);
-        __builtin_memcpy(&wv, w + 256 * sb + 4 * lane, 16);
+    if (sb < nsb) {
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             float t = v[k] * scale;
             v[k] = t * wv[k];
         }
-        kq_convert_superblock(v, sb, lane, nsb, act + (int64_t)blockIdx.x * act_row_bytes);
+        kq_convert_superblock(v, sb, lane, nsb, act + (int64_t)blockIdx.y * act_row_bytes);
     }
 }
 
 hipError_t rmsnorm_kq_act(const float* x, const float* w, void* act, int64_t rows, int64_t d, double eps, hipStream_t st) {
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(rmsnorm_kq_act_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, w, (int)d, (float)(1.0 / (double)d), (float)eps,
-                       (uint8_t*)act, (int64_t)kq_act_bytes(d));
+    hipLaunchKernelGGL(rmsnorm_kq_act_kernel, dim3((unsigned)((d / 256 + 3) / 4), (unsigned)rows), dim3(256), 0, st, x, w, (int)d,
+                       (float)(1.0 / (double)d), (float)eps, (uint8_t*)act, (int64_t)kq_act_bytes(d));
     return hipGetLastError();
 }
 
