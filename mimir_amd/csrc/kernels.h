@@ -78,6 +78,9 @@ struct Q4RopeTail {
 };
 hipError_t qgemv_q4_0_act_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
                                    const Q4RopeTail& rope, const Q4NormHead& norm, const int* tune, hipStream_t st);
+// The same tail behind a Q4_K or Q6_K product (qgemv_kquant_rope_ok says whether the shape qualifies).
+bool qgemv_kquant_rope_ok(int dt, const QGemvArgs& a);
+hipError_t qgemv_kquant_act_rope(int dt, const QGemvArgs& a, const Q4RopeTail& rope, hipStream_t st);
 hipError_t qgemv_q4_0_act_swiglu(const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K,
                                  const int* tune, hipStream_t st);
 

@@ -378,21 +378,28 @@ static mi355x_status step_any(Model& m) {
     if (!one_launch) attention_plan(B, c.heads, c.kv_heads, 1, c.context, &at.chunk, &at.nsplit);
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
-        if (b.qkv.set() && act_class(b.qkv, B) == kActKQ) {  // norm and conversion in one launch, one product into [B, q | k | v]
+        const bool qkv_kq = b.qkv.set() && act_class(b.qkv, B) == kActKQ;
+        if (qkv_kq) {  // norm and conversion in one launch
             LLM_HIP(rmsnorm_kq_act(x, b.attn_norm.buf.as<float>(), m.act[kActKQ].p, B, c.embed, c.eps, m.stream), "attn_norm");
-            if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
         } else {
             LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, B, c.embed, c.eps, m.stream), "attn_norm");
+            if (b.qkv.set())
+                if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.qkv}, done)) return st;
         }
-        if (b.qkv.set() && act_class(b.qkv, B) == kActKQ) {
-            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
-                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
-            at.q = qkv; at.q_strides[0] = qd + 2 * kvd;
-        } else if (b.qkv.set()) {  // one product into [B, q | k | v]
-            if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.qkv}, done)) return st;
-            if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
-            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
-                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        if (b.qkv.set()) {  // one product into [B, q | k | v]
+            QGemvArgs qa{b.qkv.buf.p, nullptr, m.act[kActKQ].p, qkv, B, b.qkv.n, b.qkv.k, b.qkv.k, 0};
+            if (qkv_kq && c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0 && qgemv_kquant_rope_ok(b.qkv.dtype, qa)) {
+                Q4RopeTail tail;  // the rotation and the cache writes ride on the product
+                tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
+                tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
+                tail.cache_dt = c.cache_dtype; tail.H = c.heads; tail.HK = c.kv_heads; tail.dim = c.head_dim; tail.rope_dim = c.rope_dim;
+                tail.cap = c.context;
+                LLM_HIP(qgemv_kquant_act_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
+            } else {
+                if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
+                LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                                c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+            }
             at.q = qkv; at.q_strides[0] = qd + 2 * kvd;
         } else {
             if (mi355x_status st = convert_for(m, h, B, c.embed, {&b.q, &b.k, &b.v}, done)) return st;

@@ -20,6 +20,7 @@
 // for the LDS.
 #include "device_util.h"
 #include "kernels.h"
+#include "rope_tail.h"
 
 namespace mimir {
 
@@ -340,7 +341,8 @@ struct Q4KTile {
 // with x are per chunk.
 template <int R>
 __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
-                                                               const float* resid, int N, int nsb, int64_t act_row_bytes) {
+                                                               const float* resid, int N, int nsb, int64_t act_row_bytes, Q4RopeTail rope,
+                                                               int rope_on) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -416,6 +418,16 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __
             accm[r] = add_in_order<4>(accm[r], u);
         }
     }
+    if (rope_on) {  // R even: the wavefront's rows are pairs of features; rotation and cache writes as rope_kv does them
+        if (R >= 2) {
+            const int pos = *rope.pos;
+#pragma unroll
+            for (int r = 0; r + 1 < R; r += 2)
+                if (lane == 0 && row0 + r < N)
+                    q4_rope_store(rope, pos, blockIdx.y, row0 + r, acc[r] - accm[r], acc[r + 1] - accm[r + 1], y + (int64_t)blockIdx.y * N);
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++)
         if (lane == 0 && row0 + r < N) {
@@ -456,7 +468,8 @@ struct Q6KTile {
 // 2(c/2)+4; Q6_K's scales are per chunk.
 template <int R>
 __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
-                                                               const float* resid, int N, int nsb, int64_t act_row_bytes) {
+                                                               const float* resid, int N, int nsb, int64_t act_row_bytes, Q4RopeTail rope,
+                                                               int rope_on) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -529,6 +542,15 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
             acc[r] = add_in_order<8>(acc[r], t);
         }
     }
+    if (rope_on) {
+        if (R >= 2) {
+            const int pos = *rope.pos;
+#pragma unroll
+            for (int r = 0; r + 1 < R; r += 2)
+                if (lane == 0 && row0 + r < N) q4_rope_store(rope, pos, blockIdx.y, row0 + r, acc[r], acc[r + 1], y + (int64_t)blockIdx.y * N);
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++)
         if (lane == 0 && row0 + r < N) {
@@ -545,7 +567,7 @@ void set_kquant_tune(int which, int value) {
 }
 
 template <int R>
-static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st) {
+static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, const Q4RopeTail* rope, hipStream_t st) {
     static bool raised[2] = {false, false};
     const size_t lds = kq_lds_bytes(nsb);
     const int rows_per_wg = kKqThreads / 64 * R;
@@ -556,13 +578,26 @@ static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, hipStream_t st)
         if (e != hipSuccess) return e;
         raised[dt == kQ4_K] = true;
     }
+    const Q4RopeTail tail = rope ? *rope : Q4RopeTail{};
     if (dt == kQ4_K)
         hipLaunchKernelGGL(qgemv_q4k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K), tail, rope ? 1 : 0);
     else
         hipLaunchKernelGGL(qgemv_q6k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K), tail, rope ? 1 : 0);
     return hipGetLastError();
+}
+
+// Whether qgemv_kquant_act_rope takes the product: the kernels that own pairs of rows.
+bool qgemv_kquant_rope_ok(int dt, const QGemvArgs& a) {
+    const int nsb = (int)(a.K / 256);
+    return (dt == kQ4_K || dt == kQ6_K) && a.K % 256 == 0 && kq_lds_bytes(nsb) <= kKqMaxLds && ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0;
+}
+
+// The q|k|v product of a decoding step with the rotation and the cache writes as its tail: y receives
+// the rotated queries only (see Q4RopeTail; interleaved pairs, even widths).
+hipError_t qgemv_kquant_act_rope(int dt, const QGemvArgs& a, const Q4RopeTail& rope, hipStream_t st) {
+    return launch_kq<2>(dt, a, (int)(a.K / 256), &rope, st);
 }
 
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
@@ -575,7 +610,7 @@ hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     if (g_kq_tune[1] != 1 && lds_ok) {
         int R = g_kq_tune[0];
         if (R != 1 && R != 2 && R != 4) R = a.N * a.M >= 2048 ? 2 : 1;  // measured: see the sweep keys of mi355x_tune
-        return R == 4 ? launch_kq<4>(dt, a, nsb, st) : R == 2 ? launch_kq<2>(dt, a, nsb, st) : launch_kq<1>(dt, a, nsb, st);
+        return R == 4 ? launch_kq<4>(dt, a, nsb, nullptr, st) : R == 2 ? launch_kq<2>(dt, a, nsb, nullptr, st) : launch_kq<1>(dt, a, nsb, nullptr, st);
     }
     const int waves = 4;
     dim3 grid((unsigned)((a.N + waves - 1) / waves), (unsigned)a.M);

@@ -34,6 +34,7 @@
 #include "device_util.h"
 #include "kernels.h"
 #include "q4_act.h"
+#include "rope_tail.h"
 
 namespace mimir {
 
@@ -349,35 +350,6 @@ struct Q4Job {
     float norm_inv_d, norm_eps;
     int64_t x_row_stride;
 };
-
-// Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
-__device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int m, int row, float a, float b, float* yr) {
-    const int head = row / t.dim, f = row - head * t.dim;
-    float va = a, vb = b;
-    if (head < t.H + t.HK && f < t.rope_dim) {
-        const int half = t.rope_dim >> 1, i = f >> 1;
-        const float c = t.cosv[(int64_t)pos * half + i], sn = t.sinv[(int64_t)pos * half + i];
-        const float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;  // four products, then one subtraction and one addition
-        va = ac - bs;
-        vb = as + bc;
-    }
-    if (head < t.H) {
-        yr[row] = va;
-        yr[row + 1] = vb;
-        return;
-    }
-    const bool is_k = head < t.H + t.HK;
-    const int kh = is_k ? head - t.H : head - t.H - t.HK;
-    void* cache = is_k ? t.kcache : t.vcache;
-    const int64_t at = (((int64_t)m * t.HK + kh) * t.cap + pos) * t.dim + f;
-    if (t.cache_dt == kF32) {
-        ((float*)cache)[at] = va;
-        ((float*)cache)[at + 1] = vb;
-    } else {
-        ((uint16_t*)cache)[at] = f32_to_f16_bits(va);
-        ((uint16_t*)cache)[at + 1] = f32_to_f16_bits(vb);
-    }
-}
 
 constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
 static int g_q4_batch_off = 0;  // measurement aid: 1 keeps products of several rows of x on the one-row kernel, 2 puts all on the batch kernel

@@ -1,0 +1,39 @@
+// The rotation and cache writes of a decoding step as the tail of the product that computes q, k and v
+// (rope_kv's arithmetic): shared by the kernels whose wavefronts own pairs of output rows.
+#pragma once
+
+#include "device_util.h"
+#include "kernels.h"
+
+namespace mimir {
+
+// Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
+__device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int m, int row, float a, float b, float* yr) {
+    const int head = row / t.dim, f = row - head * t.dim;
+    float va = a, vb = b;
+    if (head < t.H + t.HK && f < t.rope_dim) {
+        const int half = t.rope_dim >> 1, i = f >> 1;
+        const float c = t.cosv[(int64_t)pos * half + i], sn = t.sinv[(int64_t)pos * half + i];
+        const float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;  // four products, then one subtraction and one addition
+        va = ac - bs;
+        vb = as + bc;
+    }
+    if (head < t.H) {
+        yr[row] = va;
+        yr[row + 1] = vb;
+        return;
+    }
+    const bool is_k = head < t.H + t.HK;
+    const int kh = is_k ? head - t.H : head - t.H - t.HK;
+    void* cache = is_k ? t.kcache : t.vcache;
+    const int64_t at = (((int64_t)m * t.HK + kh) * t.cap + pos) * t.dim + f;
+    if (t.cache_dt == kF32) {
+        ((float*)cache)[at] = va;
+        ((float*)cache)[at + 1] = vb;
+    } else {
+        ((uint16_t*)cache)[at] = f32_to_f16_bits(va);
+        ((uint16_t*)cache)[at + 1] = f32_to_f16_bits(vb);
+    }
+}
+
+}  // namespace mimir
