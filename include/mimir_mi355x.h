@@ -87,7 +87,7 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * reference takes for that file dtype (io/mim/dtype.go:118-123).
  * One entry point for every M, as OpQMatMul is one operation: by dtype and
  * shape the library runs row kernels (few rows of x; one launch for one row of
- * x by Q4_0 or a small Q8_0 matrix) or, from enough rows on, kernels on the
+ * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix) or, from enough rows on, kernels on the
  * int8 matrix cores (Q4_0, Q4_K, Q6_K); which one ran changes the results only
  * by the order of float32 additions (Q4_0, Q8_0) or not at all (Q4_K, Q6_K). */
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,

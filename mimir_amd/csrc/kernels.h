@@ -103,6 +103,7 @@ hipError_t rmsnorm_kq_act(const float* x, const float* w, void* act, int64_t row
 hipError_t swiglu_kq_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 // The same from bfloat16 rows (8-byte aligned, a multiple of 4 elements apart).
 hipError_t kq_convert_act_bf16(const void* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+// With a.act null and qgemv_kquant_rope_ok(dt, a): one launch from float32 a.x (16-byte aligned rows), rounded by every workgroup.
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st);
 // The same products for many rows of x on the matrix cores (qgemm_kquant.hip); qgemv_kquant_act
 // hands over to it where qgemm_kquant_pays says it is the faster of the two.

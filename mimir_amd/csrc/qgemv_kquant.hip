@@ -59,10 +59,8 @@ __device__ __forceinline__ float add_in_order(float acc, float term) {
 }
 
 // quantizeRow for one super-block of 256 with its sums: one wavefront, lane i holding values 4i..4i+3.
-__device__ __forceinline__ void kq_convert_superblock(const f32x4 v, int sb, int lane, int nsb, uint8_t* __restrict__ row) {
-    uint32_t* q = (uint32_t*)row + (int64_t)sb * 64;
-    uint16_t* sums = (uint16_t*)(row + (int64_t)nsb * 256) + sb * 16;
-    float* dscale = (float*)(row + (int64_t)nsb * 288);
+// q: the super-block's 64 dwords of quants; sums: its 16 sums; d: its scale.
+__device__ __forceinline__ void kq_convert_superblock_to(const f32x4 v, int lane, uint32_t* q, uint16_t* sums, float* d_out) {
     float amax = 0.f;
     bool finite = true;
 #pragma unroll
@@ -92,7 +90,13 @@ __device__ __forceinline__ void kq_convert_superblock(const f32x4 v, int sb, int
     q[lane] = packed;
     int s16 = dpp_i32_quad_sum(local);  // 16 quants = 4 consecutive lanes
     if ((lane & 3) == 0) sums[lane >> 2] = (uint16_t)(int16_t)s16;
-    if (lane == 0) dscale[sb] = d;
+    if (lane == 0) *d_out = d;
+}
+
+// Into a converted row in global memory (kq_act_bytes' layout).
+__device__ __forceinline__ void kq_convert_superblock(const f32x4 v, int sb, int lane, int nsb, uint8_t* __restrict__ row) {
+    kq_convert_superblock_to(v, lane, (uint32_t*)row + (int64_t)sb * 64, (uint16_t*)(row + (int64_t)nsb * 256) + sb * 16,
+                             (float*)(row + (int64_t)nsb * 288) + sb);
 }
 
 // One wavefront per super-block.
@@ -328,6 +332,28 @@ __device__ __forceinline__ void kq_stage_act(const uint8_t* __restrict__ arow, i
     for (int c = tid; c < nsb * 9; c += kKqThreads) dst[c] = tail[c];
 }
 
+// The same row from float32 x, rounded by the workgroup itself (quantizeRow, as kq_convert_act_kernel):
+// wavefront w takes super-blocks w, w + 4, ...
+__device__ __forceinline__ void kq_convert_into_lds(const float* __restrict__ xr, int nsb, uint8_t* lds, int tid) {
+    const int lane = tid & 63;
+    constexpr int kWaves = kKqThreads / 64, kBatch = 4;  // loads requested kBatch at a time: a loop of unknown length waits for each
+    for (int sb0 = tid >> 6; sb0 < nsb; sb0 += kWaves * kBatch) {
+        f32x4 v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int sb = min(sb0 + kWaves * j, nsb - 1);
+            __builtin_memcpy(&v[j], xr + 256 * sb + 4 * lane, 16);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int sb = sb0 + kWaves * j;
+            if (sb < nsb)
+                kq_convert_superblock_to(v[j], lane, (uint32_t*)(lds + sb * kKqStride), (uint16_t*)(lds + nsb * kKqStride) + sb * 16,
+                                         (float*)(lds + nsb * (kKqStride + 32)) + sb);
+        }
+    }
+}
+
 __device__ __forceinline__ u32x4 lds_u32x4(const uint8_t* p) { return *(const u32x4*)p; }
 
 struct Q4KTile {
@@ -342,7 +368,7 @@ struct Q4KTile {
 template <int R>
 __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
                                                                const float* resid, int N, int nsb, int64_t act_row_bytes, Q4RopeTail rope,
-                                                               int rope_on) {
+                                                               int rope_on, int x_is_f32) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -363,7 +389,9 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __
         }
     };
     fetch(0);
-    kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
+    // act: rows converted beforehand, or (x_is_f32) rows of float32 x, act_row_bytes apart, which the workgroup rounds itself
+    if (x_is_f32) kq_convert_into_lds((const float*)(act + (int64_t)blockIdx.y * act_row_bytes), nsb, kq_lds, tid);
+    else kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
     __syncthreads();
     const int16_t* sums = (const int16_t*)(kq_lds + nsb * kKqStride);
     const float* xd = (const float*)(kq_lds + nsb * (kKqStride + 32));
@@ -469,7 +497,7 @@ struct Q6KTile {
 template <int R>
 __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y,
                                                                const float* resid, int N, int nsb, int64_t act_row_bytes, Q4RopeTail rope,
-                                                               int rope_on) {
+                                                               int rope_on, int x_is_f32) {
     extern __shared__ __align__(16) uint8_t kq_lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * (kKqThreads / 64) + wave) * R;
@@ -492,7 +520,9 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
         }
     };
     fetch(0);
-    kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
+    // act: rows converted beforehand, or (x_is_f32) rows of float32 x, act_row_bytes apart, which the workgroup rounds itself
+    if (x_is_f32) kq_convert_into_lds((const float*)(act + (int64_t)blockIdx.y * act_row_bytes), nsb, kq_lds, tid);
+    else kq_stage_act(act + (int64_t)blockIdx.y * act_row_bytes, nsb, kq_lds, tid);
     __syncthreads();
     const int16_t* sums = (const int16_t*)(kq_lds + nsb * kKqStride);
     const float* xd = (const float*)(kq_lds + nsb * (kKqStride + 32));
@@ -579,12 +609,15 @@ static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, const Q4RopeTai
         raised[dt == kQ4_K] = true;
     }
     const Q4RopeTail tail = rope ? *rope : Q4RopeTail{};
+    // without converted activations the kernel reads float32 x and rounds it per workgroup
+    const uint8_t* in = a.act ? (const uint8_t*)a.act : (const uint8_t*)a.x;
+    const int64_t in_row = a.act ? (int64_t)kq_act_bytes(a.K) : a.x_row_stride * 4;
     if (dt == kQ4_K)
-        hipLaunchKernelGGL(qgemv_q4k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K), tail, rope ? 1 : 0);
+        hipLaunchKernelGGL(qgemv_q4k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, in, a.y, a.resid, (int)a.N, nsb, in_row,
+                           tail, rope ? 1 : 0, a.act ? 0 : 1);
     else
-        hipLaunchKernelGGL(qgemv_q6k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act,
-                           a.y, a.resid, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K), tail, rope ? 1 : 0);
+        hipLaunchKernelGGL(qgemv_q6k_kernel<R>, grid, dim3(kKqThreads), lds, st, (const uint8_t*)a.W, in, a.y, a.resid, (int)a.N, nsb, in_row,
+                           tail, rope ? 1 : 0, a.act ? 0 : 1);
     return hipGetLastError();
 }
 
@@ -602,6 +635,11 @@ hipError_t qgemv_kquant_act_rope(int dt, const QGemvArgs& a, const Q4RopeTail& r
 
 hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
     int nsb = (int)(a.K / 256);
+    // Float32 x in place of converted rows (a.act null): only the kernels that stage the row in LDS round it themselves.
+    if (!a.act) {
+        if (!qgemv_kquant_rope_ok(dt, a) || ((uintptr_t)a.x & 15) || a.x_row_stride % 4) return hipErrorInvalidValue;
+        return a.N * a.M >= 2048 ? launch_kq<2>(dt, a, nsb, nullptr, st) : launch_kq<1>(dt, a, nsb, nullptr, st);
+    }
     // From a few rows of x on, the matrix cores (whose results are the CPU's bit for bit).
     if (!a.resid && (g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && qgemm_kquant_pays(dt, a))) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
     // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.

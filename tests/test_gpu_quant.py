@@ -467,6 +467,28 @@ def test_kquant_gemv_every_launch_shape(dt):
             assert bits_equal(r, want)
 
 
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+def test_kquant_gemv_single_row_rounds_x_in_the_product(dt):
+    """One row of x against a small matrix is one launch whose workgroups round x themselves: the
+    same bits as the two-launch form (taken when x is not 16-byte aligned) and as the CPU, with
+    zero super-blocks, ties and a NaN in x."""
+    rng = np.random.default_rng(5 + dt)
+    for n, k in ((37, 256 * 56), (515, 256 * 16), (2, 256)):
+        raw = random_blocks(rng, dt, n * k)
+        x = rng.normal(size=k).astype(np.float32)
+        x[:256] = 0
+        x[k - 256:] = (rng.integers(0, 254, 256) - 127) / 2; x[k - 1] = 127
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        for poison in (False, True):
+            if poison: x[k // 2] = np.nan
+            want = O.qmatmul(dt, raw, x, n, k)
+            xd = gpu.dev(np.concatenate([np.zeros(1, np.float32), x]))
+            gpu.say(f"kquant single row dt={dt} N={n} K={k} nan={poison}")
+            one = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
+            two = gpu.qgemv(dt, ptr, xd[1:], n, k)
+            assert bits_equal(one, want) and bits_equal(two, want)
+
+
 def test_kquant_gemv_golden_and_exact_rows(golden_dir):
     cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
     for kind, dt in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
