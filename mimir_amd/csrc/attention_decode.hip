@@ -19,7 +19,7 @@
 // output projection.
 #include "device_util.h"
 #include "kernels.h"
-#include "q4_act.h"
+#include "q4_rows_act.h"
 
 namespace mimir {
 
@@ -42,6 +42,7 @@ struct DecParams {
     int cmax, nsplit;
     const int32_t* dyn_k;
     int64_t act_row_bytes;
+    int act_rows;  // the converted result in the form for a few rows of x (q4_rows_act.h), all sequences in one buffer
 };
 
 __device__ __forceinline__ float group16_sum(float v) {
@@ -341,9 +342,13 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
             hi[e] = fin[gi * D + blk * 32 + 16 + 4 * dq + e];
         }
         const int nb = p.H * D / 32, nbp = nb | 1;
-        u32x4* plane = (u32x4*)(act + (int64_t)b * p.act_row_bytes);
-        float* xscale = (float*)(plane + kDigits * nbp);
-        q4_convert_item(lo, hi, plane, xscale, nbp, (hk * G + g0 + gi) * (D / 32) + blk, dq);
+        if (p.act_rows) {
+            rows_convert_item(lo, hi, act, nb, b, (hk * G + g0 + gi) * (D / 32) + blk, dq);
+        } else {
+            u32x4* plane = (u32x4*)(act + (int64_t)b * p.act_row_bytes);
+            float* xscale = (float*)(plane + kDigits * nbp);
+            q4_convert_item(lo, hi, plane, xscale, nbp, (hk * G + g0 + gi) * (D / 32) + blk, dq);
+        }
     }
 }
 
@@ -393,7 +398,8 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
 // bytes whose first 4096 were zero before the first launch (the tickets reset
 // themselves). act, if set, gets row b's result [H * D] in the Q4_0 product's
 // fixed-point form, act_row_bytes apart; out may then be null.
-hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st) {
+// act_rows: the form for up to eight sequences together (q4_rows_act.h; a.B <= 8), row b's result as row b of it.
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, bool act_rows) {
     DecParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];
@@ -406,6 +412,8 @@ hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, vo
     attention_decode_plan(a.B, a.H, a.HK, kmax, &p.nsplit, &p.cmax);
     p.dyn_k = a.dyn_k;
     p.act_row_bytes = act_row_bytes;
+    p.act_rows = act_rows ? 1 : 0;
+    if (act_rows && a.B > 8) return hipErrorInvalidValue;
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
     dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
     size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);

@@ -70,6 +70,7 @@ constexpr int64_t kConvertInProductRows = 8;
 // Rows of x from which the Q4_0 product of float32 x goes to the int8 matrix cores: 16 means wherever its
 // cost model says it pays; "q4_0.fx_rows" sets another threshold, which then holds for every shape.
 int g_fx_min_rows = 16;
+int g_rows_path = 0;  // "q4_0.rows_path" 1: no matrix-core kernel for two to fifteen rows of x
 int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
@@ -77,6 +78,7 @@ thread_local std::vector<hipEvent_t> t_events;
 thread_local size_t t_events_used = 0;
 namespace mimir {
 void set_llama_step_mode(int mode);  // llm.hip
+void set_llama_rows_off(int v);      // llm.hip
 bool next_timing_events(hipEvent_t* start, hipEvent_t* stop) {
     if (t_events_used + 2 > t_events.size()) return false;
     *start = t_events[t_events_used];
@@ -345,6 +347,18 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
                 HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, (hipStream_t)stream), "launch qgemm_q4_0_fx");
                 return MI355X_OK;
             }
+            if (M >= 2 && M < 16 && g_rows_path != 1 && g_tune_q4[4] != 2 && ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0 &&
+                mimir::qgemv_q4_0_rows_ok(W, 1, N, K)) {
+                // a few rows (the decoding step of a batch): W read once for eight rows of x, on the int8 matrix cores
+                void* act;
+                if (mi355x_status st = act_scratch(mimir::q4_0_rows_act_bytes(K), &act)) return st;
+                for (int64_t m0 = 0; m0 < M; m0 += 8) {
+                    const int64_t mm = M - m0 < 8 ? M - m0 : 8;
+                    HIP_TRY(mimir::q4_0_rows_convert_act(x + m0 * x_row_stride, mm, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_rows_convert_act");
+                    HIP_TRY(mimir::qgemv_q4_0_rows(W, act, y + m0 * N, nullptr, mm, N, K, 1, (hipStream_t)stream), "launch qgemv_q4_0_rows");
+                }
+                return MI355X_OK;
+            }
             if (M == 1 && ((uintptr_t)x & 15) == 0) {
                 // one row: one launch, every workgroup converts x for itself (several rows: converted once, multiplied together)
                 HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0");
@@ -371,6 +385,10 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         if (mi355x_status st = act_scratch(mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
         HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
         a.act = act;
+        if (g_rows_path != 1 && mimir::qgemv_q8_0_rows_ok(a)) {  // several rows: W read once for up to eight of them, the same sums
+            HIP_TRY(mimir::qgemv_q8_0_rows(a, (hipStream_t)stream), "launch qgemv_q8_0_rows");
+            return MI355X_OK;
+        }
         HIP_TRY(mimir::qgemv_q8_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q8_0_act");
         return MI355X_OK;
     }
@@ -628,6 +646,11 @@ mi355x_status mi355x_tune(const char* key, int value) {
         g_fx_min_rows = value > 0 ? value : 16;
         return MI355X_OK;
     }
+    if (key && strcmp(key, "q4_0.rows_path") == 0) {  // 1: off; 2: its kernel without the LDS pass
+        g_rows_path = value == 1 ? 1 : 0;
+        mimir::set_q4_rows_direct(value == 2);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "q4_0.batch_off") == 0) {
         mimir::set_q4_batch_off(value);
         return MI355X_OK;
@@ -638,6 +661,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "attention.path") == 0) {
         g_tune_attn = value;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "llama.rows") == 0) {  // 1: a batch of sequences decodes with the one-sequence kernels
+        mimir::set_llama_rows_off(value == 1);
         return MI355X_OK;
     }
     if (key && strcmp(key, "llama.step") == 0 && value >= 0 && value <= 2) {

@@ -91,6 +91,10 @@ bool q8_act_fits(int64_t K);
 size_t q8_act_bytes(int64_t K);
 hipError_t q8_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
+// Two or more rows of x against W read once (each sum formed as qgemv_q8_0_act forms it): rows converted beforehand,
+// W 4-byte aligned, an even number of blocks a row, no residual.
+bool qgemv_q8_0_rows_ok(const QGemvArgs& a);
+hipError_t qgemv_q8_0_rows(const QGemvArgs& a, hipStream_t st);
 
 // The Q4_K and Q6_K products as the reference's CPU computes them: x rounded
 // to int8 in super-blocks of 256 with the sums of each 16 quants
@@ -183,8 +187,32 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
 void set_attention_decode_splits(int n);
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
-hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st);
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st,
+                            bool act_rows = false);
 
+// The fixed-point Q4_0 product for up to eight rows of float32 x that reads W once (qgemv_q4_0_rows.hip, int8
+// matrix cores): the rows are converted together by q4_0_rows_convert_act into q4_0_rows_act_bytes(K) bytes
+// (x 16-byte aligned rows, K a multiple of 64).
+size_t q4_0_rows_act_bytes(int64_t K);
+hipError_t q4_0_rows_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
+bool qgemv_q4_0_rows_ok(const void* W, int64_t M, int64_t N, int64_t K);
+// shares > 1 (qgemv_q4_0_rows_shares_ok; no resid): K is cut into that many shares, whose sums go to y[shares, M, N]
+// for a later kernel to add in their order.
+bool qgemv_q4_0_rows_shares_ok(const void* W, int64_t M, int64_t N, int64_t K, int shares);
+hipError_t qgemv_q4_0_rows(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, int shares,
+                           hipStream_t st);
+// Up to three matrices (n[i] = 0: none) that share act and K in one launch, their rows one after the other in
+// y[shares, M, n[0] + n[1] + n[2]]: each must satisfy qgemv_q4_0_rows_shares_ok, all but the last with a multiple of 32 rows.
+hipError_t qgemv_q4_0_rows_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, const float* resid, int64_t M,
+                                 int64_t K, int shares, hipStream_t st);
+// Around that product in a decoding step of up to eight sequences, each leaving its result in the converted form:
+// RMSNorm (with shares > 0, x += parts[0] + parts[1] + ... first, parts [shares, rows, d], written back to x: the
+// residual connection behind a product cut into shares), SiLU(g) * u, and the addition of the shares alone.
+hipError_t rows_norm_act(float* x, const float* parts, int shares, const float* w, void* act, int64_t rows, int64_t d, double eps,
+                         hipStream_t st);
+hipError_t rows_swiglu_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
+hipError_t rows_add_parts(float* x, const float* parts, int shares, int64_t n, hipStream_t st);
+void set_q4_rows_direct(int v);  // measurement aid: 1 = its kernel that loads each lane's block where it lies
 // The fixed-point Q4_0 product for many rows of float32 x on the int8 matrix cores (qgemm_q4_0_fx.hip):
 // x converted by q4_0_fx_convert_act (q4_0_fx_act_bytes(K) bytes a row), K a multiple of 128.
 size_t q4_0_fx_act_bytes(int64_t K);

@@ -105,7 +105,13 @@ struct Model {
     // linears that the fixed-point kernel takes); step_graph replays the run.
     bool fast = false;
     DevBuf state, record, qkv, gu, argmax_ws;  // gu: gate|up of a step, [batch, 2 hidden]
+    // `rows`: a fast model with two to eight sequences, whose step reads every weight once for all of them
+    // (step_rows): the sequences' activations converted together, and the two shares of K of the output and
+    // down projections, [2, batch, embed].
+    bool rows = false;
+    DevBuf rows_act, parts;
     hipGraphExec_t step_graph = nullptr;
+    bool graph_rows = false;  // the captured step is step_rows
 
     ~Model() {
         if (step_graph) (void)hipGraphExecDestroy(step_graph);
@@ -170,7 +176,7 @@ mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_
         break;
     case kQ8_0:
         if (cls != kActQ8) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: q8_0 rows of %lld are too long", (long long)w.k);
-        e = qgemv_q8_0_act(a, kNoTune, m.stream);
+        e = qgemv_q8_0_rows_ok(a) ? qgemv_q8_0_rows(a, m.stream) : qgemv_q8_0_act(a, kNoTune, m.stream);  // several rows: W read once
         break;
     case kQ4_K: case kQ6_K: e = qgemv_kquant_act(w.dtype, a, m.stream); break;
     case kF32: case kF16: case kBF16: e = gemv_float(w.dtype, w.buf.p, x, y, rows, w.n, w.k, w.k, m.stream); break;
@@ -345,6 +351,57 @@ static mi355x_status step_fast(Model& m) {
         d.resid = x;
         LLM_HIP(qgemv_q4_0_act(d, kNoTune, m.stream), "ffn_down");
     }
+    return MI355X_OK;
+}
+
+static int g_llama_rows_off = 0;  // measurement aid: 1 = several sequences take step_fast as one does
+void set_llama_rows_off(int v) { g_llama_rows_off = v; }
+
+// One decoding step of two to eight sequences with Q4_0 linears (the case of step_fast): the same
+// operations, but every product reads its weights once for all the sequences, on the int8 matrix cores
+// (qgemv_q4_0_rows.hip), where step_fast's products read them once per sequence. Nine launches a block:
+// norm (adding the shares of the product before it into x) with conversion, q|k|v, rotation and cache
+// write, attention with conversion, output projection in two shares of K, norm, gate|up, SiLU * up with
+// conversion, down projection in two shares. The shares of the last down projection are added at the end.
+static mi355x_status step_rows(Model& m) {
+    const auto& c = m.c;
+    const int64_t B = c.batch;
+    const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim, row = qd + 2 * kvd;
+    float *x = m.x.as<float>(), *qkv = m.qkv.as<float>(), *gu = m.gu.as<float>(), *parts = m.parts.as<float>();
+    void* act = m.rows_act.p;
+    const int32_t* pos = m.state.as<int32_t>();
+    if (mi355x_status st = embed_rows(m, m.next_tok.as<int32_t>(), B, x, device_error_word())) return st;
+    AttnArgs at;
+    at.q = qkv; at.kv_dtype = c.cache_dtype; at.out = nullptr; at.lse = nullptr;
+    at.q_strides[0] = row; at.q_strides[1] = c.head_dim; at.q_strides[2] = 0;
+    at.k_strides[0] = at.v_strides[0] = (int64_t)c.kv_heads * c.context * c.head_dim;
+    at.k_strides[1] = at.v_strides[1] = (int64_t)c.context * c.head_dim;
+    at.k_strides[2] = at.v_strides[2] = c.head_dim;
+    at.o_strides[0] = qd; at.o_strides[1] = c.head_dim; at.o_strides[2] = 0;
+    at.B = B; at.Q = 1; at.K = 1; at.H = c.heads; at.HK = c.kv_heads; at.D = c.head_dim;
+    at.scale = 1.0 / std::sqrt((double)c.head_dim);
+    at.causal = 0; at.causal_offset = 0;
+    at.dyn_k = pos;  // position p holds p keys before this step's own
+    const int shares = 2;
+    for (int i = 0; i < c.layers; i++) {
+        Block& b = m.blocks[i];
+        LLM_HIP(rows_norm_act(x, parts, i == 0 ? 0 : shares, b.attn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "attn_norm");
+        const void* w3[3] = {b.q.buf.p, b.k.buf.p, b.v.buf.p};
+        const int64_t n3[3] = {qd, kvd, kvd};
+        LLM_HIP(qgemv_q4_0_rows_multi(w3, n3, act, qkv, nullptr, B, c.embed, 1, m.stream), "q|k|v");
+        LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                        c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        at.k = m.keys[i].p; at.v = m.values[i].p;
+        LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, true), "attention");
+        LLM_HIP(qgemv_q4_0_rows(b.o.buf.p, act, parts, nullptr, B, c.embed, qd, shares, m.stream), "attn_output");
+        LLM_HIP(rows_norm_act(x, parts, shares, b.ffn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "ffn_norm");
+        const void* w2[3] = {b.gate.buf.p, b.up.buf.p, nullptr};
+        const int64_t n2[3] = {c.hidden, c.hidden, 0};
+        LLM_HIP(qgemv_q4_0_rows_multi(w2, n2, act, gu, nullptr, B, c.embed, 1, m.stream), "gate|up");
+        LLM_HIP(rows_swiglu_act(gu, gu + c.hidden, act, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+        LLM_HIP(qgemv_q4_0_rows(b.down.buf.p, act, parts, nullptr, B, c.embed, c.hidden, shares, m.stream), "ffn_down");
+    }
+    LLM_HIP(rows_add_parts(x, parts, shares, B * c.embed, m.stream), "residual");
     return MI355X_OK;
 }
 
@@ -686,6 +743,31 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         if (mi355x_status st = fuse({&b.gate, &b.up}, b.gate_up)) return st;
     }
     LLM_HIP(m->gu.alloc((size_t)c.batch * 2 * c.hidden * 4), "hipMalloc");
+    // several sequences: every product of a step on the kernels that read W once for up to eight rows of x
+    m->rows = m->fast && c.batch >= 2 && c.batch <= 8 && qd % 32 == 0 && kvd % 32 == 0 && c.hidden % 32 == 0 && c.embed <= 8192;
+    if (m->rows) {
+        AttnArgs at;  // the shape of a step's attention, as step_rows sets it up
+        at.q = m->qkv.as<float>(); at.k = m->keys[0].p; at.v = m->values[0].p; at.kv_dtype = c.cache_dtype;
+        at.q_strides[0] = qd + 2 * kvd; at.q_strides[1] = c.head_dim; at.q_strides[2] = 0;
+        at.k_strides[0] = at.v_strides[0] = (int64_t)c.kv_heads * c.context * c.head_dim;
+        at.k_strides[1] = at.v_strides[1] = (int64_t)c.context * c.head_dim;
+        at.k_strides[2] = at.v_strides[2] = c.head_dim;
+        at.B = c.batch; at.Q = 1; at.K = 1; at.H = c.heads; at.HK = c.kv_heads; at.D = c.head_dim;
+        m->rows = attention_decode_ok(at, c.context);
+    }
+    for (int i = 0; i < c.layers && m->rows; i++) {
+        Block& b = m->blocks[i];
+        for (const Weight* w : {&b.q, &b.k, &b.v, &b.gate, &b.up})
+            if (!qgemv_q4_0_rows_shares_ok(w->buf.p, c.batch, w->n, w->k, 1)) m->rows = false;
+        for (const Weight* w : {&b.o, &b.down})
+            if (!qgemv_q4_0_rows_shares_ok(w->buf.p, c.batch, w->n, w->k, 2)) m->rows = false;
+    }
+    if (m->rows) {
+        const size_t ab = q4_0_rows_act_bytes(kmax);
+        LLM_HIP(m->rows_act.alloc(ab), "hipMalloc(activations)");
+        LLM_HIP(hipMemset(m->rows_act.p, 0, ab), "hipMemset(activations)");  // rows past the batch stay zero
+        LLM_HIP(m->parts.alloc((size_t)2 * c.batch * c.embed * 4), "hipMalloc");
+    }
     m->ready = true;
     return MI355X_OK;
 }
@@ -790,13 +872,19 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
         if (!st && e == hipSuccess) e = advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 0, m->stream);
         if (!st && e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: step state: %s", hipGetErrorName(e));
         auto one_step = [&]() -> mi355x_status {
-            if (mi355x_status s2 = m->fast ? step_fast(*m) : step_any(*m)) return s2;
+            if (mi355x_status s2 = m->rows && !g_llama_rows_off ? step_rows(*m) : m->fast ? step_fast(*m) : step_any(*m)) return s2;
             if (mi355x_status s2 = head(*m, m->x.as<float>(), B, c.embed)) return s2;
             LLM_HIP(argmax(m->logits.as<float>(), B, c.vocab, m->next_tok.as<int32_t>(), m->argmax_ws.p, m->stream), "argmax");
             LLM_HIP(advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 1, m->stream), "advance");
             return MI355X_OK;
         };
+        const bool rows_now = m->rows && !g_llama_rows_off;
+        if (m->step_graph && m->graph_rows != rows_now) {  // the measurement aid changed which step runs
+            (void)hipGraphExecDestroy(m->step_graph);
+            m->step_graph = nullptr;
+        }
         if (!st && n_new > 1 && !m->step_graph && use_graph) {
+            m->graph_rows = rows_now;
             hipGraph_t g = nullptr;
             e = hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal);
             if (e != hipSuccess) st = capi_fail((mi355x_status)e, "mi355x: llama: begin capture: %s", hipGetErrorName(e));

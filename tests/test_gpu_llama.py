@@ -219,6 +219,45 @@ def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, ca
     assert all(same), (runs[2][0], runs[0][0])
 
 
+@pytest.mark.parametrize("batch", [2, 5, 8])
+def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
+    """Two to eight sequences decode with products that read each weight once for all of them (int8 matrix
+    cores, the output and down projections cut into two shares of K that the next norm adds). Their
+    integers are those of the one-sequence kernels, only float32 sums are ordered differently, so the tokens
+    must be those of the one-sequence kernels run per sequence (llama.rows = 1), of the per-operator path,
+    and, up to near-ties, the oracle's."""
+    lib = gpu.lib()
+    c = _small_q4_config(batch, capi.F16)
+    om = OL.synthetic(_oracle_config(c), seed=2, output_dt=O.Q4_0)
+    m = Llama(c)
+    _upload_synthetic(m, om)
+    m.finalize(40)
+    prompts = np.random.default_rng(17).integers(0, c.vocab, (batch, 11))
+    runs = {}
+    try:
+        for name, key, v in (("rows graph", b"llama.rows", 0), ("rows launches", b"llama.step", 1), ("per sequence", b"llama.rows", 1),
+                             ("per operator", b"llama.step", 2)):
+            capi.check(lib.mi355x_tune(b"llama.rows", 0))
+            capi.check(lib.mi355x_tune(b"llama.step", 0))
+            capi.check(lib.mi355x_tune(key, v))
+            gpu.say(f"generate batch {batch}: {name}")
+            m.reset()
+            first, _ = m.generate(prompts, 30)
+            more, _ = m.generate(first[:, -1:], 10)  # the graph of the first call, from another cache length
+            runs[name] = np.concatenate([first, more], 1)
+    finally:
+        capi.check(lib.mi355x_tune(b"llama.rows", 0))
+        capi.check(lib.mi355x_tune(b"llama.step", 0))
+    for name in ("rows launches", "per sequence", "per operator"):
+        assert np.array_equal(runs["rows graph"], runs[name]), (name, runs["rows graph"], runs[name])
+    for b in range(batch):
+        want, margins = om.generate(prompts[b].tolist(), 30, capacity=c.context, cache_dtype=O.F16)
+        for i, (a, w) in enumerate(zip(runs["rows graph"][b, :30].tolist(), want)):
+            if a != w:
+                assert margins[i] < 1e-3 * 170.0, (b, i, a, w, margins[i])
+                break
+
+
 def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
     """The fused step lets the rotation, the norms and the conversion of SwiGLU's results ride on the products
     only where their shapes allow: interleaved pairs, rows of x one step of a wavefront long. A model with
