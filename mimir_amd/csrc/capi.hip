@@ -651,6 +651,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
         mimir::set_q4_rows_direct(value == 2);
         return MI355X_OK;
     }
+    if (key && strcmp(key, "q4_0.rows_waves") == 0) {
+        mimir::set_q4_rows_waves(value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "q4_0.batch_off") == 0) {
         mimir::set_q4_batch_off(value);
         return MI355X_OK;

@@ -212,6 +212,7 @@ hipError_t rows_norm_act(float* x, const float* parts, int shares, const float* 
                          hipStream_t st);
 hipError_t rows_swiglu_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 hipError_t rows_add_parts(float* x, const float* parts, int shares, int64_t n, hipStream_t st);
+void set_q4_rows_waves(int v);   // measurement aid: 4 or 8 wavefronts a workgroup, 0 by shape
 void set_q4_rows_direct(int v);  // measurement aid: 1 = its kernel that loads each lane's block where it lies
 // The fixed-point Q4_0 product for many rows of float32 x on the int8 matrix cores (qgemm_q4_0_fx.hip):
 // x converted by q4_0_fx_convert_act (q4_0_fx_act_bytes(K) bytes a row), K a multiple of 128.

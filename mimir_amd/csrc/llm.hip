@@ -382,7 +382,7 @@ static mi355x_status step_rows(Model& m) {
     at.scale = 1.0 / std::sqrt((double)c.head_dim);
     at.causal = 0; at.causal_offset = 0;
     at.dyn_k = pos;  // position p holds p keys before this step's own
-    const int shares = 2;
+    const int shares = 2;  // of K, for the two products with 4096 rows of W: measured against 1, 3 and 4
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
         LLM_HIP(rows_norm_act(x, parts, i == 0 ? 0 : shares, b.attn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "attn_norm");

@@ -247,7 +247,8 @@ constexpr int kWaveLds = kSlabBytes + kRunBlocks * kTailBytes;  // the slab, the
 
 // gridDim.y shares of K: with more than one, share s writes its sums to y + s * M * N and nothing is added
 // (a later kernel adds the shares in their order); resid only with one share.
-__global__ __launch_bounds__(64 * kWaves) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
+template <int WAVES>  // wavefronts of a workgroup, among which the runs of its share of K go round
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
                                                                        float* y, const float* resid,  // resid may be y
                                                                        int M, int nb) {
     extern __shared__ __align__(16) uint8_t smem[];  // per wavefront: slab and tail of its run; later the wavefronts' sums
@@ -337,8 +338,8 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_q4_0_rows_kernel(const Rows
     const uint8_t* mine = slab + l32 * kSlabStride + 20 * lh;
     const uint8_t* mine_d = slab + l32 * kSlabStride + 16 * lh;
     const uint32_t shift = lh ? 0u : 16u;
-    for (int run = run0; run < run_end; run += kWaves) {
-        const int nrun = run + kWaves < run_end ? run + kWaves : run;
+    for (int run = run0; run < run_end; run += WAVES) {
+        const int nrun = run + WAVES < run_end ? run + WAVES : run;
         fetch_w(nxt, nrun);
         // slab and tail are this wavefront's alone: every lane's reads of the last run were waited for before
         // its last MFMAs and FMAs, and a wavefront's LDS operations complete in order
@@ -384,7 +385,7 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_q4_0_rows_kernel(const Rows
     if (wave != 0) return;
     f32x4 sum = red[lane];
 #pragma unroll
-    for (int w = 1; w < kWaves; w++) {
+    for (int w = 1; w < WAVES; w++) {
         const f32x4 t = red[w * 64 + lane];
 #pragma unroll
         for (int j = 0; j < 4; j++) sum[j] = sum[j] + t[j];
@@ -548,7 +549,9 @@ hipError_t rows_add_parts(float* x, const float* parts, int shares, int64_t n, h
 }
 
 static int g_rows_direct = 0;  // measurement aid: 1 = always the kernel without the LDS pass
+static int g_rows_waves = 0;   // measurement aid: 4 or 8 = that many wavefronts a workgroup, whatever the shape
 void set_q4_rows_direct(int v) { g_rows_direct = v; }
+void set_q4_rows_waves(int v) { g_rows_waves = v; }
 
 // W 2-byte aligned (ggml blocks), pairs of blocks, at most eight rows of x.
 static bool rows_base_ok(const void* W, int64_t M, int64_t N, int64_t K) {
@@ -605,8 +608,15 @@ hipError_t qgemv_q4_0_rows_multi(const void* const W[3], const int64_t n[3], con
         if (n[i] == 0 && i < last) return hipErrorInvalidValue;
     }
     if (last < 0 || (shares > 1 && resid)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(qgemv_q4_0_rows_kernel, dim3(groups, (unsigned)shares), dim3(64 * kWaves), (size_t)kWaves * kWaveLds, st, job,
-                       (const uint8_t*)act, y, resid, (int)M, (int)(K / 32));
+    // Many workgroups: four wavefronts each, so that all are resident at once and each wavefront has runs
+    // to request ahead of; few: eight, for the parallelism.
+    const bool four = g_rows_waves == 4 || (g_rows_waves == 0 && (int64_t)groups * shares >= 384);
+    if (four)
+        hipLaunchKernelGGL(qgemv_q4_0_rows_kernel<4>, dim3(groups, (unsigned)shares), dim3(256), (size_t)4 * kWaveLds, st, job,
+                           (const uint8_t*)act, y, resid, (int)M, (int)(K / 32));
+    else
+        hipLaunchKernelGGL(qgemv_q4_0_rows_kernel<8>, dim3(groups, (unsigned)shares), dim3(512), (size_t)8 * kWaveLds, st, job,
+                           (const uint8_t*)act, y, resid, (int)M, (int)(K / 32));
     return hipGetLastError();
 }
 

@@ -233,11 +233,13 @@ __global__ __launch_bounds__(512) void qgemv_q8_0_kernel(const uint8_t* __restri
     }
 }
 
-// Several rows of x against W read once: MB converted rows staged in LDS, a wavefront per row of W (pairs of
-// blocks, W 4-byte aligned), every (row of W, row of x) sum formed exactly as the kernel above forms it.
+// Several rows of x against W read once: MB converted rows staged in LDS once per workgroup, whose wavefronts
+// then walk rows_per_wave rows of W each (pairs of blocks, W 4-byte aligned; the next row's first blocks are
+// requested before the current row is multiplied). Every (row of W, row of x) sum is formed exactly as the
+// kernel above forms it.
 template <int MB>
 __global__ __launch_bounds__(512) void qgemv_q8_0_rows_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act, float* y, int M,
-                                                              int N, int nb, int64_t act_row_bytes) {
+                                                              int N, int nb, int64_t act_row_bytes, int rows_per_wave) {
     extern __shared__ u32x4 lds_q8[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
@@ -246,67 +248,68 @@ __global__ __launch_bounds__(512) void qgemv_q8_0_rows_kernel(const uint8_t* __r
     const int n16 = (int)(act_row_bytes >> 4);
     const int64_t row_bytes = (int64_t)nb * 34;
     const int nunits = nb >> 1, nsteps = (nunits + 63) >> 6;
-    const int row = blockIdx.x * waves + wave;
-    const uint8_t* rowp = W + (int64_t)(row < N ? row : N - 1) * row_bytes;
-    Q8Pair first;  // the row's first step is requested before x is staged
-    {
-        const int u = lane < nunits ? lane : nunits - 1;
-        const uint32_t* src = (const uint32_t*)rowp + u * 17;
+    const int wg_row0 = blockIdx.x * waves * rows_per_wave;
+    auto fetch = [&](Q8Pair& f, int row, int step) {
+        int u = lane + 64 * step;
+        u = u < nunits ? u : nunits - 1;
+        const uint32_t* src = (const uint32_t*)(W + (int64_t)(row < N ? row : N - 1) * row_bytes) + u * 17;
 #pragma unroll
-        for (int k = 0; k < 4; k++) first.v[k] = *(const u32x4_a4*)(src + 4 * k);
-        first.tail = src[16];
-    }
+        for (int k = 0; k < 4; k++) f.v[k] = *(const u32x4_a4*)(src + 4 * k);
+        f.tail = src[16];
+    };
+    Q8Pair next;  // the first row's first step is requested before x is staged
+    fetch(next, wg_row0 + wave, 0);
     for (int mb = 0; mb < MB; mb++) {
         const int m = m0 + mb < M ? m0 + mb : M - 1;
         const u32x4* act_row = (const u32x4*)(act + (int64_t)m * act_row_bytes);
         for (int idx = tid; idx < n16; idx += (int)blockDim.x) lds_q8[mb * n16 + idx] = act_row[idx];
     }
     __syncthreads();
-    if (row >= N) return;
-    float acc[MB][4];
+    for (int i = 0; i < rows_per_wave; i++) {
+        const int row = wg_row0 + wave + waves * i;
+        if (row >= N) break;
+        float acc[MB][4];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int l = 0; l < 4; l++) acc[mb][l] = 0.f;
-    for (int step = 0; step < nsteps; step++) {
-        int u = lane + 64 * step;
-        const bool live = u < nunits;
-        u = live ? u : nunits - 1;
-        Q8Pair pr = first;
-        if (step > 0) {
-            const uint32_t* src = (const uint32_t*)rowp + u * 17;
+            for (int l = 0; l < 4; l++) acc[mb][l] = 0.f;
+        for (int step = 0; step < nsteps; step++) {
+            int u = lane + 64 * step;
+            const bool live = u < nunits;
+            u = live ? u : nunits - 1;
+            const Q8Pair pr = next;
+            if (step + 1 < nsteps) fetch(next, row, step + 1);
+            else fetch(next, row + waves, 0);  // past the end of W: the last row again, not used
+            uint32_t d[17];
 #pragma unroll
-            for (int k = 0; k < 4; k++) pr.v[k] = *(const u32x4_a4*)(src + 4 * k);
-            pr.tail = src[16];
+            for (int k = 0; k < 16; k++) d[k] = pr.v[k >> 2][k & 3];
+            d[16] = pr.tail;
+            uint32_t w0[8], w1[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                w0[k] = __builtin_amdgcn_alignbyte(d[k + 1], d[k], 2);
+                w1[k] = d[9 + k];
+            }
+            const float dw0 = live ? f16_bits_to_f32((uint16_t)(d[0] & 0xffffu)) : 0.f;
+            const float dw1 = live ? f16_bits_to_f32((uint16_t)(d[8] >> 16)) : 0.f;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                const u32x4* xr = lds_q8 + mb * n16;
+                const float* xd = (const float*)(xr + 2 * nbp);
+                const u32x4 xa0 = xr[2 * u], xb0 = xr[nbp + 2 * u];
+                const u32x4 xa1 = xr[2 * u + 1], xb1 = xr[nbp + 2 * u + 1];
+                const float dx0 = live ? xd[2 * u] : 0.f, dx1 = live ? xd[2 * u + 1] : 0.f;
+                q8_block(w0, xa0, xb0, dw0, dx0, acc[mb]);
+                q8_block(w1, xa1, xb1, dw1, dx1, acc[mb]);
+                __builtin_amdgcn_sched_barrier(0);  // one row of x at a time: its operands need not all be held at once
+            }
         }
-        uint32_t d[17];
-#pragma unroll
-        for (int k = 0; k < 16; k++) d[k] = pr.v[k >> 2][k & 3];
-        d[16] = pr.tail;
-        uint32_t w0[8], w1[8];
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            w0[k] = __builtin_amdgcn_alignbyte(d[k + 1], d[k], 2);
-            w1[k] = d[9 + k];
-        }
-        const float dw0 = live ? f16_bits_to_f32((uint16_t)(d[0] & 0xffffu)) : 0.f;
-        const float dw1 = live ? f16_bits_to_f32((uint16_t)(d[8] >> 16)) : 0.f;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
-            const u32x4* xr = lds_q8 + mb * n16;
-            const float* xd = (const float*)(xr + 2 * nbp);
-            const u32x4 xa0 = xr[2 * u], xb0 = xr[nbp + 2 * u];
-            const u32x4 xa1 = xr[2 * u + 1], xb1 = xr[nbp + 2 * u + 1];
-            const float dx0 = live ? xd[2 * u] : 0.f, dx1 = live ? xd[2 * u + 1] : 0.f;
-            q8_block(w0, xa0, xb0, dw0, dx0, acc[mb]);
-            q8_block(w1, xa1, xb1, dw1, dx1, acc[mb]);
+            float a0 = wave_sum(acc[mb][0]), a1 = wave_sum(acc[mb][1]), a2 = wave_sum(acc[mb][2]), a3 = wave_sum(acc[mb][3]);
+            float s02 = a0 + a2, s13 = a1 + a3;
+            if (lane == 0 && m0 + mb < M) y[(int64_t)(m0 + mb) * N + row] = s02 + s13;
         }
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        float a0 = wave_sum(acc[mb][0]), a1 = wave_sum(acc[mb][1]), a2 = wave_sum(acc[mb][2]), a3 = wave_sum(acc[mb][3]);
-        float s02 = a0 + a2, s13 = a1 + a3;
-        if (lane == 0 && m0 + mb < M) y[(int64_t)(m0 + mb) * N + row] = s02 + s13;
     }
 }
 
@@ -319,10 +322,13 @@ hipError_t qgemv_q8_0_rows(const QGemvArgs& a, hipStream_t st) {
     const int waves = 8;
     const size_t ab = q8_act_bytes(a.K);
     const int mb = a.M > 4 ? 8 : a.M > 2 ? 4 : 2;
-    dim3 grid((unsigned)((a.N + waves - 1) / waves), (unsigned)((a.M + mb - 1) / mb));
+    // rows of W per wavefront: as many as still leave every compute unit four workgroups
+    int rpw = 16;
+    while (rpw > 1 && (a.N + waves * rpw - 1) / (waves * rpw) < 1024) rpw >>= 1;
+    dim3 grid((unsigned)((a.N + waves * rpw - 1) / (waves * rpw)), (unsigned)((a.M + mb - 1) / mb));
 #define Q8ROWS(MB)                                                                                                                      \
     hipLaunchKernelGGL((qgemv_q8_0_rows_kernel<MB>), grid, dim3(64 * waves), MB * ab, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, \
-                       (int)a.M, (int)a.N, (int)(a.K / 32), (int64_t)ab)
+                       (int)a.M, (int)a.N, (int)(a.K / 32), (int64_t)ab, rpw)
     if (mb == 8) Q8ROWS(8); else if (mb == 4) Q8ROWS(4); else Q8ROWS(2);
 #undef Q8ROWS
     return hipGetLastError();

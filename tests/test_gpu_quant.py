@@ -408,6 +408,25 @@ def test_q8_0_lm_head_shape_sampled():
     assert O.argmax(got) == O.argmax(want)
 
 
+@pytest.mark.parametrize("m,n,k", [(11, 203, 4096 + 64), (2, 70, 128), (16, 9, 1280), (8, 7000, 4096)])
+def test_q8_0_rows_of_x_share_one_pass_over_w(m, n, k):
+    """Several rows of x against Q8_0 weights read once: every sum is formed as the one-row kernel forms it,
+    so the results are its bits, row by row."""
+    rng = np.random.default_rng(m + n + k)
+    raw = random_blocks(rng, O.Q8_0, n * k)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    gpu.say(f"q8_0 rows kernel M={m} N={n} K={k}")
+    got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+    want = O.qmatmul(O.Q8_0, raw, x, n, k)
+    w = O.dequantize(O.Q8_0, raw).reshape(n, k).astype(np.float64)
+    mag = np.abs(x.astype(np.float64)) @ np.abs(w).T  # what the rounding errors of the float32 sums scale with
+    assert np.all(np.abs(got - want) <= 2e-6 * mag + 1e-30)
+    xd = gpu.dev(x)
+    one = np.stack([gpu.qgemv(O.Q8_0, ptr, xd[i], n, k) for i in range(m)])
+    assert bits_equal(got, one)
+
+
 # ---- Q4_K / Q6_K -------------------------------------------------------------
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
