@@ -667,8 +667,8 @@ mi355x_status mi355x_tune(const char* key, int value) {
         g_tune_attn = value;
         return MI355X_OK;
     }
-    if (key && strcmp(key, "llama.rows") == 0) {  // 1: a batch of sequences decodes with the one-sequence kernels
-        mimir::set_llama_rows_off(value == 1);
+    if (key && strcmp(key, "llama.rows") == 0) {  // 1: a batch of sequences decodes with the one-sequence kernels; 2: the batch step without its riders
+        mimir::set_llama_rows_off(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "llama.step") == 0 && value >= 0 && value <= 2) {

@@ -205,6 +205,13 @@ hipError_t qgemv_q4_0_rows(const void* W, const void* act, float* y, const float
 // y[shares, M, n[0] + n[1] + n[2]]: each must satisfy qgemv_q4_0_rows_shares_ok, all but the last with a multiple of 32 rows.
 hipError_t qgemv_q4_0_rows_multi(const void* const W[3], const int64_t n[3], const void* act, float* y, const float* resid, int64_t M,
                                  int64_t K, int shares, hipStream_t st);
+// q, k and v in one launch with the rotation and the cache writes of a decoding step as its tail (y [M, n[0] + n[1] + n[2]]
+// receives the rotated queries only; interleaved pairs, rows in multiples of 32); and gate and up [N, K] in one launch that
+// leaves SiLU(x . gate^T) * (x . up^T) converted in act_out as the x of a product over N (N a multiple of 32).
+hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                    const Q4RopeTail& rope, hipStream_t st);
+hipError_t qgemv_q4_0_rows_swiglu_act(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N, int64_t K,
+                                      hipStream_t st);
 // Around that product in a decoding step of up to eight sequences, each leaving its result in the converted form:
 // RMSNorm (with shares > 0, x += parts[0] + parts[1] + ... first, parts [shares, rows, d], written back to x: the
 // residual connection behind a product cut into shares), SiLU(g) * u, and the addition of the shares alone.

@@ -109,9 +109,9 @@ struct Model {
     // (step_rows): the sequences' activations converted together, and the two shares of K of the output and
     // down projections, [2, batch, embed].
     bool rows = false;
-    DevBuf rows_act, parts;
+    DevBuf rows_act, rows_act2, parts;
     hipGraphExec_t step_graph = nullptr;
-    bool graph_rows = false;  // the captured step is step_rows
+    int graph_rows = 0;  // which step the graph holds: 0 step_fast or step_any, 1 step_rows, 2 step_rows without its riders
 
     ~Model() {
         if (step_graph) (void)hipGraphExecDestroy(step_graph);
@@ -355,7 +355,8 @@ static mi355x_status step_fast(Model& m) {
 }
 
 static int g_llama_rows_off = 0;  // measurement aid: 1 = several sequences take step_fast as one does
-void set_llama_rows_off(int v) { g_llama_rows_off = v; }
+static int g_llama_rows_plain = 0;  // measurement aid: 1 = step_rows with the rotation and SwiGLU as launches of their own
+void set_llama_rows_off(int v) { g_llama_rows_off = v == 1; g_llama_rows_plain = v >= 2 ? v : 0; }
 
 // One decoding step of two to eight sequences with Q4_0 linears (the case of step_fast): the same
 // operations, but every product reads its weights once for all the sequences, on the int8 matrix cores
@@ -388,18 +389,32 @@ static mi355x_status step_rows(Model& m) {
         LLM_HIP(rows_norm_act(x, parts, i == 0 ? 0 : shares, b.attn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "attn_norm");
         const void* w3[3] = {b.q.buf.p, b.k.buf.p, b.v.buf.p};
         const int64_t n3[3] = {qd, kvd, kvd};
-        LLM_HIP(qgemv_q4_0_rows_multi(w3, n3, act, qkv, nullptr, B, c.embed, 1, m.stream), "q|k|v");
-        LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
-                        c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        if (c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0 && g_llama_rows_plain != 2 && g_llama_rows_plain != 4) {  // the rotation and the cache writes ride on the product
+            Q4RopeTail tail;
+            tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
+            tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
+            tail.cache_dt = c.cache_dtype; tail.H = c.heads; tail.HK = c.kv_heads; tail.dim = c.head_dim; tail.rope_dim = c.rope_dim;
+            tail.cap = c.context;
+            LLM_HIP(qgemv_q4_0_rows_qkv_rope(w3, n3, act, qkv, B, c.embed, tail, m.stream), "q|k|v, rope and cache");
+        } else {
+            LLM_HIP(qgemv_q4_0_rows_multi(w3, n3, act, qkv, nullptr, B, c.embed, 1, m.stream), "q|k|v");
+            LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
+                            c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+        }
         at.k = m.keys[i].p; at.v = m.values[i].p;
         LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, true), "attention");
         LLM_HIP(qgemv_q4_0_rows(b.o.buf.p, act, parts, nullptr, B, c.embed, qd, shares, m.stream), "attn_output");
         LLM_HIP(rows_norm_act(x, parts, shares, b.ffn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "ffn_norm");
-        const void* w2[3] = {b.gate.buf.p, b.up.buf.p, nullptr};
-        const int64_t n2[3] = {c.hidden, c.hidden, 0};
-        LLM_HIP(qgemv_q4_0_rows_multi(w2, n2, act, gu, nullptr, B, c.embed, 1, m.stream), "gate|up");
-        LLM_HIP(rows_swiglu_act(gu, gu + c.hidden, act, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
-        LLM_HIP(qgemv_q4_0_rows(b.down.buf.p, act, parts, nullptr, B, c.embed, c.hidden, shares, m.stream), "ffn_down");
+        if (g_llama_rows_plain != 2 && g_llama_rows_plain != 3) {  // SiLU * up and the conversion ride on the product, into a buffer of their own
+            LLM_HIP(qgemv_q4_0_rows_swiglu_act(b.gate.buf.p, b.up.buf.p, act, m.rows_act2.p, B, c.hidden, c.embed, m.stream), "gate|up, conversion");
+            LLM_HIP(qgemv_q4_0_rows(b.down.buf.p, m.rows_act2.p, parts, nullptr, B, c.embed, c.hidden, shares, m.stream), "ffn_down");
+        } else {
+            const void* w2[3] = {b.gate.buf.p, b.up.buf.p, nullptr};
+            const int64_t n2[3] = {c.hidden, c.hidden, 0};
+            LLM_HIP(qgemv_q4_0_rows_multi(w2, n2, act, gu, nullptr, B, c.embed, 1, m.stream), "gate|up");
+            LLM_HIP(rows_swiglu_act(gu, gu + c.hidden, act, B, c.hidden, 2 * (int64_t)c.hidden, m.stream), "swiglu");
+            LLM_HIP(qgemv_q4_0_rows(b.down.buf.p, act, parts, nullptr, B, c.embed, c.hidden, shares, m.stream), "ffn_down");
+        }
     }
     LLM_HIP(rows_add_parts(x, parts, shares, B * c.embed, m.stream), "residual");
     return MI355X_OK;
@@ -766,6 +781,8 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         const size_t ab = q4_0_rows_act_bytes(kmax);
         LLM_HIP(m->rows_act.alloc(ab), "hipMalloc(activations)");
         LLM_HIP(hipMemset(m->rows_act.p, 0, ab), "hipMemset(activations)");  // rows past the batch stay zero
+        LLM_HIP(m->rows_act2.alloc(ab), "hipMalloc(activations)");
+        LLM_HIP(hipMemset(m->rows_act2.p, 0, ab), "hipMemset(activations)");
         LLM_HIP(m->parts.alloc((size_t)2 * c.batch * c.embed * 4), "hipMalloc");
     }
     m->ready = true;
@@ -878,7 +895,7 @@ mi355x_status mi355x_llama_generate(void* model, const int32_t* prompt, int64_t 
             LLM_HIP(advance(m->state.as<int32_t>(), m->next_tok.as<int32_t>(), m->record.as<int32_t>(), (int)B, 1, m->stream), "advance");
             return MI355X_OK;
         };
-        const bool rows_now = m->rows && !g_llama_rows_off;
+        const int rows_now = m->rows && !g_llama_rows_off ? 1 + g_llama_rows_plain : 0;
         if (m->step_graph && m->graph_rows != rows_now) {  // the measurement aid changed which step runs
             (void)hipGraphExecDestroy(m->step_graph);
             m->step_graph = nullptr;

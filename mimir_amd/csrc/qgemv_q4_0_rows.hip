@@ -32,6 +32,7 @@
 #include "device_util.h"
 #include "kernels.h"
 #include "q4_rows_act.h"
+#include "rope_tail.h"
 
 namespace mimir {
 
@@ -245,19 +246,33 @@ constexpr int kSlabStride = kRunBytes + 32;     // bytes between rows of a wavef
 constexpr int kSlabBytes = 32 * kSlabStride;
 constexpr int kWaveLds = kSlabBytes + kRunBlocks * kTailBytes;  // the slab, then the run's scales and sums of x
 
+enum RowsTail { kRowsPlain = 0, kRowsRope = 1, kRowsSwiGLU = 2 };
+
+// What the tails need beside the job.
+struct RowsTailArgs {
+    Q4RopeTail rope;              // kRowsRope: the three matrices are q, k, v; y gets the rotated queries, the caches k and v
+    uint8_t* act_out = nullptr;   // kRowsSwiGLU: the two matrices are gate and up; SiLU(gate) * up converted for the next product
+    int nb_out = 0;               //   whose rows have nb_out blocks
+};
+
 // gridDim.y shares of K: with more than one, share s writes its sums to y + s * M * N and nothing is added
 // (a later kernel adds the shares in their order); resid only with one share.
-template <int WAVES>  // wavefronts of a workgroup, among which the runs of its share of K go round
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
+// TAIL: kRowsRope, the rotation of a decoding step and its cache writes on the results (rope_kv's arithmetic,
+// interleaved pairs); kRowsSwiGLU, a workgroup multiplies its 32 rows of gate and of up and leaves SiLU(gate) * up
+// (swiglu_kernel's arithmetic) converted as block blockIdx.x of the next product's x. One share for both.
+template <int WAVES, int TAIL>  // WAVES: wavefronts of a workgroup, among which the runs of its share of K go round
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(TAIL == kRowsSwiGLU ? 3 : 4))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
                                                                        float* y, const float* resid,  // resid may be y
-                                                                       int M, int nb) {
+                                                                       int M, int nb, const RowsTailArgs tail_args) {
     extern __shared__ __align__(16) uint8_t smem[];  // per wavefront: slab and tail of its run; later the wavefronts' sums
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: what depends on it alone is scalar arithmetic
     // up to three matrices, their rows one after the other in y: this workgroup's, and its first row there
     int g = blockIdx.x, which = 0;
-    if (g >= job.groups[0]) { g -= job.groups[0]; which = 1; }
-    if (which == 1 && g >= job.groups[1]) { g -= job.groups[1]; which = 2; }
+    if (TAIL != kRowsSwiGLU) {
+        if (g >= job.groups[0]) { g -= job.groups[0]; which = 1; }
+        if (which == 1 && g >= job.groups[1]) { g -= job.groups[1]; which = 2; }
+    }
     const uint8_t* __restrict__ W = which == 0 ? job.W[0] : which == 1 ? job.W[1] : job.W[2];
     const int N = which == 0 ? job.n[0] : which == 1 ? job.n[1] : job.n[2];
     const int ybase = which == 0 ? 0 : which == 1 ? job.n[0] : job.n[0] + job.n[1];
@@ -280,27 +295,26 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
         goff[i] = (uint32_t)(row - n0) * (uint32_t)(nb * 18) + 16 * c;  // rows of W below 2^32 bytes apart from the first (checked by the host)
         loff[i] = r * kSlabStride + 16 * c;
     }
-    const uint8_t* wbase = W + (int64_t)n0 * nb * 18;
-    const uint8_t* base4;
-    int64_t stride4;
+    const int64_t group_bytes = (int64_t)n0 * nb * 18;
+    int64_t off4, stride4;  // the fifth load: relative to the matrix for the lower lanes, to act for the upper
     if (lane < 32) {
         const int p = 256 + lane, r = p / 9, c = p - 9 * r;
         const int row = n0 + r < N ? n0 + r : N - 1;
-        base4 = wbase + (int64_t)(row - n0) * nb * 18 + 16 * c;
+        off4 = group_bytes + (int64_t)(row - n0) * nb * 18 + 16 * c;
         stride4 = kRunBytes;
         loff[4] = r * kSlabStride + 16 * c;
     } else {
-        base4 = act + (int64_t)nb * kFragBytes + 16 * (lane - 32);
+        off4 = (int64_t)nb * kFragBytes + 16 * (lane - 32);
         stride4 = kRunBlocks * kTailBytes;
         loff[4] = kSlabBytes + 16 * (lane - 32);
     }
 
     struct Run { u32x4 w[5]; };
-    auto fetch_w = [&](Run& f, int run) {
-        const uint8_t* p = wbase + (int64_t)run * kRunBytes;
+    auto fetch_w = [&](Run& f, const uint8_t* wm, int run) {
+        const uint8_t* p = wm + group_bytes + (int64_t)run * kRunBytes;
 #pragma unroll
         for (int i = 0; i < 4; i++) f.w[i] = *(const u32x4*)(p + goff[i]);
-        f.w[4] = *(const u32x4*)(base4 + run * stride4);
+        f.w[4] = *(const u32x4*)((lane < 32 ? wm : act) + off4 + run * stride4);
     };
     struct XPair { i32x4 a, b; };
     auto fetch_x = [&](XPair& f, int step) {  // blocks 2 step and 2 step + 1
@@ -309,10 +323,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
         f.b = *(const i32x4*)(p + kFragBytes + xlane);
     };
 
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     const uint8_t* tail = slab + kSlabBytes + 16 * lh;
     // c: a block's digit sums against the nibbles; lane: row l32 of W, rows 4 lh + j of x. b: block of the run.
-    auto finish = [&](const i32x16& c, float dw, int b) {
+    auto finish = [&](float (&acc)[4], const i32x16& c, float dw, int b) {
         const f32x4 dx = *(const f32x4*)(tail + b * kTailBytes);
         const i32x4 off = *(const i32x4*)(tail + b * kTailBytes + 32);
 #pragma unroll
@@ -329,7 +342,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
     Run cur, nxt;
     XPair xs[4];
     if (run0 < run_end) {
-        fetch_w(cur, run0);
+        fetch_w(cur, W, run0);
 #pragma unroll
         for (int u = 0; u < 4; u++) fetch_x(xs[u], 4 * run0 + u);
     }
@@ -338,9 +351,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
     const uint8_t* mine = slab + l32 * kSlabStride + 20 * lh;
     const uint8_t* mine_d = slab + l32 * kSlabStride + 16 * lh;
     const uint32_t shift = lh ? 0u : 16u;
-    for (int run = run0; run < run_end; run += WAVES) {
-        const int nrun = run + WAVES < run_end ? run + WAVES : run;
-        fetch_w(nxt, nrun);
+    // One run of `cur` into acc, with the run (wn, nrun) requested for afterwards.
+    auto one_run = [&](float (&acc)[4], const uint8_t* wn, int nrun) {
+        fetch_w(nxt, wn, nrun);
         // slab and tail are this wavefront's alone: every lane's reads of the last run were waited for before
         // its last MFMAs and FMAs, and a wavefront's LDS operations complete in order
 #pragma unroll
@@ -372,15 +385,38 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
             // both products are issued before the first one's sums are touched
             const i32x16 ca = __builtin_amdgcn_mfma_i32_32x32x32_i8(xp.a, wa, zero, 0, 0, 0);
             const i32x16 cb = __builtin_amdgcn_mfma_i32_32x32x32_i8(xp.b, wb, zero, 0, 0, 0);
-            finish(ca, f16_bits_to_f32((uint16_t)dd[0]), 2 * j);
-            finish(cb, f16_bits_to_f32((uint16_t)dd[1]), 2 * j + 1);
+            finish(acc, ca, f16_bits_to_f32((uint16_t)dd[0]), 2 * j);
+            finish(acc, cb, f16_bits_to_f32((uint16_t)dd[1]), 2 * j + 1);
         }
         cur = nxt;
+    };
+
+    // this wavefront's runs one after the other; with the SwiGLU tail, the same runs of up after those of gate
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, gate_acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const int mine_runs = run0 < run_end ? (run_end - run0 + WAVES - 1) / WAVES : 0;
+    const int items = TAIL == kRowsSwiGLU ? 2 * mine_runs : mine_runs;
+    for (int it = 0; it < items; it++) {
+        if (TAIL == kRowsSwiGLU && it == mine_runs) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                gate_acc[j] = acc[j];
+                acc[j] = 0.f;
+            }
+        }
+        int nx = it + 1 < items ? it + 1 : it;  // the item requested ahead
+        const uint8_t* wn = TAIL == kRowsSwiGLU && nx >= mine_runs ? job.W[1] : W;
+        if (nx >= mine_runs) nx -= mine_runs;
+        one_run(acc, wn, run0 + nx * WAVES);
     }
 
     __syncthreads();  // every wavefront is done with its slab
     f32x4* red = (f32x4*)smem;
-    red[wave * 64 + lane] = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    if (TAIL == kRowsSwiGLU) {
+        red[wave * 64 + lane] = f32x4{gate_acc[0], gate_acc[1], gate_acc[2], gate_acc[3]};
+        red[(WAVES + wave) * 64 + lane] = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    } else {
+        red[wave * 64 + lane] = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    }
     __syncthreads();
     if (wave != 0) return;
     f32x4 sum = red[lane];
@@ -390,16 +426,98 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4)))
 #pragma unroll
         for (int j = 0; j < 4; j++) sum[j] = sum[j] + t[j];
     }
-    if (n < N) {
-        float* yo = y + (int64_t)blockIdx.y * M * ny + ybase;
+    if (TAIL == kRowsPlain) {
+        if (n < N) {
+            float* yo = y + (int64_t)blockIdx.y * M * ny + ybase;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int m = 4 * lh + j;
+                if (m < M) {
+                    float v = sum[j];
+                    if (resid) v = v + resid[(int64_t)m * ny + ybase + n];
+                    yo[(int64_t)m * ny + n] = v;
+                }
+            }
+        }
+    } else if (TAIL == kRowsRope) {
+        // rows (n, n + 1), n even, are a pair of features: the even lane takes its neighbour's sums and stores both
+        const int pos = *tail_args.rope.pos;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
+            const float other = dpp_f32<0xb1>(sum[j]);  // quad_perm [1,0,3,2]
             const int m = 4 * lh + j;
-            if (m < M) {
-                float v = sum[j];
-                if (resid) v = v + resid[(int64_t)m * ny + ybase + n];
-                yo[(int64_t)m * ny + n] = v;
+            if ((lane & 1) == 0 && n < N && m < M) q4_rope_store(tail_args.rope, pos, m, ybase + n, sum[j], other, y + (int64_t)m * ny);
+        }
+    } else {
+        f32x4 up = red[WAVES * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) {
+            const f32x4 t = red[(WAVES + w) * 64 + lane];
+#pragma unroll
+            for (int j = 0; j < 4; j++) up[j] = up[j] + t[j];
+        }
+        // this workgroup's 32 results of row m are block blockIdx.x of the next product's row m: the lanes of a half
+        // hold its elements. Largest magnitude and sum over the half's 32 lanes, digits through LDS into the operand's
+        // 16-byte pieces (lane 32 h + 8 d + m of the block: digit d of elements 16 h.. of row m).
+        uint8_t* stage = smem + 2 * WAVES * 64 * 16;  // 64 pieces
+        const float nl2e = (float)(-1.4426950408889634);
+        float scale_j[4];
+        int sum_j[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float v = 0.f;
+            if (n < N) {
+                const float e = __builtin_exp2f(sum[j] * nl2e);
+                const float sg = 1.0f / (1.0f + e);
+                const float a = sum[j] * sg;
+                v = a * up[j];
             }
+            // magnitudes as integers order like the floats, with infinities and NaNs above every finite value
+            uint32_t mag = __builtin_bit_cast(uint32_t, v) & 0x7fffffffu;
+            mag = max(mag, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mag, 0xb1, 0xf, 0xf, true));
+            mag = max(mag, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mag, 0x4e, 0xf, 0xf, true));
+            mag = max(mag, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mag, 0x141, 0xf, 0xf, true));
+            mag = max(mag, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mag, 0x140, 0xf, 0xf, true));
+            mag = max(mag, (uint32_t)__builtin_amdgcn_ds_swizzle((int)mag, 0x401F));  // lane ^ 16
+            const float amax = __builtin_bit_cast(float, mag);
+            float scale, inv;
+            if (mag >= 0x7f800000u) {  // a NaN or an infinity in the block: its products are NaN
+                scale = __builtin_nanf("");
+                inv = 0.f;
+                v = 0.f;
+            } else if (amax < 0x1p-100f) {
+                scale = 0.f;
+                inv = 0.f;
+            } else {
+                scale = amax / (float)kFixMax;
+                inv = (float)kFixMax / amax;
+            }
+            int a = (int)__builtin_rintf(v * inv);
+            a = a > kFixMax ? kFixMax : a < -kFixMax ? -kFixMax : a;
+            int t = a;
+            t += __builtin_amdgcn_update_dpp(0, t, 0xb1, 0xf, 0xf, true);
+            t += __builtin_amdgcn_update_dpp(0, t, 0x4e, 0xf, 0xf, true);
+            t += __builtin_amdgcn_update_dpp(0, t, 0x141, 0xf, 0xf, true);
+            t += __builtin_amdgcn_update_dpp(0, t, 0x140, 0xf, 0xf, true);
+            t += __builtin_amdgcn_ds_swizzle(t, 0x401F);
+            scale_j[j] = scale;
+            sum_j[j] = t;
+            const int d0 = (int)(int8_t)a;
+            const int a1 = (a - d0) >> 8;
+            const int d1 = (int)(int8_t)a1;
+            const int d2 = (a1 - d1) >> 8;
+            const int m = 4 * lh + j;
+            uint8_t* at = stage + (32 * (l32 >> 4) + m) * 16 + (l32 & 15);
+            at[0] = (uint8_t)d0;
+            at[8 * 16] = (uint8_t)d1;
+            at[16 * 16] = (uint8_t)d2;
+        }
+        uint8_t* out = tail_args.act_out + (int64_t)blockIdx.x * kFragBytes;
+        if ((lane & 31) < 24) *(u32x4*)(out + 16 * lane) = *(const u32x4*)(stage + 16 * lane);
+        if (l32 == 0) {
+            uint8_t* to = tail_args.act_out + (int64_t)tail_args.nb_out * kFragBytes + (int64_t)blockIdx.x * kTailBytes;
+            *(f32x4*)(to + 16 * lh) = f32x4{scale_j[0], scale_j[1], scale_j[2], scale_j[3]};
+            *(i32x4*)(to + 32 + 16 * lh) = i32x4{8 * sum_j[0], 8 * sum_j[1], 8 * sum_j[2], 8 * sum_j[3]};
         }
     }
 }
@@ -570,6 +688,22 @@ bool qgemv_q4_0_rows_ok(const void* W, int64_t M, int64_t N, int64_t K) {
            (qgemv_q4_0_rows_shares_ok(W, M, N, K, 1) || (size_t)(K / 32) * kTailBytes + kWaves * 64 * 16 <= 64 * 1024);
 }
 
+// Many workgroups: four wavefronts each, so that all are resident at once and each wavefront has runs to request
+// ahead of; few: eight, for the parallelism.
+static hipError_t launch_rows(const RowsJob& job, unsigned groups, int shares, int tail, const RowsTailArgs& t, const void* act, float* y,
+                              const float* resid, int64_t M, int64_t K, hipStream_t st) {
+    const bool four = tail != kRowsSwiGLU && (g_rows_waves == 4 || (g_rows_waves == 0 && (int64_t)groups * shares >= 384));
+    const dim3 grid(groups, (unsigned)shares);
+#define ROWS_LAUNCH(WV, TL)                                                                                                       \
+    hipLaunchKernelGGL((qgemv_q4_0_rows_kernel<WV, TL>), grid, dim3(64 * WV), (size_t)WV * kWaveLds, st, job, (const uint8_t*)act, y, \
+                       resid, (int)M, (int)(K / 32), t)
+    if (tail == kRowsSwiGLU) ROWS_LAUNCH(4, kRowsSwiGLU);
+    else if (tail == kRowsRope) { if (four) ROWS_LAUNCH(4, kRowsRope); else ROWS_LAUNCH(8, kRowsRope); }
+    else { if (four) ROWS_LAUNCH(4, kRowsPlain); else ROWS_LAUNCH(8, kRowsPlain); }
+#undef ROWS_LAUNCH
+    return hipGetLastError();
+}
+
 // act: q4_0_rows_convert_act's buffer. y[M, N] = x . W^T (+ resid, which may be y itself). With shares > 1
 // (qgemv_q4_0_rows_shares_ok, no resid): y[shares, M, N], share s of K summed into y[s].
 hipError_t qgemv_q4_0_rows(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, int shares,
@@ -608,16 +742,39 @@ hipError_t qgemv_q4_0_rows_multi(const void* const W[3], const int64_t n[3], con
         if (n[i] == 0 && i < last) return hipErrorInvalidValue;
     }
     if (last < 0 || (shares > 1 && resid)) return hipErrorInvalidValue;
-    // Many workgroups: four wavefronts each, so that all are resident at once and each wavefront has runs
-    // to request ahead of; few: eight, for the parallelism.
-    const bool four = g_rows_waves == 4 || (g_rows_waves == 0 && (int64_t)groups * shares >= 384);
-    if (four)
-        hipLaunchKernelGGL(qgemv_q4_0_rows_kernel<4>, dim3(groups, (unsigned)shares), dim3(256), (size_t)4 * kWaveLds, st, job,
-                           (const uint8_t*)act, y, resid, (int)M, (int)(K / 32));
-    else
-        hipLaunchKernelGGL(qgemv_q4_0_rows_kernel<8>, dim3(groups, (unsigned)shares), dim3(512), (size_t)8 * kWaveLds, st, job,
-                           (const uint8_t*)act, y, resid, (int)M, (int)(K / 32));
-    return hipGetLastError();
+    return launch_rows(job, groups, shares, kRowsPlain, RowsTailArgs{}, act, y, resid, M, K, st);
+}
+
+// q, k and v in one launch with the rotation and the cache writes of a decoding step as its tail: y [M, n[0] + n[1] + n[2]]
+// receives the rotated queries only (interleaved pairs, even row counts).
+hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], const void* act, float* y, int64_t M, int64_t K,
+                                    const Q4RopeTail& rope, hipStream_t st) {
+    RowsJob job;
+    unsigned groups = 0;
+    for (int i = 0; i < 3; i++) {
+        if (n[i] <= 0 || n[i] % 32 != 0 || !qgemv_q4_0_rows_shares_ok(W[i], M, n[i], K, 1)) return hipErrorInvalidValue;
+        job.W[i] = (const uint8_t*)W[i];
+        job.n[i] = (int)n[i];
+        job.groups[i] = (int)(n[i] / 32);
+        groups += (unsigned)job.groups[i];
+    }
+    RowsTailArgs t;
+    t.rope = rope;
+    return launch_rows(job, groups, 1, kRowsRope, t, act, y, nullptr, M, K, st);
+}
+
+// SiLU(x . gate^T) * (x . up^T), gate and up [N, K], converted into act_out as the x of a product over N (N a multiple of 32).
+hipError_t qgemv_q4_0_rows_swiglu_act(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N, int64_t K,
+                                      hipStream_t st) {
+    if (N % 32 != 0 || !qgemv_q4_0_rows_shares_ok(gate, M, N, K, 1) || !qgemv_q4_0_rows_shares_ok(up, M, N, K, 1)) return hipErrorInvalidValue;
+    RowsJob job;
+    job.W[0] = (const uint8_t*)gate; job.W[1] = (const uint8_t*)up; job.W[2] = nullptr;
+    job.n[0] = (int)N; job.n[1] = 0; job.n[2] = 0;
+    job.groups[0] = (int)(N / 32); job.groups[1] = job.groups[2] = 0;
+    RowsTailArgs t;
+    t.act_out = (uint8_t*)act_out;
+    t.nb_out = (int)(N / 32);
+    return launch_rows(job, (unsigned)(N / 32), 1, kRowsSwiGLU, t, act, nullptr, nullptr, M, K, st);
 }
 
 }  // namespace mimir

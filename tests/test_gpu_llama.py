@@ -222,8 +222,9 @@ def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, ca
 @pytest.mark.parametrize("batch", [2, 5, 8])
 def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
     """Two to eight sequences decode with products that read each weight once for all of them (int8 matrix
-    cores, the output and down projections cut into two shares of K that the next norm adds). Their
-    integers are those of the one-sequence kernels, only float32 sums are ordered differently, so the tokens
+    cores, the output and down projections cut into two shares of K that the next norm adds; the rotation
+    with the cache writes and SiLU * up with its conversion ride on the products, or run as launches of
+    their own). Their integers are those of the one-sequence kernels, only float32 sums are ordered differently, so the tokens
     must be those of the one-sequence kernels run per sequence (llama.rows = 1), of the per-operator path,
     and, up to near-ties, the oracle's."""
     lib = gpu.lib()
@@ -235,8 +236,8 @@ def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
     prompts = np.random.default_rng(17).integers(0, c.vocab, (batch, 11))
     runs = {}
     try:
-        for name, key, v in (("rows graph", b"llama.rows", 0), ("rows launches", b"llama.step", 1), ("per sequence", b"llama.rows", 1),
-                             ("per operator", b"llama.step", 2)):
+        for name, key, v in (("rows graph", b"llama.rows", 0), ("rows launches", b"llama.step", 1), ("rows without riders", b"llama.rows", 2),
+                             ("per sequence", b"llama.rows", 1), ("per operator", b"llama.step", 2)):
             capi.check(lib.mi355x_tune(b"llama.rows", 0))
             capi.check(lib.mi355x_tune(b"llama.step", 0))
             capi.check(lib.mi355x_tune(key, v))
@@ -248,7 +249,7 @@ def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
     finally:
         capi.check(lib.mi355x_tune(b"llama.rows", 0))
         capi.check(lib.mi355x_tune(b"llama.step", 0))
-    for name in ("rows launches", "per sequence", "per operator"):
+    for name in ("rows launches", "rows without riders", "per sequence", "per operator"):
         assert np.array_equal(runs["rows graph"], runs[name]), (name, runs["rows graph"], runs[name])
     for b in range(batch):
         want, margins = om.generate(prompts[b].tolist(), 30, capacity=c.context, cache_dtype=O.F16)
