@@ -262,6 +262,51 @@ def bench_blocks_kquant(rng, dtype_bytes, n_elems):
     return raw.reshape(-1)
 
 
+def rows_bench(lib, capi, torch, m=8, shapes=((14336, 4096), (4096, 14336), (4096, 4096), (6144, 4096), (28672, 4096)), iters=200, only=None):
+    """The Q4_0 product of a few rows of x (a decoding step of a batch), mi355x_qgemv as a whole (conversion
+    of x and product, two launches) over rotating copies of W: the kernel that reads W once for eight rows
+    on the int8 matrix cores, its variant that loads each lane's block where it lies, and the one-row kernel
+    run per row. `only` (a variant's name): a few launches of that variant and nothing else, for counter runs."""
+    rng = np.random.default_rng(0)
+    st = torch.cuda.Stream()
+    out = {}
+    variants = (("rows_kernel", 0), ("rows_kernel_no_lds_pass", 2), ("one_row_kernel_per_row", 1))
+    try:
+        for n, k in shapes:
+            raw = bench_blocks_q4_0(rng, n * k)
+            nbuf = max(2, min(32, int(300e6 // raw.size)))
+            w0 = torch.from_numpy(raw).to("cuda:0")
+            bufs = [w0] + [w0.clone() for _ in range(nbuf - 1)]
+            x = torch.randn(m, k, device="cuda:0")
+            y = torch.empty(m, n, device="cuda:0")
+            torch.cuda.synchronize()
+            res = {}
+            for name, path in variants:
+                if only and name != only:
+                    continue
+                capi.check(lib.mi355x_tune(b"q4_0.rows_path", path))
+                with torch.cuda.stream(st):
+                    call = lambda i: capi.check(lib.mi355x_qgemv(capi.Q4_0, bufs[i % nbuf].data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, st.cuda_stream))
+                    for i in range(4 if only else 10):
+                        call(i)
+                    st.synchronize()
+                    if only:
+                        continue
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(st)
+                    for i in range(iters):
+                        call(i)
+                    e1.record(st)
+                    st.synchronize()
+                us = e0.elapsed_time(e1) / iters * 1e3
+                res[name] = {"us": round(us, 2), "W_GBps": round(raw.size / (us * 1e-6) / 1e9, 1)}
+            out[f"M{m}_N{n}_K{k}"] = res
+            del bufs, w0, x, y
+    finally:
+        capi.check(lib.mi355x_tune(b"q4_0.rows_path", 0))
+    return out
+
+
 def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096), (2048, 14336)), k=4096, iters=50):
     """The prompt-sized products with bfloat16 activations and results, mi355x_qgemm_bf16 as a whole
     (for Q4_K and Q6_K that includes the casts and the int8 rounding of x): TFLOP/s (2 M N K) between
@@ -369,6 +414,10 @@ def main():
     ap.add_argument("--counters", type=int, default=0, metavar="N",
                     help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
     ap.add_argument("--gemm", action="store_true", help="also time the prompt-sized Q4_0 product on the matrix cores (M = 512, 2048)")
+    ap.add_argument("--rows", action="store_true", help="also time the Q4_0 product of eight rows of x (a batch's decoding step) at the model's shapes")
+    ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
+                    help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
+                         "rows_kernel, rows_kernel_no_lds_pass or one_row_kernel_per_row")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
@@ -389,6 +438,10 @@ def main():
         raise SystemExit("bench.py: no GPU visible")
     capi.check(lib.mi355x_init(0))
 
+    if args.rows_counters:
+        rows_bench(lib, capi, torch, shapes=((14336, 4096),), only=args.rows_counters)
+        print(json.dumps({"rows_counters": args.rows_counters, "launches": 4, "W_bytes": 14336 * 4096 // 32 * 18}))
+        return
     n, k = 14336, 4096
     g = Gemv(lib, capi, torch, n, k, args.bufs)
     g.check()
@@ -450,6 +503,8 @@ def main():
     del g
     if args.gemm:
         out["prefill_gemm"] = gemm_bench(lib, capi, torch)
+    if args.rows:
+        out["batch_rows_gemv"] = rows_bench(lib, capi, torch)
     if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check if args.decode_linear == "q4_0" else 0,
                                      linear=args.decode_linear)
