@@ -87,9 +87,11 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * reference takes for that file dtype (io/mim/dtype.go:118-123).
  * One entry point for every M, as OpQMatMul is one operation: by dtype and
  * shape the library runs row kernels (few rows of x; one launch for one row of
- * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix) or, from enough rows on, kernels on the
- * int8 matrix cores (Q4_0, Q4_K, Q6_K); which one ran changes the results only
- * by the order of float32 additions (Q4_0, Q8_0) or not at all (Q4_K, Q6_K). */
+ * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix; Q8_0 weights are read
+ * once for up to eight rows) or kernels on the int8 matrix cores (Q4_0 from two
+ * rows on, which read W once for eight rows; Q4_K, Q6_K from enough rows on);
+ * which one ran changes the results only by the order of float32 additions
+ * (Q4_0), or not at all (Q8_0 among its row kernels, Q4_K, Q6_K). */
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
 
@@ -285,6 +287,10 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
  * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
  * kernel, 2 puts them all on the kernel that shares W among rows of x.
+ * "q4_0.rows_path" = 1 keeps Q4_0 and Q8_0 products of two to fifteen rows of
+ * x off the kernels that read W once for eight rows, 2 selects the Q4_0 one's
+ * variant without the pass through LDS; "q4_0.rows_waves" = 4 or 8 fixes its
+ * wavefronts a workgroup.
  * "attention.splits" = n fixes the shares of the keys in decode attention.
  * "q4_0.fx_rows" = n sends Q4_0 products of at least n rows of float32 x to the
  * int8 matrix cores whatever the shape (0: the built-in cost model).
@@ -298,7 +304,10 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * "llama.step" chooses how mi355x_llama_generate runs its decoding steps: 0 the
  * fused launches replayed as a HIP graph where every block's linears are Q4_0
  * (else the per-operator path), 1 the same launches without the graph, 2 the
- * per-operator path always. */
+ * per-operator path always. "llama.rows" = 1 makes two to eight sequences decode
+ * with the one-sequence kernels run per sequence instead of the step that reads
+ * every weight once for all of them, 2 keeps that step but runs the rotation
+ * and SwiGLU as launches of their own (3, 4: only SwiGLU, only the rotation). */
 MI355X_API mi355x_status mi355x_tune(const char* key, int value);
 /* Between timed_begin and timed_end, each launch of the fixed-point Q4_0 GEMV
  * kernel made by the calling thread (at most max_launches of them; not under
