@@ -261,7 +261,7 @@ struct RowsTailArgs {
 // interleaved pairs); kRowsSwiGLU, a workgroup multiplies its 32 rows of gate and of up and leaves SiLU(gate) * up
 // (swiglu_kernel's arithmetic) converted as block blockIdx.x of the next product's x. One share for both.
 template <int WAVES, int TAIL>  // WAVES: wavefronts of a workgroup, among which the runs of its share of K go round
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(TAIL == kRowsSwiGLU ? 3 : 4))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
                                                                        float* y, const float* resid,  // resid may be y
                                                                        int M, int nb, const RowsTailArgs tail_args) {
     extern __shared__ __align__(16) uint8_t smem[];  // per wavefront: slab and tail of its run; later the wavefronts' sums
@@ -324,10 +324,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(TAIL
     };
 
     const uint8_t* tail = slab + kSlabBytes + 16 * lh;
-    // c: a block's digit sums against the nibbles; lane: row l32 of W, rows 4 lh + j of x. b: block of the run.
-    auto finish = [&](float (&acc)[4], const i32x16& c, float dw, int b) {
-        const f32x4 dx = *(const f32x4*)(tail + b * kTailBytes);
-        const i32x4 off = *(const i32x4*)(tail + b * kTailBytes + 32);
+    // c: a block's digit sums against the nibbles; lane: row l32 of W, rows 4 lh + j of x. dx, off: the block's scales and 8 * sums of x.
+    auto finish = [&](float (&acc)[4], const i32x16& c, float dw, const f32x4 dx, const i32x4 off) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             // sum of x (n - 8), below 2^31 in magnitude (32 * 8 * kFixMax); the partial terms may wrap
@@ -358,14 +356,19 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(TAIL
         // its last MFMAs and FMAs, and a wavefront's LDS operations complete in order
 #pragma unroll
         for (int i = 0; i < 5; i++) *(u32x4*)(slab + loff[i]) = cur.w[i];
+        // The LDS reads of a step are issued a step ahead of their use, the scales and sums of x before the
+        // MFMAs whose results they meet: a wavefront has few neighbours on its SIMD to fill its waits with.
+        uint32_t r[5], dword;
+        auto read_block = [&](int j) {
+#pragma unroll
+            for (int i = 0; i < 5; i++) r[i] = *(const uint32_t*)(mine + 36 * j + 4 * i);
+            dword = *(const uint32_t*)(mine_d + 36 * j);
+        };
+        read_block(0);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const XPair xp = xs[j];
             fetch_x(xs[j], 4 * nrun + j);
-            uint32_t r[5];
-#pragma unroll
-            for (int i = 0; i < 5; i++) r[i] = *(const uint32_t*)(mine + 36 * j + 4 * i);
-            const uint32_t dword = *(const uint32_t*)(mine_d + 36 * j);
             i32x4 wa, wb;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -379,14 +382,17 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(TAIL
             // float in place, this compiler read the first of the two for both)
             const uint32_t dbits = (dword >> (16 - shift)) & 0xffffu;
             const auto dd = __builtin_amdgcn_permlane32_swap(dbits, dbits, false, false);
+            if (j < 3) read_block(j + 1);
+            const f32x4 dxa = *(const f32x4*)(tail + (2 * j) * kTailBytes), dxb = *(const f32x4*)(tail + (2 * j + 1) * kTailBytes);
+            const i32x4 offa = *(const i32x4*)(tail + (2 * j) * kTailBytes + 32), offb = *(const i32x4*)(tail + (2 * j + 1) * kTailBytes + 32);
             i32x16 zero;
 #pragma unroll
             for (int i = 0; i < 16; i++) zero[i] = 0;
             // both products are issued before the first one's sums are touched
             const i32x16 ca = __builtin_amdgcn_mfma_i32_32x32x32_i8(xp.a, wa, zero, 0, 0, 0);
             const i32x16 cb = __builtin_amdgcn_mfma_i32_32x32x32_i8(xp.b, wb, zero, 0, 0, 0);
-            finish(acc, ca, f16_bits_to_f32((uint16_t)dd[0]), 2 * j);
-            finish(acc, cb, f16_bits_to_f32((uint16_t)dd[1]), 2 * j + 1);
+            finish(acc, ca, f16_bits_to_f32((uint16_t)dd[0]), dxa, offa);
+            finish(acc, cb, f16_bits_to_f32((uint16_t)dd[1]), dxb, offb);
         }
         cur = nxt;
     };
