@@ -89,9 +89,10 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * shape the library runs row kernels (few rows of x; one launch for one row of
  * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix; Q8_0 weights are read
  * once for up to eight rows) or kernels on the int8 matrix cores (Q4_0 from two
- * rows on, which read W once for eight rows; Q4_K, Q6_K from enough rows on);
- * which one ran changes the results only by the order of float32 additions
- * (Q4_0), or not at all (Q8_0 among its row kernels, Q4_K, Q6_K). */
+ * rows on, which read W once for eight rows; two to eight rows by a large Q8_0
+ * matrix; Q4_K, Q6_K from enough rows on); which one ran changes the results
+ * only by the order of float32 additions (Q4_0, Q8_0), or not at all (Q8_0
+ * among its row kernels, Q4_K, Q6_K). */
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
 
@@ -291,6 +292,8 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * x off the kernels that read W once for eight rows, 2 selects the Q4_0 one's
  * variant without the pass through LDS; "q4_0.rows_waves" = 4 or 8 fixes its
  * wavefronts a workgroup.
+ * "q8_0.mfma" = 1 sends every Q8_0 product of two to eight rows of x that the
+ * matrix-core kernel takes to it, 2 none (0: matrices of 64 M weights or more).
  * "attention.splits" = n fixes the shares of the keys in decode attention.
  * "q4_0.fx_rows" = n sends Q4_0 products of at least n rows of float32 x to the
  * int8 matrix cores whatever the shape (0: the built-in cost model).

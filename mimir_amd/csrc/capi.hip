@@ -385,6 +385,10 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
         if (mi355x_status st = act_scratch(mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
         HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
         a.act = act;
+        if (g_rows_path != 1 && mimir::qgemv_q8_0_mfma_pays(a)) {  // a large matrix and two to eight rows: the int8 matrix cores
+            HIP_TRY(mimir::qgemv_q8_0_mfma(a, (hipStream_t)stream), "launch qgemv_q8_0_mfma");
+            return MI355X_OK;
+        }
         if (g_rows_path != 1 && mimir::qgemv_q8_0_rows_ok(a)) {  // several rows: W read once for up to eight of them, the same sums
             HIP_TRY(mimir::qgemv_q8_0_rows(a, (hipStream_t)stream), "launch qgemv_q8_0_rows");
             return MI355X_OK;
@@ -649,6 +653,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     if (key && strcmp(key, "q4_0.rows_path") == 0) {  // 1: off; 2: its kernel without the LDS pass
         g_rows_path = value == 1 ? 1 : 0;
         mimir::set_q4_rows_direct(value == 2);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q8_0.mfma") == 0) {
+        mimir::set_q8_mfma(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.rows_waves") == 0) {

@@ -95,6 +95,13 @@ hipError_t qgemv_q8_0_act(const QGemvArgs& a, const int* tune, hipStream_t st);
 // W 4-byte aligned, an even number of blocks a row, no residual.
 bool qgemv_q8_0_rows_ok(const QGemvArgs& a);
 hipError_t qgemv_q8_0_rows(const QGemvArgs& a, hipStream_t st);
+// Two to eight rows of x on the int8 matrix cores (qgemv_q8_0_mfma.hip): the CPU's integer lane sums, the float32 sums
+// of a row's blocks in another order than the kernels above add them. K a multiple of 256, W 16-byte aligned.
+// qgemv_q8_0_mfma_pays: large enough a matrix for it to be the faster (or as "q8_0.mfma" says: 1 always, 2 never).
+bool qgemv_q8_0_mfma_ok(const QGemvArgs& a);
+bool qgemv_q8_0_mfma_pays(const QGemvArgs& a);
+void set_q8_mfma(int v);
+hipError_t qgemv_q8_0_mfma(const QGemvArgs& a, hipStream_t st);
 
 // The Q4_K and Q6_K products as the reference's CPU computes them: x rounded
 // to int8 in super-blocks of 256 with the sums of each 16 quants

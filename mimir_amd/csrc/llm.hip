@@ -176,7 +176,8 @@ mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_
         break;
     case kQ8_0:
         if (cls != kActQ8) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: q8_0 rows of %lld are too long", (long long)w.k);
-        e = qgemv_q8_0_rows_ok(a) ? qgemv_q8_0_rows(a, m.stream) : qgemv_q8_0_act(a, kNoTune, m.stream);  // several rows: W read once
+        // several rows: W read once, on the matrix cores where the matrix is large
+        e = qgemv_q8_0_mfma_pays(a) ? qgemv_q8_0_mfma(a, m.stream) : qgemv_q8_0_rows_ok(a) ? qgemv_q8_0_rows(a, m.stream) : qgemv_q8_0_act(a, kNoTune, m.stream);
         break;
     case kQ4_K: case kQ6_K: e = qgemv_kquant_act(w.dtype, a, m.stream); break;
     case kF32: case kF16: case kBF16: e = gemv_float(w.dtype, w.buf.p, x, y, rows, w.n, w.k, w.k, m.stream); break;

@@ -427,6 +427,32 @@ def test_q8_0_rows_of_x_share_one_pass_over_w(m, n, k):
     assert bits_equal(got, one)
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 203, 4096), (2, 32, 256), (5, 1000, 1280), (8, 33, 14336), (3, 1, 512)])
+def test_q8_0_rows_on_the_matrix_cores(m, n, k):
+    """Two to eight rows of x against Q8_0 weights on the int8 matrix cores (the head of a batch's decoding
+    step; forced here for small matrices too): the CPU's integer lane sums, float32 sums of a row's
+    blocks in another order, so close to the oracle and to the one-row kernel, not their bits."""
+    l = gpu.lib()
+    rng = np.random.default_rng(3 * m + n + k)
+    raw = random_blocks(rng, O.Q8_0, n * k)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    x[0, :32] = 0
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    try:
+        capi.check(l.mi355x_tune(b"q8_0.mfma", 1))
+        gpu.say(f"q8_0 matrix-core rows kernel M={m} N={n} K={k}")
+        got = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+        capi.check(l.mi355x_tune(b"q8_0.mfma", 2))
+        rows = gpu.qgemv(O.Q8_0, ptr, gpu.dev(x), n, k)
+    finally:
+        capi.check(l.mi355x_tune(b"q8_0.mfma", 0))
+    want = O.qmatmul(O.Q8_0, raw, x, n, k)
+    w = O.dequantize(O.Q8_0, raw).reshape(n, k).astype(np.float64)
+    mag = np.abs(x.astype(np.float64)) @ np.abs(w).T
+    assert np.all(np.abs(got - want) <= 2e-6 * mag + 1e-30)
+    assert np.all(np.abs(got - rows) <= 2e-6 * mag + 1e-30)
+
+
 # ---- Q4_K / Q6_K -------------------------------------------------------------
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
