@@ -251,6 +251,24 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear=
             "first_tokens": out[0, :8].tolist()}
 
 
+def layer_step_bench(capi, cached=2048, new=33):
+    """One decoder layer's decoding step against caches holding `cached` positions (batch 1 and 8): the whole
+    model's step timed with two and with six layers, the difference divided by four, so that embedding, head and
+    argmax drop out. The caches are filled by a prompt of `cached` tokens."""
+    out = {}
+    for batch in (1, 8):
+        ms = {}
+        for layers in (2, 6):
+            m = build_llama(capi, layers=layers, batch=batch, context=cached + new, max_tokens=cached)
+            toks = np.random.default_rng(0).integers(0, m.config.vocab, (batch, cached))
+            _, (_, t_decode) = m.generate(toks, new)
+            ms[layers] = t_decode / (new - 1) * 1e3
+            del m
+        out[f"batch{batch}"] = {"us_per_layer": round((ms[6] - ms[2]) / 4 * 1e3, 2), "ms_per_step_2_layers": round(ms[2], 4), "ms_per_step_6_layers": round(ms[6], 4)}
+    out["cached_positions"] = cached
+    return out
+
+
 def bench_blocks_kquant(rng, dtype_bytes, n_elems):
     """Random Q4_K (144-byte) or Q6_K (210-byte) super-blocks: every field uniform, the binary16 scales |N(0, 0.02)|."""
     raw = rng.integers(0, 256, size=(n_elems // 256, dtype_bytes), dtype=np.uint8)
@@ -418,6 +436,7 @@ def main():
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
                     help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
                          "rows_kernel, rows_kernel_no_lds_pass or one_row_kernel_per_row")
+    ap.add_argument("--layer-step", action="store_true", help="also time one decoder layer's decoding step against 2048 cached positions (batch 1, 8)")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
@@ -505,6 +524,8 @@ def main():
         out["prefill_gemm"] = gemm_bench(lib, capi, torch)
     if args.rows:
         out["batch_rows_gemv"] = rows_bench(lib, capi, torch)
+    if args.layer_step:
+        out["layer_step"] = layer_step_bench(capi)
     if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check if args.decode_linear == "q4_0" else 0,
                                      linear=args.decode_linear)
