@@ -442,6 +442,7 @@ def main():
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
     ap.add_argument("--decode-check", type=int, default=0, metavar="N",
                     help="compare the first N greedy tokens with the CPU oracle's (minutes of CPU time for the 512-token prompt)")
+    ap.add_argument("--no-decode-batch8", action="store_true", help="skip the second decoding run, with eight sequences")
     ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--decode-batch", type=int, default=1)
     ap.add_argument("--decode-linear", choices=("q4_0", "q4_K", "q6_K"), default="q4_0",
@@ -529,6 +530,9 @@ def main():
     if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check if args.decode_linear == "q4_0" else 0,
                                      linear=args.decode_linear)
+        if args.decode_batch == 1 and args.decode_linear == "q4_0" and args.decode_layers == 32 and not args.no_decode_batch8:
+            # the same model with eight sequences: every weight read once a step for all of them
+            out["decode_batch8"] = decode_bench(capi, layers=32, batch=8)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n, k, seconds=10.0)
     print(json.dumps(out), flush=True)
