@@ -419,12 +419,14 @@ static bool tall_tiles(const QGemvArgs& a) {
     return a.M > 128 && ((a.M + 255) / 256) * ((a.N + kTN - 1) / kTN) >= 256;
 }
 
-// The row-by-row kernels read W once per row of x, at about 8 TB/s once it sits in the caches; a
-// workgroup here spends about 2.1 us (5.5 with 256-row tiles) per super-block of K, 256 workgroups
-// at a time. Measured on 4096 x 4096 to 14336 x 4096 weights, 2 to 64 rows.
+// The row-by-row kernels read W once per row of x, at about 5.8 TB/s (Q4_K) or 5.1 TB/s (Q6_K) while it sits in
+// the caches; a workgroup here spends about 2.1 us (5.5 with 256-row tiles) per super-block of K, 256 workgroups
+// at a time. Measured on 4096 x 4096, 4096 x 14336 and 14336 x 4096 weights, 2 to 64 rows (at 14336 x 4096 and
+// eight rows: 49 and 79 us by rows, 35 and 37 us here).
 bool qgemm_kquant_pays(int dt, const QGemvArgs& a) {
-    if (a.M < 8) return false;
-    const double nsb = (double)(a.K / 256), rows_us = (double)a.M * (double)a.N * nsb * (dt == kQ4_K ? 144 : 210) / 8.0e6;
+    if (a.M < 4) return false;
+    const double nsb = (double)(a.K / 256);
+    const double rows_us = (double)a.M * (double)a.N * nsb * (dt == kQ4_K ? 144 : 210) / (dt == kQ4_K ? 5.8e6 : 5.1e6);
     const bool tall = tall_tiles(a);
     const int64_t tiles = ((a.M + (tall ? 255 : 127)) / (tall ? 256 : 128)) * ((a.N + kTN - 1) / kTN);
     return (double)((tiles + 255) / 256) * nsb * (tall ? 5.5 : 2.1) < rows_us;
