@@ -89,7 +89,8 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * shape the library runs row kernels (few rows of x; one launch for one row of
  * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix; Q8_0 weights are read
  * once for up to eight rows) or kernels on the int8 matrix cores (Q4_0 from two
- * rows on, which read W once for eight rows; two to eight rows by a large Q8_0
+ * rows on: up to some tens of rows a kernel that reads W once per eight rows,
+ * beyond them a tiled one; two to eight rows by a large Q8_0
  * matrix; Q4_K, Q6_K from enough rows on); which one ran changes the results
  * only by the order of float32 additions (Q4_0, Q8_0), or not at all (Q8_0
  * among its row kernels, Q4_K, Q6_K). */
@@ -288,10 +289,11 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
  * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
  * kernel, 2 puts them all on the kernel that shares W among rows of x.
- * "q4_0.rows_path" = 1 keeps Q4_0 and Q8_0 products of two to fifteen rows of
- * x off the kernels that read W once for eight rows, 2 selects the Q4_0 one's
- * variant without the pass through LDS; "q4_0.rows_waves" = 4 or 8 fixes its
- * wavefronts a workgroup.
+ * "q4_0.rows_path" = 1 keeps Q4_0 and Q8_0 products of a few rows of x off the
+ * kernels that read W once for eight rows, 2 selects the Q4_0 one's variant
+ * without the pass through LDS; "q4_0.rows_waves" = 4 or 8 fixes its wavefronts
+ * a workgroup; "q4_0.rows_max" = n sends Q4_0 products of fewer than n rows to
+ * it (0: up to where the tiled kernel's cost model undercuts its own).
  * "q8_0.mfma" = 1 sends every Q8_0 product of two to eight rows of x that the
  * matrix-core kernel takes to it, 2 none (0: matrices of 64 M weights or more).
  * "attention.splits" = n fixes the shares of the keys in decode attention.

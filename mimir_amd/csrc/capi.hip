@@ -70,6 +70,7 @@ constexpr int64_t kConvertInProductRows = 8;
 // Rows of x from which the Q4_0 product of float32 x goes to the int8 matrix cores: 16 means wherever its
 // cost model says it pays; "q4_0.fx_rows" sets another threshold, which then holds for every shape.
 int g_fx_min_rows = 16;
+int g_rows_max = 0;    // "q4_0.rows_max" n: Q4_0 products of fewer than n rows of x take the kernel that reads W once per eight rows (0: by cost)
 int g_rows_path = 0;  // "q4_0.rows_path" 1: no matrix-core kernel for two to fifteen rows of x
 int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
@@ -338,6 +339,31 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
     switch (dtype) {
     case MI355X_Q4_0:
         if (g_tune_q4[4] != 1 && mimir::q4_0_fixed_point_ok(W, K)) {
+            // A few rows (the decoding step of a batch): W read once per eight rows of x, on the int8 matrix cores; up to
+            // where the tiled kernel for many rows is the faster by both kernels' measured costs (some tens of rows).
+            const bool wide_x = ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0;
+            const bool fx_forced = g_fx_min_rows != 16 && M >= g_fx_min_rows;
+            bool rows = M >= 2 && g_rows_path != 1 && g_tune_q4[4] != 2 && wide_x && !fx_forced && mimir::qgemv_q4_0_rows_ok(W, 1, N, K);
+            if (rows && g_rows_max > 0) rows = M < g_rows_max;
+            else if (rows && M >= 16 && mimir::qgemm_q4_0_fx_ok(W, M, N, K))
+                rows = mimir::qgemv_q4_0_rows_cost_us(M, N, K) < mimir::qgemm_q4_0_fx_cost_us(M, N, K);
+            if (rows) {
+                const bool one_launch = mimir::qgemv_q4_0_rows_shares_ok(W, M, N, K, 1);  // else the variant that takes eight rows a launch
+                const int64_t groups = (M + 7) / 8;
+                void* act;
+                if (mi355x_status st = act_scratch(mimir::q4_0_rows_act_bytes(K) * (size_t)(one_launch ? groups : 1), &act)) return st;
+                if (one_launch) {
+                    HIP_TRY(mimir::q4_0_rows_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_rows_convert_act");
+                    HIP_TRY(mimir::qgemv_q4_0_rows(W, act, y, nullptr, M, N, K, 1, (hipStream_t)stream), "launch qgemv_q4_0_rows");
+                    return MI355X_OK;
+                }
+                for (int64_t m0 = 0; m0 < M; m0 += 8) {
+                    const int64_t mm = M - m0 < 8 ? M - m0 : 8;
+                    HIP_TRY(mimir::q4_0_rows_convert_act(x + m0 * x_row_stride, mm, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_rows_convert_act");
+                    HIP_TRY(mimir::qgemv_q4_0_rows(W, act, y + m0 * N, nullptr, mm, N, K, 1, (hipStream_t)stream), "launch qgemv_q4_0_rows");
+                }
+                return MI355X_OK;
+            }
             if (g_tune_q4[4] != 2 && M >= g_fx_min_rows && (g_fx_min_rows != 16 ? mimir::qgemm_q4_0_fx_ok(W, M, N, K) : mimir::qgemm_q4_0_fx_pays(W, M, N, K)) &&
                 ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0) {
                 // many rows: the same fixed-point arithmetic on the int8 matrix cores
@@ -345,18 +371,6 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
                 if (mi355x_status st = act_scratch(mimir::q4_0_fx_act_bytes(K) * (size_t)M, &act)) return st;
                 HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_fx_convert_act");
                 HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, (hipStream_t)stream), "launch qgemm_q4_0_fx");
-                return MI355X_OK;
-            }
-            if (M >= 2 && M < 16 && g_rows_path != 1 && g_tune_q4[4] != 2 && ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0 &&
-                mimir::qgemv_q4_0_rows_ok(W, 1, N, K)) {
-                // a few rows (the decoding step of a batch): W read once for eight rows of x, on the int8 matrix cores
-                void* act;
-                if (mi355x_status st = act_scratch(mimir::q4_0_rows_act_bytes(K), &act)) return st;
-                for (int64_t m0 = 0; m0 < M; m0 += 8) {
-                    const int64_t mm = M - m0 < 8 ? M - m0 : 8;
-                    HIP_TRY(mimir::q4_0_rows_convert_act(x + m0 * x_row_stride, mm, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_rows_convert_act");
-                    HIP_TRY(mimir::qgemv_q4_0_rows(W, act, y + m0 * N, nullptr, mm, N, K, 1, (hipStream_t)stream), "launch qgemv_q4_0_rows");
-                }
                 return MI355X_OK;
             }
             if (M == 1 && ((uintptr_t)x & 15) == 0) {
@@ -657,6 +671,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "q8_0.mfma") == 0) {
         mimir::set_q8_mfma(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.rows_max") == 0) {
+        g_rows_max = value > 0 ? value : 0;
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.rows_waves") == 0) {

@@ -197,12 +197,14 @@ size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st,
                             bool act_rows = false);
 
-// The fixed-point Q4_0 product for up to eight rows of float32 x that reads W once (qgemv_q4_0_rows.hip, int8
-// matrix cores): the rows are converted together by q4_0_rows_convert_act into q4_0_rows_act_bytes(K) bytes
+// The fixed-point Q4_0 product of a few rows of float32 x that reads W once per eight of them (qgemv_q4_0_rows.hip,
+// int8 matrix cores): each group of eight rows is converted together by q4_0_rows_convert_act into q4_0_rows_act_bytes(K) bytes,
+// group after group; the plain product takes any number of groups in one launch, its tails and shapes without whole runs one
 // (x 16-byte aligned rows, K a multiple of 64).
 size_t q4_0_rows_act_bytes(int64_t K);
 hipError_t q4_0_rows_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 bool qgemv_q4_0_rows_ok(const void* W, int64_t M, int64_t N, int64_t K);
+double qgemv_q4_0_rows_cost_us(int64_t M, int64_t N, int64_t K);  // about what M rows take, conversion included
 // shares > 1 (qgemv_q4_0_rows_shares_ok; no resid): K is cut into that many shares, whose sums go to y[shares, M, N]
 // for a later kernel to add in their order.
 bool qgemv_q4_0_rows_shares_ok(const void* W, int64_t M, int64_t N, int64_t K, int shares);
@@ -233,7 +235,8 @@ void set_q4_rows_direct(int v);  // measurement aid: 1 = its kernel that loads e
 size_t q4_0_fx_act_bytes(int64_t K);
 hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 bool qgemm_q4_0_fx_ok(const void* W, int64_t M, int64_t N, int64_t K);
-bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K);  // and is the faster choice
+bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K);  // and is the faster choice against the one-row kernels
+double qgemm_q4_0_fx_cost_us(int64_t M, int64_t N, int64_t K);           // about what it takes, conversion aside
 hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
 // Prompt-sized Q4_0 product on the matrix cores (qgemm_q4_0.hip): X [M, K]

@@ -290,11 +290,15 @@ bool qgemm_q4_0_fx_ok(const void* W, int64_t M, int64_t N, int64_t K) {
 // Whether this kernel beats the row kernels: those take about 1 us per row of x and 8.7 MB of W; a
 // workgroup here about 2.8 us per step of 128 of K, 256 workgroups at a time (measured at 4096 x 4096
 // to 14336 x 4096, 32 to 2048 rows).
+double qgemm_q4_0_fx_cost_us(int64_t M, int64_t N, int64_t K) {
+    const int64_t tiles = ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
+    return (double)((tiles + 255) / 256) * (double)(K / kStepK) * 2.8;
+}
+
 bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K) {
     if (M < 16 || !qgemm_q4_0_fx_ok(W, M, N, K)) return false;
     const double rows_us = (double)M * ((double)N * (double)(K / 32) * 18.0) / 8.7e6;
-    const int64_t tiles = ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
-    return (double)((tiles + 255) / 256) * (double)(K / kStepK) * 2.8 < rows_us;
+    return qgemm_q4_0_fx_cost_us(M, N, K) < rows_us;
 }
 
 // act: q4_0_fx_convert_act's rows. y = x . W^T (+ resid, which may be y itself).

@@ -63,8 +63,10 @@ size_t q4_0_rows_act_bytes(int64_t K) { return q4_0_rows_act_size(K); }
 // The integers and scales are those of q4_convert_item and of fx_convert_kernel. Rows from M on are
 // written as zeros, so that a launch always defines the whole buffer.
 __global__ __launch_bounds__(256) void q4_0_rows_convert_kernel(const float* __restrict__ x, int64_t x_row_stride, int M, int K,
-                                                                uint8_t* __restrict__ act) {
-    const int m = blockIdx.y, nb = K >> 5;
+                                                                uint8_t* act) {
+    const int nb = K >> 5;
+    const int m = blockIdx.y + kRows * blockIdx.z;  // row of x; blockIdx.z: its group of eight, converted into a buffer of its own
+    act += (int64_t)blockIdx.z * nb * (kFragBytes + kTailBytes);
     const float* xr = x + (int64_t)(m < M ? m : 0) * x_row_stride;
     uint8_t* tail = act + (int64_t)nb * kFragBytes;
     const int nq = K >> 2;
@@ -112,20 +114,22 @@ __global__ __launch_bounds__(256) void q4_0_rows_convert_kernel(const float* __r
         sum = group8_sum_i32(sum);  // below 2^28
         const int b = t >> 3, q = t & 7;
         uint32_t* frag = (uint32_t*)(act + (int64_t)b * kFragBytes) + (q & 3);
-        const int lane0 = 32 * (q >> 2) + m;
+        const int lane0 = 32 * (q >> 2) + (int)blockIdx.y;
 #pragma unroll
         for (int j = 0; j < 3; j++) frag[4 * (lane0 + 8 * j)] = d[j];
         frag[4 * (lane0 + 24)] = 0;
         if (q == 0) {
-            ((float*)(tail + (int64_t)b * kTailBytes))[m] = scale;
-            ((int32_t*)(tail + (int64_t)b * kTailBytes))[8 + m] = 8 * sum;
+            ((float*)(tail + (int64_t)b * kTailBytes))[blockIdx.y] = scale;
+            ((int32_t*)(tail + (int64_t)b * kTailBytes))[8 + blockIdx.y] = 8 * sum;
         }
     }
 }
 
 hipError_t q4_0_rows_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
     int gx = (int)((K / 4 + 255) / 256);
-    hipLaunchKernelGGL(q4_0_rows_convert_kernel, dim3((unsigned)gx, kRows), dim3(256), 0, st, x, x_row_stride, (int)M, (int)K, (uint8_t*)act);
+    // more than eight rows: a buffer of q4_0_rows_act_bytes(K) per group of eight, one after the other
+    hipLaunchKernelGGL(q4_0_rows_convert_kernel, dim3((unsigned)gx, kRows, (unsigned)((M + kRows - 1) / kRows)), dim3(256), 0, st, x, x_row_stride,
+                       (int)M, (int)K, (uint8_t*)act);
     return hipGetLastError();
 }
 
@@ -261,10 +265,13 @@ struct RowsTailArgs {
 // interleaved pairs); kRowsSwiGLU, a workgroup multiplies its 32 rows of gate and of up and leaves SiLU(gate) * up
 // (swiglu_kernel's arithmetic) converted as block blockIdx.x of the next product's x. One share for both.
 template <int WAVES, int TAIL>  // WAVES: wavefronts of a workgroup, among which the runs of its share of K go round
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act,
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3))) void qgemv_q4_0_rows_kernel(const RowsJob job, const uint8_t* __restrict__ act_all,
                                                                        float* y, const float* resid,  // resid may be y
-                                                                       int M, int nb, const RowsTailArgs tail_args) {
+                                                                       int M_all, int nb, const RowsTailArgs tail_args) {
     extern __shared__ __align__(16) uint8_t smem[];  // per wavefront: slab and tail of its run; later the wavefronts' sums
+    // blockIdx.z: the group of eight rows of x (plain tail only), each converted into a buffer of its own
+    const uint8_t* __restrict__ act = act_all + (int64_t)blockIdx.z * nb * (kFragBytes + kTailBytes);
+    const int M = M_all - kRows * (int)blockIdx.z < kRows ? M_all - kRows * (int)blockIdx.z : kRows;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: what depends on it alone is scalar arithmetic
     // up to three matrices, their rows one after the other in y: this workgroup's, and its first row there
@@ -434,13 +441,14 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
     }
     if (TAIL == kRowsPlain) {
         if (n < N) {
-            float* yo = y + (int64_t)blockIdx.y * M * ny + ybase;
+            const int64_t row0 = (int64_t)kRows * blockIdx.z;
+            float* yo = y + ((int64_t)blockIdx.y * M_all + row0) * ny + ybase;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int m = 4 * lh + j;
                 if (m < M) {
                     float v = sum[j];
-                    if (resid) v = v + resid[(int64_t)m * ny + ybase + n];
+                    if (resid) v = v + resid[(row0 + m) * ny + ybase + n];
                     yo[(int64_t)m * ny + n] = v;
                 }
             }
@@ -679,7 +687,7 @@ void set_q4_rows_waves(int v) { g_rows_waves = v; }
 
 // W 2-byte aligned (ggml blocks), pairs of blocks, at most eight rows of x.
 static bool rows_base_ok(const void* W, int64_t M, int64_t N, int64_t K) {
-    return K > 0 && K % 64 == 0 && K <= (1 << 20) && ((uintptr_t)W & 1) == 0 && M > 0 && M <= kRows && N > 0 && N <= (1ll << 30);
+    return K > 0 && K % 64 == 0 && K <= (1 << 20) && ((uintptr_t)W & 1) == 0 && M > 0 && M <= kRows * 65535 && N > 0 && N <= (1ll << 30);
 }
 
 // Whether the product can be cut into `shares` shares of K whose sums a later kernel adds: the kernel that
@@ -694,12 +702,14 @@ bool qgemv_q4_0_rows_ok(const void* W, int64_t M, int64_t N, int64_t K) {
            (qgemv_q4_0_rows_shares_ok(W, M, N, K, 1) || (size_t)(K / 32) * kTailBytes + kWaves * 64 * 16 <= 64 * 1024);
 }
 
+static int64_t grid_z(int64_t M) { return (M + kRows - 1) / kRows; }
+
 // Many workgroups: four wavefronts each, so that all are resident at once and each wavefront has runs to request
 // ahead of; few: eight, for the parallelism.
 static hipError_t launch_rows(const RowsJob& job, unsigned groups, int shares, int tail, const RowsTailArgs& t, const void* act, float* y,
                               const float* resid, int64_t M, int64_t K, hipStream_t st) {
-    const bool four = tail != kRowsSwiGLU && (g_rows_waves == 4 || (g_rows_waves == 0 && (int64_t)groups * shares >= 384));
-    const dim3 grid(groups, (unsigned)shares);
+    const bool four = tail != kRowsSwiGLU && (g_rows_waves == 4 || (g_rows_waves == 0 && (int64_t)groups * shares * grid_z(M) >= 384));
+    const dim3 grid(groups, (unsigned)shares, (unsigned)((M + kRows - 1) / kRows));
 #define ROWS_LAUNCH(WV, TL)                                                                                                       \
     hipLaunchKernelGGL((qgemv_q4_0_rows_kernel<WV, TL>), grid, dim3(64 * WV), (size_t)WV * kWaveLds, st, job, (const uint8_t*)act, y, \
                        resid, (int)M, (int)(K / 32), t)
@@ -721,12 +731,18 @@ hipError_t qgemv_q4_0_rows(const void* W, const void* act, float* y, const float
         const int64_t n1[3] = {N, 0, 0};
         return qgemv_q4_0_rows_multi(w1, n1, act, y, resid, M, K, shares, st);
     }
-    if (shares != 1) return hipErrorInvalidValue;
+    if (shares != 1 || M > kRows) return hipErrorInvalidValue;  // this kernel: a group of eight rows a launch
     const size_t lds = (size_t)nb * kTailBytes + kWaves * 64 * 16;
     if (lds > 64 * 1024) return hipErrorInvalidValue;
     hipLaunchKernelGGL(qgemv_q4_0_rows_direct_kernel, dim3((unsigned)((N + 31) / 32)), wg, lds, st, (const uint8_t*)W, (const uint8_t*)act, y,
                        resid, (int)M, (int)N, nb);
     return hipGetLastError();
+}
+
+// About what a product of M rows takes, conversion included: 5 us and a pass over W per eight rows at 4.2 TB/s
+// (measured at 4096 x 4096, 4096 x 14336 and 14336 x 4096, 8 to 128 rows: 131, 125 and 41 us at 128 rows).
+double qgemv_q4_0_rows_cost_us(int64_t M, int64_t N, int64_t K) {
+    return (double)((M + kRows - 1) / kRows) * ((double)N * (double)(K / 32) * 18.0 / 4.2e6) + 5.0;
 }
 
 // Up to three matrices (n[i] = 0: none) that share act and K, their rows one after the other in
@@ -758,7 +774,7 @@ hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], 
     RowsJob job;
     unsigned groups = 0;
     for (int i = 0; i < 3; i++) {
-        if (n[i] <= 0 || n[i] % 32 != 0 || !qgemv_q4_0_rows_shares_ok(W[i], M, n[i], K, 1)) return hipErrorInvalidValue;
+        if (M > kRows || n[i] <= 0 || n[i] % 32 != 0 || !qgemv_q4_0_rows_shares_ok(W[i], M, n[i], K, 1)) return hipErrorInvalidValue;
         job.W[i] = (const uint8_t*)W[i];
         job.n[i] = (int)n[i];
         job.groups[i] = (int)(n[i] / 32);
@@ -772,7 +788,7 @@ hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], 
 // SiLU(x . gate^T) * (x . up^T), gate and up [N, K], converted into act_out as the x of a product over N (N a multiple of 32).
 hipError_t qgemv_q4_0_rows_swiglu_act(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N, int64_t K,
                                       hipStream_t st) {
-    if (N % 32 != 0 || !qgemv_q4_0_rows_shares_ok(gate, M, N, K, 1) || !qgemv_q4_0_rows_shares_ok(up, M, N, K, 1)) return hipErrorInvalidValue;
+    if (M > kRows || N % 32 != 0 || !qgemv_q4_0_rows_shares_ok(gate, M, N, K, 1) || !qgemv_q4_0_rows_shares_ok(up, M, N, K, 1)) return hipErrorInvalidValue;
     RowsJob job;
     job.W[0] = (const uint8_t*)gate; job.W[1] = (const uint8_t*)up; job.W[2] = nullptr;
     job.n[0] = (int)N; job.n[1] = 0; job.n[2] = 0;

@@ -24,7 +24,7 @@ def per_row(l, raw_ptr, x, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(2, 32, 64), (8, 40, 128), (5, 203, 4096 + 64), (8, 515, 4096), (3, 70, 14336), (9, 64, 512),
-                                   (15, 33, 1024), (8, 1, 64)])
+                                   (15, 33, 1024), (8, 1, 64), (29, 100, 512), (40, 64, 4096 + 64)])
 def test_rows_kernel_matches_oracle_and_one_row_kernel(m, n, k):
     rng = np.random.default_rng(m * 1000 + n + k)
     raw = random_blocks(rng, O.Q4_0, n * k)  # scales of either sign, zero and subnormal
@@ -36,6 +36,13 @@ def test_rows_kernel_matches_oracle_and_one_row_kernel(m, n, k):
     w = O.dequantize(O.Q4_0, raw).reshape(n, k).astype(np.float64)
     mag = np.abs(x.astype(np.float64)) @ np.abs(w).T  # what the rounding errors scale with
     assert np.all(np.abs(got - want) <= 2e-6 * mag + 1e-30)
+    if m >= 16:  # the cost model may prefer the tiled kernel at this size: ask for the rows kernel
+        capi.check(gpu.lib().mi355x_tune(b"q4_0.rows_max", 1000))
+        try:
+            got2 = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+        finally:
+            capi.check(gpu.lib().mi355x_tune(b"q4_0.rows_max", 0))
+        assert np.all(np.abs(got2 - want) <= 2e-6 * mag + 1e-30)
     one = per_row(gpu.lib(), ptr, gpu.dev(x), n, k)
     assert np.all(np.abs(got - one) <= 1e-6 * mag + 1e-30)  # the same integers, another order of float32 additions
 
