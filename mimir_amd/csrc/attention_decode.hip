@@ -343,7 +343,8 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
         }
         const int nb = p.H * D / 32, nbp = nb | 1;
         if (p.act_rows) {
-            rows_convert_item(lo, hi, act, nb, b, (hk * G + g0 + gi) * (D / 32) + blk, dq);
+            // sequence b: row b % 8 of its group of eight, which has a buffer of its own
+            rows_convert_item(lo, hi, act + (int64_t)(b >> 3) * q4_0_rows_act_size((int64_t)nb * 32), nb, b & 7, (hk * G + g0 + gi) * (D / 32) + blk, dq);
         } else {
             u32x4* plane = (u32x4*)(act + (int64_t)b * p.act_row_bytes);
             float* xscale = (float*)(plane + kDigits * nbp);
@@ -398,7 +399,7 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
 // bytes whose first 4096 were zero before the first launch (the tickets reset
 // themselves). act, if set, gets row b's result [H * D] in the Q4_0 product's
 // fixed-point form, act_row_bytes apart; out may then be null.
-// act_rows: the form for up to eight sequences together (q4_rows_act.h; a.B <= 8), row b's result as row b of it.
+// act_rows: the form for eight sequences together (q4_rows_act.h), a buffer per group of eight: row b's result as row b % 8 of group b / 8.
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, bool act_rows) {
     DecParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
@@ -413,7 +414,6 @@ hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, vo
     p.dyn_k = a.dyn_k;
     p.act_row_bytes = act_row_bytes;
     p.act_rows = act_rows ? 1 : 0;
-    if (act_rows && a.B > 8) return hipErrorInvalidValue;
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
     dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
     size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);

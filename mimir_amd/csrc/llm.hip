@@ -105,7 +105,7 @@ struct Model {
     // linears that the fixed-point kernel takes); step_graph replays the run.
     bool fast = false;
     DevBuf state, record, qkv, gu, argmax_ws;  // gu: gate|up of a step, [batch, 2 hidden]
-    // `rows`: a fast model with two to eight sequences, whose step reads every weight once for all of them
+    // `rows`: a fast model with two to sixty-four sequences, whose step reads every weight once per eight of them
     // (step_rows): the sequences' activations converted together, and the two shares of K of the output and
     // down projections, [2, batch, embed].
     bool rows = false;
@@ -359,8 +359,8 @@ static int g_llama_rows_off = 0;  // measurement aid: 1 = several sequences take
 static int g_llama_rows_plain = 0;  // measurement aid: 1 = step_rows with the rotation and SwiGLU as launches of their own
 void set_llama_rows_off(int v) { g_llama_rows_off = v == 1; g_llama_rows_plain = v >= 2 ? v : 0; }
 
-// One decoding step of two to eight sequences with Q4_0 linears (the case of step_fast): the same
-// operations, but every product reads its weights once for all the sequences, on the int8 matrix cores
+// One decoding step of two to sixty-four sequences with Q4_0 linears (the case of step_fast): the same
+// operations, but every product reads its weights once per eight sequences (from HBM once), on the int8 matrix cores
 // (qgemv_q4_0_rows.hip), where step_fast's products read them once per sequence. Nine launches a block:
 // norm (adding the shares of the product before it into x) with conversion, q|k|v, rotation and cache
 // write, attention with conversion, output projection in two shares of K, norm, gate|up, SiLU * up with
@@ -760,7 +760,7 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     }
     LLM_HIP(m->gu.alloc((size_t)c.batch * 2 * c.hidden * 4), "hipMalloc");
     // several sequences: every product of a step on the kernels that read W once for up to eight rows of x
-    m->rows = m->fast && c.batch >= 2 && c.batch <= 8 && qd % 32 == 0 && kvd % 32 == 0 && c.hidden % 32 == 0 && c.embed <= 8192;
+    m->rows = m->fast && c.batch >= 2 && c.batch <= 64 && qd % 32 == 0 && kvd % 32 == 0 && c.hidden % 32 == 0 && c.embed <= 8192;
     if (m->rows) {
         AttnArgs at;  // the shape of a step's attention, as step_rows sets it up
         at.q = m->qkv.as<float>(); at.k = m->keys[0].p; at.v = m->values[0].p; at.kv_dtype = c.cache_dtype;
@@ -779,7 +779,7 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
             if (!qgemv_q4_0_rows_shares_ok(w->buf.p, c.batch, w->n, w->k, 2)) m->rows = false;
     }
     if (m->rows) {
-        const size_t ab = q4_0_rows_act_bytes(kmax);
+        const size_t ab = q4_0_rows_act_bytes(kmax) * (size_t)((c.batch + 7) / 8);  // a buffer per group of eight sequences
         LLM_HIP(m->rows_act.alloc(ab), "hipMalloc(activations)");
         LLM_HIP(hipMemset(m->rows_act.p, 0, ab), "hipMemset(activations)");  // rows past the batch stay zero
         LLM_HIP(m->rows_act2.alloc(ab), "hipMalloc(activations)");

@@ -269,7 +269,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
                                                                        float* y, const float* resid,  // resid may be y
                                                                        int M_all, int nb, const RowsTailArgs tail_args) {
     extern __shared__ __align__(16) uint8_t smem[];  // per wavefront: slab and tail of its run; later the wavefronts' sums
-    // blockIdx.z: the group of eight rows of x (plain tail only), each converted into a buffer of its own
+    // blockIdx.z: the group of eight rows of x, each converted into a buffer of its own
     const uint8_t* __restrict__ act = act_all + (int64_t)blockIdx.z * nb * (kFragBytes + kTailBytes);
     const int M = M_all - kRows * (int)blockIdx.z < kRows ? M_all - kRows * (int)blockIdx.z : kRows;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
@@ -459,8 +459,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const float other = dpp_f32<0xb1>(sum[j]);  // quad_perm [1,0,3,2]
-            const int m = 4 * lh + j;
-            if ((lane & 1) == 0 && n < N && m < M) q4_rope_store(tail_args.rope, pos, m, ybase + n, sum[j], other, y + (int64_t)m * ny);
+            const int m = 4 * lh + j, seq = kRows * (int)blockIdx.z + m;
+            if ((lane & 1) == 0 && n < N && m < M) q4_rope_store(tail_args.rope, pos, seq, ybase + n, sum[j], other, y + (int64_t)seq * ny);
         }
     } else {
         f32x4 up = red[WAVES * 64 + lane];
@@ -526,10 +526,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
             at[8 * 16] = (uint8_t)d1;
             at[16 * 16] = (uint8_t)d2;
         }
-        uint8_t* out = tail_args.act_out + (int64_t)blockIdx.x * kFragBytes;
+        uint8_t* group_out = tail_args.act_out + (int64_t)blockIdx.z * tail_args.nb_out * (kFragBytes + kTailBytes);
+        uint8_t* out = group_out + (int64_t)blockIdx.x * kFragBytes;
         if ((lane & 31) < 24) *(u32x4*)(out + 16 * lane) = *(const u32x4*)(stage + 16 * lane);
         if (l32 == 0) {
-            uint8_t* to = tail_args.act_out + (int64_t)tail_args.nb_out * kFragBytes + (int64_t)blockIdx.x * kTailBytes;
+            uint8_t* to = group_out + (int64_t)tail_args.nb_out * kFragBytes + (int64_t)blockIdx.x * kTailBytes;
             *(f32x4*)(to + 16 * lh) = f32x4{scale_j[0], scale_j[1], scale_j[2], scale_j[3]};
             *(i32x4*)(to + 32 + 16 * lh) = i32x4{8 * sum_j[0], 8 * sum_j[1], 8 * sum_j[2], 8 * sum_j[3]};
         }
@@ -543,11 +544,12 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
 // becomes x[m] + parts[0][m] + parts[1][m] + ... (the shares of K of the product before, added in
 // their order) and is written back: the residual connection.
 __global__ __launch_bounds__(256) void rows_norm_act_kernel(float* __restrict__ x, const float* __restrict__ parts, int shares,
-                                                            int64_t share_stride, const float* __restrict__ w,
-                                                            uint8_t* __restrict__ act, int d, float inv_d, float eps) {
+                                                            int64_t share_stride, const float* __restrict__ w, uint8_t* act, int d,
+                                                            float inv_d, float eps) {
     __shared__ float part[4];
     const int m = blockIdx.x, t0 = threadIdx.x, nq = d >> 3, nb = d >> 5;
     float* xr = x + (int64_t)m * d;
+    act += (int64_t)(m / kRows) * nb * (kFragBytes + kTailBytes);  // the row's group of eight has a buffer of its own
     NormRow r;
     float ss = 0.f;
 #pragma unroll
@@ -611,7 +613,7 @@ __global__ __launch_bounds__(256) void rows_norm_act_kernel(float* __restrict__ 
                 l4[k] = a * r.wl[i][k];
                 h4[k] = c * r.wh[i][k];
             }
-            rows_convert_item(l4, h4, act, nb, m, t >> 2, t & 3);
+            rows_convert_item(l4, h4, act, nb, m % kRows, t >> 2, t & 3);
         }
     }
 }
@@ -619,11 +621,12 @@ __global__ __launch_bounds__(256) void rows_norm_act_kernel(float* __restrict__ 
 // SiLU(g) * u (llm/model.go:446-448, the arithmetic of swiglu_kernel) into the converted form: g and u
 // rows `stride` floats apart, n a multiple of 32.
 __global__ __launch_bounds__(256) void rows_swiglu_act_kernel(const float* __restrict__ g, const float* __restrict__ u, int64_t stride,
-                                                              uint8_t* __restrict__ act, int n) {
+                                                              uint8_t* act, int n) {
     const float nl2e = (float)(-1.4426950408889634);
     const int m = blockIdx.y, nq = n >> 3, nb = n >> 5;
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= nq) return;  // whole quads: nq is a multiple of 4
+    act += (int64_t)(m / kRows) * nb * (kFragBytes + kTailBytes);
     const int o = 32 * (t >> 2) + 4 * (t & 3);
     f32x4 gl, gh, ul, uh;
     __builtin_memcpy(&gl, g + m * stride + o, 16);
@@ -642,7 +645,7 @@ __global__ __launch_bounds__(256) void rows_swiglu_act_kernel(const float* __res
         a = gh[k] * sg;
         h4[k] = a * uh[k];
     }
-    rows_convert_item(l4, h4, act, nb, m, t >> 2, t & 3);
+    rows_convert_item(l4, h4, act, nb, m % kRows, t >> 2, t & 3);
 }
 
 // x += parts[0] + parts[1] + ..., added in that order, n floats.
@@ -660,7 +663,7 @@ __global__ __launch_bounds__(256) void rows_add_parts_kernel(float* __restrict__
 hipError_t rows_norm_act(float* x, const float* parts, int shares, const float* w, void* act, int64_t rows, int64_t d, double eps,
                          hipStream_t st) {
     if (rows <= 0) return hipSuccess;
-    if (rows > kRows || d % 32 != 0 || d > 8 * 256 * kNormItems) return hipErrorInvalidValue;
+    if (rows > kRows * 65535 || d % 32 != 0 || d > 8 * 256 * kNormItems) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rows_norm_act_kernel, dim3((unsigned)rows), dim3(256), 0, st, x, parts, parts ? shares : 0, rows * d, w, (uint8_t*)act,
                        (int)d, (float)(1.0 / (double)d), (float)eps);
     return hipGetLastError();
@@ -668,7 +671,7 @@ hipError_t rows_norm_act(float* x, const float* parts, int shares, const float* 
 
 hipError_t rows_swiglu_act(const float* g, const float* u, void* act, int64_t rows, int64_t n, int64_t stride, hipStream_t st) {
     if (rows <= 0) return hipSuccess;
-    if (rows > kRows || n % 32 != 0) return hipErrorInvalidValue;
+    if (rows > 65535 || n % 32 != 0) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rows_swiglu_act_kernel, dim3((unsigned)((n / 8 + 255) / 256), (unsigned)rows), dim3(256), 0, st, g, u, stride,
                        (uint8_t*)act, (int)n);
     return hipGetLastError();
@@ -774,7 +777,7 @@ hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], 
     RowsJob job;
     unsigned groups = 0;
     for (int i = 0; i < 3; i++) {
-        if (M > kRows || n[i] <= 0 || n[i] % 32 != 0 || !qgemv_q4_0_rows_shares_ok(W[i], M, n[i], K, 1)) return hipErrorInvalidValue;
+        if (n[i] <= 0 || n[i] % 32 != 0 || !qgemv_q4_0_rows_shares_ok(W[i], M, n[i], K, 1)) return hipErrorInvalidValue;
         job.W[i] = (const uint8_t*)W[i];
         job.n[i] = (int)n[i];
         job.groups[i] = (int)(n[i] / 32);
@@ -788,7 +791,7 @@ hipError_t qgemv_q4_0_rows_qkv_rope(const void* const W[3], const int64_t n[3], 
 // SiLU(x . gate^T) * (x . up^T), gate and up [N, K], converted into act_out as the x of a product over N (N a multiple of 32).
 hipError_t qgemv_q4_0_rows_swiglu_act(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N, int64_t K,
                                       hipStream_t st) {
-    if (M > kRows || N % 32 != 0 || !qgemv_q4_0_rows_shares_ok(gate, M, N, K, 1) || !qgemv_q4_0_rows_shares_ok(up, M, N, K, 1)) return hipErrorInvalidValue;
+    if (N % 32 != 0 || !qgemv_q4_0_rows_shares_ok(gate, M, N, K, 1) || !qgemv_q4_0_rows_shares_ok(up, M, N, K, 1)) return hipErrorInvalidValue;
     RowsJob job;
     job.W[0] = (const uint8_t*)gate; job.W[1] = (const uint8_t*)up; job.W[2] = nullptr;
     job.n[0] = (int)N; job.n[1] = 0; job.n[2] = 0;

@@ -40,14 +40,18 @@ constexpr int kSlabStride = kRunBytes + 32;    // 304 bytes = 76 dwords: rows fa
 constexpr int kSlabBytes = 32 * kSlabStride;
 constexpr int kLoads = (32 * kPieces + 63) / 64;  // 9: the last one half full
 
-__global__ __launch_bounds__(64 * kWaves) void qgemv_q8_0_mfma_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ act,
-                                                                       float* __restrict__ y, int M, int N, int nb, int64_t act_row_bytes) {
+__global__ __launch_bounds__(64 * kWaves) void qgemv_q8_0_mfma_kernel(const uint8_t* __restrict__ W, const uint8_t* act, float* y, int M, int N,
+                                                                       int nb, int64_t act_row_bytes) {
     extern __shared__ __align__(16) uint8_t smem[];  // a slab per wavefront; later the wavefronts' sums
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n0 = blockIdx.x * 32, n = n0 + l32;
     const int nruns = nb / kRunBlocks, nbp = nb | 1;
     uint8_t* slab = smem + wave * kSlabBytes;
+    // blockIdx.y: the group of eight rows of x
+    act += (int64_t)8 * blockIdx.y * act_row_bytes;
+    y += (int64_t)8 * blockIdx.y * N;
+    M = M - 8 * (int)blockIdx.y < 8 ? M - 8 * (int)blockIdx.y : 8;
 
     // piece p = 64 i + lane of a run: row p / 17 of the 32, bytes 16 (p % 17).. of its 272
     uint32_t goff[kLoads], loff[kLoads];
@@ -175,10 +179,10 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_q8_0_mfma_kernel(const uint
 
 }  // namespace
 
-// Rows of x converted beforehand (q8_convert_act), at most eight; whole runs of eight blocks; W 16-byte aligned.
+// Rows of x converted beforehand (q8_convert_act), taken eight at a time; whole runs of eight blocks; W 16-byte aligned.
 bool qgemv_q8_0_mfma_ok(const QGemvArgs& a) {
     const int64_t nb = a.K / 32;
-    return a.M >= 2 && a.M <= 8 && a.act && !a.resid && a.K % 256 == 0 && nb > 0 && ((uintptr_t)a.W & 15) == 0 && 32 * nb * 34 < ((int64_t)1 << 32) &&
+    return a.M >= 2 && a.M <= 8 * 65535 && a.act && !a.resid && a.K % 256 == 0 && nb > 0 && ((uintptr_t)a.W & 15) == 0 && 32 * nb * 34 < ((int64_t)1 << 32) &&
            a.N > 0 && a.N <= (1ll << 30);
 }
 
@@ -192,7 +196,7 @@ bool qgemv_q8_0_mfma_pays(const QGemvArgs& a) {
 
 hipError_t qgemv_q8_0_mfma(const QGemvArgs& a, hipStream_t st) {
     const size_t lds = (size_t)kWaves * kSlabBytes + kWaves * 64 * 4;
-    hipLaunchKernelGGL(qgemv_q8_0_mfma_kernel, dim3((unsigned)((a.N + 31) / 32)), dim3(64 * kWaves), lds, st, (const uint8_t*)a.W,
+    hipLaunchKernelGGL(qgemv_q8_0_mfma_kernel, dim3((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 7) / 8)), dim3(64 * kWaves), lds, st, (const uint8_t*)a.W,
                        (const uint8_t*)a.act, a.y, (int)a.M, (int)a.N, (int)(a.K / 32), (int64_t)q8_act_bytes(a.K));
     return hipGetLastError();
 }

@@ -219,9 +219,9 @@ def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, ca
     assert all(same), (runs[2][0], runs[0][0])
 
 
-@pytest.mark.parametrize("batch", [2, 5, 8])
+@pytest.mark.parametrize("batch", [2, 5, 8, 11, 16])
 def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
-    """Two to eight sequences decode with products that read each weight once for all of them (int8 matrix
+    """Two to sixty-four sequences decode with products that read each weight once per eight of them (int8 matrix
     cores, the output and down projections cut into two shares of K that the next norm adds; the rotation
     with the cache writes and SiLU * up with its conversion ride on the products, or run as launches of
     their own). Their integers are those of the one-sequence kernels, only float32 sums are ordered differently, so the tokens
