@@ -673,6 +673,14 @@ mi355x_status mi355x_tune(const char* key, int value) {
         mimir::set_q8_mfma(value);
         return MI355X_OK;
     }
+    if (key && strcmp(key, "kquant.mfma_rows_waves") == 0) {
+        mimir::set_kquant_rows_waves(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "kquant.mfma_rows") == 0) {
+        mimir::set_kquant_rows(value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "q4_0.rows_max") == 0) {
         g_rows_max = value > 0 ? value : 0;
         return MI355X_OK;

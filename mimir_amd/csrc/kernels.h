@@ -125,6 +125,14 @@ hipError_t qgemm_kquant(int dt, const QGemvArgs& a, hipStream_t st, bool out_bf1
 // which 0: rows of W per wavefront (1, 2, 4; 0 = by shape); which 1: value 1 = always the kernels that keep x in
 // global memory, 2 = never the matrix-core kernel, 3 = always the matrix-core kernel.
 void set_kquant_tune(int which, int value);
+// Two rows of x or more against Q4_K or Q6_K weights, eight to a pass over W, on the int8 matrix cores with the CPU's bits
+// (qgemv_kquant_rows.hip); qgemv_kquant_act hands over where qgemv_kquant_rows_pays says so ("kquant.mfma_rows": 1 never, 2 wherever
+// the kernel takes the shape).
+bool qgemv_kquant_rows_ok(int dt, const QGemvArgs& a);
+bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a);
+hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st);
+void set_kquant_rows(int v);
+void set_kquant_rows_waves(int v);
 
 // y = x . W^T for a float32, binary16 or bfloat16 W [N, K].
 hipError_t gemv_float(int dt, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride,

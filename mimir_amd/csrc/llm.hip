@@ -461,7 +461,9 @@ static mi355x_status step_any(Model& m) {
         }
         if (b.qkv.set()) {  // one product into [B, q | k | v]
             QGemvArgs qa{b.qkv.buf.p, nullptr, m.act[kActKQ].p, qkv, B, b.qkv.n, b.qkv.k, b.qkv.k, 0};
-            if (qkv_kq && c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0 && qgemv_kquant_rope_ok(b.qkv.dtype, qa)) {
+            // From three sequences on, where W can be read once for eight of them, that beats the tail that saves a launch.
+            const bool read_once = B >= 3 && qkv_kq && qgemv_kquant_rows_pays(b.qkv.dtype, qa);
+            if (qkv_kq && !read_once && c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0 && qgemv_kquant_rope_ok(b.qkv.dtype, qa)) {
                 Q4RopeTail tail;  // the rotation and the cache writes ride on the product
                 tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
                 tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;

@@ -640,6 +640,8 @@ hipError_t qgemv_kquant_act(int dt, const QGemvArgs& a, hipStream_t st) {
         if (!qgemv_kquant_rope_ok(dt, a) || ((uintptr_t)a.x & 15) || a.x_row_stride % 4) return hipErrorInvalidValue;
         return a.N * a.M >= 2048 ? launch_kq<2>(dt, a, nsb, nullptr, st) : launch_kq<1>(dt, a, nsb, nullptr, st);
     }
+    // A few rows of x: W read once per eight of them.
+    if (g_kq_tune[0] == 0 && g_kq_tune[1] == 0 && qgemv_kquant_rows_pays(dt, a)) return qgemv_kquant_rows(dt, a, st);
     // From a few rows of x on, the matrix cores (whose results are the CPU's bit for bit).
     if (!a.resid && (g_kq_tune[1] == 3 || (g_kq_tune[1] == 0 && qgemm_kquant_pays(dt, a))) && qgemm_kquant_ok(dt, a)) return qgemm_kquant(dt, a, st);
     // Q4_K blocks are read with aligned 128-bit loads: 144-byte blocks keep a 16-byte aligned W aligned.

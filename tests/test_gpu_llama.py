@@ -293,7 +293,7 @@ def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
     assert np.array_equal(runs[1], runs[2]) and np.array_equal(runs[0], runs[2])
 
 
-@pytest.mark.parametrize("linear_dt,batch", [(O.Q4_K, 1), (O.Q6_K, 2), (O.Q8_0, 1)])
+@pytest.mark.parametrize("linear_dt,batch", [(O.Q4_K, 1), (O.Q6_K, 2), (O.Q8_0, 1), (O.Q4_K, 5), (O.Q4_K, 11), (O.Q6_K, 9)])
 def test_k_quant_and_q8_0_models_decode_from_a_graph(linear_dt, batch):
     """Models whose linears are not Q4_0 take the generic decoding step: q|k|v and gate|up as one product
     each over weights kept together, norm and SwiGLU with the int8 conversion in the same launch (K-quants),

@@ -534,6 +534,34 @@ def test_kquant_gemv_single_row_rounds_x_in_the_product(dt):
             assert bits_equal(one, want) and bits_equal(two, want)
 
 
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("m,n,k", [(2, 33, 256), (5, 100, 512), (8, 203, 4096), (11, 64, 256 * 9), (20, 31, 256 * 56), (40, 130, 1024)])
+def test_kquant_rows_of_x_share_one_pass_over_w_on_the_matrix_cores(dt, m, n, k):
+    """Rows of x, eight at a time, against Q4_K or Q6_K weights read once on the int8 matrix cores (the decoding
+    step of a batch; forced here beyond the rows it is chosen for): the CPU's integer sums, and its float32
+    operations in its order, so the oracle's bits and those of the one-row kernels. x holds a zero
+    super-block, ties and, in one row, a NaN."""
+    l = gpu.lib()
+    rng = np.random.default_rng(dt + 7 * m + n + k)
+    raw = random_blocks(rng, dt, n * k)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    x[0, :256] = 0
+    x[1, k - 256:] = (rng.integers(0, 254, 256) - 127) / 2; x[1, k - 1] = 127
+    if m > 2: x[m - 1, k // 2] = np.nan
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(dt, raw, x, n, k)
+    try:
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows", 2))
+        gpu.say(f"kquant matrix-core rows kernel dt={dt} M={m} N={n} K={k}")
+        got = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
+        got_act = gpu.qgemv_act(dt, ptr, gpu.dev(x), n, k)
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows", 1))
+        rows = gpu.qgemv(dt, ptr, gpu.dev(x), n, k)
+    finally:
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows", 0))
+    assert bits_equal(got, want) and bits_equal(got_act, want) and bits_equal(rows, want)
+
+
 def test_kquant_gemv_golden_and_exact_rows(golden_dir):
     cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
     for kind, dt in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
