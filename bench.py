@@ -281,47 +281,64 @@ def bench_blocks_kquant(rng, dtype_bytes, n_elems):
 
 
 def rows_bench(lib, capi, torch, m=8, shapes=((14336, 4096), (4096, 14336), (4096, 4096), (6144, 4096), (28672, 4096)), iters=200, only=None):
-    """The Q4_0 product of a few rows of x (a decoding step of a batch), mi355x_qgemv as a whole (conversion
-    of x and product, two launches) over rotating copies of W: the kernel that reads W once for eight rows
+    """The product of a few rows of x (a decoding step of a batch), mi355x_qgemv as a whole (conversion
+    of x and product, two launches) over rotating copies of W. Q4_0: the kernel that reads W once for eight rows
     on the int8 matrix cores, its variant that loads each lane's block where it lies, and the one-row kernel
-    run per row. `only` (a variant's name): a few launches of that variant and nothing else, for counter runs."""
+    run per row. Q4_K, Q6_K: the kernel that reads W once for eight rows, the tiled matrix-core kernel and the
+    one-row kernels run per row. `only` (a variant's name): a few launches of that variant and nothing else, for
+    counter runs."""
     rng = np.random.default_rng(0)
     st = torch.cuda.Stream()
     out = {}
-    variants = (("rows_kernel", 0), ("rows_kernel_no_lds_pass", 2), ("one_row_kernel_per_row", 1))
+    # name, dtype, bytes of a block of W and weights in it, the tune keys that select the variant
+    variants = (("rows_kernel", capi.Q4_0, 18, 32, ((b"q4_0.rows_path", 0),)),
+                ("rows_kernel_no_lds_pass", capi.Q4_0, 18, 32, ((b"q4_0.rows_path", 2),)),
+                ("one_row_kernel_per_row", capi.Q4_0, 18, 32, ((b"q4_0.rows_path", 1),)),
+                ("q4_K_rows_kernel", capi.Q4_K, 144, 256, ()),
+                ("q4_K_tiled_kernel", capi.Q4_K, 144, 256, ((b"kquant.path", 3),)),
+                ("q4_K_one_row_kernel_per_row", capi.Q4_K, 144, 256, ((b"kquant.path", 2), (b"kquant.mfma_rows", 1))),
+                ("q6_K_rows_kernel", capi.Q6_K, 210, 256, ()),
+                ("q6_K_tiled_kernel", capi.Q6_K, 210, 256, ((b"kquant.path", 3),)),
+                ("q6_K_one_row_kernel_per_row", capi.Q6_K, 210, 256, ((b"kquant.path", 2), (b"kquant.mfma_rows", 1))))
+    reset = ((b"q4_0.rows_path", 0), (b"kquant.path", 0), (b"kquant.mfma_rows", 0))
     try:
         for n, k in shapes:
-            raw = bench_blocks_q4_0(rng, n * k)
-            nbuf = max(2, min(32, int(300e6 // raw.size)))
-            w0 = torch.from_numpy(raw).to("cuda:0")
-            bufs = [w0] + [w0.clone() for _ in range(nbuf - 1)]
-            x = torch.randn(m, k, device="cuda:0")
-            y = torch.empty(m, n, device="cuda:0")
-            torch.cuda.synchronize()
             res = {}
-            for name, path in variants:
-                if only and name != only:
+            for dt in (capi.Q4_0, capi.Q4_K, capi.Q6_K):
+                mine = [v for v in variants if v[1] == dt and (not only or v[0] == only)]
+                if not mine:
                     continue
-                capi.check(lib.mi355x_tune(b"q4_0.rows_path", path))
-                with torch.cuda.stream(st):
-                    call = lambda i: capi.check(lib.mi355x_qgemv(capi.Q4_0, bufs[i % nbuf].data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, st.cuda_stream))
-                    for i in range(4 if only else 10):
-                        call(i)
-                    st.synchronize()
-                    if only:
-                        continue
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record(st)
-                    for i in range(iters):
-                        call(i)
-                    e1.record(st)
-                    st.synchronize()
-                us = e0.elapsed_time(e1) / iters * 1e3
-                res[name] = {"us": round(us, 2), "W_GBps": round(raw.size / (us * 1e-6) / 1e9, 1)}
+                bb, per = mine[0][2], mine[0][3]
+                raw = bench_blocks_q4_0(rng, n * k) if dt == capi.Q4_0 else bench_blocks_kquant(rng, bb, n * k)
+                nbuf = max(2, min(32, int(300e6 // raw.size)))
+                w0 = torch.from_numpy(raw).to("cuda:0")
+                bufs = [w0] + [w0.clone() for _ in range(nbuf - 1)]
+                x = torch.randn(m, k, device="cuda:0")
+                y = torch.empty(m, n, device="cuda:0")
+                torch.cuda.synchronize()
+                for name, _, _, _, keys in mine:
+                    for key, v in reset + keys:
+                        capi.check(lib.mi355x_tune(key, v))
+                    with torch.cuda.stream(st):
+                        call = lambda i: capi.check(lib.mi355x_qgemv(dt, bufs[i % nbuf].data_ptr(), x.data_ptr(), y.data_ptr(), m, n, k, k, st.cuda_stream))
+                        for i in range(4 if only else 10):
+                            call(i)
+                        st.synchronize()
+                        if only:
+                            continue
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record(st)
+                        for i in range(iters):
+                            call(i)
+                        e1.record(st)
+                        st.synchronize()
+                    us = e0.elapsed_time(e1) / iters * 1e3
+                    res[name] = {"us": round(us, 2), "W_GBps": round(raw.size / (us * 1e-6) / 1e9, 1)}
+                del bufs, w0, x, y
             out[f"M{m}_N{n}_K{k}"] = res
-            del bufs, w0, x, y
     finally:
-        capi.check(lib.mi355x_tune(b"q4_0.rows_path", 0))
+        for key, v in reset:
+            capi.check(lib.mi355x_tune(key, v))
     return out
 
 
@@ -435,7 +452,7 @@ def main():
     ap.add_argument("--rows", action="store_true", help="also time the Q4_0 product of eight rows of x (a batch's decoding step) at the model's shapes")
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
                     help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
-                         "rows_kernel, rows_kernel_no_lds_pass or one_row_kernel_per_row")
+                         "rows_kernel, rows_kernel_no_lds_pass, one_row_kernel_per_row (Q4_0), q4_K_rows_kernel, q6_K_rows_kernel, ...")
     ap.add_argument("--layer-step", action="store_true", help="also time one decoder layer's decoding step against 2048 cached positions (batch 1, 8)")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
@@ -460,7 +477,8 @@ def main():
 
     if args.rows_counters:
         rows_bench(lib, capi, torch, shapes=((14336, 4096),), only=args.rows_counters)
-        print(json.dumps({"rows_counters": args.rows_counters, "launches": 4, "W_bytes": 14336 * 4096 // 32 * 18}))
+        per_weight = {"q4_K": 144 / 256, "q6_K": 210 / 256}.get(args.rows_counters[:4], 18 / 32)
+        print(json.dumps({"rows_counters": args.rows_counters, "launches": 4, "W_bytes": int(14336 * 4096 * per_weight)}))
         return
     n, k = 14336, 4096
     g = Gemv(lib, capi, torch, n, k, args.bufs)

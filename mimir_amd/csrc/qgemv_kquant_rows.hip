@@ -16,13 +16,12 @@
 // sub-block sums for four rows of x; the scales are per lane, so sc_j times the
 // sum is one multiply-add, and m_j times the two sums of 16 one v_dot2.
 //
-// A workgroup of eight wavefronts (four for Q6_K) owns 32 rows of W; a wavefront
-// takes every eighth super-block and leaves its float32 terms per output (two
+// A workgroup of four or eight wavefronts owns 32 rows of W; its wavefronts take
+// the super-blocks round robin and leave their float32 terms per output (two
 // for Q4_K, one for Q6_K) in LDS; when all are there the first wavefront adds
-// them in the super-blocks' order, which is the CPU's. x of a super-block (2.3 KB
-// for eight rows) is staged per wavefront in LDS; a lane loads its row's header
-// and its half of each group of nibbles where they lie (five aligned 16-byte
-// loads a super-block; for Q6_K see WBlock<kQ6_K>).
+// them in the super-blocks' order, which is the CPU's. x of a super-block (2.6 KB
+// for eight rows) and W of it (32 rows, loaded as whole cache lines) pass through
+// LDS that is the wavefront's own, so no barrier but the one before the sums.
 #include "device_util.h"
 #include "kernels.h"
 
@@ -37,8 +36,12 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef short s16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kRows = 8;                        // rows of x a group holds
-constexpr int kXq = 0, kXs = 2048, kXd = 2304;  // a super-block of x for eight rows in LDS: quants [8][256], sums [8][16] int16, scales [8]
-constexpr int kXBytes = 2336;
+// A super-block of x for eight rows in LDS: quants [8][256] with rows 288 bytes apart (72 dwords: the sixteen 16-byte pieces the
+// lanes of a matrix-core operand read, eight rows by two halves, fall on all 64 banks; 256 apart they would share four), sums [8][16]
+// int16, scales [8].
+constexpr int kXRow = 288;
+constexpr int kXq = 0, kXs = 8 * kXRow, kXd = kXs + 256;
+constexpr int kXBytes = kXd + 32;
 
 // scale_min_k4 (backend/cpu/quant.go:129-134) on the twelve scale bytes held as three dwords.
 __device__ __forceinline__ int q4k_sc(uint32_t s0, uint32_t s2, int j) {
@@ -50,21 +53,21 @@ __device__ __forceinline__ int q4k_mn(uint32_t s1, uint32_t s2, int j) {
     return j < 4 ? (int)((s1 >> sh) & 63) : (int)(((s2 >> (sh + 4)) & 0xf) | (((s1 >> (sh + 6)) & 3) << 4));
 }
 
-// What a lane holds of its row's super-block between the loads and the arithmetic, how it loads it, and the float32 terms it
-// makes of it for its four rows of x (x of the super-block lies in the wavefront's LDS at xl).
+// W comes through LDS: a wavefront loads a super-block of its 32 rows as 16-byte pieces in row order (consecutive lanes, consecutive
+// pieces of a row: whole cache lines per request, where a load of a lane's own row would touch 64 lines for 16 bytes each and wait for
+// the cache's tag lookups), stores them into a slab of its own and reads its row's pieces back. WBlock<DT> says how a row's
+// super-block is cut into pieces and makes the float32 terms of a lane's four rows of x from its row in the slab (wl) and the
+// super-block of x in LDS (xl).
 template <int DT> struct WBlock;
 
 template <> struct WBlock<kQ4_K> {
     static constexpr int kBytes = 144, kTerms = 2;
-    u32x4 hdr, q[4];  // d, dmin, scales; the lane's 16 bytes of nibbles of each of the four groups of 64
-    __device__ __forceinline__ void load(const uint8_t* wb, int lh) {
-        hdr = *(const u32x4*)wb;
-#pragma unroll
-        for (int g = 0; g < 4; g++) q[g] = *(const u32x4*)(wb + 16 + 32 * g + 16 * lh);
-    }
+    static constexpr int kPieces = 9, kStride = 144;  // rows 36 dwords apart: the 16 lanes of a 128-bit read's phase fall on all 64 banks
+    __device__ __forceinline__ static int piece_offset(int c) { return 16 * c; }
     // t[0] = d_w d_x float(sumi), t[1] = dmin_w d_x float(summ)
-    __device__ __forceinline__ void terms(const uint8_t* xl, int l32, int lh, f32x4* t) const {
-        const uint8_t* xrow = xl + kXq + (l32 & 7) * 256 + 16 * lh;  // this lane's operand row of x (rows 8.. of the operand repeat rows 0..7)
+    __device__ __forceinline__ static void terms(const uint8_t* wl, const uint8_t* xl, int l32, int lh, f32x4* t) {
+        const u32x4 hdr = *(const u32x4*)wl;  // d, dmin, scales
+        const uint8_t* xrow = xl + kXq + (l32 & 7) * kXRow + 16 * lh;  // this lane's operand row of x (rows 8.. of the operand repeat rows 0..7)
         const uint32_t s0 = hdr[1], s1 = hdr[2], s2 = hdr[3];
         int sumi[4] = {0, 0, 0, 0}, summ[4] = {0, 0, 0, 0};
         // the sums of 16 of this lane's four rows of x: dword c holds chunks 2c and 2c + 1
@@ -77,11 +80,12 @@ template <> struct WBlock<kQ4_K> {
         const f32x4 xd = *(const f32x4*)(xl + kXd + 16 * lh);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
+            const u32x4 q = *(const u32x4*)(wl + 16 + 32 * g + 16 * lh);  // the lane's 16 bytes of nibbles of group g
             i32x4 wlo, whi;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                wlo[i] = (int)(q[g][i] & 0x0F0F0F0Fu);
-                whi[i] = (int)((q[g][i] >> 4) & 0x0F0F0F0Fu);
+                wlo[i] = (int)(q[i] & 0x0F0F0F0Fu);
+                whi[i] = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
             }
             const i32x4 xa = *(const i32x4*)(xrow + 64 * g), xb = *(const i32x4*)(xrow + 64 * g + 32);
             i32x16 zero;
@@ -94,7 +98,8 @@ template <> struct WBlock<kQ4_K> {
             const uint32_t ma2 = (uint32_t)ma * 0x00010001u, mb2 = (uint32_t)mb * 0x00010001u;
 #pragma unroll
             for (int jj = 0; jj < 4; jj++) {
-                sumi[jj] += sca * ca[jj] + scb * cb[jj];
+                // 24-bit multiplies (full rate; a 32-bit one takes four times as long): |sum| <= 32 * 15 * 127, scales below 64
+                sumi[jj] += __mul24(sca, ca[jj]) + __mul24(scb, cb[jj]);
                 // sub-block 2g is chunks 4g, 4g + 1 (dword 2g of the sums), sub-block 2g + 1 chunks 4g + 2, 4g + 3
                 const uint32_t pa = sv[jj][g >> 1][2 * (g & 1)], pb = sv[jj][g >> 1][2 * (g & 1) + 1];
                 summ[jj] = __builtin_amdgcn_sdot2(__builtin_bit_cast(s16x2, pa), __builtin_bit_cast(s16x2, ma2), summ[jj], false);
@@ -112,34 +117,20 @@ template <> struct WBlock<kQ4_K> {
 };
 
 // Q6_K (qdotQ6KGo, backend/cpu/qmatmul.go:180-200): 210-byte blocks, so a row's blocks start on even addresses only and the
-// 16-byte loads below are unaligned ones. Half h2 of a super-block (128 weights) is 64 bytes of ql and 32 of qh: slab s = 0..3 of the
-// half (32 weights) has its low four bits in the low (s < 2) or high nibbles of ql[64 h2 + 32 (s & 1) ..] and its upper two at bit 2 s
-// of qh[32 h2 ..]; a scale per chunk of 16, a zero point of 32. The matrix-core product must keep the two chunks of a slab apart: the
-// operand's row 8 c + m holds row m of x with everything but chunk c of the slab zeroed, so the result's rows 0..7 are chunk 0's sums
-// and rows 8..15 chunk 1's (rows 16..31 are unused).
+// 16-byte loads are unaligned ones: thirteen pieces from the block's start and a fourteenth over its last 16 bytes (194..209), which
+// lands behind them in the slab (bytes 208..223 of the row there: the scale d at 222). Half h2 of a super-block (128 weights) is 64
+// bytes of ql and 32 of qh: slab s = 0..3 of the half (32 weights) has its low four bits in the low (s < 2) or high nibbles of
+// ql[64 h2 + 32 (s & 1) ..] and its upper two at bit 2 s of qh[32 h2 ..]; a scale per chunk of 16, a zero point of 32. The matrix-core
+// product must keep the two chunks of a slab apart: the operand's row 8 c + m holds row m of x with everything but chunk c of the slab
+// zeroed, so the result's rows 0..7 are chunk 0's sums and rows 8..15 chunk 1's (rows 16..31 are unused).
 template <> struct WBlock<kQ6_K> {
     static constexpr int kBytes = 210, kTerms = 1;
-    u32x4 ql[2][2], qh[2], sc;
-    uint32_t d;
-    __device__ __forceinline__ static u32x4 load16(const uint8_t* p) {
-        u32x4 v;
-        __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
-        return v;
-    }
-    __device__ __forceinline__ void load(const uint8_t* wb, int lh) {
-#pragma unroll
-        for (int h2 = 0; h2 < 2; h2++) {
-            ql[h2][0] = load16(wb + 64 * h2 + 16 * lh);
-            ql[h2][1] = load16(wb + 64 * h2 + 32 + 16 * lh);
-            qh[h2] = load16(wb + 128 + 32 * h2 + 16 * lh);
-        }
-        sc = load16(wb + 192);
-        d = *(const uint16_t*)(wb + 208);
-    }
+    static constexpr int kPieces = 14, kStride = 240;  // 60 dwords: as above
+    __device__ __forceinline__ static int piece_offset(int c) { return c < 13 ? 16 * c : 194; }
     // t[0] = d_w d_x float(sum over the chunks of sc (q . x - 32 sum of x))
-    __device__ __forceinline__ void terms(const uint8_t* xl, int l32, int lh, f32x4* t) const {
+    __device__ __forceinline__ static void terms(const uint8_t* wl, const uint8_t* xl, int l32, int lh, f32x4* t) {
         const bool keep = (l32 >> 3) == lh;  // operand rows 0..7 keep the first 16 of a slab (held by lanes of half 0), rows 8..15 the second
-        const uint8_t* xrow = xl + kXq + (l32 & 7) * 256 + 16 * lh;
+        const uint8_t* xrow = xl + kXq + (l32 & 7) * kXRow + 16 * lh;
         int sumi[4] = {0, 0, 0, 0}, summ[4] = {0, 0, 0, 0};
         u32x4 sv[4][2];
 #pragma unroll
@@ -148,14 +139,17 @@ template <> struct WBlock<kQ6_K> {
             sv[jj][1] = *(const u32x4*)(xl + kXs + (4 * lh + jj) * 32 + 16);
         }
         const f32x4 xd = *(const f32x4*)(xl + kXd + 16 * lh);
+        const u32x4 sc = *(const u32x4*)(wl + 192);
 #pragma unroll
-        for (int h2 = 0; h2 < 2; h2++)
+        for (int h2 = 0; h2 < 2; h2++) {
+            const u32x4 ql[2] = {*(const u32x4*)(wl + 64 * h2 + 16 * lh), *(const u32x4*)(wl + 64 * h2 + 32 + 16 * lh)};
+            const u32x4 qh = *(const u32x4*)(wl + 128 + 32 * h2 + 16 * lh);
 #pragma unroll
             for (int s = 0; s < 4; s++) {
                 i32x4 w, xa = *(const i32x4*)(xrow + 128 * h2 + 32 * s);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const uint32_t lo = (ql[h2][s & 1][i] >> (s & 2 ? 4 : 0)) & 0x0F0F0F0Fu, hi = (qh[h2][i] >> (2 * s)) & 0x03030303u;
+                    const uint32_t lo = (ql[s & 1][i] >> (s & 2 ? 4 : 0)) & 0x0F0F0F0Fu, hi = (qh[i] >> (2 * s)) & 0x03030303u;
                     w[i] = (int)(lo | (hi << 4));  // 0..63
                     xa[i] = keep ? xa[i] : 0;
                 }
@@ -169,12 +163,13 @@ template <> struct WBlock<kQ6_K> {
                 const uint32_t pair = ((uint32_t)sca & 0xffffu) | ((uint32_t)scb << 16);
 #pragma unroll
                 for (int jj = 0; jj < 4; jj++) {
-                    sumi[jj] += sca * c[jj] + scb * c[4 + jj];
+                    sumi[jj] += __mul24(sca, c[jj]) + __mul24(scb, c[4 + jj]);  // |sum| <= 16 * 63 * 127, int8 scales
                     const uint32_t ps = sv[jj][h2][s];  // a copy: __builtin_bit_cast of a vector's element takes element 0 with this compiler
                     summ[jj] = __builtin_amdgcn_sdot2(__builtin_bit_cast(s16x2, ps), __builtin_bit_cast(s16x2, pair), summ[jj], false);
                 }
             }
-        const float dw = f16_bits_to_f32((uint16_t)d);
+        }
+        const float dw = f16_bits_to_f32(*(const uint16_t*)(wl + 222));
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             const float dd = dw * xd[jj];
@@ -183,30 +178,45 @@ template <> struct WBlock<kQ6_K> {
     }
 };
 
-// The pieces of x of a super-block a lane fetches for the wavefront's LDS.
-struct XPieces {
+// What a lane fetches of a super-block: its pieces of W, and of x for the wavefront's LDS.
+template <int LOADS> struct Stage {
+    u32x4 w[LOADS];
     u32x4 xq[2];  // two 16-byte pieces of the eight rows' quants
     u32x4 xs;     // lanes 0..15: a piece of their sums
     float xd;     // lanes 0..7: a row's scale
 };
 
-template <int DT, int kWaves>
+// DEPTH: super-blocks a wavefront has requested or in work at a time.
+template <int DT, int kWaves, int DEPTH>
 __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_t* __restrict__ W, const uint8_t* act, float* y, const float* resid,
                                                                      int M_all, int N, int nsb, int64_t act_row_bytes) {
     typedef WBlock<DT> WB;
-    constexpr int kT = WB::kTerms;
-    extern __shared__ __align__(16) uint8_t smem[];  // terms [nsb][kT][64] of four floats, then a super-block of x per wavefront
+    constexpr int kT = WB::kTerms, kAll = 32 * WB::kPieces, kLoads = (kAll + 63) / 64, kSlab = 32 * WB::kStride;
+    typedef Stage<kLoads> St;
+    extern __shared__ __align__(16) uint8_t smem[];  // terms [nsb][kT][64] of four floats, then per wavefront a super-block of x and the slab of W
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // blockIdx.z: the group of eight rows of x
     const int64_t row0 = (int64_t)kRows * blockIdx.z;
     act += row0 * act_row_bytes;
     const int M = M_all - (int)row0 < kRows ? M_all - (int)row0 : kRows;
-    const int n = blockIdx.x * 32 + l32;
-    const uint8_t* wrow = W + (int64_t)(n < N ? n : N - 1) * nsb * WB::kBytes;
+    const int n0 = blockIdx.x * 32, n = n0 + l32;
     f32x4* terms = (f32x4*)smem;
-    uint8_t* xl = smem + (size_t)nsb * kT * 1024 + wave * kXBytes;
+    uint8_t* xl = smem + (size_t)nsb * kT * 1024 + wave * (kXBytes + kSlab);
+    uint8_t* slab = xl + kXBytes;
 
+    // piece p = 64 i + lane of a super-block of the 32 rows: row p / kPieces, piece p % kPieces of it
+    const uint8_t* wbase = W + (int64_t)n0 * nsb * WB::kBytes;
+    uint32_t goff[kLoads], loff[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; i++) {
+        int p = 64 * i + lane;
+        p = p < kAll ? p : kAll - 1;  // a last load that is not full repeats the last piece in its upper lanes
+        const int r = p / WB::kPieces, c = p - WB::kPieces * r;
+        const int row = n0 + r < N ? n0 + r : N - 1;
+        goff[i] = (uint32_t)(row - n0) * (uint32_t)(nsb * WB::kBytes) + WB::piece_offset(c);  // 32 rows of W within 4 GB (checked by the host)
+        loff[i] = r * WB::kStride + 16 * c;
+    }
     // pieces of x a lane fetches: quants p = lane, 64 + lane (row p / 16, bytes 16 (p % 16)..); sums (lanes below 16:
     // row lane / 2, half lane % 2); scale (lanes below 8: row lane). Rows from M on repeat the last one.
     const uint8_t* xsrc[2];
@@ -219,42 +229,76 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
     const uint8_t* ssrc = act + (int64_t)(rs & 7) * act_row_bytes + (int64_t)nsb * 256 + 16 * (lane & 1);
     const uint8_t* dsrc = act + (int64_t)(rd & 7) * act_row_bytes + (int64_t)nsb * 288;
 
-    auto fetch = [&](WB& w, XPieces& f, int sb) {
-        w.load(wrow + (int64_t)sb * WB::kBytes, lh);
+    auto fetch = [&](St& f, int sb) {
+        const uint8_t* wb = wbase + (int64_t)sb * WB::kBytes;
+#pragma unroll
+        for (int i = 0; i < kLoads; i++) {
+            if (DT == kQ4_K) f.w[i] = *(const u32x4*)(wb + goff[i]);
+            else __builtin_memcpy(&f.w[i], __builtin_assume_aligned(wb + goff[i], 2), 16);
+        }
 #pragma unroll
         for (int i = 0; i < 2; i++) f.xq[i] = *(const u32x4*)(xsrc[i] + (int64_t)sb * 256);
         if (lane < 16) f.xs = *(const u32x4*)(ssrc + (int64_t)sb * 32);
         if (lane < 8) f.xd = ((const float*)dsrc)[sb];
     };
-
-    WB wcur, wnxt;
-    XPieces xcur, xnxt;
-    if (wave < nsb) fetch(wcur, xcur, wave);
-    for (int sb = wave; sb < nsb; sb += kWaves) {
-        fetch(wnxt, xnxt, sb + kWaves < nsb ? sb + kWaves : sb);
-        // x of the super-block into this wavefront's LDS (its own: a wavefront's LDS operations complete in order)
+    auto work = [&](const St& f, int sb) {
+        // W and x of the super-block into this wavefront's LDS (its own: a wavefront's LDS operations complete in order)
 #pragma unroll
-        for (int i = 0; i < 2; i++) *(u32x4*)(xl + kXq + 16 * (64 * i + lane)) = xcur.xq[i];
-        if (lane < 16) *(u32x4*)(xl + kXs + 16 * lane) = xcur.xs;
-        if (lane < 8) *(float*)(xl + kXd + 4 * lane) = xcur.xd;
+        for (int i = 0; i < kLoads; i++)
+            if (64 * (i + 1) <= kAll || lane < kAll - 64 * i) *(u32x4*)(slab + loff[i]) = f.w[i];
+#pragma unroll
+        for (int i = 0; i < 2; i++) *(u32x4*)(xl + kXq + ((64 * i + lane) >> 4) * kXRow + 16 * (lane & 15)) = f.xq[i];
+        if (lane < 16) *(u32x4*)(xl + kXs + 16 * lane) = f.xs;
+        if (lane < 8) *(float*)(xl + kXd + 4 * lane) = f.xd;
         f32x4 t[kT];
-        wcur.terms(xl, l32, lh, t);
+        WB::terms(slab + l32 * WB::kStride, xl, l32, lh, t);
 #pragma unroll
         for (int i = 0; i < kT; i++) terms[(sb * kT + i) * 64 + lane] = t[i];
-        wcur = wnxt;
-        xcur = xnxt;
+    };
+    if constexpr (DEPTH == 2) {  // one in work, the next requested
+        St cur, nxt;
+        if (wave < nsb) fetch(cur, wave);
+        for (int sb = wave; sb < nsb; sb += kWaves) {
+            fetch(nxt, sb + kWaves < nsb ? sb + kWaves : sb);
+            work(cur, sb);
+            cur = nxt;
+        }
+    } else {  // DEPTH register sets, each refilled when its super-block is done
+        St f[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++)
+            if (wave + d * kWaves < nsb) fetch(f[d], wave + d * kWaves);
+        for (int sb0 = wave; sb0 < nsb; sb0 += DEPTH * kWaves) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; d++) {
+                const int sb = sb0 + d * kWaves;  // the same for the whole wavefront
+                if (sb >= nsb) break;
+                work(f[d], sb);
+                if (sb + DEPTH * kWaves < nsb) fetch(f[d], sb + DEPTH * kWaves);
+            }
+        }
     }
     __syncthreads();
     if (wave != 0) return;
     f32x4 acc[kT];
 #pragma unroll
     for (int i = 0; i < kT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int sb = 0; sb < nsb; sb++) {  // the CPU's order
+    // the CPU's order; eight super-blocks' terms are requested together so that the chain of additions does not wait for LDS each time
+    for (int sb0 = 0; sb0 < nsb; sb0 += 8) {
+        f32x4 t[8][kT];
 #pragma unroll
-        for (int i = 0; i < kT; i++) {
-            const f32x4 t = terms[(sb * kT + i) * 64 + lane];
+        for (int j = 0; j < 8; j++) {
+            const int sb = sb0 + j < nsb ? sb0 + j : nsb - 1;
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) acc[i][jj] = acc[i][jj] + t[jj];
+            for (int i = 0; i < kT; i++) t[j][i] = terms[(sb * kT + i) * 64 + lane];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if (sb0 + j >= nsb) break;
+#pragma unroll
+            for (int i = 0; i < kT; i++)
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) acc[i][jj] = acc[i][jj] + t[j][i][jj];
         }
     }
     if (n < N) {
@@ -276,18 +320,23 @@ static int g_kq_rows = 0;  // measurement aid: 1 = never, 2 = for any number of 
 void set_kquant_rows(int v) { g_kq_rows = v; }
 
 static int g_kq_rows_waves = 0;  // measurement aid: 4 or 8 wavefronts to a workgroup whatever the type
-void set_kquant_rows_waves(int v) { g_kq_rows_waves = v; }
-// Q6_K's kernel holds more of W in registers (three wavefronts to a SIMD): four wavefronts to a workgroup let three workgroups share a
-// compute unit where eight would leave it to one.
-static int rows_waves(int dt) { return g_kq_rows_waves == 4 || g_kq_rows_waves == 8 ? g_kq_rows_waves : dt == kQ4_K ? 8 : 4; }
-static size_t rows_lds(int dt, int64_t nsb) { return (size_t)nsb * (dt == kQ4_K ? 2 : 1) * 1024 + 8 * kXBytes; }
+static int g_kq_rows_depth = 0;  // measurement aid: 2 or 3 super-blocks under way whatever the shape
+void set_kquant_rows_waves(int v) {
+    if (v == 0) g_kq_rows_depth = g_kq_rows_waves = 0;
+    else if (v == 2 || v == 3) g_kq_rows_depth = v;
+    else g_kq_rows_waves = v;
+}
+// LDS of a workgroup: the terms, and per wavefront a super-block of x and the slab of W.
+static size_t rows_lds(int dt, int64_t nsb, int waves) {
+    return (size_t)nsb * (dt == kQ4_K ? 2 : 1) * 1024 + (size_t)waves * (kXBytes + 32 * (dt == kQ4_K ? WBlock<kQ4_K>::kStride : WBlock<kQ6_K>::kStride));
+}
 
 // Two rows of x or more, converted (kq_convert_act); the terms of 32 rows of W in LDS; Q4_K's W 16-byte aligned, Q6_K's on an even address.
 bool qgemv_kquant_rows_ok(int dt, const QGemvArgs& a) {
     const int64_t nsb = a.K / 256;
     return (dt == kQ4_K || dt == kQ6_K) && g_kq_rows != 1 && a.M >= 2 && a.M <= 8 * 65535 && a.act && a.K % 256 == 0 && nsb > 0 &&
            ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0 && ((uintptr_t)a.act & 15) == 0 && a.N > 0 && a.N <= (1ll << 30) &&
-           rows_lds(dt, nsb) <= 160 * 1024;
+           rows_lds(dt, nsb, 4) <= 160 * 1024 && 32 * nsb * 210 < ((int64_t)1 << 32);
 }
 
 // Where it is the faster choice. A pass over W for eight rows of x runs at about 3.3 TB/s (Q4_K; 14336 x 4096 in 11 us, 28672 x 4096
@@ -300,29 +349,44 @@ bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a) {
     if (a.M > 64) return false;
     const double nsb = (double)(a.K / 256), groups = (double)((a.M + kRows - 1) / kRows);
     const double rows_us = groups * (double)a.N * nsb * (dt == kQ4_K ? 144 / 3.3e6 : 210 / 2.6e6);
-    const int64_t tiles = ((a.M + 127) / 128) * ((a.N + 127) / 128);
-    return rows_us < (double)((tiles + 255) / 256) * nsb * 2.1;
+    // (its 2.1 us hold up to some 128 tiles at a time: 112 tiles take 35 us at K = 4096, 224 take 63)
+    const double tiles = (double)(((a.M + 127) / 128) * ((a.N + 127) / 128));
+    return rows_us < (tiles > 128 ? tiles / 128 : 1.0) * nsb * 2.1;
 }
 
-template <int DT, int WAVES>
+template <int DT, int WAVES, int DEPTH>
 static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st) {
     const int nsb = (int)(a.K / 256);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, DEPTH>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         raised = true;
     }
-    const size_t lds = (size_t)nsb * WBlock<DT>::kTerms * 1024 + WAVES * kXBytes;
-    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)), dim3(64 * WAVES),
-                       lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, a.resid, (int)a.M, (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+    const size_t lds = rows_lds(DT, nsb, WAVES);
+    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES, DEPTH>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)),
+                       dim3(64 * WAVES), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, a.resid, (int)a.M, (int)a.N, nsb,
+                       (int64_t)kq_act_bytes(a.K));
     return hipGetLastError();
 }
 
+// Wavefronts a workgroup and super-blocks under way, as measured at eight rows of x (us with the conversion of x, Q4_K | Q6_K, for 4
+// wavefronts and 2 under way, 4 and 3, 8 and 2, 8 and 3): 14336 x 4096 11.1 11.9 14.2 13.8 | 16.3 17.1 19.4 17.6; 4096 x 4096 7.7 7.8
+// 7.1 7.1 | 10.2 10.9 9.4 8.9; 28672 x 4096 20.3 21.4 26.8 26.5 | 34.3 33.7 42.3 38.1; 4096 x 14336 20.6 19.8 (no room for eight) |
+// 26.6 28.3 22.1 22.8. Eight where the workgroups are at most one to a compute unit, four where they are many.
 hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st) {
-    const bool eight = rows_waves(dt) == 8;
-    if (dt == kQ4_K) return eight ? launch_kq_rows<kQ4_K, 8>(a, st) : launch_kq_rows<kQ4_K, 4>(a, st);
-    return eight ? launch_kq_rows<kQ6_K, 8>(a, st) : launch_kq_rows<kQ6_K, 4>(a, st);
+    const int64_t nsb = a.K / 256, wgs = (a.N + 31) / 32 * ((a.M + kRows - 1) / kRows);
+    int waves = wgs <= 256 ? 8 : 4;
+    int depth = dt == kQ6_K && waves == 8 && nsb <= 32 ? 3 : 2;
+    if (g_kq_rows_waves == 4 || g_kq_rows_waves == 8) waves = g_kq_rows_waves;
+    if (rows_lds(dt, nsb, waves) > 160 * 1024) waves = 4;
+    if (g_kq_rows_depth == 2 || g_kq_rows_depth == 3) depth = g_kq_rows_depth;
+    if (dt == kQ4_K) {
+        if (waves == 8) return depth == 3 ? launch_kq_rows<kQ4_K, 8, 3>(a, st) : launch_kq_rows<kQ4_K, 8, 2>(a, st);
+        return depth == 3 ? launch_kq_rows<kQ4_K, 4, 3>(a, st) : launch_kq_rows<kQ4_K, 4, 2>(a, st);
+    }
+    if (waves == 8) return depth == 3 ? launch_kq_rows<kQ6_K, 8, 3>(a, st) : launch_kq_rows<kQ6_K, 8, 2>(a, st);
+    return depth == 3 ? launch_kq_rows<kQ6_K, 4, 3>(a, st) : launch_kq_rows<kQ6_K, 4, 2>(a, st);
 }
 
 }  // namespace mimir
