@@ -449,7 +449,7 @@ def main():
     ap.add_argument("--counters", type=int, default=0, metavar="N",
                     help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
     ap.add_argument("--gemm", action="store_true", help="also time the prompt-sized Q4_0 product on the matrix cores (M = 512, 2048)")
-    ap.add_argument("--rows", action="store_true", help="also time the Q4_0 product of eight rows of x (a batch's decoding step) at the model's shapes")
+    ap.add_argument("--rows", action="store_true", help="also time the Q4_0, Q4_K and Q6_K products of eight rows of x (a batch's decoding step) at the model's shapes")
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
                     help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
                          "rows_kernel, rows_kernel_no_lds_pass, one_row_kernel_per_row (Q4_0), q4_K_rows_kernel, q6_K_rows_kernel, ...")

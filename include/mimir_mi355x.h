@@ -306,7 +306,7 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * "kquant.mfma_rows" = 1 keeps Q4_K / Q6_K products of a few rows of x off the
  * kernel that reads W once per eight rows, 2 sends them there for any number of
  * rows from two on; "kquant.mfma_rows_waves" = 4 or 8 fixes its wavefronts a
- * workgroup, 2 or 3 the super-blocks a wavefront has under way (0: both by shape).
+ * workgroup, 1 keeps its partial sums in LDS whatever K is (0: both by shape).
  * "qgemm.path" = 1 makes mi355x_qgemm_bf16 take its general route for every shape.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).

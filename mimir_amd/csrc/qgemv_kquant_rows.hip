@@ -186,14 +186,17 @@ template <int LOADS> struct Stage {
     float xd;     // lanes 0..7: a row's scale
 };
 
-// DEPTH: super-blocks a wavefront has requested or in work at a time.
-template <int DT, int kWaves, int DEPTH>
+// CHAIN > 0: a wavefront takes a contiguous run of at most CHAIN super-blocks and keeps its terms in registers; the sums then pass
+// from wavefront to wavefront through LDS in the super-blocks' order (a barrier a wavefront). LDS holds no terms then, so more
+// workgroups share a compute unit and long rows leave room for eight wavefronts. CHAIN = 0: super-blocks round robin, terms
+// [nsb][kT][64] in LDS, summed by the first wavefront (any K that fits).
+template <int DT, int kWaves, int CHAIN>
 __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_t* __restrict__ W, const uint8_t* act, float* y, const float* resid,
                                                                      int M_all, int N, int nsb, int64_t act_row_bytes) {
     typedef WBlock<DT> WB;
     constexpr int kT = WB::kTerms, kAll = 32 * WB::kPieces, kLoads = (kAll + 63) / 64, kSlab = 32 * WB::kStride;
     typedef Stage<kLoads> St;
-    extern __shared__ __align__(16) uint8_t smem[];  // terms [nsb][kT][64] of four floats, then per wavefront a super-block of x and the slab of W
+    extern __shared__ __align__(16) uint8_t smem[];  // terms (or the sums handed on), then per wavefront a super-block of x and the slab of W
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // blockIdx.z: the group of eight rows of x
@@ -202,7 +205,7 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
     const int M = M_all - (int)row0 < kRows ? M_all - (int)row0 : kRows;
     const int n0 = blockIdx.x * 32, n = n0 + l32;
     f32x4* terms = (f32x4*)smem;
-    uint8_t* xl = smem + (size_t)nsb * kT * 1024 + wave * (kXBytes + kSlab);
+    uint8_t* xl = smem + (size_t)(CHAIN ? 1 : nsb) * kT * 1024 + wave * (kXBytes + kSlab);
     uint8_t* slab = xl + kXBytes;
 
     // piece p = 64 i + lane of a super-block of the 32 rows: row p / kPieces, piece p % kPieces of it
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
         if (lane < 16) f.xs = *(const u32x4*)(ssrc + (int64_t)sb * 32);
         if (lane < 8) f.xd = ((const float*)dsrc)[sb];
     };
-    auto work = [&](const St& f, int sb) {
+    auto work = [&](const St& f, f32x4* t) {
         // W and x of the super-block into this wavefront's LDS (its own: a wavefront's LDS operations complete in order)
 #pragma unroll
         for (int i = 0; i < kLoads; i++)
@@ -250,55 +253,78 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
         for (int i = 0; i < 2; i++) *(u32x4*)(xl + kXq + ((64 * i + lane) >> 4) * kXRow + 16 * (lane & 15)) = f.xq[i];
         if (lane < 16) *(u32x4*)(xl + kXs + 16 * lane) = f.xs;
         if (lane < 8) *(float*)(xl + kXd + 4 * lane) = f.xd;
-        f32x4 t[kT];
         WB::terms(slab + l32 * WB::kStride, xl, l32, lh, t);
-#pragma unroll
-        for (int i = 0; i < kT; i++) terms[(sb * kT + i) * 64 + lane] = t[i];
     };
-    if constexpr (DEPTH == 2) {  // one in work, the next requested
-        St cur, nxt;
-        if (wave < nsb) fetch(cur, wave);
-        for (int sb = wave; sb < nsb; sb += kWaves) {
-            fetch(nxt, sb + kWaves < nsb ? sb + kWaves : sb);
-            work(cur, sb);
-            cur = nxt;
-        }
-    } else {  // DEPTH register sets, each refilled when its super-block is done
-        St f[DEPTH];
-#pragma unroll
-        for (int d = 0; d < DEPTH; d++)
-            if (wave + d * kWaves < nsb) fetch(f[d], wave + d * kWaves);
-        for (int sb0 = wave; sb0 < nsb; sb0 += DEPTH * kWaves) {
-#pragma unroll
-            for (int d = 0; d < DEPTH; d++) {
-                const int sb = sb0 + d * kWaves;  // the same for the whole wavefront
-                if (sb >= nsb) break;
-                work(f[d], sb);
-                if (sb + DEPTH * kWaves < nsb) fetch(f[d], sb + DEPTH * kWaves);
-            }
-        }
-    }
-    __syncthreads();
-    if (wave != 0) return;
     f32x4 acc[kT];
 #pragma unroll
     for (int i = 0; i < kT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // the CPU's order; eight super-blocks' terms are requested together so that the chain of additions does not wait for LDS each time
-    for (int sb0 = 0; sb0 < nsb; sb0 += 8) {
-        f32x4 t[8][kT];
+    if constexpr (CHAIN > 0) {
+        const int sb_lo = wave * nsb / kWaves, count = (wave + 1) * nsb / kWaves - sb_lo;  // at most CHAIN (the host's choice of CHAIN)
+        St f[2];
+        f32x4 tt[CHAIN][kT];
+        if (count > 0) fetch(f[0], sb_lo);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int sb = sb0 + j < nsb ? sb0 + j : nsb - 1;
-#pragma unroll
-            for (int i = 0; i < kT; i++) t[j][i] = terms[(sb * kT + i) * 64 + lane];
+        for (int j = 0; j < CHAIN; j++) {
+            if (j < count) {  // the same for the whole wavefront
+                if (j + 1 < count) fetch(f[(j + 1) & 1], sb_lo + j + 1);
+                work(f[j & 1], tt[j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one super-block's work at a time: interleaved they would not fit the registers
         }
+        // wavefront w adds its terms, the CPU's next ones, to the sums of those before it and hands them on
+        for (int w = 0; w < kWaves; w++) {
+            if (w == wave) {
+                if (w > 0) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            if (sb0 + j >= nsb) break;
+                    for (int i = 0; i < kT; i++) acc[i] = terms[i * 64 + lane];
+                }
 #pragma unroll
-            for (int i = 0; i < kT; i++)
+                for (int j = 0; j < CHAIN; j++) {
+                    if (j < count) {
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) acc[i][jj] = acc[i][jj] + t[j][i][jj];
+                        for (int i = 0; i < kT; i++)
+#pragma unroll
+                            for (int jj = 0; jj < 4; jj++) acc[i][jj] = acc[i][jj] + tt[j][i][jj];
+                    }
+                }
+                if (w + 1 < kWaves) {
+#pragma unroll
+                    for (int i = 0; i < kT; i++) terms[i * 64 + lane] = acc[i];
+                }
+            }
+            if (w + 1 < kWaves) __syncthreads();
+        }
+        if (wave != kWaves - 1) return;
+    } else {
+        St cur, nxt;  // one in work, the next requested
+        if (wave < nsb) fetch(cur, wave);
+        for (int sb = wave; sb < nsb; sb += kWaves) {
+            fetch(nxt, sb + kWaves < nsb ? sb + kWaves : sb);
+            f32x4 t[kT];
+            work(cur, t);
+#pragma unroll
+            for (int i = 0; i < kT; i++) terms[(sb * kT + i) * 64 + lane] = t[i];
+            cur = nxt;
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        // the CPU's order; eight super-blocks' terms are requested together so that the chain of additions does not wait for LDS each time
+        for (int sb0 = 0; sb0 < nsb; sb0 += 8) {
+            f32x4 t[8][kT];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int sb = sb0 + j < nsb ? sb0 + j : nsb - 1;
+#pragma unroll
+                for (int i = 0; i < kT; i++) t[j][i] = terms[(sb * kT + i) * 64 + lane];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (sb0 + j >= nsb) break;
+#pragma unroll
+                for (int i = 0; i < kT; i++)
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) acc[i][jj] = acc[i][jj] + t[j][i][jj];
+            }
         }
     }
     if (n < N) {
@@ -319,16 +345,18 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
 static int g_kq_rows = 0;  // measurement aid: 1 = never, 2 = for any number of rows the kernel takes
 void set_kquant_rows(int v) { g_kq_rows = v; }
 
-static int g_kq_rows_waves = 0;  // measurement aid: 4 or 8 wavefronts to a workgroup whatever the type
-static int g_kq_rows_depth = 0;  // measurement aid: 2 or 3 super-blocks under way whatever the shape
+static int g_kq_rows_waves = 0;  // measurement aid: 4 or 8 wavefronts to a workgroup whatever the shape
+static int g_kq_rows_chain = 0;  // measurement aid: 1 = terms in LDS whatever the shape
 void set_kquant_rows_waves(int v) {
-    if (v == 0) g_kq_rows_depth = g_kq_rows_waves = 0;
-    else if (v == 2 || v == 3) g_kq_rows_depth = v;
+    if (v == 0) g_kq_rows_chain = g_kq_rows_waves = 0;
+    else if (v == 1) g_kq_rows_chain = 1;
     else g_kq_rows_waves = v;
 }
-// LDS of a workgroup: the terms, and per wavefront a super-block of x and the slab of W.
-static size_t rows_lds(int dt, int64_t nsb, int waves) {
-    return (size_t)nsb * (dt == kQ4_K ? 2 : 1) * 1024 + (size_t)waves * (kXBytes + 32 * (dt == kQ4_K ? WBlock<kQ4_K>::kStride : WBlock<kQ6_K>::kStride));
+
+// LDS of a workgroup: the terms (or the sums handed on), and per wavefront a super-block of x and the slab of W.
+static size_t rows_lds(int dt, int64_t nsb, int waves, bool chain) {
+    return (size_t)(chain ? 1 : nsb) * (dt == kQ4_K ? 2 : 1) * 1024 +
+           (size_t)waves * (kXBytes + 32 * (dt == kQ4_K ? WBlock<kQ4_K>::kStride : WBlock<kQ6_K>::kStride));
 }
 
 // Two rows of x or more, converted (kq_convert_act); the terms of 32 rows of W in LDS; Q4_K's W 16-byte aligned, Q6_K's on an even address.
@@ -336,7 +364,7 @@ bool qgemv_kquant_rows_ok(int dt, const QGemvArgs& a) {
     const int64_t nsb = a.K / 256;
     return (dt == kQ4_K || dt == kQ6_K) && g_kq_rows != 1 && a.M >= 2 && a.M <= 8 * 65535 && a.act && a.K % 256 == 0 && nsb > 0 &&
            ((uintptr_t)a.W & (dt == kQ4_K ? 15 : 1)) == 0 && ((uintptr_t)a.act & 15) == 0 && a.N > 0 && a.N <= (1ll << 30) &&
-           rows_lds(dt, nsb, 4) <= 160 * 1024 && 32 * nsb * 210 < ((int64_t)1 << 32);
+           (nsb <= 64 || rows_lds(dt, nsb, 4, false) <= 160 * 1024) && 32 * nsb * 210 < ((int64_t)1 << 32);
 }
 
 // Where it is the faster choice. A pass over W for eight rows of x runs at about 3.3 TB/s (Q4_K; 14336 x 4096 in 11 us, 28672 x 4096
@@ -354,39 +382,35 @@ bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a) {
     return rows_us < (tiles > 128 ? tiles / 128 : 1.0) * nsb * 2.1;
 }
 
-template <int DT, int WAVES, int DEPTH>
+template <int DT, int WAVES, int CHAIN>
 static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st) {
     const int nsb = (int)(a.K / 256);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, DEPTH>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, CHAIN>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         raised = true;
     }
-    const size_t lds = rows_lds(DT, nsb, WAVES);
-    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES, DEPTH>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)),
-                       dim3(64 * WAVES), lds, st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, a.resid, (int)a.M, (int)a.N, nsb,
-                       (int64_t)kq_act_bytes(a.K));
+    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES, CHAIN>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)),
+                       dim3(64 * WAVES), rows_lds(DT, nsb, WAVES, CHAIN > 0), st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, a.resid, (int)a.M,
+                       (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
     return hipGetLastError();
 }
 
-// Wavefronts a workgroup and super-blocks under way, as measured at eight rows of x (us with the conversion of x, Q4_K | Q6_K, for 4
-// wavefronts and 2 under way, 4 and 3, 8 and 2, 8 and 3): 14336 x 4096 11.1 11.9 14.2 13.8 | 16.3 17.1 19.4 17.6; 4096 x 4096 7.7 7.8
-// 7.1 7.1 | 10.2 10.9 9.4 8.9; 28672 x 4096 20.3 21.4 26.8 26.5 | 34.3 33.7 42.3 38.1; 4096 x 14336 20.6 19.8 (no room for eight) |
-// 26.6 28.3 22.1 22.8. Eight where the workgroups are at most one to a compute unit, four where they are many.
+// Eight wavefronts where the workgroups are at most one to a compute unit or the rows are long, four where they are many (measured at
+// eight rows of x, us with the conversion of x, Q4_K | Q6_K, four and eight wavefronts: 14336 x 4096 11.1 14.2 | 16.0 19.2; 4096 x 4096
+// 7.6 7.1 | 10.1 9.3; 28672 x 4096 20.5 27.3 | 33.5 41.8). Rows of more than four super-blocks a wavefront (K above 8192 with eight) keep
+// the terms in registers, in runs of up to eight super-blocks (4096 x 14336: 16.3 | 21.3 us, 19.9 | 21.9 with the terms in LDS, which leave
+// room for four wavefronts only); shorter ones gain nothing from it (the registers cost what the LDS gives), longer ones have no choice.
 hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st) {
     const int64_t nsb = a.K / 256, wgs = (a.N + 31) / 32 * ((a.M + kRows - 1) / kRows);
-    int waves = wgs <= 256 ? 8 : 4;
-    int depth = dt == kQ6_K && waves == 8 && nsb <= 32 ? 3 : 2;
+    int waves = wgs <= 256 || nsb > 32 ? 8 : 4;
     if (g_kq_rows_waves == 4 || g_kq_rows_waves == 8) waves = g_kq_rows_waves;
-    if (rows_lds(dt, nsb, waves) > 160 * 1024) waves = 4;
-    if (g_kq_rows_depth == 2 || g_kq_rows_depth == 3) depth = g_kq_rows_depth;
-    if (dt == kQ4_K) {
-        if (waves == 8) return depth == 3 ? launch_kq_rows<kQ4_K, 8, 3>(a, st) : launch_kq_rows<kQ4_K, 8, 2>(a, st);
-        return depth == 3 ? launch_kq_rows<kQ4_K, 4, 3>(a, st) : launch_kq_rows<kQ4_K, 4, 2>(a, st);
-    }
-    if (waves == 8) return depth == 3 ? launch_kq_rows<kQ6_K, 8, 3>(a, st) : launch_kq_rows<kQ6_K, 8, 2>(a, st);
-    return depth == 3 ? launch_kq_rows<kQ6_K, 4, 3>(a, st) : launch_kq_rows<kQ6_K, 4, 2>(a, st);
+    bool chain = g_kq_rows_chain != 1 && nsb > 4 * waves && nsb <= 64;
+    if (chain) waves = 8;
+    else if (rows_lds(dt, nsb, waves, false) > 160 * 1024) waves = 4;
+    if (dt == kQ4_K) return chain ? launch_kq_rows<kQ4_K, 8, 8>(a, st) : waves == 8 ? launch_kq_rows<kQ4_K, 8, 0>(a, st) : launch_kq_rows<kQ4_K, 4, 0>(a, st);
+    return chain ? launch_kq_rows<kQ6_K, 8, 8>(a, st) : waves == 8 ? launch_kq_rows<kQ6_K, 8, 0>(a, st) : launch_kq_rows<kQ6_K, 4, 0>(a, st);
 }
 
 }  // namespace mimir

@@ -535,12 +535,15 @@ def test_kquant_gemv_single_row_rounds_x_in_the_product(dt):
 
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
-@pytest.mark.parametrize("m,n,k", [(2, 33, 256), (5, 100, 512), (8, 203, 4096), (11, 64, 256 * 9), (20, 31, 256 * 56), (40, 130, 1024)])
+@pytest.mark.parametrize("m,n,k", [(2, 33, 256), (5, 100, 512), (8, 203, 4096), (11, 64, 256 * 9), (20, 31, 256 * 56), (40, 130, 1024),
+                                   (3, 40, 256 * 37), (4, 33, 256 * 70), (9, 300, 256 * 33)])
 def test_kquant_rows_of_x_share_one_pass_over_w_on_the_matrix_cores(dt, m, n, k):
     """Rows of x, eight at a time, against Q4_K or Q6_K weights read once on the int8 matrix cores (the decoding
     step of a batch; forced here beyond the rows it is chosen for): the CPU's integer sums, and its float32
     operations in its order, so the oracle's bits and those of the one-row kernels. x holds a zero
-    super-block, ties and, in one row, a NaN."""
+    super-block, ties and, in one row, a NaN. Rows of up to 32 super-blocks keep their partial sums in
+    LDS, longer ones (to 64) in registers, handed from wavefront to wavefront; beyond that LDS again, or
+    another kernel where it has no room."""
     l = gpu.lib()
     rng = np.random.default_rng(dt + 7 * m + n + k)
     raw = random_blocks(rng, dt, n * k)
