@@ -19,6 +19,7 @@
 // output projection.
 #include "device_util.h"
 #include "kernels.h"
+#include "kq_act.h"
 #include "q4_rows_act.h"
 
 namespace mimir {
@@ -43,6 +44,7 @@ struct DecParams {
     const int32_t* dyn_k;
     int64_t act_row_bytes;
     int act_rows;  // the converted result in the form for a few rows of x (q4_rows_act.h), all sequences in one buffer
+    int act_kq;    // the converted result as int8 super-blocks for Q4_K / Q6_K products (kq_act.h), rows act_row_bytes apart
 };
 
 __device__ __forceinline__ float group16_sum(float v) {
@@ -331,6 +333,15 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     if (g < ng && lse && lane == 0) lse[(int64_t)b * p.H + h] = L == 0.f ? -__builtin_inff() : M + __builtin_logf(L);
     if (!act) return;
     __syncthreads();
+    if (p.act_kq) {
+        // the heads of this workgroup are whole super-blocks of 256 of the row (checked by the host): a wavefront each
+        const int nsup = ng * D / 256, wv = tid >> 6;
+        if (wv < nsup) {
+            const f32x4 v = *(const f32x4*)(fin + 256 * wv + 4 * lane);
+            kq_convert_superblock(v, (hk * G + g0) * D / 256 + wv, lane, p.H * D / 256, act + (int64_t)b * p.act_row_bytes);
+        }
+        return;
+    }
     // item t: head t / (D/8), block (t % (D/8)) / 4 of the head, dword t % 4
     const int nit = ng * (D / 8);
     if (tid < nit) {
@@ -395,12 +406,19 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
     return lds <= 60 * 1024 && kmax <= INT32_MAX / 2;
 }
 
+// Whether the result can leave in the K-quants' int8 form: the heads a workgroup finishes are whole super-blocks of the row.
+bool attention_decode_kq_ok(const AttnArgs& a) {
+    const int G = a.H / a.HK, per = G < kHeads ? G : kHeads;
+    return (G <= kHeads || G % kHeads == 0) && (per * a.D) % 256 == 0 && (G * a.D) % 256 == 0;
+}
+
 // a.K keys (plus *a.dyn_k), at most kmax. workspace: attention_decode_workspace_bytes
 // bytes whose first 4096 were zero before the first launch (the tickets reset
 // themselves). act, if set, gets row b's result [H * D] in the Q4_0 product's
 // fixed-point form, act_row_bytes apart; out may then be null.
-// act_rows: the form for eight sequences together (q4_rows_act.h), a buffer per group of eight: row b's result as row b % 8 of group b / 8.
-hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, bool act_rows) {
+// act_form: kAttnActQ4 that form; kAttnActRows the form for eight sequences together (q4_rows_act.h), a buffer per group of eight: row b's
+// result as row b % 8 of group b / 8; kAttnActKQ int8 super-blocks for the K-quant products (where attention_decode_kq_ok).
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, int act_form) {
     DecParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];
@@ -413,7 +431,8 @@ hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, vo
     attention_decode_plan(a.B, a.H, a.HK, kmax, &p.nsplit, &p.cmax);
     p.dyn_k = a.dyn_k;
     p.act_row_bytes = act_row_bytes;
-    p.act_rows = act_rows ? 1 : 0;
+    p.act_rows = act_form == kAttnActRows ? 1 : 0;
+    p.act_kq = act_form == kAttnActKQ ? 1 : 0;
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
     dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
     size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);

@@ -202,8 +202,10 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
 void set_attention_decode_splits(int n);
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
+enum { kAttnActQ4 = 0, kAttnActRows = 1, kAttnActKQ = 2 };
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st,
-                            bool act_rows = false);
+                            int act_form = kAttnActQ4);
+bool attention_decode_kq_ok(const AttnArgs& a);
 
 // The fixed-point Q4_0 product of a few rows of float32 x that reads W once per eight of them (qgemv_q4_0_rows.hip,
 // int8 matrix cores): each group of eight rows is converted together by q4_0_rows_convert_act into q4_0_rows_act_bytes(K) bytes,

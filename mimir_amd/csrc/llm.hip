@@ -403,7 +403,7 @@ static mi355x_status step_rows(Model& m) {
                             c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
         }
         at.k = m.keys[i].p; at.v = m.values[i].p;
-        LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, true), "attention");
+        LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, kAttnActRows), "attention");
         LLM_HIP(qgemv_q4_0_rows(b.o.buf.p, act, parts, nullptr, B, c.embed, qd, shares, m.stream), "attn_output");
         LLM_HIP(rows_norm_act(x, parts, shares, b.ffn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "ffn_norm");
         if (g_llama_rows_plain != 2 && g_llama_rows_plain != 3) {  // SiLU * up and the conversion ride on the product, into a buffer of their own
@@ -486,9 +486,15 @@ static mi355x_status step_any(Model& m) {
             at.q = q; at.q_strides[0] = qd;
         }
         at.k = m.keys[i].p; at.v = m.values[i].p;
-        if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream), "attention");
-        else LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
-        if (mi355x_status st = convert_for(m, a, B, qd, {&b.o}, done)) return st;
+        // K-quant output projection: attention leaves its result as the int8 super-blocks that product reads
+        const bool a_kq = one_launch && act_class(b.o, B) == kActKQ && attention_decode_kq_ok(at);
+        if (a_kq) {
+            LLM_HIP(attention_decode(at, c.context, m.act[0].p, m.act[kActKQ].p, (int64_t)kq_act_bytes(qd), m.stream, kAttnActKQ), "attention");
+        } else {
+            if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream), "attention");
+            else LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
+            if (mi355x_status st = convert_for(m, a, B, qd, {&b.o}, done)) return st;
+        }
         if (act_class(b.o, B) != kActNone) {  // the residual rides on the product
             if (mi355x_status st = linear(m, b.o, a, x, B, x)) return st;
         } else {

@@ -20,6 +20,7 @@
 // for the LDS.
 #include "device_util.h"
 #include "kernels.h"
+#include "kq_act.h"
 #include "rope_tail.h"
 
 namespace mimir {
@@ -35,11 +36,6 @@ size_t kq_act_bytes(int64_t K) {
     return (size_t)((nsb * (256 + 32 + 4) + 15) / 16 * 16);
 }
 
-__device__ __forceinline__ int dpp_i32_quad_sum(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0xb1, 0xf, 0xf, true);
-    v += __builtin_amdgcn_update_dpp(0, v, 0x4e, 0xf, 0xf, true);
-    return v;
-}
 __device__ __forceinline__ int dpp_i32_group8_sum(int v) {
     v = dpp_i32_quad_sum(v);
     v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true);
@@ -56,47 +52,6 @@ __device__ __forceinline__ float add_in_order(float acc, float term) {
     for (int q = 0; q < 64 / STRIDE; q++)
         acc = acc + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, term), q * STRIDE));
     return acc;
-}
-
-// quantizeRow for one super-block of 256 with its sums: one wavefront, lane i holding values 4i..4i+3.
-// q: the super-block's 64 dwords of quants; sums: its 16 sums; d: its scale.
-__device__ __forceinline__ void kq_convert_superblock_to(const f32x4 v, int lane, uint32_t* q, uint16_t* sums, float* d_out) {
-    float amax = 0.f;
-    bool finite = true;
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        float a = __builtin_fabsf(v[k]);
-        finite = finite && a < __builtin_inff();
-        if (a > amax) amax = a;
-    }
-    amax = wave_max(amax);
-    float bad = wave_max(finite ? 0.f : 1.f);
-    float d = 0.f;
-    uint32_t packed = 0;
-    int local = 0;
-    if (bad != 0.f) {
-        d = __builtin_nanf("");
-    } else if (amax != 0.f) {
-        d = amax / 127.0f;
-        float id = 127.0f / amax;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            int r = (int)__builtin_rintf(v[k] * id);
-            r = r > 127 ? 127 : r < -127 ? -127 : r;
-            packed |= (uint32_t)(r & 0xff) << (8 * k);
-            local += r;
-        }
-    }
-    q[lane] = packed;
-    int s16 = dpp_i32_quad_sum(local);  // 16 quants = 4 consecutive lanes
-    if ((lane & 3) == 0) sums[lane >> 2] = (uint16_t)(int16_t)s16;
-    if (lane == 0) *d_out = d;
-}
-
-// Into a converted row in global memory (kq_act_bytes' layout).
-__device__ __forceinline__ void kq_convert_superblock(const f32x4 v, int sb, int lane, int nsb, uint8_t* __restrict__ row) {
-    kq_convert_superblock_to(v, lane, (uint32_t*)row + (int64_t)sb * 64, (uint16_t*)(row + (int64_t)nsb * 256) + sb * 16,
-                             (float*)(row + (int64_t)nsb * 288) + sb);
 }
 
 // One wavefront per super-block.

@@ -293,15 +293,19 @@ def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
     assert np.array_equal(runs[1], runs[2]) and np.array_equal(runs[0], runs[2])
 
 
-@pytest.mark.parametrize("linear_dt,batch", [(O.Q4_K, 1), (O.Q6_K, 2), (O.Q8_0, 1), (O.Q4_K, 5), (O.Q4_K, 11), (O.Q6_K, 9)])
-def test_k_quant_and_q8_0_models_decode_from_a_graph(linear_dt, batch):
+@pytest.mark.parametrize("linear_dt,batch,heads,head_dim", [(O.Q4_K, 1, 4, 64), (O.Q6_K, 2, 4, 64), (O.Q8_0, 1, 4, 64), (O.Q4_K, 5, 4, 64),
+                                                            (O.Q4_K, 11, 4, 64), (O.Q6_K, 9, 4, 64), (O.Q4_K, 1, 4, 128), (O.Q6_K, 3, 8, 64),
+                                                            (O.Q4_K, 9, 16, 128)])
+def test_k_quant_and_q8_0_models_decode_from_a_graph(linear_dt, batch, heads, head_dim):
     """Models whose linears are not Q4_0 take the generic decoding step: q|k|v and gate|up as one product
     each over weights kept together, norm and SwiGLU with the int8 conversion in the same launch (K-quants),
     residuals in the products' epilogues, the position on the device, the whole step replayed as a graph. It
-    must choose the tokens of the per-operator path (position from the host) and of the oracle."""
+    must choose the tokens of the per-operator path (position from the host) and of the oracle. Where the query
+    heads of a key-value head are whole super-blocks of 256 (the last three shapes), attention leaves its result
+    in the int8 form the K-quant output projection reads."""
     lib = gpu.lib()
     c = capi.LlamaConfig()
-    c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = 512, 1024, 2, 4, 2, 64, 64, 301
+    c.embed, c.hidden, c.layers, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.vocab = 512, 1024, 2, heads, 2, head_dim, head_dim, 301
     c.context, c.interleaved, c.cache_dtype, c.batch = 64, 1, capi.F16, batch
     c.rope_base, c.rope_scale, c.eps = 10000.0, 1.0, 1e-5
     om = OL.synthetic(_oracle_config(c), seed=7, linear_dt=linear_dt)
