@@ -131,6 +131,9 @@ void set_kquant_tune(int which, int value);
 bool qgemv_kquant_rows_ok(int dt, const QGemvArgs& a);
 bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a);
 hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st);
+// With the rotation and the cache writes of a decoding step as its tail (y receives the rotated queries only).
+bool qgemv_kquant_rows_rope_ok(int dt, const QGemvArgs& a);
+hipError_t qgemv_kquant_rows_rope(int dt, const QGemvArgs& a, const Q4RopeTail& rope, hipStream_t st);
 void set_kquant_rows(int v);
 void set_kquant_rows_waves(int v);
 

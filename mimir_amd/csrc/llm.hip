@@ -463,13 +463,16 @@ static mi355x_status step_any(Model& m) {
             QGemvArgs qa{b.qkv.buf.p, nullptr, m.act[kActKQ].p, qkv, B, b.qkv.n, b.qkv.k, b.qkv.k, 0};
             // From three sequences on, where W can be read once for eight of them, that beats the tail that saves a launch.
             const bool read_once = B >= 3 && qkv_kq && qgemv_kquant_rows_pays(b.qkv.dtype, qa);
-            if (qkv_kq && !read_once && c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0 && qgemv_kquant_rope_ok(b.qkv.dtype, qa)) {
+            const bool pairs = c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0;
+            const bool once_rope = read_once && pairs && qgemv_kquant_rows_rope_ok(b.qkv.dtype, qa);
+            if (once_rope || (qkv_kq && !read_once && pairs && qgemv_kquant_rope_ok(b.qkv.dtype, qa))) {
                 Q4RopeTail tail;  // the rotation and the cache writes ride on the product
                 tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
                 tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
                 tail.cache_dt = c.cache_dtype; tail.H = c.heads; tail.HK = c.kv_heads; tail.dim = c.head_dim; tail.rope_dim = c.rope_dim;
                 tail.cap = c.context;
-                LLM_HIP(qgemv_kquant_act_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
+                if (once_rope) LLM_HIP(qgemv_kquant_rows_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
+                else LLM_HIP(qgemv_kquant_act_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
             } else {
                 if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
                 LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,

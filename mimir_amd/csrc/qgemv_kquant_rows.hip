@@ -24,6 +24,7 @@
 // LDS that is the wavefront's own, so no barrier but the one before the sums.
 #include "device_util.h"
 #include "kernels.h"
+#include "rope_tail.h"
 
 namespace mimir {
 
@@ -190,9 +191,11 @@ template <int LOADS> struct Stage {
 // from wavefront to wavefront through LDS in the super-blocks' order (a barrier a wavefront). LDS holds no terms then, so more
 // workgroups share a compute unit and long rows leave room for eight wavefronts. CHAIN = 0: super-blocks round robin, terms
 // [nsb][kT][64] in LDS, summed by the first wavefront (any K that fits).
-template <int DT, int kWaves, int CHAIN>
+// ROPE: W is q | k | v of a decoding step; the rotation and the cache writes ride on the results (rope_kv's arithmetic, interleaved
+// pairs), y gets the rotated queries only.
+template <int DT, int kWaves, int CHAIN, bool ROPE = false>
 __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_t* __restrict__ W, const uint8_t* act, float* y, const float* resid,
-                                                                     int M_all, int N, int nsb, int64_t act_row_bytes) {
+                                                                     int M_all, int N, int nsb, int64_t act_row_bytes, const Q4RopeTail rope) {
     typedef WBlock<DT> WB;
     constexpr int kT = WB::kTerms, kAll = 32 * WB::kPieces, kLoads = (kAll + 63) / 64, kSlab = 32 * WB::kStride;
     typedef Stage<kLoads> St;
@@ -327,6 +330,18 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
             }
         }
     }
+    if constexpr (ROPE) {
+        // rows (n, n + 1), n even, are a pair of features: the even lane takes its neighbour's result and stores both
+        const int pos = *rope.pos;
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const float v = kT == 2 ? acc[0][jj] - acc[kT - 1][jj] : acc[0][jj];
+            const float other = dpp_f32<0xb1>(v);  // quad_perm [1,0,3,2]
+            const int m = 4 * lh + jj, seq = (int)row0 + m;
+            if ((lane & 1) == 0 && n < N && m < M) q4_rope_store(rope, pos, seq, n, v, other, y + (int64_t)seq * N);
+        }
+        return;
+    }
     if (n < N) {
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
@@ -382,18 +397,18 @@ bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a) {
     return rows_us < (tiles > 128 ? tiles / 128 : 1.0) * nsb * 2.1;
 }
 
-template <int DT, int WAVES, int CHAIN>
-static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st) {
+template <int DT, int WAVES, int CHAIN, bool ROPE = false>
+static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st, const Q4RopeTail* rope = nullptr) {
     const int nsb = (int)(a.K / 256);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, CHAIN>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, CHAIN, ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES, CHAIN>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)),
+    hipLaunchKernelGGL((qgemv_kq_rows_kernel<DT, WAVES, CHAIN, ROPE>), dim3((unsigned)((a.N + 31) / 32), 1, (unsigned)((a.M + kRows - 1) / kRows)),
                        dim3(64 * WAVES), rows_lds(DT, nsb, WAVES, CHAIN > 0), st, (const uint8_t*)a.W, (const uint8_t*)a.act, a.y, a.resid, (int)a.M,
-                       (int)a.N, nsb, (int64_t)kq_act_bytes(a.K));
+                       (int)a.N, nsb, (int64_t)kq_act_bytes(a.K), rope ? *rope : Q4RopeTail{});
     return hipGetLastError();
 }
 
@@ -402,13 +417,40 @@ static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st) {
 // 7.6 7.1 | 10.1 9.3; 28672 x 4096 20.5 27.3 | 33.5 41.8). Rows of more than four super-blocks a wavefront (K above 8192 with eight) keep
 // the terms in registers, in runs of up to eight super-blocks (4096 x 14336: 16.3 | 21.3 us, 19.9 | 21.9 with the terms in LDS, which leave
 // room for four wavefronts only); shorter ones gain nothing from it (the registers cost what the LDS gives), longer ones have no choice.
-hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st) {
+static void rows_shape(int dt, const QGemvArgs& a, int* waves_out, bool* chain_out) {
     const int64_t nsb = a.K / 256, wgs = (a.N + 31) / 32 * ((a.M + kRows - 1) / kRows);
     int waves = wgs <= 256 || nsb > 32 ? 8 : 4;
     if (g_kq_rows_waves == 4 || g_kq_rows_waves == 8) waves = g_kq_rows_waves;
     bool chain = g_kq_rows_chain != 1 && nsb > 4 * waves && nsb <= 64;
     if (chain) waves = 8;
     else if (rows_lds(dt, nsb, waves, false) > 160 * 1024) waves = 4;
+    *waves_out = waves;
+    *chain_out = chain;
+}
+
+// The q | k | v product of a decoding step with the rotation and the cache writes as its tail (see Q4RopeTail; interleaved pairs,
+// even widths): where the rows kernel takes the shape with its terms in LDS (K up to 8192).
+bool qgemv_kquant_rows_rope_ok(int dt, const QGemvArgs& a) {
+    if (!qgemv_kquant_rows_ok(dt, a) || a.resid || a.N % 2) return false;
+    int waves;
+    bool chain;
+    rows_shape(dt, a, &waves, &chain);
+    return !chain;
+}
+
+hipError_t qgemv_kquant_rows_rope(int dt, const QGemvArgs& a, const Q4RopeTail& rope, hipStream_t st) {
+    int waves;
+    bool chain;
+    rows_shape(dt, a, &waves, &chain);
+    if (chain) return hipErrorInvalidValue;
+    if (dt == kQ4_K) return waves == 8 ? launch_kq_rows<kQ4_K, 8, 0, true>(a, st, &rope) : launch_kq_rows<kQ4_K, 4, 0, true>(a, st, &rope);
+    return waves == 8 ? launch_kq_rows<kQ6_K, 8, 0, true>(a, st, &rope) : launch_kq_rows<kQ6_K, 4, 0, true>(a, st, &rope);
+}
+
+hipError_t qgemv_kquant_rows(int dt, const QGemvArgs& a, hipStream_t st) {
+    int waves;
+    bool chain;
+    rows_shape(dt, a, &waves, &chain);
     if (dt == kQ4_K) return chain ? launch_kq_rows<kQ4_K, 8, 8>(a, st) : waves == 8 ? launch_kq_rows<kQ4_K, 8, 0>(a, st) : launch_kq_rows<kQ4_K, 4, 0>(a, st);
     return chain ? launch_kq_rows<kQ6_K, 8, 8>(a, st) : waves == 8 ? launch_kq_rows<kQ6_K, 8, 0>(a, st) : launch_kq_rows<kQ6_K, 4, 0>(a, st);
 }
