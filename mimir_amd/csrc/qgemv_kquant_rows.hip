@@ -19,9 +19,11 @@
 // A workgroup of four or eight wavefronts owns 32 rows of W; its wavefronts take
 // the super-blocks round robin and leave their float32 terms per output (two
 // for Q4_K, one for Q6_K) in LDS; when all are there the first wavefront adds
-// them in the super-blocks' order, which is the CPU's. x of a super-block (2.6 KB
-// for eight rows) and W of it (32 rows, loaded as whole cache lines) pass through
-// LDS that is the wavefront's own, so no barrier but the one before the sums.
+// them in the super-blocks' order, which is the CPU's. (Long rows: contiguous
+// runs of super-blocks, terms in registers, the sums handed from wavefront to
+// wavefront in that order; see the kernel.) x of a super-block (2.6 KB for eight
+// rows) and W of it (32 rows, loaded as whole cache lines) pass through LDS that
+// is the wavefront's own, so no barrier but those around the sums.
 #include "device_util.h"
 #include "kernels.h"
 #include "rope_tail.h"
@@ -413,7 +415,7 @@ static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st, const Q4Rop
 }
 
 // Eight wavefronts where the workgroups are at most one to a compute unit or the rows are long, four where they are many (measured at
-// eight rows of x, us with the conversion of x, Q4_K | Q6_K, four and eight wavefronts: 14336 x 4096 11.1 14.2 | 16.0 19.2; 4096 x 4096
+// eight rows of x already converted, us a call, Q4_K | Q6_K, four and eight wavefronts: 14336 x 4096 11.1 14.2 | 16.0 19.2; 4096 x 4096
 // 7.6 7.1 | 10.1 9.3; 28672 x 4096 20.5 27.3 | 33.5 41.8). Rows of more than four super-blocks a wavefront (K above 8192 with eight) keep
 // the terms in registers, in runs of up to eight super-blocks (4096 x 14336: 16.3 | 21.3 us, 19.9 | 21.9 with the terms in LDS, which leave
 // room for four wavefronts only); shorter ones gain nothing from it (the registers cost what the LDS gives), longer ones have no choice.
