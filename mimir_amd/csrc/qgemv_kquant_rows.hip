@@ -185,8 +185,8 @@ template <> struct WBlock<kQ6_K> {
 template <int LOADS> struct Stage {
     u32x4 w[LOADS];
     u32x4 xq[2];  // two 16-byte pieces of the eight rows' quants
-    u32x4 xs;     // lanes 0..15: a piece of their sums
-    float xd;     // lanes 0..7: a row's scale
+    u32x4 xs;     // a piece of their sums (lanes 0..15 store theirs)
+    float xd;     // a row's scale (lanes 0..7 store theirs)
 };
 
 // CHAIN > 0: a wavefront takes a contiguous run of at most CHAIN super-blocks and keeps its terms in registers; the sums then pass
@@ -233,9 +233,11 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
         const int p = 64 * i + lane, r = p >> 4;
         xsrc[i] = act + (int64_t)(r < M ? r : M - 1) * act_row_bytes + 16 * (p & 15);
     }
-    const int rs = (lane >> 1) < M ? (lane >> 1) : M - 1, rd = lane < M ? lane : M - 1;  // used by lanes below 16 and 8
-    const uint8_t* ssrc = act + (int64_t)(rs & 7) * act_row_bytes + (int64_t)nsb * 256 + 16 * (lane & 1);
-    const uint8_t* dsrc = act + (int64_t)(rd & 7) * act_row_bytes + (int64_t)nsb * 288;
+    // (every lane loads, the upper ones what lower ones load too: with a load under a branch the compiler waits for all loads under
+    // way, the next super-block's with them, before it touches this one's)
+    const int rs = ((lane >> 1) & 7) < M ? ((lane >> 1) & 7) : M - 1, rd = (lane & 7) < M ? (lane & 7) : M - 1;
+    const uint8_t* ssrc = act + (int64_t)rs * act_row_bytes + (int64_t)nsb * 256 + 16 * (lane & 1);
+    const uint8_t* dsrc = act + (int64_t)rd * act_row_bytes + (int64_t)nsb * 288;
 
     auto fetch = [&](St& f, int sb) {
         const uint8_t* wb = wbase + (int64_t)sb * WB::kBytes;
@@ -246,8 +248,8 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) f.xq[i] = *(const u32x4*)(xsrc[i] + (int64_t)sb * 256);
-        if (lane < 16) f.xs = *(const u32x4*)(ssrc + (int64_t)sb * 32);
-        if (lane < 8) f.xd = ((const float*)dsrc)[sb];
+        f.xs = *(const u32x4*)(ssrc + (int64_t)sb * 32);
+        f.xd = ((const float*)dsrc)[sb];
     };
     auto work = [&](const St& f, f32x4* t) {
         // W and x of the super-block into this wavefront's LDS (its own: a wavefront's LDS operations complete in order)
