@@ -66,18 +66,19 @@ __device__ __forceinline__ float group8_max(float v) {
 
 // A row's sum of squares as a workgroup of 256 threads adds it: thread t takes x[t], x[t + 256], ...
 // in that order (the wavefronts' and the workgroup's sums follow at the caller). The loads go out in
-// batches of eight: a loop of unknown length would wait for each before requesting the next.
+// batches of sixteen (a row of 4096 in one): a loop of unknown length would wait for each before requesting the next.
 __device__ __forceinline__ float strided_sum_squares(const float* __restrict__ xr, int d, int t) {
     float ss = 0.f;
-    for (int i0 = t; i0 < d; i0 += 8 * 256) {
-        float v[8];
+    constexpr int kBatch = 16;
+    for (int i0 = t; i0 < d; i0 += kBatch * 256) {
+        float v[kBatch];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < kBatch; u++) {
             const int i = i0 + 256 * u;
             v[u] = i < d ? xr[i] : 0.f;  // + 0 changes no sum
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < kBatch; u++) {
             float sq = v[u] * v[u];
             ss = ss + sq;
         }
