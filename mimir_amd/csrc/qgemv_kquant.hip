@@ -386,8 +386,9 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q4k_kernel(const uint8_t* __
                 lo1 = __builtin_amdgcn_sdot4((int)(w1 & 0x0F0F0F0Fu), (int)xc[i], lo1, false);
                 hi1 = __builtin_amdgcn_sdot4((int)((w1 >> 4) & 0x0F0F0F0Fu), (int)xe[i], hi1, false);
             }
-            int sumi = sc_a * lo0 + sc_b * hi0 + sc_c * lo1 + sc_e * hi1;
-            int summ = m_a * sa + m_b * sb_ + m_c * sc_ + m_e * se;
+            // 24-bit multiplies (full rate; a 32-bit one takes four times as long): scales and mins below 64, sums within 16 * 15 * 127
+            int sumi = __mul24(sc_a, lo0) + __mul24(sc_b, hi0) + __mul24(sc_c, lo1) + __mul24(sc_e, hi1);
+            int summ = __mul24(m_a, sa) + __mul24(m_b, sb_) + __mul24(m_c, sc_) + __mul24(m_e, se);
             sumi = dpp_i32_quad_sum(live ? sumi : 0);
             summ = dpp_i32_quad_sum(live ? summ : 0);
             float t = 0.f, u = 0.f;
@@ -517,7 +518,7 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
             const uint32_t pair = n ? cur[r].sc.take(2, mis[r]) : cur[r].sc.take(0, mis[r]);
             const uint32_t pair4 = n ? cur[r].sc.take(3, mis[r]) : cur[r].sc.take(1, mis[r]);
             const int sc_l = (int)(int8_t)(pair >> (8 * c)), sc_h = (int)(int8_t)(pair4 >> (8 * c));
-            int sumi = sc_l * (dl - 32 * sl) + sc_h * (dh - 32 * sh_);
+            int sumi = __mul24(sc_l, dl - 32 * sl) + __mul24(sc_h, dh - 32 * sh_);  // int8 scales, |dl - 32 sl| below 2^18: 24-bit multiplies
             sumi = dpp_i32_group8_sum(live ? sumi : 0);
             float t = 0.f;
             if (part == 0 && live) {
