@@ -298,6 +298,18 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
         void* act;
         if (mi355x_status s2 = act_scratch(mimir::kq_act_bytes(K) * (size_t)M, &act)) return s2;
         mimir::QGemvArgs a{W, nullptr, act, (float*)Y, M, N, K, 0, 0};
+        if (mimir::qgemv_kquant_rows_pays(dtype, a)) {  // a few rows: W read once per eight of them, the same bits, one rounding after
+            float* yf = (float*)Y;
+            if (!f32) {
+                if (mi355x_status s2 = gemm_scratch(((size_t)M * N * 4 + 255) & ~(size_t)255, &ws)) return s2;
+                yf = (float*)ws;
+            }
+            a.y = yf;
+            HIP_TRY(mimir::kq_convert_act_bf16(X, M, K, x_row_stride, act, st), "launch kq_convert_act");
+            HIP_TRY(mimir::qgemv_kquant_rows(dtype, a, st), "launch qgemv_kquant_rows");
+            if (!f32) HIP_TRY(mimir::f32_to_bf16(yf, Y, M * N, st), "launch cast");
+            return MI355X_OK;
+        }
         if (mimir::qgemm_kquant_ok(dtype, a) && mimir::qgemm_kquant_pays(dtype, a)) {
             HIP_TRY(mimir::kq_convert_act_bf16(X, M, K, x_row_stride, act, st), "launch kq_convert_act");
             HIP_TRY(mimir::qgemm_kquant(dtype, a, st, !f32), "launch qgemm_kquant");

@@ -117,12 +117,14 @@ def test_few_rows_on_the_matrix_cores_and_many_on_the_row_kernels(dt):
 
 
 @pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
-def test_prompt_sized_products_take_the_matrix_cores_and_bf16_rounds_once(dt):
+@pytest.mark.parametrize("m", [512, 11])
+def test_prompt_sized_products_take_the_matrix_cores_and_bf16_rounds_once(dt, m):
     """Left to itself the library sends a prompt-sized product to the matrix cores (the CPU's bits), and
     mi355x_qgemm_bf16 is the reference's sequence for a half x: cast to float32, product, one rounding
-    (tensor/quant.go:45-48)."""
+    (tensor/quant.go:45-48). Eleven rows take the kernel that reads W once per eight rows of x, from
+    bfloat16 rows too."""
     import torch
-    m, n, k = 512, 1024, 2048
+    n, k = 1024, 2048
     rng = np.random.default_rng(31 + dt)
     raw = random_blocks(rng, dt, n * k)
     xb = O.f32_to_bf16(rng.normal(size=(m, k)).astype(np.float32))

@@ -565,6 +565,42 @@ def test_kquant_rows_of_x_share_one_pass_over_w_on_the_matrix_cores(dt, m, n, k)
     assert bits_equal(got, want) and bits_equal(got_act, want) and bits_equal(rows, want)
 
 
+@pytest.mark.parametrize("dt", [O.Q4_K, O.Q6_K])
+def test_kquant_rows_kernel_at_the_largest_integer_sums(dt):
+    """Every quant and scale at its largest magnitude with x at +-127 per super-block (backend/cpu/quant_test.go:164-204), through the
+    kernel that reads W once per eight rows of x: its 24-bit multiplies and int32 sums hold what the CPU's int32 arithmetic holds."""
+    l = gpu.lib()
+    m, n, k = 11, 64, 256 * 40
+    bb = O.block_bytes(dt)
+    raw = np.zeros(n * k // 256 * bb, np.uint8).reshape(-1, bb)
+    if dt == O.Q4_K:
+        raw[:, 4:16] = 0xFF          # every scale and min 63
+        raw[:, 16:144] = 0xFF        # every quant 15
+        raw[:, 0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+        raw[:, 2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+        raw[1::2, 16:144] = 0        # and every quant 0
+    else:
+        raw[:, 0:192] = 0xFF         # every quant 63 (31 after the offset)
+        raw[1::2, 0:192] = 0         # every quant 0 (-32)
+        raw[:, 192:208] = 0x80       # every scale -128
+        raw[2::3, 192:208] = 0x7F    # or 127
+        raw[:, 208:210] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    raw = raw.reshape(-1)
+    x = np.where(np.arange(m * k).reshape(m, k) % 3 == 0, -127.0, 127.0).astype(np.float32)
+    x[1::2] = 127.0
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(dt, raw, x, n, k)
+    try:
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows", 2))
+        for key, v in ((b"kquant.mfma_rows_waves", 0), (b"kquant.mfma_rows_waves", 1)):  # partial sums in registers (K = 10240), then in LDS
+            capi.check(l.mi355x_tune(key, v))
+            gpu.say(f"kquant rows kernel extremes dt={dt} {key.decode()}={v}")
+            assert bits_equal(gpu.qgemv(dt, ptr, gpu.dev(x), n, k), want)
+    finally:
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows", 0))
+        capi.check(l.mi355x_tune(b"kquant.mfma_rows_waves", 0))
+
+
 def test_kquant_gemv_golden_and_exact_rows(golden_dir):
     cases = golden_cases(os.path.join(golden_dir, "quant.mim"))
     for kind, dt in (("q4_K", O.Q4_K), ("q6_K", O.Q6_K)):
