@@ -148,6 +148,9 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
             for (int f = 0; f < FPL; f++) qr[g][f] = 0.f;
         }
     }
+    // rows of a head's keys and values lie within 2^31 elements and fewer than 2^23 apart (checked by the host): 24-bit multiplies
+    // and 32-bit offsets in place of 64-bit address arithmetic per row
+    const int kp = (int)p.k_p, vp = (int)p.v_p;
     const KV* kbase = k + b * p.k_b + (int64_t)hk * p.k_h + part * FPL;
     const KV* vbase = v + b * p.v_b + (int64_t)hk * p.v_h + part * FPL;
 
@@ -159,19 +162,19 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int jj = kKeyGroups * u + kg;
-        load_raw<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kraw[u]);
+        load_raw<KV, FPL>(kbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), kp), kraw[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; u++) {
         const int jj = kKeyGroups * u + kg;
-        load_raw<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vraw[u]);
+        load_raw<KV, FPL>(vbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), vp), vraw[u]);
     }
     for (int jj0 = 0; jj0 < nj; jj0 += U * kKeyGroups) {
         if (jj0 > 0) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int jj = jj0 + kKeyGroups * u + kg;
-                load_raw<KV, FPL>(kbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.k_p, kraw[u]);
+                load_raw<KV, FPL>(kbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), kp), kraw[u]);
             }
         }
 #pragma unroll
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int jj = jj0 + kKeyGroups * u + kg;
-                load_raw<KV, FPL>(vbase + (int64_t)(j0 + (jj < nj ? jj : 0)) * p.v_p, vraw[u]);
+                load_raw<KV, FPL>(vbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), vp), vraw[u]);
             }
         }
 #pragma unroll
@@ -403,6 +406,9 @@ bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
     int ns, cm;
     attention_decode_plan(a.B, a.H, a.HK, kmax, &ns, &cm);
     size_t lds = (size_t)(kHeads * cm + kKeyGroups * kHeads * a.D) * sizeof(float);
+    if (a.k_strides[2] <= 0 || a.v_strides[2] <= 0 || a.k_strides[2] >= (1 << 23) || a.v_strides[2] >= (1 << 23) || kmax >= (1 << 23) ||
+        kmax * a.k_strides[2] >= ((int64_t)1 << 31) || kmax * a.v_strides[2] >= ((int64_t)1 << 31))
+        return false;
     return lds <= 60 * 1024 && kmax <= INT32_MAX / 2;
 }
 
