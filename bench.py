@@ -350,8 +350,10 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
     out = {}
     rng = np.random.default_rng(0)
     st = torch.cuda.Stream()
-    kinds = (("q4_0", capi.Q4_0, 2500.0, "frac_of_bf16_peak"), ("q4_K", capi.Q4_K, 5000.0, "frac_of_int8_peak"),
-             ("q6_K", capi.Q6_K, 5000.0, "frac_of_int8_peak"))
+    # "q4_0_binary16_weights": the same call with "qgemm.f16" = 1 (every weight rounded once to binary16, one
+    # multiplication a weight; results within 1e-3, not exact)
+    kinds = (("q4_0", capi.Q4_0, 2500.0, "frac_of_bf16_peak"), ("q4_0_binary16_weights", capi.Q4_0, 2500.0, "frac_of_f16_peak"),
+             ("q4_K", capi.Q4_K, 5000.0, "frac_of_int8_peak"), ("q6_K", capi.Q6_K, 5000.0, "frac_of_int8_peak"))
     # float32 activations by Q4_0 (what the decoder's prompt pass multiplies): mi355x_qgemv, whose 24-bit
     # fixed-point x takes three int8 multiplications a weight
     res = {}
@@ -378,6 +380,7 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
     out["q4_0_f32_x"] = res
     for name, dt, peak, frac_key in kinds:
         res = {}
+        capi.check(lib.mi355x_tune(b"qgemm.f16", 1 if name == "q4_0_binary16_weights" else 0))
         for m, n in shapes:
             if dt == capi.Q4_0:
                 raw = bench_blocks_q4_0(rng, n * k)
@@ -403,6 +406,7 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
             res[f"M{m}_N{n}_K{k}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1), frac_key: round(tf / peak, 4)}
             del w, x, y
         out[name] = res
+    capi.check(lib.mi355x_tune(b"qgemm.f16", 0))
     return out
 
 

@@ -308,6 +308,11 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * rows from two on; "kquant.mfma_rows_waves" = 4 or 8 fixes its wavefronts a
  * workgroup, 1 keeps its partial sums in LDS whatever K is (0: both by shape).
  * "qgemm.path" = 1 makes mi355x_qgemm_bf16 take its general route for every shape.
+ * "qgemm.f16" = 1 makes mi355x_qgemm_bf16's Q4_0 matrix-core kernel round every
+ * weight once to binary16 instead of multiplying it exactly (each weight within
+ * 2^-11 of itself; at K = 4096 the results are off by about 2e-4 of their root mean
+ * square, 1e-3 of it at worst; block scales beyond 8188 in magnitude overflow): half the matrix instructions,
+ * about 1.5 times the speed. Off by default.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).
  * "llama.step" chooses how mi355x_llama_generate runs its decoding steps: 0 the

@@ -73,6 +73,7 @@ int g_fx_min_rows = 16;
 int g_rows_max = 0;    // "q4_0.rows_max" n: Q4_0 products of fewer than n rows of x take the kernel that reads W once per eight rows (0: by cost)
 int g_rows_path = 0;  // "q4_0.rows_path" 1: no matrix-core kernel for two to fifteen rows of x
 int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
+int g_tune_gemm_f16 = 0;  // 1: the Q4_0 matrix-core product with weights rounded to binary16
 int g_tune_attn = 0;  // 1: the general kernels also for one query position
 }
 thread_local std::vector<hipEvent_t> t_events;
@@ -290,7 +291,10 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     }
     void* ws;
     if (dtype == MI355X_Q4_0 && g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
-        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, st), "launch qgemm_q4_0");
+        void* half_ws = nullptr;
+        if (g_tune_gemm_f16 == 1)
+            if (mi355x_status s2 = gemm_scratch(mimir::qgemm_q4_0_half_ws_bytes(M, K), &half_ws)) return s2;
+        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, half_ws, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
     if ((dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) && g_tune_gemm != 1 && ((uintptr_t)X & 7) == 0 && x_row_stride % 4 == 0) {
@@ -670,6 +674,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "qgemm.path") == 0) {
         g_tune_gemm = value;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "qgemm.f16") == 0) {
+        g_tune_gemm_f16 = value == 1 ? 1 : 0;
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.fx_rows") == 0) {

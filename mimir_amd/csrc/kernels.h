@@ -253,10 +253,13 @@ double qgemm_q4_0_fx_cost_us(int64_t M, int64_t N, int64_t K);           // abou
 hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
 // Prompt-sized Q4_0 product on the matrix cores (qgemm_q4_0.hip): X [M, K]
-// bfloat16, Y [M, N] bfloat16 or float32.
+// bfloat16, Y [M, N] bfloat16 or float32. Exact up to the order of the float32 sums when half_ws is null; with
+// half_ws (qgemm_q4_0_half_ws_bytes(M, K) bytes of device memory, 256-byte aligned) the weights are rounded to
+// binary16 (2^-11 of each) and X goes through half_ws as row-scaled binary16.
 bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K, int64_t x_row_stride);
+size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t K);
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
-                           hipStream_t st);
+                           void* half_ws, hipStream_t st);
 hipError_t bf16_rows_to_f32(const void* x, float* y, int64_t M, int64_t K, int64_t x_row_stride, hipStream_t st);
 hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 

@@ -33,6 +33,19 @@
 // (lane % 32), the lane's half (lane / 32) choosing which eight of the sixteen;
 // its result holds column (lane % 32) and rows 8 (i / 4) + 4 (lane / 32) + i % 4
 // in register i.
+//
+// A second, approximate form (template argument HALF, chosen by the caller; never
+// by default) rounds each weight once to binary16 and multiplies with
+// v_mfma_f32_32x32x16_f16: one plane instead of two, and a nibble becomes a weight
+// in three packed instructions per pair. A weight is then off by at most 2^-11 of
+// itself (the results by about 2e-4 of their root mean square at K = 4096 and by
+// 1e-3 of it at worst: at the edge of the 1e-3 asked of this product, which is why
+// it is not the default); |d| above 8188 overflows. X is brought to binary16
+// beforehand by a pass of its own that scales each row by a power of two, so that
+// its largest element lands in [2^14, 2^15): bfloat16's 8 significant bits fit
+// binary16's 11, so the conversion is exact for every element within 2^28 of the
+// row's largest, whatever the row's range, and the results are scaled back
+// (exactly) when they are written.
 #include "device_util.h"
 #include "kernels.h"
 
@@ -42,6 +55,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -49,7 +64,7 @@ constexpr int kBN = 128;        // columns of Y (rows of W) per workgroup
 constexpr int kKS = 64;         // K per step: two Q4_0 blocks
 constexpr int kLd = kKS + 8;    // bfloat16 elements per LDS row
 
-constexpr size_t stage_bytes(int BM) { return (size_t)(BM + 2 * kBN) * kLd * 2; }  // X, hi, lo
+constexpr size_t stage_bytes(int BM, bool half = false) { return (size_t)(BM + (half ? 1 : 2) * kBN) * kLd * 2; }  // X, hi, lo (binary16: X, w)
 
 // The barrier of the main loop. __syncthreads() also waits for every global load
 // in flight (its fence covers all memory), which would stall each step for a
@@ -66,11 +81,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return u;
 }
 
-template <int MT, bool OUT_F32>  // MT 32-row tiles per multiplying wavefront: the workgroup's tile is (64 MT) x 128
+// MT 32-row tiles per multiplying wavefront: the workgroup's tile is (64 MT) x 128. HALF: X is binary16 (rows
+// scaled, row m's results to be multiplied by row_scale[m]) and the weights are rounded to binary16.
+template <int MT, bool OUT_F32, bool HALF>
 __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W,
                                                             void* __restrict__ Yv, int M, int N, int K, int64_t x_row_stride,
-                                                            int tiles_m, int ntiles) {
+                                                            int tiles_m, int ntiles, const float* __restrict__ row_scale) {
     constexpr int BM = 64 * MT;
+    constexpr size_t kStage = stage_bytes(BM, HALF);
     constexpr int AV = BM * 8 / 256;      // 16-byte pieces of the X tile per thread (4 or 2): piece p is row p / 8, bytes 16 (p % 8)..
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -113,9 +131,9 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
     // buffers): nine lanes share a row's 144 bytes, so a wavefront load touches
     // about ten cache lines instead of 64, and each feeder then picks its block
     // out of LDS. With 256-row tiles every feeder loads its own 18 bytes.
-    constexpr bool PANEL = MT <= 2;
+    constexpr bool PANEL = MT <= 2 || HALF;  // one plane of weights leaves room for the panel beside 256-row tiles too
     constexpr int kPanelBytes = kBN * 144, kPanelPieces = kBN * 9;
-    uint8_t* raw = smem + 2 * stage_bytes(BM);
+    uint8_t* raw = smem + 2 * kStage;
     struct Fetched {  // what one step needs from memory
         u32x4 ra[AV], rq;
         uint16_t rd;
@@ -152,7 +170,7 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         }
     };
     auto stage = [&](int buf, const Fetched& f, int step) {
-        uint16_t* As = (uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
+        uint16_t* As = (uint16_t*)(smem + (size_t)buf * kStage);
         uint16_t* Bh = As + BM * kLd;
         uint16_t* Bl = Bh + kBN * kLd;
         const u32x4* ra = f.ra;
@@ -171,6 +189,29 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         // times d is the weight, exactly; its upper 16 bits are a bfloat16 (hi,
         // truncated, not rounded: w - hi then has at most 7 significant bits and
         // its upper 16 bits are lo, exactly).
+        if (HALF) {
+            // the nibble into the mantissa of binary16's 1024 (v_perm, two at a time), minus 1032 is n - 8, times d
+            // rounds once: the weight to the nearest binary16
+            const _Float16 dh = __builtin_bit_cast(_Float16, rd);
+            const f16x2 d2 = {dh, dh}, off = {(_Float16)1032.f, (_Float16)1032.f};
+            u32x4 wq[4];
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t nib = (rq[i] >> (4 * half)) & 0x0f0f0f0fu;
+                    const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
+                    const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
+                    const f16x2 w0 = (__builtin_bit_cast(f16x2, p0) - off) * d2;
+                    const f16x2 w1 = (__builtin_bit_cast(f16x2, p1) - off) * d2;
+                    wq[2 * half + (i >> 1)][2 * (i & 1)] = __builtin_bit_cast(uint32_t, w0);
+                    wq[2 * half + (i >> 1)][2 * (i & 1) + 1] = __builtin_bit_cast(uint32_t, w1);
+                }
+            uint16_t* hrow = Bh + w_col * kLd + w_blk * 32;
+#pragma unroll
+            for (int v = 0; v < 4; v++) *(u32x4*)(hrow + 8 * v) = wq[v];
+            return;
+        }
         const float d = f16_bits_to_f32(rd);
         u32x4 hi[4], lo[4];  // elements 0..7, 8..15 (low nibbles), 16..23, 24..31 (high nibbles)
 #pragma unroll
@@ -212,14 +253,16 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
     // LDS while the MFMAs of slice i run (two sets of fragment registers), so
     // that only the first slice's reads are waited for.
     auto compute = [&](int buf) {
-        const uint16_t* As = (const uint16_t*)(smem + (size_t)buf * stage_bytes(BM));
+        const uint16_t* As = (const uint16_t*)(smem + (size_t)buf * kStage);
         const uint16_t* Bh = As + BM * kLd;
         const uint16_t* Bl = Bh + kBN * kLd;
         bf16x8 a[2][MT], bh[2][2], bl[2][2];
         auto read_slice = [&](int set, int sl) {  // slice sl: block sl / 2, half sl % 2
             const int koff = (sl >> 1) * 32 + (sl & 1) * 16 + lh * 8;
+            if (!HALF) {
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++) bl[set][nt] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + koff);
+                for (int nt = 0; nt < 2; nt++) bl[set][nt] = *(const bf16x8*)(Bl + (wn * 64 + nt * 32 + l32) * kLd + koff);
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) a[set][mt] = *(const bf16x8*)(As + (wm * (32 * MT) + mt * 32 + l32) * kLd + koff);
 #pragma unroll
@@ -229,6 +272,17 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
 #pragma unroll
         for (int sl = 0; sl < 4; sl++) {
             if (sl < 3) read_slice((sl + 1) & 1, sl + 1);
+            if (HALF) {
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < 2; nt++) {
+                        const bf16x8 av = a[sl & 1][mt], bv = bh[sl & 1][nt];
+                        total[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, av), __builtin_bit_cast(f16x8, bv),
+                                                                               total[mt][nt], 0, 0, 0);
+                    }
+                continue;
+            }
             // the tiles in turn for each operand pair, so that consecutive MFMAs are independent
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
@@ -243,13 +297,14 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         }
         // the order asked of the scheduler: slice 0's reads, then slice by slice the
         // next slice's reads ahead of this slice's MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x100, MT + 4, 0);
+        constexpr int kReads = MT + (HALF ? 2 : 4), kMfmas = (HALF ? 2 : 4) * MT;
+        __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
 #pragma unroll
         for (int sl = 0; sl < 3; sl++) {
-            __builtin_amdgcn_sched_group_barrier(0x100, MT + 4, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 4 * MT, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfmas, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 4 * MT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmas, 0);
     };
 
     // Buffer kb & 1 holds step kb. Within step kb the feeders fill the other
@@ -312,8 +367,10 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
             for (int i = 0; i < 16; i++) {
                 const int m = m0 + wm * (32 * MT) + mt * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
                 if (m < M && n < N) {
-                    if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n] = total[mt][nt][i];
-                    else ((uint16_t*)Yv)[(int64_t)m * N + n] = f32_to_bf16_bits(total[mt][nt][i]);
+                    float v = total[mt][nt][i];
+                    if (HALF) v *= row_scale[m];
+                    if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n] = v;
+                    else ((uint16_t*)Yv)[(int64_t)m * N + n] = f32_to_bf16_bits(v);
                 }
             }
         }
@@ -323,6 +380,57 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f32_kernel(const uint16_t* _
                                                                int64_t x_row_stride) {
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < M * K; t += (int64_t)gridDim.x * 256)
         y[t] = bf16_bits_to_f32(x[(t / K) * x_row_stride + t % K]);
+}
+
+// A row of bfloat16 to binary16, scaled by the power of two that brings the row's largest finite magnitude into
+// [2^14, 2^15) (clamped to what float32 can hold both ways); scale_back[m] undoes it. One workgroup a row; K in
+// pieces of eight elements.
+__global__ __launch_bounds__(256) void bf16_rows_to_f16_scaled_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                      float* __restrict__ scale_back, int64_t K, int64_t x_row_stride) {
+    __shared__ uint32_t part[4];
+    const int64_t m = blockIdx.x;
+    const uint16_t* row = x + m * x_row_stride;
+    const int pieces = (int)(K >> 3);
+    uint32_t top = 0;  // the largest finite magnitude's bits (bfloat16 magnitudes order as integers)
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        u32x4 v;
+        __builtin_memcpy(&v, __builtin_assume_aligned(row + 8 * (int64_t)p, 16), 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t a = v[i] & 0x7fffu, b = (v[i] >> 16) & 0x7fffu;
+            if (a < 0x7f80u && a > top) top = a;
+            if (b < 0x7f80u && b > top) top = b;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)top, o, 64);
+        top = other > top ? other : top;
+    }
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = top;
+    __syncthreads();
+    top = part[0];
+#pragma unroll
+    for (int i = 1; i < 4; i++) top = part[i] > top ? part[i] : top;
+    int e = 0;
+    if (top != 0) {
+        const int ex = (int)(top >> 7) - 127;  // floor(log2) of a normal magnitude; subnormals count as 2^-117
+        e = 14 - ex;
+        e = e > 126 ? 126 : e < -126 ? -126 : e;
+    }
+    const float up = __uint_as_float((uint32_t)(e + 127) << 23);
+    if (threadIdx.x == 0) scale_back[m] = __uint_as_float((uint32_t)(127 - e) << 23);
+    uint16_t* out = y + m * K;
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        u32x4 v, r;
+        __builtin_memcpy(&v, __builtin_assume_aligned(row + 8 * (int64_t)p, 16), 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const f16x2 h = {(_Float16)(__uint_as_float(v[i] << 16) * up), (_Float16)(__uint_as_float(v[i] & 0xffff0000u) * up)};
+            r[i] = __builtin_bit_cast(uint32_t, h);
+        }
+        *(u32x4*)(out + 8 * (int64_t)p) = r;
+    }
 }
 
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n) {
@@ -353,8 +461,22 @@ bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K
 
 // X [M, K] bfloat16 (rows x_row_stride elements apart), W [N, K] Q4_0 with
 // finite scales, Y [M, N] bfloat16, or float32 if out_f32.
+// With half_ws (qgemm_q4_0_half_ws_bytes(M, K) bytes, 16-byte aligned) the product takes its approximate form:
+// X converted into half_ws first, weights rounded to binary16.
+size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t K) { return (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * 4; }
+
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
-                           hipStream_t st) {
+                           void* half_ws, hipStream_t st) {
+    const bool half = half_ws != nullptr;
+    const float* row_scale = nullptr;
+    if (half) {
+        float* sb = (float*)((uint8_t*)half_ws + (((size_t)M * K * 2 + 255) & ~(size_t)255));
+        hipLaunchKernelGGL(bf16_rows_to_f16_scaled_kernel, dim3((unsigned)M), dim3(256), 0, st, (const uint16_t*)X, (uint16_t*)half_ws, sb, K,
+                           x_row_stride);
+        X = half_ws;
+        x_row_stride = K;
+        row_scale = sb;
+    }
     // the tallest tiles that still give every compute unit work: a taller tile
     // reads less from LDS per MFMA (a wavefront multiplies 32 MT x 64 of it)
     const int64_t tiles_n = (N + kBN - 1) / kBN;
@@ -363,23 +485,30 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
     const int tiles_m = (int)((M + BM - 1) / BM);
     const int ntiles = (int)(tiles_m * tiles_n);
     dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
-    const size_t lds = 2 * stage_bytes(BM) + (MT <= 2 ? 2 * kBN * 144 : 0);
+    const size_t lds = 2 * stage_bytes(BM, half) + (MT <= 2 || half ? 2 * kBN * 144 : 0);
     {  // more dynamic LDS than a kernel gets by default
         static bool raised = false;
         if (!raised) {
             const int most = 160 * 1024;
             hipError_t e = hipSuccess;
-#define QGEMM_RAISE(MT_, F32_) \
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_kernel<MT_, F32_>, hipFuncAttributeMaxDynamicSharedMemorySize, most)
+#define QGEMM_RAISE(MT_, F32_)                                                                                                                  \
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_kernel<MT_, F32_, false>, hipFuncAttributeMaxDynamicSharedMemorySize, most); \
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_kernel<MT_, F32_, true>, hipFuncAttributeMaxDynamicSharedMemorySize, most)
             QGEMM_RAISE(1, true); QGEMM_RAISE(1, false); QGEMM_RAISE(2, true); QGEMM_RAISE(2, false); QGEMM_RAISE(4, true); QGEMM_RAISE(4, false);
 #undef QGEMM_RAISE
             if (e != hipSuccess) return e;
             raised = true;
         }
     }
-#define QGEMM_LAUNCH(MT_, F32_)                                                                                                     \
-    hipLaunchKernelGGL((qgemm_q4_0_kernel<MT_, F32_>), grid, dim3(512), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y, (int)M, \
-                       (int)N, (int)K, x_row_stride, tiles_m, ntiles)
+#define QGEMM_LAUNCH(MT_, F32_)                                                                                                              \
+    do {                                                                                                                                     \
+        if (half)                                                                                                                            \
+            hipLaunchKernelGGL((qgemm_q4_0_kernel<MT_, F32_, true>), grid, dim3(512), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y,     \
+                               (int)M, (int)N, (int)K, x_row_stride, tiles_m, ntiles, row_scale);                                            \
+        else                                                                                                                                 \
+            hipLaunchKernelGGL((qgemm_q4_0_kernel<MT_, F32_, false>), grid, dim3(512), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y,    \
+                               (int)M, (int)N, (int)K, x_row_stride, tiles_m, ntiles, row_scale);                                            \
+    } while (0)
     if (MT == 4) {
         if (out_f32) QGEMM_LAUNCH(4, true); else QGEMM_LAUNCH(4, false);
     } else if (MT == 2) {
