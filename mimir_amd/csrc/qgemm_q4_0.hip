@@ -477,10 +477,11 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
         x_row_stride = K;
         row_scale = sb;
     }
-    // the tallest tiles that still give every compute unit work: a taller tile
-    // reads less from LDS per MFMA (a wavefront multiplies 32 MT x 64 of it)
+    // the tallest tiles that still give three quarters of the compute units work: a taller tile reads less from
+    // LDS per MFMA (a wavefront multiplies 32 MT x 64 of it), which is worth more than the idle quarter (measured at
+    // 512 x 14336 and 2048 x 4096: 224 and 256 tiles of 256 rows beat 448 and 512 tiles of 128 rows by a fifth)
     const int64_t tiles_n = (N + kBN - 1) / kBN;
-    const int MT = ((M + 255) / 256) * tiles_n >= 384 ? 4 : ((M + 127) / 128) * tiles_n >= 384 ? 2 : 1;
+    const int MT = ((M + 255) / 256) * tiles_n >= 192 ? 4 : ((M + 127) / 128) * tiles_n >= 192 ? 2 : 1;
     const int BM = 64 * MT;
     const int tiles_m = (int)((M + BM - 1) / BM);
     const int ntiles = (int)(tiles_m * tiles_n);

@@ -75,7 +75,8 @@ def check_bf16(got, want_bits, bound):
     assert differ.mean() <= 0.01, float(differ.mean())
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (32, 128, 512), (70, 200, 768), (1, 130, 4096), (200, 384, 1024), (129, 257, 1280), (33, 65, 96), (40, 130, 192)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (32, 128, 512), (70, 200, 768), (1, 130, 4096), (200, 384, 1024), (129, 257, 1280), (33, 65, 96), (40, 130, 192),
+                                   (250, 12790, 512)])  # the last: 128-row tiles
 def test_small_and_ragged_shapes(m, n, k):
     rng = np.random.default_rng(m * 7 + n)
     w = random_blocks(rng, O.Q4_0, n * k)
@@ -247,7 +248,8 @@ def check_binary16_form(w, x, n, k, got32):
     check_f32(got32, want, bound + slack, "against the reference")
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (70, 200, 768), (1, 130, 4096), (200, 384, 1024), (129, 257, 1280), (300, 3200, 512)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (70, 200, 768), (1, 130, 4096), (200, 384, 1024), (129, 257, 1280), (300, 3200, 512),
+                                   (250, 12790, 512)])  # the last: 128-row tiles
 def test_binary16_form_small_and_ragged_shapes(m, n, k):
     rng = np.random.default_rng(m * 11 + n)
     w = scales_within_binary16(rng, n * k)
