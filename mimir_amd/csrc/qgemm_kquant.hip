@@ -392,7 +392,7 @@ hipError_t launch(const QGemvArgs& a, int nsb, hipStream_t st) {
     // What the registers allow: 256 a lane at two wavefronts a SIMD.
     constexpr int DEPTH = MT == 1 ? 2 : 1;
     typedef Layout<128 * MT> L;
-    static bool raised = false;
+    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)qgemm_kquant_kernel<DT, MT, DEPTH, OUT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, L::total);
         if (e != hipSuccess) return e;

@@ -488,7 +488,7 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
     dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
     const size_t lds = 2 * stage_bytes(BM, half) + (MT <= 2 || half ? 2 * kBN * 144 : 0);
     {  // more dynamic LDS than a kernel gets by default
-        static bool raised = false;
+        static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
         if (!raised) {
             const int most = 160 * 1024;
             hipError_t e = hipSuccess;

@@ -303,7 +303,7 @@ bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K) {
 
 // act: q4_0_fx_convert_act's rows. y = x . W^T (+ resid, which may be y itself).
 hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, hipStream_t st) {
-    static bool raised = false;
+    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)qgemm_q4_0_fx_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Layout::total);
         if (e != hipSuccess) return e;

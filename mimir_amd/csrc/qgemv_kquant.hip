@@ -554,7 +554,7 @@ void set_kquant_tune(int which, int value) {
 
 template <int R>
 static hipError_t launch_kq(int dt, const QGemvArgs& a, int nsb, const Q4RopeTail* rope, hipStream_t st) {
-    static bool raised[2] = {false, false};
+    static std::atomic<bool> raised[2];  // zero at start; threads may race here: both then set the same attribute
     const size_t lds = kq_lds_bytes(nsb);
     const int rows_per_wg = kKqThreads / 64 * R;
     dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.M);

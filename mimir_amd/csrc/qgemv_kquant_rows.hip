@@ -404,7 +404,7 @@ bool qgemv_kquant_rows_pays(int dt, const QGemvArgs& a) {
 template <int DT, int WAVES, int CHAIN, bool ROPE = false>
 static hipError_t launch_kq_rows(const QGemvArgs& a, hipStream_t st, const Q4RopeTail* rope = nullptr) {
     const int nsb = (int)(a.K / 256);
-    static bool raised = false;
+    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)qgemv_kq_rows_kernel<DT, WAVES, CHAIN, ROPE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;

@@ -716,7 +716,7 @@ static int q4_batch_rows(int64_t M, int64_t K) {
 
 template <int R, int MODE, int MB>
 static hipError_t launch_q4_0_i4_batch(const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st) {
-    static bool raised = false;
+    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
     const size_t act_bytes = q4_0_act_bytes(K), lds_bytes = MB * act_bytes + MB * 128;
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)qgemv_q4_0_i4_batch_kernel<R, MODE, MB>, hipFuncAttributeMaxDynamicSharedMemorySize,
