@@ -311,8 +311,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * "qgemm.f16" = 1 makes mi355x_qgemm_bf16's Q4_0 matrix-core kernel round every
  * weight once to binary16 instead of multiplying it exactly (each weight within
  * 2^-11 of itself; at K = 4096 the results are off by about 2e-4 of their root mean
- * square, 1e-3 of it at worst; block scales beyond 8188 in magnitude overflow): half the matrix instructions,
- * about 1.5 times the speed. Off by default.
+ * square, 1e-3 of it at worst; block scales beyond 8188 in magnitude overflow):
+ * half the matrix instructions, 1.3 to 1.4 times the speed. Off by default; the
+ * setting is process-wide.
  * "attention.path" = 1 makes mi355x_attention use its general kernels also for
  * one query position (which otherwise takes a single-launch kernel).
  * "llama.step" chooses how mi355x_llama_generate runs its decoding steps: 0 the
