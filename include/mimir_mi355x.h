@@ -16,6 +16,14 @@
  *    default stream. Launches return once queued, like Backend.Run
  *    (backend/backend.go:152-168); mi355x_sync waits and reports device-side
  *    errors, like Backend.Sync (backend/rocm/rocm_linux.go:349-375).
+ *  - Entry points that need memory beyond their arguments (mi355x_qgemv,
+ *    mi355x_qgemm_bf16, mi355x_attention, mi355x_argmax) keep it per device and
+ *    stream: calls on different streams share nothing, calls on one stream are
+ *    ordered by it. Such a block grows on demand with hipMalloc, which HIP
+ *    refuses while the stream is being captured: run a call once at its
+ *    largest size before recording it into a graph (the block a graph was
+ *    recorded with is never freed, so the graph stays valid however the
+ *    scratch grows afterwards).
  *  - dtype codes are the reference's DType enumeration
  *    (backend/backend.go:72-90) with Q4_0 appended.
  *  - Block-quantized buffers hold ggml's block layout unchanged
@@ -173,14 +181,20 @@ MI355X_API mi355x_status mi355x_rope(const float* x, float* y, int64_t rows, int
 MI355X_API mi355x_status mi355x_kv_write(const float* src, void* cache, int cache_dtype, int64_t B, int heads, int64_t S, int dim,
                               int64_t capacity, int64_t pos, int64_t src_b_stride, int64_t src_h_stride, int64_t src_p_stride,
                               void* stream);
-/* OpAttention (backend/op.go:117-129; backend/attention.go:25-143) without a
- * mask: queries [B, H, Q, D], keys and values [B, HK, K, D] of kv_dtype (F32 or
- * F16), out [B, H, Q, D], each read through strides {batch, head, position}
- * with contiguous features; lse, if not NULL, [B, H, Q] contiguous. Key j is
- * hidden from query i when causal and j > i + causal_offset. D at most 256. */
-MI355X_API mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const void* v, int kv_dtype,
-                               const int64_t* kv_strides, float* out, const int64_t* out_strides, float* lse, int64_t B, int H,
-                               int HK, int64_t Q, int64_t K, int D, double scale, int causal, int64_t causal_offset, void* stream);
+/* OpAttention (backend/op.go:117-129; backend/attention.go:25-143):
+ * softmax(scale * q . k^T + mask) . v. Queries [B, H, Q, D], keys [B, HK, K, D]
+ * and values [B, HK, K, DV] of kv_dtype (F32 or F16), out [B, H, Q, DV], each
+ * read through its strides {batch, head, position} in elements with contiguous
+ * features; lse, if not NULL, [B, H, Q] contiguous: the logsumexp of each row's
+ * scores. mask, if not NULL, is float32 [B, H, Q, K] read through mask_strides
+ * {batch, head, query, key} (0 broadcasts a dimension) and added to the scores;
+ * key j is also hidden from query i when causal and j > i + causal_offset. A
+ * row that sees no key gets zeros and -Inf; with K == 0 that is every row, and
+ * k, v and their strides may be NULL. D and DV at most 256. */
+MI355X_API mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const int64_t* k_strides, const void* v,
+                               const int64_t* v_strides, int kv_dtype, const float* mask, const int64_t* mask_strides, float* out,
+                               const int64_t* out_strides, float* lse, int64_t B, int H, int HK, int64_t Q, int64_t K, int D, int DV, double scale,
+                               int causal, int64_t causal_offset, void* stream);
 /* Block.mlp's activation (llm/model.go:446-448): out = SiLU(gate) * up, rows of
  * gate and up in_row_stride floats apart, out contiguous. */
 MI355X_API mi355x_status mi355x_swiglu(const float* gate, const float* up, float* out, int64_t rows, int64_t n, int64_t in_row_stride, void* stream);
@@ -242,8 +256,9 @@ MI355X_API mi355x_status mi355x_llama_generate(void* model, const int32_t* promp
  * Operations: MI355X_OP_QMATMUL (In[0] float32 [..., K] through any view, In[1]
  * block-quantized [N, K] read contiguously from a block boundary),
  * MI355X_OP_CAST and MI355X_OP_GATHER of a block-quantized In[0] through any
- * view, MI355X_OP_ATTENTION (q, k, v; the output holds the result [B..., H, Q, D]
- * followed by the logsumexp [B..., H, Q]). Anything else fails with
+ * view, MI355X_OP_ATTENTION (q, k, v and the optional additive mask In[3]
+ * [B..., H, Q, K]; the output holds the result [B..., H, Q, DV] followed by the
+ * logsumexp [B..., H, Q]). Anything else fails with
  * MI355X_ERR_INTERNAL. Errors: a foreign or freed buffer is MI355X_ERR_DTYPE, a
  * size that does not match MI355X_ERR_SHAPE, a gather index out of range
  * MI355X_ERR_INDEX at the next sync (rocm_linux.go:275-375).

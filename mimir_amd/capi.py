@@ -43,7 +43,8 @@ SYMBOLS = {
     "mi355x_rmsnorm": (C.c_uint32, [_vp, _vp, _vp, _i64, _i64, C.c_double, _vp]),
     "mi355x_rope": (C.c_uint32, [_vp, _vp, _i64, _i64, _int, _int, _int, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
     "mi355x_kv_write": (C.c_uint32, [_vp, _vp, _int, _i64, _int, _i64, _int, _i64, _i64, _i64, _i64, _i64, _vp]),
-    "mi355x_attention": (C.c_uint32, [_vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _i64, _int, _int, _i64, _i64, _int, C.c_double, _int, _i64, _vp]),
+    "mi355x_attention": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _i64, _i64, _int, _int,
+                                      C.c_double, _int, _i64, _vp]),
     "mi355x_swiglu": (C.c_uint32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_add": (C.c_uint32, [_vp, _vp, _vp, _i64, _vp]),
     "mi355x_argmax": (C.c_uint32, [_vp, _i64, _i64, _vp, _vp]),

@@ -14,10 +14,11 @@
 // load covers eight consecutive keys; values: lanes take consecutive features,
 // so each load is one contiguous key row.
 //
-// As the reference: the query is scaled first; p = exp(s - max); the result is
-// (sum p v) * (1 / sum p); the logsumexp is max + log(sum p); a row that sees
-// no key gets zeros and -Inf. Key j is hidden from query i when causal and
-// j > i + causal_offset.
+// As the reference: the query is scaled first; the additive mask [B, H, Q, K], if
+// any, is added to the scores (backend/cpu/attention.go:268-292); p = exp(s -
+// max); the result is (sum p v) * (1 / sum p); the logsumexp is max + log(sum p);
+// a row that sees no key gets zeros and -Inf. Key j is hidden from query i when
+// causal and j > i + causal_offset. Values may have another width (DV) than keys.
 #include "device_util.h"
 #include "kernels.h"
 
@@ -39,7 +40,8 @@ struct AttnParams {
     int64_t k_b, k_h, k_p;     // strides of k in elements
     int64_t v_b, v_h, v_p;     // strides of v in elements
     int64_t o_b, o_h, o_i;     // strides of out in floats
-    int B, H, HK, Q, K, D;
+    int64_t m_b, m_h, m_i, m_j; // strides of the mask in floats
+    int B, H, HK, Q, K, D, DV;
     float scale;
     int causal;
     int64_t causal_offset;
@@ -50,13 +52,14 @@ struct AttnParams {
 // Partial results of one (query row, head, split): m, l, then o[D].
 template <typename KV>
 __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float* __restrict__ q, const KV* __restrict__ k,
-                                                                    const KV* __restrict__ v, float* __restrict__ ws,
-                                                                    float* __restrict__ out, float* __restrict__ lse, AttnParams p) {
+                                                                    const KV* __restrict__ v, const float* __restrict__ mask,
+                                                                    float* __restrict__ ws, float* __restrict__ out, float* __restrict__ lse,
+                                                                    AttnParams p) {
     extern __shared__ float smem[];
-    const int D = p.D, G = p.H / p.HK, chunk = p.chunk;
+    const int D = p.D, DV = p.DV, G = p.H / p.HK, chunk = p.chunk;
     float* qs = smem;                       // [4][D], scaled
     float* sc = qs + kAttnHeads * D;        // [4][chunk]
-    float* red = sc + kAttnHeads * chunk;   // [4][kAttnThreads / 64 ... ] and slices of o: max(32, 4 * D) floats
+    float* red = sc + kAttnHeads * chunk;   // [4][kAttnThreads / 64 ... ] and slices of o: max(32, 4 * DV) floats
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int split = blockIdx.x;
     const int ngq = (G + kAttnHeads - 1) / kAttnHeads;
@@ -98,7 +101,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
 #pragma unroll
         for (int g = 0; g < kAttnHeads; g++) {
             float t = group8_sum(s[g]);
-            if (part == 0 && live) sc[g * chunk + jj] = t;
+            if (part == 0 && live) {
+                if (mask && g < ng) t = t + mask[b * p.m_b + (int64_t)(hk * G + g0 + g) * p.m_h + i * p.m_i + (int64_t)(j0 + jj) * p.m_j];
+                sc[g * chunk + jj] = t;
+            }
         }
     }
     __syncthreads();
@@ -130,10 +136,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
     __syncthreads();
 
     // values: thread (d, slice) sums the keys jj = slice, slice + nslice, ...
-    const int nslice = kAttnThreads / D > 0 ? kAttnThreads / D : 1;  // D <= 256
-    const int d = tid % D, slice = tid / D;
+    const int nslice = kAttnThreads / DV > 0 ? kAttnThreads / DV : 1;  // DV <= 256
+    const int d = tid % DV, slice = tid / DV;
     float o[kAttnHeads] = {0.f, 0.f, 0.f, 0.f};
-    if (slice < nslice && tid < nslice * D) {
+    if (slice < nslice && tid < nslice * DV) {
         const KV* vbase = v + b * p.v_b + (int64_t)hk * p.v_h + d;
         for (int jj = slice; jj < nj; jj += nslice) {
             float vv = kv_load<KV>(vbase + (int64_t)(j0 + jj) * p.v_p);
@@ -153,18 +159,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
     if (nslice > 1) {
         if (slice > 0 && slice < nslice) {
 #pragma unroll
-            for (int g = 0; g < kAttnHeads; g++) oslices[((slice - 1) * kAttnHeads + g) * D + d] = o[g];
+            for (int g = 0; g < kAttnHeads; g++) oslices[((slice - 1) * kAttnHeads + g) * DV + d] = o[g];
         }
         __syncthreads();
         if (slice == 0) {
             for (int s2 = 1; s2 < nslice; s2++)
 #pragma unroll
-                for (int g = 0; g < kAttnHeads; g++) o[g] += oslices[((s2 - 1) * kAttnHeads + g) * D + d];
+                for (int g = 0; g < kAttnHeads; g++) o[g] += oslices[((s2 - 1) * kAttnHeads + g) * DV + d];
         }
     }
     (void)m_g;
     (void)l_g;
-    if (slice != 0 || tid >= D) return;
+    if (slice != 0 || tid >= DV) return;
 #pragma unroll
     for (int g = 0; g < kAttnHeads; g++) {
         if (g >= ng) break;
@@ -179,7 +185,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
                 if (lse && d == 0) lse[((int64_t)b * p.H + h) * p.Q + i] = m4[g] + __builtin_logf(l4[g]);
             }
         } else {
-            float* w = ws + ((((int64_t)b * p.Q + i) * p.H + h) * p.nsplit + split) * (D + 2);
+            float* w = ws + ((((int64_t)b * p.Q + i) * p.H + h) * p.nsplit + split) * (DV + 2);
             if (d == 0) {
                 w[0] = m4[g];
                 w[1] = l4[g];
@@ -192,7 +198,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(const float*
 // out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M); one workgroup per (row, head).
 __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ ws, float* __restrict__ out,
                                                            float* __restrict__ lse, AttnParams p) {
-    const int D = p.D, d = threadIdx.x;
+    const int D = p.DV, d = threadIdx.x;
     const int64_t rh = blockIdx.x;  // (b * Q + i) * H + h
     const int h = (int)(rh % p.H);
     const int64_t bi = rh / p.H;
@@ -222,6 +228,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
     }
 }
 
+// D: the width of the values.
 size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit) {
     return nsplit <= 1 ? 0 : (size_t)(B * Q * H * nsplit * (D + 2)) * sizeof(float);
 }
@@ -244,7 +251,9 @@ hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st) {
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];
     p.v_b = a.v_strides[0]; p.v_h = a.v_strides[1]; p.v_p = a.v_strides[2];
     p.o_b = a.o_strides[0]; p.o_h = a.o_strides[1]; p.o_i = a.o_strides[2];
-    p.B = (int)a.B; p.H = a.H; p.HK = a.HK; p.Q = (int)a.Q; p.K = (int)a.K; p.D = a.D;
+    const int DV = a.DV > 0 ? a.DV : a.D;
+    p.m_b = a.m_strides[0]; p.m_h = a.m_strides[1]; p.m_i = a.m_strides[2]; p.m_j = a.m_strides[3];
+    p.B = (int)a.B; p.H = a.H; p.HK = a.HK; p.Q = (int)a.Q; p.K = (int)a.K; p.D = a.D; p.DV = DV;
     p.scale = (float)a.scale;
     p.causal = a.causal;
     p.causal_offset = a.causal_offset;
@@ -253,20 +262,43 @@ hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st) {
     p.dyn_k = a.dyn_k;
     int G = a.H / a.HK, ngq = (G + kAttnHeads - 1) / kAttnHeads;
     dim3 grid((unsigned)a.nsplit, (unsigned)(a.HK * ngq), (unsigned)(a.B * a.Q));
-    int redf = 4 * a.D > 32 ? 4 * a.D : 32;
-    int nslice = kAttnThreads / a.D > 0 ? kAttnThreads / a.D : 1;
-    if ((nslice - 1) * kAttnHeads * a.D > redf) redf = (nslice - 1) * kAttnHeads * a.D;
+    int redf = 4 * DV > 32 ? 4 * DV : 32;
+    int nslice = kAttnThreads / DV > 0 ? kAttnThreads / DV : 1;
+    if ((nslice - 1) * kAttnHeads * DV > redf) redf = (nslice - 1) * kAttnHeads * DV;
     size_t lds = (size_t)(kAttnHeads * a.D + kAttnHeads * a.chunk + redf) * sizeof(float);
     if (a.kv_dtype == kF16)
         hipLaunchKernelGGL(attn_partial_kernel<uint16_t>, grid, dim3(kAttnThreads), lds, st, a.q, (const uint16_t*)a.k,
-                           (const uint16_t*)a.v, (float*)workspace, a.out, a.lse, p);
+                           (const uint16_t*)a.v, a.mask, (float*)workspace, a.out, a.lse, p);
     else
-        hipLaunchKernelGGL(attn_partial_kernel<float>, grid, dim3(kAttnThreads), lds, st, a.q, (const float*)a.k, (const float*)a.v,
+        hipLaunchKernelGGL(attn_partial_kernel<float>, grid, dim3(kAttnThreads), lds, st, a.q, (const float*)a.k, (const float*)a.v, a.mask,
                            (float*)workspace, a.out, a.lse, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.nsplit == 1) return e;
     hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)(a.B * a.Q * a.H)), dim3(256), 0, st, (const float*)workspace, a.out,
                        a.lse, p);
+    return hipGetLastError();
+}
+
+// No keys at all: every row gets zeros and a logsumexp of -Inf (backend/cpu/attention.go:472-476,494-497), and
+// nothing reads k or v. One thread per output element.
+__global__ __launch_bounds__(256) void attn_empty_kernel(float* __restrict__ out, float* __restrict__ lse, int64_t o_b, int64_t o_h, int64_t o_i,
+                                                         int H, int Q, int DV, int64_t n) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const int d = (int)(t % DV);
+    const int64_t row = t / DV;  // (b * H + h) * Q + i
+    const int i = (int)(row % Q);
+    const int h = (int)(row / Q % H);
+    const int64_t b = row / Q / H;
+    out[b * o_b + h * o_h + i * o_i + d] = 0.f;
+    if (lse && d == 0) lse[row] = -__builtin_inff();
+}
+
+hipError_t attention_empty(const AttnArgs& a, hipStream_t st) {
+    const int DV = a.DV > 0 ? a.DV : a.D;
+    const int64_t n = a.B * a.H * a.Q * DV;
+    hipLaunchKernelGGL(attn_empty_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a.out, a.lse, a.o_strides[0], a.o_strides[1],
+                       a.o_strides[2], a.H, (int)a.Q, DV, n);
     return hipGetLastError();
 }
 

@@ -369,7 +369,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 
 }  // namespace
 
-static int g_force_splits = 0;  // measurement aid: a fixed number of shares
+static std::atomic<int> g_force_splits{0};  // measurement aid: a fixed number of shares
 void set_attention_decode_splits(int n) { g_force_splits = n; }
 
 // Shares of the keys and the most keys a share can hold, for at most kmax keys.
@@ -395,6 +395,7 @@ size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit) {
 // or 128 features, rows of the caches and of q aligned for 16-byte loads.
 bool attention_decode_ok(const AttnArgs& a, int64_t kmax) {
     if (a.Q != 1 || (a.D != 64 && a.D != 128) || a.B <= 0 || a.B > 65535) return false;
+    if (a.mask || (a.DV > 0 && a.DV != a.D) || kmax <= 0 || !a.k || !a.v) return false;  // the general kernels take those
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
     if (a.B * a.HK * ngq > kCounterBytes / 4 || (int64_t)a.HK * ngq > 65535) return false;
     const int es = a.kv_dtype == kF16 ? 2 : 4;

@@ -434,8 +434,8 @@ Status Backend::issue(const Kernel& k, const std::vector<Buffer*>& outs, const s
     }
     case Op::Attention: {
         // NewAttentionShape (backend/attention.go:36-62)
-        if (k.in.size() == 4) return Status::fail(Err::Internal, "attention with a mask is not on this path");
-        if (k.in.size() != 3) return Status::fail(Err::Internal, "attention: %zu inputs", k.in.size());
+        if (k.in.size() != 3 && k.in.size() != 4) return Status::fail(Err::Internal, "attention: %zu inputs", k.in.size());
+        const bool masked = k.in.size() == 4;
         const View &vq = k.in[0], &vk = k.in[1], &vv = k.in[2];
         const int r = (int)vq.shape.size();
         bool ok = r >= 3 && (int)vk.shape.size() == r && (int)vv.shape.size() == r;
@@ -447,23 +447,38 @@ Status Backend::issue(const Kernel& k, const std::vector<Buffer*>& outs, const s
         if (vk.shape[r - 1] != D || HK < 1 || H % HK != 0)
             return Status::fail(Err::Shape, "attention of queries %s, keys %s, values %s", shape_str(vq.shape).c_str(), shape_str(vk.shape).c_str(),
                                 shape_str(vv.shape).c_str());
+        if (masked) {  // [B..., H, Q, K] (backend/attention.go:53-55)
+            const View& vm = k.in[3];
+            bool mok = (int)vm.shape.size() == r && vm.shape[r - 3] == H && vm.shape[r - 2] == Q && vm.shape[r - 1] == Kn;
+            for (int d = 0; mok && d < r - 3; d++) mok = vm.shape[d] == vq.shape[d];
+            if (!mok) return Status::fail(Err::Shape, "attention of queries %s, keys %s and mask %s", shape_str(vq.shape).c_str(), shape_str(vk.shape).c_str(),
+                                          shape_str(vm.shape).c_str());
+            if (ins[3]->dtype() != MI355X_F32) return Status::fail(Err::DType, "attention with a mask of dtype %d", ins[3]->dtype());
+        }
         if (ins[0]->dtype() != MI355X_F32 || k.dtype != MI355X_F32 || ins[1]->dtype() != ins[2]->dtype() ||
             (ins[1]->dtype() != MI355X_F32 && ins[1]->dtype() != MI355X_F16))
             return Status::fail(Err::DType, "attention of dtype %d over keys of dtype %d", ins[0]->dtype(), ins[1]->dtype());
-        int64_t B = 0, qb = 0, kb = 0, vb = 0, B2 = 0, B3 = 0;
-        if (DV != D || !leading_rows(vq, 3, &B, &qb) || !leading_rows(vk, 3, &B2, &kb) || !leading_rows(vv, 3, &B3, &vb) ||
-            (D > 1 && (vq.strides[r - 1] != 1 || vk.strides[r - 1] != 1 || vv.strides[r - 1] != 1)) || vk.strides[r - 3] != vv.strides[r - 3] ||
-            vk.strides[r - 2] != vv.strides[r - 2] || kb != vb)
+        int64_t B = 0, qb = 0, kb = 0, vb = 0, mb = 0, B2 = 0, B3 = 0, B4 = 0;
+        if (!leading_rows(vq, 3, &B, &qb) || !leading_rows(vk, 3, &B2, &kb) || !leading_rows(vv, 3, &B3, &vb) ||
+            (masked && !leading_rows(k.in[3], 3, &B4, &mb)) ||
+            (D > 1 && (vq.strides[r - 1] != 1 || vk.strides[r - 1] != 1)) || (DV > 1 && vv.strides[r - 1] != 1))
             return Status::fail(Err::Internal, "attention: views of this layout are not on this path");
-        if (n_out != B * H * Q * (D + 1)) return Status::fail(Err::Internal, "attention into %s", shape_str(k.shape).c_str());
+        if (n_out != B * H * Q * (DV + 1)) return Status::fail(Err::Internal, "attention into %s", shape_str(k.shape).c_str());
         if (n_out == 0) return {};
         int64_t qs[3] = {qb, vq.strides[r - 3], vq.strides[r - 2]}, ks[3] = {kb, vk.strides[r - 3], vk.strides[r - 2]};
-        int64_t os[3] = {H * Q * D, Q * D, D};
+        int64_t vs[3] = {vb, vv.strides[r - 3], vv.strides[r - 2]};
+        int64_t os[3] = {H * Q * DV, Q * DV, DV}, ms[4] = {0, 0, 0, 0};
+        const float* mask = nullptr;
+        if (masked) {
+            const View& vm = k.in[3];
+            ms[0] = mb; ms[1] = vm.strides[r - 3]; ms[2] = vm.strides[r - 2]; ms[3] = vm.strides[r - 1];
+            mask = (const float*)in[3] + vm.offset;
+        }
         const size_t esz = ins[1]->dtype() == MI355X_F16 ? 2 : 4;
         float* o = (float*)out;
-        return from_code(mi355x_attention((const float*)in[0] + vq.offset, qs, (const uint8_t*)in[1] + vk.offset * esz,
-                                          (const uint8_t*)in[2] + vv.offset * esz, ins[1]->dtype(), ks, o, os, o + B * H * Q * D, B, (int)H, (int)HK, Q,
-                                          Kn, (int)D, k.attrs.scale, k.attrs.causal ? 1 : 0, k.attrs.causal_offset, stream_),
+        return from_code(mi355x_attention((const float*)in[0] + vq.offset, qs, (const uint8_t*)in[1] + vk.offset * esz, ks,
+                                          (const uint8_t*)in[2] + vv.offset * esz, vs, ins[1]->dtype(), mask, ms, o, os, o + B * H * Q * DV, B, (int)H,
+                                          (int)HK, Q, Kn, (int)D, (int)DV, k.attrs.scale, k.attrs.causal ? 1 : 0, k.attrs.causal_offset, stream_),
                          "attention");
     }
     }

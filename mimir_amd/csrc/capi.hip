@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <vector>
 #include <string>
@@ -40,41 +41,51 @@ mi355x_status hip_fail(hipError_t e, const char* what) {
 
 constexpr int kMaxDevices = 16;
 
+// Scratch memory of the entry points that need some beyond their arguments (converted activations,
+// partial results and tickets of split attention and argmax, float32 copies of qgemm_bf16's general
+// route). One set per device and stream: calls on different streams never share a block, calls on one
+// stream are ordered by it. A block that has become too small is replaced by a larger one and is never
+// freed: work already queued, and HIP graphs a caller has instantiated over an entry point, may still
+// read and write it, tickets included (a graph keeps the block it was recorded with and stays valid).
+// Growth at least doubles a block, so what is kept aside stays below the size of the live block.
+struct ScratchBlock {
+    void* p = nullptr;
+    size_t bytes = 0;
+};
+struct StreamScratch {
+    ScratchBlock act, attn, gemm, argmax;
+};
+
 // Per-device state: the error word kernels OR bits into, read back at sync.
 struct DeviceState {
     bool ready = false;
     uint32_t* err_dev = nullptr;
     uint32_t* err_host = nullptr;  // pinned
-    // Converted activations of mi355x_qgemv's fixed-point path: grown on
-    // demand, shared by every call on this device (calls that overlap on two
-    // streams of one device race on it).
-    void* act = nullptr;
-    size_t act_bytes = 0;
-    // Partial results of split attention, grown and shared likewise.
-    void* attn = nullptr;
-    size_t attn_bytes = 0;
-    // Float32 copies of activations and results for qgemm_bf16's general route.
-    void* gemm = nullptr;
-    size_t gemm_bytes = 0;
-    // Tickets and candidates of the split argmax.
-    void* argmax = nullptr;
-    size_t argmax_bytes = 0;
+    std::map<void*, StreamScratch> scratch;  // by stream handle
+    std::vector<void*> retired;              // outgrown blocks, kept until the process ends
 };
 
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
-int g_tune_q4[5] = {0, 0, 0, 0, 0};
+std::atomic<int> g_tune_q4_live[5] = {{0}, {0}, {0}, {0}, {0}};
+// A call's own copy of the launch-plan overrides, so that one call sees one plan.
+struct TuneQ4 {
+    int v[5];
+    TuneQ4() { for (int i = 0; i < 5; i++) v[i] = g_tune_q4_live[i].load(std::memory_order_relaxed); }
+    operator const int*() const { return v; }
+    int operator[](int i) const { return v[i]; }
+};
 // Up to this many rows of x the Q4_0 product converts x inside its own launch (each workgroup
 // for itself); beyond, one conversion launch serves all workgroups.
 constexpr int64_t kConvertInProductRows = 8;
 // Rows of x from which the Q4_0 product of float32 x goes to the int8 matrix cores: 16 means wherever its
 // cost model says it pays; "q4_0.fx_rows" sets another threshold, which then holds for every shape.
-int g_fx_min_rows = 16;
-int g_rows_max = 0;    // "q4_0.rows_max" n: Q4_0 products of fewer than n rows of x take the kernel that reads W once per eight rows (0: by cost)
-int g_rows_path = 0;  // "q4_0.rows_path" 1: no matrix-core kernel for two to fifteen rows of x
-int g_tune_gemm = 0;  // 1: qgemm_bf16 always takes its general route
-int g_tune_gemm_f16 = 0;  // 1: the Q4_0 matrix-core product with weights rounded to binary16
-int g_tune_attn = 0;  // 1: the general kernels also for one query position
+std::atomic<int> g_fx_min_rows{16};
+std::atomic<int> g_rows_max{0};    // "q4_0.rows_max" n: Q4_0 products of fewer than n rows of x take the kernel that reads W once per eight rows (0: by cost)
+std::atomic<int> g_rows_path{0};  // "q4_0.rows_path" 1: no matrix-core kernel for two to fifteen rows of x
+std::atomic<int> g_tune_gemm{0};  // 1: qgemm_bf16 always takes its general route
+std::atomic<int> g_tune_gemm_f16{0};  // 1: the Q4_0 matrix-core product with weights rounded to binary16
+std::atomic<int> g_tune_attn{0};  // 1: the general kernels also for one query position
 }
 thread_local std::vector<hipEvent_t> t_events;
 thread_local size_t t_events_used = 0;
@@ -111,69 +122,62 @@ mi355x_status current_state(DeviceState** out) {
     return MI355X_OK;
 }
 
-// Returns the device's activation scratch, at least `bytes` long.
-mi355x_status act_scratch(size_t bytes, void** out) {
+// Returns the calling stream's block `which` of the current device, at least `bytes` long (at least `floor`
+// when it has to be allocated); the first `zero_prefix` bytes of a new block are zeroed (tickets).
+// Allocates, so it fails under stream capture when the block has to grow: a caller that records a
+// graph runs the call once beforehand, as run_batch does.
+mi355x_status stream_scratch(void* stream, ScratchBlock StreamScratch::*which, size_t bytes, size_t floor, size_t zero_prefix, const char* what,
+                             void** out) {
     DeviceState* s;
     if (mi355x_status st = current_state(&s)) return st;
     std::lock_guard<std::mutex> lock(g_mu);
-    if (s->act_bytes < bytes) {
-        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+    ScratchBlock& b = s->scratch[stream].*which;
+    if (b.bytes < bytes) {
+        size_t want = bytes < floor ? floor : bytes;
+        if (want < 2 * b.bytes) want = 2 * b.bytes;
         void* p = nullptr;
-        HIP_TRY(hipMalloc(&p, want), "hipMalloc(activation scratch)");
-        if (s->act) HIP_TRY(hipFree(s->act), "hipFree(activation scratch)");  // waits for work that reads it
-        s->act = p;
-        s->act_bytes = want;
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) return fail((mi355x_status)e, "mi355x: hipMalloc(%s scratch, %zu bytes): %s", what, want, hipGetErrorName(e));
+        if (zero_prefix) {
+            e = hipMemset(p, 0, zero_prefix);
+            if (e != hipSuccess) {
+                (void)hipFree(p);  // nothing has seen it yet
+                return fail((mi355x_status)e, "mi355x: hipMemset(%s tickets): %s", what, hipGetErrorName(e));
+            }
+        }
+        if (b.p) s->retired.push_back(b.p);
+        b.p = p;
+        b.bytes = want;
     }
-    *out = s->act;
+    *out = b.p;
     return MI355X_OK;
 }
 
-mi355x_status attn_scratch(size_t bytes, void** out) {
-    DeviceState* s;
-    if (mi355x_status st = current_state(&s)) return st;
-    std::lock_guard<std::mutex> lock(g_mu);
-    if (s->attn_bytes < bytes) {
-        size_t want = bytes < (4u << 20) ? (4u << 20) : bytes;
-        void* p = nullptr;
-        HIP_TRY(hipMalloc(&p, want), "hipMalloc(attention scratch)");
-        HIP_TRY(hipMemset(p, 0, mimir::kAttnTicketBytes), "hipMemset(attention tickets)");  // the decode kernel's tickets
-        if (s->attn) HIP_TRY(hipFree(s->attn), "hipFree(attention scratch)");
-        s->attn = p;
-        s->attn_bytes = want;
-    }
-    *out = s->attn;
+mi355x_status act_scratch(void* stream, size_t bytes, void** out) {
+    return stream_scratch(stream, &StreamScratch::act, bytes, 1u << 20, 0, "activation", out);
+}
+// Where a product's converted activations go: the stream's growing block, or a fixed block of
+// fixed_bytes bytes (then nothing is allocated and a larger need is an error).
+struct ActSource {
+    void* stream;
+    void* fixed;
+    size_t fixed_bytes;
+};
+mi355x_status act_for(const ActSource& src, size_t bytes, void** out) {
+    if (!src.fixed) return act_scratch(src.stream, bytes, out);
+    if (bytes > src.fixed_bytes)
+        return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_noalloc: the converted activations take %zu bytes, the fixed scratch holds %zu", bytes, src.fixed_bytes);
+    *out = src.fixed;
     return MI355X_OK;
 }
-
-mi355x_status gemm_scratch(size_t bytes, void** out) {
-    DeviceState* s;
-    if (mi355x_status st = current_state(&s)) return st;
-    std::lock_guard<std::mutex> lock(g_mu);
-    if (s->gemm_bytes < bytes) {
-        void* p = nullptr;
-        HIP_TRY(hipMalloc(&p, bytes), "hipMalloc(gemm scratch)");
-        if (s->gemm) HIP_TRY(hipFree(s->gemm), "hipFree(gemm scratch)");
-        s->gemm = p;
-        s->gemm_bytes = bytes;
-    }
-    *out = s->gemm;
-    return MI355X_OK;
+mi355x_status attn_scratch(void* stream, size_t bytes, void** out) {
+    return stream_scratch(stream, &StreamScratch::attn, bytes, 4u << 20, mimir::kAttnTicketBytes, "attention", out);
 }
-
-mi355x_status argmax_scratch(size_t bytes, void** out) {
-    DeviceState* s;
-    if (mi355x_status st = current_state(&s)) return st;
-    std::lock_guard<std::mutex> lock(g_mu);
-    if (s->argmax_bytes < bytes) {
-        void* p = nullptr;
-        HIP_TRY(hipMalloc(&p, bytes), "hipMalloc(argmax scratch)");
-        HIP_TRY(hipMemset(p, 0, mimir::kArgmaxTicketBytes), "hipMemset(argmax tickets)");
-        if (s->argmax) HIP_TRY(hipFree(s->argmax), "hipFree(argmax scratch)");
-        s->argmax = p;
-        s->argmax_bytes = bytes;
-    }
-    *out = s->argmax;
-    return MI355X_OK;
+mi355x_status gemm_scratch(void* stream, size_t bytes, void** out) {
+    return stream_scratch(stream, &StreamScratch::gemm, bytes, 0, 0, "gemm", out);
+}
+mi355x_status argmax_scratch(void* stream, size_t bytes, void** out) {
+    return stream_scratch(stream, &StreamScratch::argmax, bytes, 0, mimir::kArgmaxTicketBytes, "argmax", out);
 }
 
 }  // namespace
@@ -293,19 +297,19 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     if (dtype == MI355X_Q4_0 && g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
         void* half_ws = nullptr;
         if (g_tune_gemm_f16 == 1)
-            if (mi355x_status s2 = gemm_scratch(mimir::qgemm_q4_0_half_ws_bytes(M, K), &half_ws)) return s2;
+            if (mi355x_status s2 = gemm_scratch(stream, mimir::qgemm_q4_0_half_ws_bytes(M, K), &half_ws)) return s2;
         HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, half_ws, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
     if ((dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) && g_tune_gemm != 1 && ((uintptr_t)X & 7) == 0 && x_row_stride % 4 == 0) {
         // the int8 rounding reads the bfloat16 rows directly and the matrix-core kernel rounds its results
         void* act;
-        if (mi355x_status s2 = act_scratch(mimir::kq_act_bytes(K) * (size_t)M, &act)) return s2;
+        if (mi355x_status s2 = act_scratch(stream, mimir::kq_act_bytes(K) * (size_t)M, &act)) return s2;
         mimir::QGemvArgs a{W, nullptr, act, (float*)Y, M, N, K, 0, 0};
         if (mimir::qgemv_kquant_rows_pays(dtype, a)) {  // a few rows: W read once per eight of them, the same bits, one rounding after
             float* yf = (float*)Y;
             if (!f32) {
-                if (mi355x_status s2 = gemm_scratch(((size_t)M * N * 4 + 255) & ~(size_t)255, &ws)) return s2;
+                if (mi355x_status s2 = gemm_scratch(stream, ((size_t)M * N * 4 + 255) & ~(size_t)255, &ws)) return s2;
                 yf = (float*)ws;
             }
             a.y = yf;
@@ -324,7 +328,7 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     // Q8_0, Q4_K and Q6_K that is the reference's own sequence (cast, int8 rounding of x, integer dot
     // products, cast), and the K-quants take their matrix-core kernel from a few rows on.
     const size_t xb = ((size_t)M * K * 4 + 255) & ~(size_t)255, yb = ((size_t)M * N * 4 + 255) & ~(size_t)255;
-    if (mi355x_status s2 = gemm_scratch(xb + yb, &ws)) return s2;
+    if (mi355x_status s2 = gemm_scratch(stream, xb + yb, &ws)) return s2;
     float* xf = (float*)ws;
     float* yf = f32 ? (float*)Y : (float*)((uint8_t*)ws + xb);
     HIP_TRY(mimir::bf16_rows_to_f32(X, xf, M, K, x_row_stride, st), "launch cast");
@@ -333,8 +337,9 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     return MI355X_OK;
 }
 
-mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
-                           int64_t x_row_stride, void* stream) {
+static mi355x_status qgemv_impl(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride,
+                                void* stream, const ActSource& src) {
+    const TuneQ4 g_tune_q4;  // this call's copy of the launch-plan overrides
     if (!mimir::is_quantized(dtype)) return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by weights of dtype %d", dtype);
     int bs = mimir::block_size(dtype);
     if (M < 0 || N < 0 || K < 0 || K % bs != 0)
@@ -367,7 +372,7 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
                 const bool one_launch = mimir::qgemv_q4_0_rows_shares_ok(W, M, N, K, 1);  // else the variant that takes eight rows a launch
                 const int64_t groups = (M + 7) / 8;
                 void* act;
-                if (mi355x_status st = act_scratch(mimir::q4_0_rows_act_bytes(K) * (size_t)(one_launch ? groups : 1), &act)) return st;
+                if (mi355x_status st = act_for(src, mimir::q4_0_rows_act_bytes(K) * (size_t)(one_launch ? groups : 1), &act)) return st;
                 if (one_launch) {
                     HIP_TRY(mimir::q4_0_rows_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_rows_convert_act");
                     HIP_TRY(mimir::qgemv_q4_0_rows(W, act, y, nullptr, M, N, K, 1, (hipStream_t)stream), "launch qgemv_q4_0_rows");
@@ -384,7 +389,7 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
                 ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0) {
                 // many rows: the same fixed-point arithmetic on the int8 matrix cores
                 void* act;
-                if (mi355x_status st = act_scratch(mimir::q4_0_fx_act_bytes(K) * (size_t)M, &act)) return st;
+                if (mi355x_status st = act_for(src, mimir::q4_0_fx_act_bytes(K) * (size_t)M, &act)) return st;
                 HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_fx_convert_act");
                 HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, (hipStream_t)stream), "launch qgemm_q4_0_fx");
                 return MI355X_OK;
@@ -395,7 +400,7 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
                 return MI355X_OK;
             }
             void* act;
-            if (mi355x_status st = act_scratch(mimir::q4_0_act_bytes(K) * (size_t)M, &act)) return st;
+            if (mi355x_status st = act_for(src, mimir::q4_0_act_bytes(K) * (size_t)M, &act)) return st;
             HIP_TRY(mimir::q4_0_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_convert_act");
             a.act = act;
             HIP_TRY(mimir::qgemv_q4_0_act(a, g_tune_q4, (hipStream_t)stream), "launch qgemv_q4_0_act");
@@ -412,7 +417,7 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
             return MI355X_OK;
         }
         void* act;
-        if (mi355x_status st = act_scratch(mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
+        if (mi355x_status st = act_for(src, mimir::q8_act_bytes(K) * (size_t)M, &act)) return st;
         HIP_TRY(mimir::q8_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q8_convert_act");
         a.act = act;
         if (g_rows_path != 1 && mimir::qgemv_q8_0_mfma_pays(a)) {  // a large matrix and two to eight rows: the int8 matrix cores
@@ -435,7 +440,7 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
             return MI355X_OK;
         }
         void* act;
-        if (mi355x_status st = act_scratch(mimir::kq_act_bytes(K) * (size_t)M, &act)) return st;
+        if (mi355x_status st = act_for(src, mimir::kq_act_bytes(K) * (size_t)M, &act)) return st;
         HIP_TRY(mimir::kq_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch kq_convert_act");
         a.act = act;
         HIP_TRY(mimir::qgemv_kquant_act(dtype, a, (hipStream_t)stream), "launch qgemv_kquant_act");
@@ -444,6 +449,11 @@ mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, i
     default:
         return fail(MI355X_ERR_DTYPE, "mi355x: qgemv by weights of dtype %d", dtype);
     }
+}
+
+mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
+                           int64_t x_row_stride, void* stream) {
+    return qgemv_impl(dtype, W, x, y, M, N, K, x_row_stride, stream, ActSource{stream, nullptr, 0});
 }
 
 size_t mi355x_act_bytes(int dtype, int64_t K) {
@@ -469,6 +479,7 @@ mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K
 }
 
 mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    const TuneQ4 g_tune_q4;  // this call's copy of the launch-plan overrides
     if (M < 0 || N < 0 || K <= 0 || M > 65535 || N > (int64_t)1 << 30)
         return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act of %lld rows by [%lld, %lld]", (long long)M, (long long)N, (long long)K);
     if (M == 0 || N == 0) return MI355X_OK;
@@ -501,6 +512,7 @@ static mi355x_status fused_args_ok(const char* what, int dtype, const void* act,
 }
 
 mi355x_status mi355x_qgemv_act_add(int dtype, const void* W, const void* act, const float* resid, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    const TuneQ4 g_tune_q4;  // this call's copy of the launch-plan overrides
     if (mi355x_status st = fused_args_ok("qgemv_act_add", dtype, act, y, M, K)) return st;
     if (N < 0 || N > (int64_t)1 << 30) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_add of %lld rows", (long long)N);
     if (M == 0 || N == 0) return MI355X_OK;
@@ -513,6 +525,7 @@ mi355x_status mi355x_qgemv_act_add(int dtype, const void* W, const void* act, co
 
 mi355x_status mi355x_qgemv_act_multi(int dtype, const void* W0, const void* W1, const void* W2, int64_t n0, int64_t n1, int64_t n2,
                                      const void* act, float* y, int64_t M, int64_t K, void* stream) {
+    const TuneQ4 g_tune_q4;  // this call's copy of the launch-plan overrides
     if (mi355x_status st = fused_args_ok("qgemv_act_multi", dtype, act, y, M, K)) return st;
     const void* W[3] = {W0, W1, W2};
     const int64_t n[3] = {n0, n1, n2};
@@ -529,6 +542,7 @@ mi355x_status mi355x_qgemv_act_multi(int dtype, const void* W0, const void* W1, 
 }
 
 mi355x_status mi355x_qgemv_act_swiglu(int dtype, const void* gate, const void* up, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+    const TuneQ4 g_tune_q4;  // this call's copy of the launch-plan overrides
     if (mi355x_status st = fused_args_ok("qgemv_act_swiglu", dtype, act, y, M, K)) return st;
     if (N < 0 || N > (int64_t)1 << 28) return fail(MI355X_ERR_SHAPE, "mi355x: qgemv_act_swiglu of %lld rows", (long long)N);
     if (M == 0 || N == 0) return MI355X_OK;
@@ -599,37 +613,47 @@ mi355x_status mi355x_kv_write(const float* src, void* cache, int cache_dtype, in
     return MI355X_OK;
 }
 
-mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const void* v, int kv_dtype,
-                               const int64_t* kv_strides, float* out, const int64_t* out_strides, float* lse, int64_t B, int H,
-                               int HK, int64_t Q, int64_t K, int D, double scale, int causal, int64_t causal_offset, void* stream) {
+mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const int64_t* k_strides, const void* v,
+                               const int64_t* v_strides, int kv_dtype, const float* mask, const int64_t* mask_strides, float* out,
+                               const int64_t* out_strides, float* lse, int64_t B, int H, int HK, int64_t Q, int64_t K, int D, int DV, double scale,
+                               int causal, int64_t causal_offset, void* stream) {
     if (kv_dtype != MI355X_F32 && kv_dtype != MI355X_F16) return fail(MI355X_ERR_DTYPE, "mi355x: attention over keys of dtype %d", kv_dtype);
     // backend/attention.go:36-62
-    if (B < 0 || Q < 0 || K < 0 || H <= 0 || HK <= 0 || H % HK != 0 || D <= 0 || D > 256)
-        return fail(MI355X_ERR_SHAPE, "mi355x: attention of %d heads on %d key heads of %d features (at most 256)", H, HK, D);
+    if (B < 0 || Q < 0 || K < 0 || H <= 0 || HK <= 0 || H % HK != 0 || D <= 0 || D > 256 || DV <= 0 || DV > 256)
+        return fail(MI355X_ERR_SHAPE, "mi355x: attention of %d heads on %d key heads of %d features and values of %d (at most 256)", H, HK, D, DV);
     if (B == 0 || Q == 0) return MI355X_OK;
     if (B * Q > 65535 || (int64_t)HK * ((H / HK + 3) / 4) > 65535)
         return fail(MI355X_ERR_SHAPE, "mi355x: attention of %lld query rows: too many for one launch", (long long)(B * Q));
-    if (!q || !out || !q_strides || !kv_strides || !out_strides || (K > 0 && (!k || !v))) return fail(MI355X_ERR_INTERNAL, "mi355x: attention: null pointer");
+    if (!q || !out || !q_strides || !out_strides || (K > 0 && (!k || !v || !k_strides || !v_strides)) || (mask && !mask_strides))
+        return fail(MI355X_ERR_INTERNAL, "mi355x: attention: null pointer");
     mimir::AttnArgs a;
     a.q = q; a.k = k; a.v = v; a.kv_dtype = kv_dtype; a.out = out; a.lse = lse;
     for (int i = 0; i < 3; i++) {
         a.q_strides[i] = q_strides[i];
-        a.k_strides[i] = a.v_strides[i] = kv_strides[i];
+        a.k_strides[i] = K > 0 ? k_strides[i] : 0;
+        a.v_strides[i] = K > 0 ? v_strides[i] : 0;
         a.o_strides[i] = out_strides[i];
     }
-    a.B = B; a.Q = Q; a.K = K; a.H = H; a.HK = HK; a.D = D;
+    a.B = B; a.Q = Q; a.K = K; a.H = H; a.HK = HK; a.D = D; a.DV = DV;
     a.scale = scale; a.causal = causal; a.causal_offset = causal_offset;
+    a.mask = K > 0 ? mask : nullptr;
+    if (a.mask)
+        for (int i = 0; i < 4; i++) a.m_strides[i] = mask_strides[i];
+    if (K == 0) {  // no row sees a key: zeros and -Inf, and nothing reads k or v (which may be null)
+        HIP_TRY(mimir::attention_empty(a, (hipStream_t)stream), "launch attention_empty");
+        return MI355X_OK;
+    }
     void* ws = nullptr;
     if (g_tune_attn != 1 && mimir::attention_decode_ok(a, K)) {  // one query position: a single launch
         int cmax;
         mimir::attention_decode_plan(B, H, HK, K, &a.nsplit, &cmax);
-        if (mi355x_status st = attn_scratch(mimir::attention_decode_workspace_bytes(B, H, D, a.nsplit), &ws)) return st;
+        if (mi355x_status st = attn_scratch(stream, mimir::attention_decode_workspace_bytes(B, H, D, a.nsplit), &ws)) return st;
         HIP_TRY(mimir::attention_decode(a, K, ws, nullptr, 0, (hipStream_t)stream), "launch attention_decode");
         return MI355X_OK;
     }
     mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
     // the scratch begins with the decode kernel's tickets
-    if (mi355x_status st = attn_scratch(mimir::kAttnTicketBytes + mimir::attention_workspace_bytes(B, H, Q, D, a.nsplit), &ws)) return st;
+    if (mi355x_status st = attn_scratch(stream, mimir::kAttnTicketBytes + mimir::attention_workspace_bytes(B, H, Q, DV, a.nsplit), &ws)) return st;
     HIP_TRY(mimir::attention(a, (uint8_t*)ws + mimir::kAttnTicketBytes, (hipStream_t)stream), "launch attention");
     return MI355X_OK;
 }
@@ -656,7 +680,7 @@ mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_
     if (!logits || !out) return fail(MI355X_ERR_INTERNAL, "mi355x: argmax: null pointer");
     void* ws = nullptr;
     if (rows <= 1024)
-        if (mi355x_status st = argmax_scratch(mimir::argmax_workspace_bytes(1024), &ws)) return st;
+        if (mi355x_status st = argmax_scratch(stream, mimir::argmax_workspace_bytes(1024), &ws)) return st;
     HIP_TRY(mimir::argmax(logits, rows, n, out, ws, (hipStream_t)stream), "launch argmax");
     return MI355X_OK;
 }
@@ -665,7 +689,7 @@ mi355x_status mi355x_tune(const char* key, int value) {
     static const char* keys[5] = {"q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path"};
     for (int i = 0; i < 5; i++)
         if (key && strcmp(key, keys[i]) == 0) {
-            g_tune_q4[i] = value;
+            g_tune_q4_live[i] = value;
             return MI355X_OK;
         }
     if (key && (strcmp(key, "kquant.rows") == 0 || strcmp(key, "kquant.path") == 0)) {

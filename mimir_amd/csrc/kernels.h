@@ -191,10 +191,15 @@ struct AttnArgs {
     int64_t causal_offset;
     int chunk, nsplit;
     const int32_t* dyn_k = nullptr;  // device int: that many more keys than K
+    int DV = 0;                      // features of a value (0: D)
+    const float* mask = nullptr;     // added to the scores, [B, H, Q, K] read through m_strides {batch, head, query, key}
+    int64_t m_strides[4] = {0, 0, 0, 0};
 };
 void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, int* nsplit);
 size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit);
 hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
+// K == 0: zeros and a logsumexp of -Inf for every row; reads neither keys nor values.
+hipError_t attention_empty(const AttnArgs& a, hipStream_t st);
 
 // One query position per sequence in a single launch (attention_decode.hip).
 // The workspace begins with kAttnTicketBytes of tickets that must be zero before

@@ -355,8 +355,8 @@ static mi355x_status step_fast(Model& m) {
     return MI355X_OK;
 }
 
-static int g_llama_rows_off = 0;  // measurement aid: 1 = several sequences take step_fast as one does
-static int g_llama_rows_plain = 0;  // measurement aid: 1 = step_rows with the rotation and SwiGLU as launches of their own
+static std::atomic<int> g_llama_rows_off{0};  // measurement aid: 1 = several sequences take step_fast as one does
+static std::atomic<int> g_llama_rows_plain{0};  // measurement aid: 1 = step_rows with the rotation and SwiGLU as launches of their own
 void set_llama_rows_off(int v) { g_llama_rows_off = v == 1; g_llama_rows_plain = v >= 2 ? v : 0; }
 
 // One decoding step of two to sixty-four sequences with Q4_0 linears (the case of step_fast): the same
@@ -560,7 +560,7 @@ using mimir::Model;
 // How mi355x_llama_generate runs its decoding steps: 0 the fused launches
 // replayed as a graph where the model qualifies, 1 the same launches issued one
 // by one, 2 the general per-operator path.
-static int g_llama_step_mode = 0;
+static std::atomic<int> g_llama_step_mode{0};
 namespace mimir {
 void set_llama_step_mode(int mode) { g_llama_step_mode = mode; }
 }

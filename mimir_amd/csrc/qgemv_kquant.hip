@@ -547,7 +547,7 @@ __global__ __launch_bounds__(kKqThreads) void qgemv_q6k_kernel(const uint8_t* __
 
 // [0] rows per wavefront (0: by shape). [1] 1: always the kernels without LDS, 2: never the
 // matrix-core kernel, 3: the matrix-core kernel for any number of rows.
-static int g_kq_tune[2] = {0, 0};
+static std::atomic<int> g_kq_tune[2] = {{0}, {0}};
 void set_kquant_tune(int which, int value) {
     if (which >= 0 && which < 2) g_kq_tune[which] = value;
 }

@@ -361,11 +361,11 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_kq_rows_kernel(const uint8_
 
 }  // namespace
 
-static int g_kq_rows = 0;  // measurement aid: 1 = never, 2 = for any number of rows the kernel takes
+static std::atomic<int> g_kq_rows{0};  // measurement aid: 1 = never, 2 = for any number of rows the kernel takes
 void set_kquant_rows(int v) { g_kq_rows = v; }
 
-static int g_kq_rows_waves = 0;  // measurement aid: 4 or 8 wavefronts to a workgroup whatever the shape
-static int g_kq_rows_chain = 0;  // measurement aid: 1 = terms in LDS whatever the shape
+static std::atomic<int> g_kq_rows_waves{0};  // measurement aid: 4 or 8 wavefronts to a workgroup whatever the shape
+static std::atomic<int> g_kq_rows_chain{0};  // measurement aid: 1 = terms in LDS whatever the shape
 void set_kquant_rows_waves(int v) {
     if (v == 0) g_kq_rows_chain = g_kq_rows_waves = 0;
     else if (v == 1) g_kq_rows_chain = 1;

@@ -352,7 +352,7 @@ struct Q4Job {
 };
 
 constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
-static int g_q4_batch_off = 0;  // measurement aid: 1 keeps products of several rows of x on the one-row kernel, 2 puts all on the batch kernel
+static std::atomic<int> g_q4_batch_off{0};  // measurement aid: 1 keeps products of several rows of x on the one-row kernel, 2 puts all on the batch kernel
 void set_q4_batch_off(int v) { g_q4_batch_off = v; }
 
 template <int R, int PC, int MODE, int HEAD = kHeadAct>

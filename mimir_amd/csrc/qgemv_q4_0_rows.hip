@@ -683,8 +683,8 @@ hipError_t rows_add_parts(float* x, const float* parts, int shares, int64_t n, h
     return hipGetLastError();
 }
 
-static int g_rows_direct = 0;  // measurement aid: 1 = always the kernel without the LDS pass
-static int g_rows_waves = 0;   // measurement aid: 4 or 8 = that many wavefronts a workgroup, whatever the shape
+static std::atomic<int> g_rows_direct{0};  // measurement aid: 1 = always the kernel without the LDS pass
+static std::atomic<int> g_rows_waves{0};   // measurement aid: 4 or 8 = that many wavefronts a workgroup, whatever the shape
 void set_q4_rows_direct(int v) { g_rows_direct = v; }
 void set_q4_rows_waves(int v) { g_rows_waves = v; }
 

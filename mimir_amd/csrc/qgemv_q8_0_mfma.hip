@@ -186,7 +186,7 @@ bool qgemv_q8_0_mfma_ok(const QGemvArgs& a) {
            a.N > 0 && a.N <= (1ll << 30);
 }
 
-static int g_q8_mfma = 0;  // measurement aid: 1 = wherever the kernel takes the shape, 2 = never
+static std::atomic<int> g_q8_mfma{0};  // measurement aid: 1 = wherever the kernel takes the shape, 2 = never
 void set_q8_mfma(int v) { g_q8_mfma = v; }
 
 bool qgemv_q8_0_mfma_pays(const QGemvArgs& a) {

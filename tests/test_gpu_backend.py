@@ -13,7 +13,7 @@ import oracle as O
 from mimir_amd import capi
 from mimir_amd.backend import (OP_ATTENTION, OP_CAST, OP_GATHER, OP_QMATMUL, Backend, BackendError, Batch, Kernel, View)
 from tests import gpu
-from tests.helpers import bits_equal, check_close, exact_rows, random_blocks
+from tests.helpers import bench_blocks, bits_equal, check_close, exact_rows, random_blocks
 
 pytestmark = pytest.mark.gpu
 
@@ -154,10 +154,91 @@ def test_attention_output_layout(be):
         wo, wl = O.attention(q, kk, vv, 0.125, causal=True, causal_offset=Kn - Q, kv_dt=odt, k_len=Kn)
         check_close(got[: B * H * Q * D], wo, 1e-5, "attention")
         check_close(got[B * H * Q * D:], wl, 1e-5, "logsumexp")
-    with pytest.raises(BackendError) as e:  # a mask is not on this path
-        be.run(Kernel(OP_ATTENTION, capi.F32, [B * H * Q * (D + 1)], [View.contiguous([B, H, Q, D]), kview, kview, View.contiguous([B, H, Q, Kn])]),
-               [out], [qb, kb, vb, f32_buffer(be, np.zeros(B * H * Q * Kn))])
-    assert e.value.code == capi.ERR_INTERNAL
+
+
+def test_attention_mask_value_width_and_no_keys(be):
+    """OpAttention's other inputs (backend/op.go:117-129): the additive mask In[3] [B, H, Q, K], here expanded over
+    the heads with stride 0 and holding -Inf entries; values of another width than the keys; and K = 0, where
+    every row is zeros and -Inf and the key buffers are never read (NewAttentionShape allows it)."""
+    rng = np.random.default_rng(26)
+    B, H, HK, Q, Kn, D, DV = 2, 4, 2, 3, 19, 32, 48
+    q = rng.normal(size=(B, H, Q, D)).astype(np.float32)
+    kf = rng.normal(size=(B, HK, Kn, D)).astype(np.float32); vf = rng.normal(size=(B, HK, Kn, DV)).astype(np.float32)
+    mask = rng.normal(size=(B, 1, Q, Kn)).astype(np.float32)
+    mask[rng.random(mask.shape) < 0.25] = -np.inf
+    mask[1, 0, 2, :] = -np.inf
+    qb, kb, vb, mb = f32_buffer(be, q), f32_buffer(be, kf), f32_buffer(be, vf), f32_buffer(be, mask)
+    out = be.alloc(capi.F32, B * H * Q * (DV + 1))
+    mview = View.contiguous([B, 1, Q, Kn]).expand([B, H, Q, Kn])
+    gpu.say("attention through the backend with a mask and values of another width")
+    be.run(Kernel(OP_ATTENTION, capi.F32, [B * H * Q * (DV + 1)], [View.contiguous([B, H, Q, D]), View.contiguous([B, HK, Kn, D]),
+                                                                    View.contiguous([B, HK, Kn, DV]), mview], scale=0.2, causal=True, causal_offset=Kn - Q),
+           [out], [qb, kb, vb, mb])
+    got = out_f32(be, out)
+    wo, wl = O.attention(q, kf, vf, 0.2, causal=True, causal_offset=Kn - Q, mask=mask)
+    check_close(got[: B * H * Q * DV], wo, 1e-5, "attention")
+    check_close(got[B * H * Q * DV:], wl, 1e-5, "logsumexp")
+    # a mask of the wrong shape, and one that is not float32
+    for bad_view, bad_buf, code in ((View.contiguous([B, H, Q, Kn + 1]), f32_buffer(be, np.zeros(B * H * Q * (Kn + 1))), capi.ERR_SHAPE),):
+        with pytest.raises(BackendError) as e:
+            be.run(Kernel(OP_ATTENTION, capi.F32, [B * H * Q * (DV + 1)], [View.contiguous([B, H, Q, D]), View.contiguous([B, HK, Kn, D]),
+                                                                            View.contiguous([B, HK, Kn, DV]), bad_view]), [out], [qb, kb, vb, bad_buf])
+        assert e.value.code == code
+    # no keys: views [B, HK, 0, D] over buffers of one element
+    empty = be.alloc(capi.F32, 0)
+    out0 = be.alloc(capi.F32, B * H * Q * (D + 1))
+    be.upload(out0, np.full(B * H * Q * (D + 1), np.nan, np.float32))
+    gpu.say("attention through the backend without keys")
+    be.run(Kernel(OP_ATTENTION, capi.F32, [B * H * Q * (D + 1)], [View.contiguous([B, H, Q, D]), View.contiguous([B, HK, 0, D]),
+                                                                   View.contiguous([B, HK, 0, D])], scale=0.2, causal=True), [out0], [qb, empty, empty])
+    got = out_f32(be, out0)
+    assert not got[: B * H * Q * D].any() and np.all(got[B * H * Q * D:] == -np.inf)
+
+
+def test_recorded_batch_survives_scratch_growth(be):
+    """A batch that has become a graph keeps the scratch blocks it was recorded with: calls that outgrow the
+    library's scratch afterwards (activations and attention partials) must leave the graph's replays right."""
+    rng = np.random.default_rng(27)
+    l = gpu.lib()
+    k, n, B, H, HK, D, cap = 1024, 64, 1, 8, 2, 64, 512
+    wraw = bench_blocks(rng, O.Q8_0, n * k)
+    w = be.alloc(capi.Q8_0, n * k); be.upload(w, wraw)
+    x = rng.normal(size=(2, k)).astype(np.float32)
+    q = rng.normal(size=(B, H, 1, D)).astype(np.float32)
+    kf = rng.normal(size=(B, HK, cap, D)).astype(np.float32); vf = rng.normal(size=(B, HK, cap, D)).astype(np.float32)
+    xb, qb, kb, vb = f32_buffer(be, x), f32_buffer(be, q), f32_buffer(be, kf), f32_buffer(be, vf)
+    y = be.alloc(capi.F32, 2 * n); a = be.alloc(capi.F32, B * H * (D + 1))
+    ks = [Kernel(OP_QMATMUL, capi.F32, [2, n], [View.contiguous([2, k]), View.contiguous([n, k])]),
+          Kernel(OP_ATTENTION, capi.F32, [B * H * (D + 1)], [View.contiguous([B, H, 1, D]), View.contiguous([B, HK, cap, D]), View.contiguous([B, HK, cap, D])],
+                 scale=0.125)]
+    batch = Batch(be, ks, [[y], [a]], [[xb, w], [qb, kb, vb]])
+    want_y = O.qmatmul(O.Q8_0, wraw, x, n, k)
+    wo, wl = O.attention(q, kf, vf, 0.125)
+
+    def check(tag):
+        be.upload(y, np.full(2 * n, np.nan, np.float32)); be.upload(a, np.full(B * H * (D + 1), np.nan, np.float32))
+        gpu.say(f"recorded batch, {tag}")
+        be.run_batch(batch)
+        check_close(out_f32(be, y).reshape(2, n), want_y, 1e-4, tag)  # float32 sums of a row's blocks in another order
+        got = out_f32(be, a)
+        check_close(got[: B * H * D], wo, 1e-5, tag); check_close(got[B * H * D:], wl, 1e-5, tag)
+
+    before = be.graph_replays()
+    for it in range(3):
+        check(f"run {it}")
+    assert be.graph_replays() - before == 2
+    # outgrow both blocks on the backend's stream: 2000 rows of converted activations (2.3 MB) and the partials of 256 query rows
+    big_m, big_q = 2000, 256
+    bx = f32_buffer(be, rng.normal(size=(big_m, k)).astype(np.float32)); by = be.alloc(capi.F32, big_m * n)
+    be.run(Kernel(OP_QMATMUL, capi.F32, [big_m, n], [View.contiguous([big_m, k]), View.contiguous([n, k])]), [by], [bx, w])
+    bq = f32_buffer(be, rng.normal(size=(B, H, big_q, D)).astype(np.float32)); bo = be.alloc(capi.F32, B * H * big_q * (D + 1))
+    be.run(Kernel(OP_ATTENTION, capi.F32, [B * H * big_q * (D + 1)], [View.contiguous([B, H, big_q, D]), View.contiguous([B, HK, cap, D]),
+                                                                       View.contiguous([B, HK, cap, D])], scale=0.125), [bo], [bq, kb, vb])
+    be.sync()
+    for it in range(2):
+        check(f"replay {it} after the scratch grew")
+    assert be.graph_replays() - before == 4
+    batch.close()
 
 
 def test_check_run_and_ownership(be):

@@ -23,8 +23,10 @@ ATOL, RTOL = 1e-5, 1e-4
 
 def close(got, want, what=""):
     assert got.shape == want.shape, (got.shape, want.shape)
-    err = np.abs(got.astype(np.float64) - want)
-    assert np.all(err <= ATOL + RTOL * np.abs(want)), f"{what}: worst {err.max():.3e}"
+    inf = np.isinf(want)
+    assert np.array_equal(got[inf], want[inf]), f"{what}: infinities differ"
+    err = np.abs(got[~inf].astype(np.float64) - want[~inf])
+    assert np.all(err <= ATOL + RTOL * np.abs(want[~inf])), f"{what}: worst {err.max():.3e}"
 
 
 @pytest.fixture(scope="module")
@@ -126,22 +128,81 @@ def test_kv_write_casts_like_the_reference():
     assert l.mi355x_kv_write(sd.data_ptr(), cache.data_ptr(), capi.F32, B, KVH, S, D, cap, cap - 2, KVH * S * D, S * D, D, gpu.stream()) == capi.ERR_SHAPE
 
 
-def attention(q, k, v, scale, causal=False, offset=0, kv_dt=capi.F32, k_len=None, want_lse=True):
-    """q [B,H,Q,D], k/v [B,HK,cap,D] contiguous numpy (uint16 bits for F16)."""
+def attention(q, k, v, scale, causal=False, offset=0, kv_dt=capi.F32, k_len=None, want_lse=True, mask=None):
+    """q [B,H,Q,D], k [B,HK,cap,D] and v [B,HK,cap,DV] contiguous numpy (uint16 bits for F16); mask broadcastable
+    to [B,H,Q,K] (dimensions of size 1 are read with stride 0)."""
     l = gpu.lib()
     B, H, Q, D = q.shape
-    HK, cap = k.shape[1], k.shape[2]
+    HK, cap, DV = k.shape[1], k.shape[2], v.shape[3]
     K = cap if k_len is None else k_len
     qd = gpu.dev(q)
     kd = gpu.dev(k.view(np.int16) if kv_dt == capi.F16 else k); vd = gpu.dev(v.view(np.int16) if kv_dt == capi.F16 else v)
-    out = torch.full((B, H, Q, D), float("nan"), dtype=torch.float32, device="cuda:0")
+    out = torch.full((B, H, Q, DV), float("nan"), dtype=torch.float32, device="cuda:0")
     lse = torch.full((B, H, Q), float("nan"), dtype=torch.float32, device="cuda:0")
-    arr = lambda *a: (C.c_int64 * 3)(*a)
-    capi.check(l.mi355x_attention(qd.data_ptr(), arr(H * Q * D, Q * D, D), kd.data_ptr(), vd.data_ptr(), kv_dt, arr(HK * cap * D, cap * D, D),
-                                  out.data_ptr(), arr(H * Q * D, Q * D, D), lse.data_ptr() if want_lse else None, B, H, HK, Q, K, D,
+    arr = lambda *a: (C.c_int64 * len(a))(*a)
+    md, ms = None, None
+    if mask is not None:
+        m4 = np.ascontiguousarray(mask, np.float32).reshape((1,) * (4 - np.ndim(mask)) + np.shape(mask))
+        md = gpu.dev(m4)
+        ms = arr(*[0 if m4.shape[i] == 1 else int(np.prod(m4.shape[i + 1:])) for i in range(4)])
+    capi.check(l.mi355x_attention(qd.data_ptr(), arr(H * Q * D, Q * D, D), kd.data_ptr(), arr(HK * cap * D, cap * D, D), vd.data_ptr(),
+                                  arr(HK * cap * DV, cap * DV, DV), kv_dt, md.data_ptr() if md is not None else None, ms,
+                                  out.data_ptr(), arr(H * Q * DV, Q * DV, DV), lse.data_ptr() if want_lse else None, B, H, HK, Q, K, D, DV,
                                   scale, int(causal), offset, gpu.stream()))
     gpu.sync()
     return out.cpu().numpy(), lse.cpu().numpy()
+
+
+def test_attention_golden_mask(cases):
+    """The reference's masked case (nn/transformer_test.go:36-38): an additive float mask as In[3]."""
+    c = cases["sdpa_mask"]
+    q, k, v, mask = (t.data for t in c["in"][:4])
+    gpu.say(f"sdpa_mask q={q.shape} mask={mask.shape}")
+    out, lse = attention(q, k, v, 1 / np.sqrt(q.shape[-1]), mask=mask)
+    close(out, c["out"].data, "sdpa_mask")
+    _, wl = O.attention(q, k, v, 1 / np.sqrt(q.shape[-1]), mask=mask)
+    close(lse, wl, "sdpa_mask lse")
+
+
+@pytest.mark.parametrize("B,H,HK,Q,K,D,DV", [(2, 4, 2, 5, 37, 16, 24), (1, 8, 2, 1, 300, 64, 128), (1, 3, 1, 7, 70, 128, 8), (2, 32, 8, 1, 129, 128, 128)])
+def test_attention_mask_and_value_width(B, H, HK, Q, K, D, DV):
+    """Values of another width than the keys, and an additive mask with -Inf entries (whole rows among them),
+    per head, broadcast over heads, and broadcast over batch and heads; with and without causality."""
+    rng = np.random.default_rng(B * 100 + K)
+    q = rng.normal(size=(B, H, Q, D)).astype(np.float32)
+    k = rng.normal(size=(B, HK, K, D)).astype(np.float32); v = rng.normal(size=(B, HK, K, DV)).astype(np.float32)
+    scale = 1 / np.sqrt(D)
+    full = rng.normal(size=(B, H, Q, K)).astype(np.float32)
+    full[rng.random(full.shape) < 0.3] = -np.inf
+    full[0, 0, 0, :] = -np.inf  # a row that sees nothing: zeros and -Inf
+    for name, mask in (("none", None), ("full", full), ("heads", full[:, :1]), ("rows", full[:1, :1])):
+        for causal, off in ((False, 0), (True, K - Q)):
+            gpu.say(f"attention B={B} H={H} HK={HK} Q={Q} K={K} D={D} DV={DV} mask={name} causal={causal}")
+            out, lse = attention(q, k, v, scale, causal=causal, offset=off, mask=mask)
+            wo, wl = O.attention(q, k, v, scale, causal=causal, causal_offset=off, mask=mask)
+            close(out, wo, name); close(lse, wl, name + " lse")
+    assert np.all(out[0, 0, 0] == 0) and lse[0, 0, 0] == -np.inf
+
+
+@pytest.mark.parametrize("B,H,HK,Q,D", [(1, 32, 8, 1, 128), (2, 4, 2, 3, 16)])
+def test_attention_without_keys(B, H, HK, Q, D):
+    """K = 0 (NewAttentionShape allows it, backend/attention.go:36-62): zeros and a logsumexp of -Inf, with
+    allocated key buffers and with none at all."""
+    l = gpu.lib()
+    rng = np.random.default_rng(9)
+    qd = gpu.dev(rng.normal(size=(B, H, Q, D)).astype(np.float32))
+    kd = torch.zeros(4, dtype=torch.float32, device="cuda:0")
+    arr = lambda *a: (C.c_int64 * len(a))(*a)
+    for kv in (kd.data_ptr(), None):
+        for kv_dt in (capi.F32, capi.F16):
+            out = torch.full((B, H, Q, D), float("nan"), dtype=torch.float32, device="cuda:0")
+            lse = torch.full((B, H, Q), float("nan"), dtype=torch.float32, device="cuda:0")
+            gpu.say(f"attention without keys B={B} H={H} Q={Q} D={D} kv={'set' if kv else 'null'} dt={kv_dt}")
+            capi.check(l.mi355x_attention(qd.data_ptr(), arr(H * Q * D, Q * D, D), kv, arr(0, 0, D) if kv else None, kv, arr(0, 0, D) if kv else None,
+                                          kv_dt, None, None, out.data_ptr(), arr(H * Q * D, Q * D, D), lse.data_ptr(), B, H, HK, Q, 0, D, D,
+                                          1 / np.sqrt(D), 1, 0, gpu.stream()))
+            gpu.sync()
+            assert not out.cpu().numpy().any() and np.all(lse.cpu().numpy() == -np.inf)
 
 
 @pytest.mark.parametrize("name,kw", [

@@ -167,9 +167,7 @@ def test_random_init_q4_0_model_matches_oracle_and_greedy_tokens(batch):
         want, margins = om.generate(prompts[b].tolist(), 24, capacity=c.context, cache_dtype=O.F16)
         scale = 170.0
         for i, (a, w) in enumerate(zip(toks[b].tolist(), want)):
-            if a != w:
-                assert margins[i] < 0.02 * scale, (b, i, a, w, margins[i])
-                break  # the sequences part here by construction
+            assert a == w, f"token {i}: device {a}, oracle {w}, oracle's margin there {margins[i]:.4g}"
 
 
 @pytest.mark.parametrize("batch,cache", [(1, capi.F32), (2, capi.F16)])
@@ -207,9 +205,7 @@ def test_fused_and_graph_replayed_steps_choose_the_per_operator_tokens(batch, ca
     want, margins = om.generate(prompts[0].tolist(), 30, capacity=c.context, cache_dtype=O.F32 if cache == capi.F32 else O.F16)
     got = runs[2][0][0, :30].tolist()
     for i, (a, w) in enumerate(zip(got, want)):
-        if a != w:
-            assert margins[i] < 1e-3 * 170.0, (i, a, w, margins[i])
-            break
+        assert a == w, f"token {i}: device {a}, oracle {w}, oracle's margin there {margins[i]:.4g}"
     # attention splits the keys differently when the position comes from the
     # device (a fixed plan for the whole context), so a sum may round another
     # way; tokens differ only if two logits tie to that precision
@@ -254,9 +250,7 @@ def test_batch_step_that_reads_weights_once_chooses_the_same_tokens(batch):
     for b in range(batch):
         want, margins = om.generate(prompts[b].tolist(), 30, capacity=c.context, cache_dtype=O.F16)
         for i, (a, w) in enumerate(zip(runs["rows graph"][b, :30].tolist(), want)):
-            if a != w:
-                assert margins[i] < 1e-3 * 170.0, (b, i, a, w, margins[i])
-                break
+            assert a == w, f"token {i}: device {a}, oracle {w}, oracle's margin there {margins[i]:.4g}"
 
 
 def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
@@ -287,9 +281,7 @@ def test_fused_steps_without_their_riders_choose_the_per_operator_tokens():
         capi.check(lib.mi355x_tune(b"llama.step", 0))
     want, margins = om.generate(prompts[0].tolist(), 20, capacity=c.context, cache_dtype=O.F16)
     for i, (a, w) in enumerate(zip(runs[2][0].tolist(), want)):
-        if a != w:
-            assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
-            break
+        assert a == w, f"token {i}: device {a}, oracle {w}, oracle's margin there {margins[i]:.4g}"
     assert np.array_equal(runs[1], runs[2]) and np.array_equal(runs[0], runs[2])
 
 
@@ -326,7 +318,5 @@ def test_k_quant_and_q8_0_models_decode_from_a_graph(linear_dt, batch, heads, he
         capi.check(lib.mi355x_tune(b"llama.step", 0))
     want, margins = om.generate(prompts[0].tolist(), 20, capacity=c.context, cache_dtype=O.F16)
     for i, (a, w) in enumerate(zip(runs[2][0][0, :20].tolist(), want)):
-        if a != w:
-            assert margins[i] < 0.02 * 170.0, (i, a, w, margins[i])
-            break
+        assert a == w, f"token {i}: device {a}, oracle {w}, oracle's margin there {margins[i]:.4g}"
     assert np.array_equal(runs[1][0], runs[2][0]) and np.array_equal(runs[0][0], runs[2][0]) and np.array_equal(runs[0][1], runs[2][0])

@@ -168,6 +168,31 @@ def test_prefill_shapes(n):
         assert np.array_equal(got4[:512], got) and np.array_equal(got4[512:1024], got[::-1]) and np.array_equal(got4[1024:1536], got)
 
 
+def test_prefill_shape_2048_by_14336():
+    """The shape the prompt-sized product's figures are quoted on: M = 2048 tokens by N = 14336, K = 4096,
+    weights and activations as the configurations draw them. The oracle takes two bands of 256 output columns,
+    one of them across a tile boundary of every tile height, over all 2048 rows; the exact form (float32 sums and
+    their bfloat16 rounding) and the form with weights rounded to binary16."""
+    rng = np.random.default_rng(3)
+    m, n, k = 2048, 14336, 4096
+    w = bench_blocks(rng, O.Q4_0, n * k)
+    x = bf16_bits(rng.normal(size=(m, k)))
+    gpu.say("qgemm_bf16 2048x4096 by 14336x4096")
+    got = qgemm(w, x, n, k)
+    got32 = qgemm(w, x, n, k, capi.F32)
+    with binary16_weights():
+        gpu.say("qgemm_bf16 2048x4096 by 14336x4096, binary16 weights")
+        half32 = qgemm(w, x, n, k, capi.F32)
+    for lo in (0, 9088 - 128):
+        hi = lo + 256
+        wb = w.reshape(n, -1)[lo:hi].reshape(-1)
+        want_f32 = reference_f32(wb, x, hi - lo, k)
+        err = np.abs(got32[:, lo:hi] - want_f32)
+        assert np.all(err <= 1e-4 * np.maximum(1, np.abs(want_f32))), (lo, float(err.max()))
+        check_bf16(got[:, lo:hi], O.q4_0_matmul_bf16(wb, x, hi - lo, k), 1e-4 * np.maximum(1, np.abs(want_f32)))
+        check_binary16_form(wb, x, hi - lo, k, half32[:, lo:hi])
+
+
 def test_tall_tiles():
     """M = 2048 by N = 6144 takes the 256-row tiles: a band of columns against
     the oracle, and ragged edges (M = 2000, N = 6100) against the same rows and

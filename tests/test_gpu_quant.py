@@ -153,6 +153,63 @@ def test_q4_0_fixed_point_kernel_special_values():
     assert np.isnan(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)).all()
 
 
+@pytest.mark.parametrize("m", [1, 8, 64])
+def test_q4_0_fixed_point_outliers_inside_a_block(m):
+    """The fixed-point kernels keep 24 bits per block of 32 activations, not per element: an element
+    10^6 times its neighbours takes the block's scale, and the neighbours keep what is left of the 24 bits.
+    The error per element is at most 2^-23 of the block's largest magnitude (half a unit of a grid of 7829367
+    steps, and the rounding of the scaling), so the result is within 2^-23 * sum_b amax_b * sum_{e in b} |w_e| of the float32 product's exact
+    value, whatever the weights are. Three cases a float32 product would keep exactly and this one cannot:
+    the outlier's own weight is zero (nibble 8), so that only the neighbours count; every other weight is
+    zero, so that only the outlier counts; and random weights. Each is held to that bound plus the float32
+    product's own 2e-6 * sum |x| |w|, and to the conformance rule tol * max(1, |want|) with tol 1e-3 where
+    the bound itself is inside it. One row of x (v_dot8), eight (int8 matrix cores, W read once) and 64
+    (the tiled kernel)."""
+    rng = np.random.default_rng(31 + m)
+    n, k = 64, 4096
+    nb = k // 32
+    base = bench_blocks(rng, O.Q4_0, n * k).reshape(n, nb, 18)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    pos = rng.integers(0, 32, nb)  # the outlier's place in each block
+    x.reshape(m, nb, 32)[:, np.arange(nb), pos] *= np.float32(1e6)
+
+    def with_nibbles(blocks, e, value):
+        """Sets the nibble of element e[b] of block b of every row to value."""
+        out = blocks.copy()
+        for b in range(nb):
+            byte, high = 2 + (e[b] % 16), e[b] >= 16
+            col = out[:, b, byte]
+            out[:, b, byte] = (col & 0x0f) | (value << 4) if high else (col & 0xf0) | value
+        return out
+
+    zeros = np.full((n, nb, 18), 0x88, np.uint8); zeros[:, :, :2] = base[:, :, :2]  # every weight (8 - 8) * d
+    only = zeros.copy()
+    for b in range(nb):  # only the outlier's weight is not zero
+        byte, high = 2 + (pos[b] % 16), pos[b] >= 16
+        only[:, b, byte] = base[:, b, byte] & (0xf0 if high else 0x0f) | (0x08 if high else 0x80)
+    cases = {"outlier's weight zero": with_nibbles(base, pos, 8), "only the outlier's weight": only, "random weights": base}
+    for name, blocks in cases.items():
+        raw = blocks.reshape(-1)
+        buf, ptr = gpu.dev_bytes_at(raw, 0)
+        gpu.say(f"q4_0 fixed-point outliers in every block, m={m}: {name}")
+        got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+        want = O.qmatmul(O.Q4_0, raw, x, n, k)
+        wf = np.abs(O.dequantize(O.Q4_0, raw).reshape(n, nb, 32).astype(np.float64))
+        amax = np.abs(x.reshape(m, nb, 32)).max(2).astype(np.float64)                        # [m, nb]
+        fixed = 2.0 ** -23 * np.einsum("mb,nb->mn", amax, wf.sum(2))                         # the fixed-point grid
+        f32 = 2e-6 * np.einsum("mbe,nbe->mn", np.abs(x.reshape(m, nb, 32)).astype(np.float64), wf)  # float32 sums in two orders
+        err = np.abs(got.astype(np.float64) - want)
+        assert np.all(err <= fixed + f32 + 1e-30), (name, float((err / (fixed + f32 + 1e-30)).max()))
+        inside = fixed + f32 <= 1e-3 * np.maximum(1, np.abs(want))
+        assert np.all(err[inside] <= 1e-3 * np.maximum(1, np.abs(want[inside]))), name
+        if name == "only the outlier's weight":  # the outliers are exact in 24 bits: nothing is lost at all beyond float32's sums
+            assert np.all(err <= f32 + 1e-30), float((err / (f32 + 1e-30)).max())
+        if name == "outlier's weight zero":
+            # what a float32 product keeps and this one loses: the neighbours' low bits, at most the bound above,
+            # which here is about 1e-1 of the result (the neighbours are 1e-6 of their block's scale)
+            print(f"[outliers m={m}] worst error {err.max():.3e}, bound {float((fixed + f32).max()):.3e}, largest |want| {np.abs(want).max():.3e}")
+
+
 def test_q4_0_gemv_without_lds_staging():
     rng = np.random.default_rng(6)
     n, k = 64, 4096
