@@ -23,7 +23,7 @@
  *    refuses while the stream is being captured: run a call once at its
  *    largest size before recording it into a graph (the block a graph was
  *    recorded with is never freed, so the graph stays valid however the
- *    scratch grows afterwards).
+ *    scratch grows afterwards), or use mi355x_qgemv_noalloc.
  *  - dtype codes are the reference's DType enumeration
  *    (backend/backend.go:72-90) with Q4_0 appended.
  *  - Block-quantized buffers hold ggml's block layout unchanged
@@ -104,6 +104,19 @@ MI355X_API mi355x_status mi355x_sync(void* stream);
  * among its row kernels, Q4_K, Q6_K). */
 MI355X_API mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream);
+
+/* mi355x_qgemv for callers that cannot allocate device memory: code under HIP
+ * graph capture, serving loops and harnesses that forbid hipMalloc. It has no
+ * counterpart in the reference. Same arguments, kernels and results as
+ * mi355x_qgemv, but the converted activations go to a fixed block of 1 MiB inside
+ * the library's code object instead of a scratch buffer that grows, and nothing
+ * is allocated or freed: mi355x_init must have run on the device, and a product
+ * whose converted activations exceed the block (M * mi355x_act_bytes(dtype, K),
+ * for Q4_0 rounded up to groups of eight rows where W is read once per eight)
+ * fails with MI355X_ERR_SHAPE. Every call on a device uses that device's one
+ * block: calls that overlap on one device (two streams) race on it. */
+MI355X_API mi355x_status mi355x_qgemv_noalloc(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
+                                   int64_t x_row_stride, void* stream);
 
 /* The product in two steps, for callers that multiply one x by several
  * matrices (q, k and v; gate and up). mi355x_convert_act turns each row of x

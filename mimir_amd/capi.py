@@ -32,6 +32,7 @@ SYMBOLS = {
     "mi355x_download": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "mi355x_sync": (C.c_uint32, [_vp]),
     "mi355x_qgemv": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "mi355x_qgemv_noalloc": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mi355x_act_bytes": (_sz, [_int, _i64]),
     "mi355x_convert_act": (C.c_uint32, [_int, _vp, _i64, _i64, _i64, _vp, _vp]),
     "mi355x_qgemv_act": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),

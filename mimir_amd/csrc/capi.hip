@@ -41,6 +41,13 @@ mi355x_status hip_fail(hipError_t e, const char* what) {
 
 constexpr int kMaxDevices = 16;
 
+// The converted activations of mi355x_qgemv_noalloc: a fixed block in the code object's own
+// device memory, so that the entry point allocates nothing. Every device the library runs on
+// holds its own copy at its own address (DeviceState::fixed, looked up when the device's state
+// is created); in host code the array's name is only a handle for that lookup, never an address.
+constexpr size_t kNoallocScratchBytes = (size_t)1 << 20;
+static __device__ __align__(256) unsigned char g_noalloc_scratch[kNoallocScratchBytes];
+
 // Scratch memory of the entry points that need some beyond their arguments (converted activations,
 // partial results and tickets of split attention and argmax, float32 copies of qgemm_bf16's general
 // route). One set per device and stream: calls on different streams never share a block, calls on one
@@ -63,6 +70,7 @@ struct DeviceState {
     uint32_t* err_host = nullptr;  // pinned
     std::map<void*, StreamScratch> scratch;  // by stream handle
     std::vector<void*> retired;              // outgrown blocks, kept until the process ends
+    void* fixed = nullptr;                   // this device's copy of g_fixed_scratch
 };
 
 std::mutex g_mu;
@@ -116,6 +124,7 @@ mi355x_status current_state(DeviceState** out) {
         HIP_TRY(hipMalloc((void**)&s.err_dev, 256), "hipMalloc(error word)");
         HIP_TRY(hipMemset(s.err_dev, 0, 256), "hipMemset(error word)");
         HIP_TRY(hipHostMalloc((void**)&s.err_host, 256, hipHostMallocDefault), "hipHostMalloc(error word)");
+        HIP_TRY(hipGetSymbolAddress(&s.fixed, HIP_SYMBOL(g_noalloc_scratch)), "hipGetSymbolAddress(fixed scratch)");
         s.ready = true;
     }
     *out = &s;
@@ -454,6 +463,21 @@ static mi355x_status qgemv_impl(int dtype, const void* W, const float* x, float*
 mi355x_status mi355x_qgemv(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
                            int64_t x_row_stride, void* stream) {
     return qgemv_impl(dtype, W, x, y, M, N, K, x_row_stride, stream, ActSource{stream, nullptr, 0});
+}
+
+// mi355x_qgemv without an allocation: the device's state must exist already (mi355x_init), and the
+// converted activations go to the device's fixed block.
+mi355x_status mi355x_qgemv_noalloc(int dtype, const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K,
+                                   int64_t x_row_stride, void* stream) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+    void* fixed = nullptr;
+    if (dev >= 0 && dev < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_mu);
+        if (g_dev[dev].ready) fixed = g_dev[dev].fixed;
+    }
+    if (!fixed) return fail(MI355X_ERR_INTERNAL, "mi355x: qgemv_noalloc: call mi355x_init(%d) first (creating the device's state allocates)", dev);
+    return qgemv_impl(dtype, W, x, y, M, N, K, x_row_stride, stream, ActSource{stream, fixed, kNoallocScratchBytes});
 }
 
 size_t mi355x_act_bytes(int dtype, int64_t K) {
