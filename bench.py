@@ -468,6 +468,8 @@ def main():
     ap.add_argument("--decode-batch", type=int, default=1)
     ap.add_argument("--decode-linear", choices=("q4_0", "q4_K", "q6_K"), default="q4_0",
                     help="block dtype of the decoder's linear weights (the oracle check is for q4_0)")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="a launch-plan override for mi355x_tune before anything runs (may be repeated), e.g. q4_0.stream=1")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives or sharding are built)")
@@ -478,6 +480,9 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible")
     capi.check(lib.mi355x_init(0))
+    for kv in args.tune:
+        key, _, val = kv.partition("=")
+        capi.check(lib.mi355x_tune(key.encode(), int(val)))
 
     if args.rows_counters:
         rows_bench(lib, capi, torch, shapes=((14336, 4096),), only=args.rows_counters)
@@ -521,7 +526,7 @@ def main():
                    "N": n, "K": k, "M": 1, "wall_ms_per_step": round(step_wall_ms, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "qgemv_q4_0_i4_kernel<4, 1, 0, 2>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
+                     "kernel": "qgemv_q4_0_stream_kernel<0, 2, 4>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
                      "us_min": round(kern_min, 3), "us_max": round(kern_max, 3),
                      # the product over activations converted beforehand (as a decoding step's launches take them),
                      # back to back in a graph, the wait between dependent kernels included

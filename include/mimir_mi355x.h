@@ -315,6 +315,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * Overrides the launch plan of mi355x_qgemv for sweeps: key is one of
  * "q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path" (1 forces
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
+ * "q4_0.stream" = 1 keeps Q4_0 products of one to four rows of x off the kernel
+ * that runs one workgroup per compute unit (the older, finer-grained launch shape
+ * then takes them).
  * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
  * kernel, 2 puts them all on the kernel that shares W among rows of x.
  * "q4_0.rows_path" = 1 keeps Q4_0 and Q8_0 products of a few rows of x off the
@@ -358,6 +361,12 @@ MI355X_API mi355x_status mi355x_tune(const char* key, int value);
  * for the device and writes the milliseconds of each launch, in order. */
 MI355X_API mi355x_status mi355x_timed_begin(int max_launches);
 MI355X_API mi355x_status mi355x_timed_end(float* ms_each, int* n_launches);
+/* While stamps is not NULL, every launch of the whole-chip Q4_0 decode kernel (one to four rows of x by a Q4_0
+ * matrix) writes five int64 readings of the device's 100 MHz clock per workgroup to stamps[5 * workgroup ..]: at
+ * entry, once x is staged in LDS, after its first row of W, after its last, and at exit. The caller provides
+ * 40 bytes per workgroup of the largest launch (at most two workgroups per compute unit) and reads them back
+ * after the launch; NULL stops it. Process-wide. */
+MI355X_API mi355x_status mi355x_gemv_stamps(void* stamps);
 /* Reads `bytes` bytes at p with 128-bit loads from `grid` workgroups of
  * `threads` threads and folds them into scratch (at least grid*threads/64
  * floats): the practical ceiling of a streaming read on this device. */

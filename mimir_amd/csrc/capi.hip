@@ -757,6 +757,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
         mimir::set_q4_rows_waves(value);
         return MI355X_OK;
     }
+    if (key && strcmp(key, "q4_0.stream") == 0) {  // 1: off
+        mimir::set_q4_stream_off(value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "q4_0.batch_off") == 0) {
         mimir::set_q4_batch_off(value);
         return MI355X_OK;
@@ -800,6 +804,13 @@ mi355x_status mi355x_timed_end(float* ms_each, int* n_launches) {
     t_events_used = 0;
     *n_launches = (int)n;
     HIP_TRY(e, "timed_end");
+    return MI355X_OK;
+}
+
+// Where the launches of the Q4_0 product's whole-chip kernel leave five timestamps per workgroup
+// (qgemv_q4_0_stream.hip), or null to stop.
+mi355x_status mi355x_gemv_stamps(void* stamps) {
+    mimir::set_q4_stream_stamps((long long*)stamps);
     return MI355X_OK;
 }
 

@@ -64,6 +64,13 @@ struct Q4NormHead {
 };
 bool q4_0_norm_head_ok(int64_t K);
 void set_q4_batch_off(int v);  // 1: products of several rows of x stay on the one-row kernel
+// The same products on the kernel shaped for the whole chip (qgemv_q4_0_stream.hip): one to four rows of x, a
+// workgroup per compute unit, x kept in registers. Returns false where it does not take the shape (the caller then
+// launches qgemv_q4_0_i4_kernel); otherwise *err is the launch's status. mode: a Q4Mode.
+struct Q4Job;
+bool q4_0_stream_dispatch(int mode, const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st, hipError_t* err);
+void set_q4_stream_off(int v);             // measurement aid: 1 keeps every product off that kernel
+void set_q4_stream_stamps(long long* p);   // measurement aid: device memory for five timestamps per workgroup of its launches (null: none)
 bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
                                          int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st);

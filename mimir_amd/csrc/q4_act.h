@@ -25,24 +25,43 @@ __host__ __device__ inline size_t q4_0_act_row_bytes(int64_t K) {
 
 // The eight values a thread holds (elements 4i..4i+3 and 16+4i..16+4i+3 of a
 // block) to kDigits dwords of digits. Z = (X + kFixBias) ^ kFixBias has the
-// two's-complement balanced digit j of X in nibble j.
+// two's-complement balanced digit j of X in nibble j, so byte m of Z holds digits
+// 2m and 2m+1; dword j of the result wants digit j of the value at position p in
+// nibble p (positions 0, 2, 4, 6: lo[0..3]; 1, 3, 5, 7: hi[0..3]). Bytes m of the
+// four lo values are gathered into one dword and those of the four hi values into
+// another (a 4 x 4 byte transposition: seven v_perm_b32 each), then two
+// dwords of digits come out of each such pair by masks and shifts.
 __device__ __forceinline__ void fix_digits(const float lo[4], const float hi[4], float inv, uint32_t out[kDigits]) {
-    uint32_t z[8];
+    uint32_t ze[4], zo[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         // x * inv may round half a unit past kFixMax for the block's largest value: clamp
         int a = (int)__builtin_rintf(lo[k] * inv), b = (int)__builtin_rintf(hi[k] * inv);
         a = a > kFixMax ? kFixMax : a < -kFixMax ? -kFixMax : a;
         b = b > kFixMax ? kFixMax : b < -kFixMax ? -kFixMax : b;
-        z[2 * k] = ((uint32_t)(a + (int)kFixBias)) ^ kFixBias;      // nibble position 2k
-        z[2 * k + 1] = ((uint32_t)(b + (int)kFixBias)) ^ kFixBias;  // nibble position 2k+1
+        ze[k] = ((uint32_t)(a + (int)kFixBias)) ^ kFixBias;  // nibble position 2k
+        zo[k] = ((uint32_t)(b + (int)kFixBias)) ^ kFixBias;  // nibble position 2k+1
+    }
+    // v_perm_b32(s0, s1, sel): result byte i is byte sel.byte[i] of the eight bytes {s1 (0..3), s0 (4..7)}
+    uint32_t e[3], o[3];
+    {
+        const uint32_t t01l = __builtin_amdgcn_perm(ze[1], ze[0], 0x05010400u), t01h = __builtin_amdgcn_perm(ze[1], ze[0], 0x07030602u);
+        const uint32_t t23l = __builtin_amdgcn_perm(ze[3], ze[2], 0x05010400u), t23h = __builtin_amdgcn_perm(ze[3], ze[2], 0x07030602u);
+        e[0] = __builtin_amdgcn_perm(t23l, t01l, 0x05040100u);
+        e[1] = __builtin_amdgcn_perm(t23l, t01l, 0x07060302u);
+        e[2] = __builtin_amdgcn_perm(t23h, t01h, 0x05040100u);
+    }
+    {
+        const uint32_t t01l = __builtin_amdgcn_perm(zo[1], zo[0], 0x05010400u), t01h = __builtin_amdgcn_perm(zo[1], zo[0], 0x07030602u);
+        const uint32_t t23l = __builtin_amdgcn_perm(zo[3], zo[2], 0x05010400u), t23h = __builtin_amdgcn_perm(zo[3], zo[2], 0x07030602u);
+        o[0] = __builtin_amdgcn_perm(t23l, t01l, 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(t23l, t01l, 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(t23h, t01h, 0x05040100u);
     }
 #pragma unroll
-    for (int j = 0; j < kDigits; j++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int p = 0; p < 8; p++) w |= ((z[p] >> (4 * j)) & 15u) << (4 * p);
-        out[j] = w;
+    for (int m = 0; m < 3; m++) {
+        out[2 * m] = (e[m] & 0x0F0F0F0Fu) | ((o[m] << 4) & 0xF0F0F0F0u);
+        out[2 * m + 1] = ((e[m] >> 4) & 0x0F0F0F0Fu) | (o[m] & 0xF0F0F0F0u);
     }
 }
 
@@ -52,21 +71,25 @@ __device__ __forceinline__ void fix_digits(const float lo[4], const float hi[4],
 // of a block must sit in four consecutive lanes, all active: the block's
 // largest magnitude is a quad reduction.
 __device__ __forceinline__ void q4_convert_item(float lo[4], float hi[4], u32x4* plane, float* xscale, int nbp, int b, int d) {
-    float amax = 0.f;
-    bool finite = true;
+    // The largest magnitude as the largest bit pattern without its sign: the order of non-negative floats is that of
+    // their bits, and every infinity or NaN lies above every finite value, so one maximum says both how large the block
+    // is and whether all of it is finite.
+    uint32_t top = 0;
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        float a0 = __builtin_fabsf(lo[k]), a1 = __builtin_fabsf(hi[k]);
-        finite = finite && a0 < __builtin_inff() && a1 < __builtin_inff();  // false for NaN too
-        amax = fmaxf(amax, fmaxf(a0, a1));
+        const uint32_t a0 = __builtin_bit_cast(uint32_t, lo[k]) & 0x7fffffffu, a1 = __builtin_bit_cast(uint32_t, hi[k]) & 0x7fffffffu;
+        top = top > a0 ? top : a0;
+        top = top > a1 ? top : a1;
     }
-    amax = fmaxf(amax, dpp_f32<0xb1>(amax));
-    amax = fmaxf(amax, dpp_f32<0x4e>(amax));
-    float bad = finite ? 0.f : 1.f;
-    bad = fmaxf(bad, dpp_f32<0xb1>(bad));
-    bad = fmaxf(bad, dpp_f32<0x4e>(bad));
+    {
+        const uint32_t t1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)top, 0xb1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+        top = top > t1 ? top : t1;
+        const uint32_t t2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)top, 0x4e, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+        top = top > t2 ? top : t2;
+    }
+    const float amax = __builtin_bit_cast(float, top);
     float scale, inv;
-    if (bad != 0.f) {  // a NaN or an infinity in the block: its products are NaN
+    if (top >= 0x7f800000u) {  // a NaN or an infinity in the block: its products are NaN
         scale = __builtin_nanf("");
         inv = 0.f;
 #pragma unroll

@@ -34,6 +34,7 @@
 #include "device_util.h"
 #include "kernels.h"
 #include "q4_act.h"
+#include "q4_job.h"
 #include "rope_tail.h"
 
 namespace mimir {
@@ -252,9 +253,6 @@ __global__ __launch_bounds__(256) void q4_0_convert_act_kernel(const float* __re
     }
 }
 
-// A 128-bit load that is only dword aligned (gfx950 serves it at full rate).
-typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
-
 hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
     int nb = (int)(K / 32);
     int gx = (nb * 4 + 255) / 256;
@@ -263,95 +261,6 @@ hipError_t q4_0_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_
     return hipGetLastError();
 }
 
-template <int RR, int PC>
-struct Q4PairTile {
-    u32x4 a[RR][PC], b[RR][PC];
-    uint32_t c[RR][PC];
-};
-
-// Lane `lane` owns blocks 2p, 2p+1 with p = lane + 64 * pc of each row: nine
-// aligned dwords. Plain (cached) loads: the three touch the same cache lines,
-// which must stay cached between them.
-template <int RR, int PC>
-__device__ __forceinline__ void q4_load_pairs(Q4PairTile<RR, PC>& t, const uint8_t* const rowp[RR], int npairs, int pc0, int lane) {
-#pragma unroll
-    for (int pc = 0; pc < PC; pc++) {
-        int p = lane + 64 * (pc0 + pc);
-        p = p < npairs ? p : npairs - 1;
-#pragma unroll
-        for (int r = 0; r < RR; r++) {
-            const uint32_t* src = (const uint32_t*)rowp[r] + p * 9;
-            t.a[r][pc] = *(const u32x4_a4*)src;
-            t.b[r][pc] = *(const u32x4_a4*)(src + 4);
-            t.c[r][pc] = src[8];
-        }
-    }
-}
-
-// For the two blocks of a pair: sum over the block of (n - 8) * X, X the
-// fixed-point activations. Digit planes run from the most significant down,
-// each four v_dot8 accumulating on sixteen times the sum so far; the two
-// blocks' chains are independent and interleaved so that neither waits on
-// its own previous result.
-__device__ __forceinline__ void q4_pair_dot(const uint32_t q0[4], const uint32_t q1[4], const u32x4 d0[kDigits],
-                                            const u32x4 d1[kDigits], int& out0, int& out1) {
-    int w0[4], w1[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        w0[i] = (int)(q0[i] ^ 0x88888888u);
-        w1[i] = (int)(q1[i] ^ 0x88888888u);
-    }
-    int t0 = 0, t1 = 0;
-#pragma unroll
-    for (int j = kDigits - 1; j >= 0; j--) {
-        t0 *= 16;
-        t1 *= 16;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            t0 = __builtin_amdgcn_sdot8(w0[i], (int)d0[j][i], t0, false);
-            t1 = __builtin_amdgcn_sdot8(w1[i], (int)d1[j][i], t1, false);
-        }
-    }
-    out0 = t0;  // |t| <= 32 * 8 * 7829367 < 2^31
-    out1 = t1;
-}
-
-// What one launch of the fixed-point kernel computes, for each row m of x:
-//   kPlain    y[m, :] = x[m, :] . W0^T (+ resid[m, :])
-//   kMulti    y[m, :] = x[m, :] . [W0; W1; W2]^T: up to three matrices that share
-//             K, their rows concatenated (queries, keys and values of a block)
-//   kSwiGLU   y[m, r] = SiLU(x[m, :] . W0[r]) * (x[m, :] . W1[r]): gate and up
-//             of a SwiGLU feed-forward (llm/model.go:446-448), the activation
-//             applied as tensor/elementwise.go:520-525,583-585 computes it
-//   kRope     kMulti for the q, k, v projections of a decoding step, then what
-//             rope_kv does with the result: pairs of features (2i, 2i+1) of the
-//             query and key heads rotated by the angle of the position read on
-//             the device (nn/transformer.go:146-257, interleaved layout), queries
-//             left in y, keys and values cast into their caches at that position
-//             (KVCache.Write, nn/transformer.go:464). Rows per wavefront even.
-enum Q4Mode { kPlain = 0, kMulti = 1, kSwiGLU = 2, kRope = 3 };
-
-struct Q4Job {
-    const uint8_t* W[3];
-    int n[3];
-    int total;           // rows of y
-    const float* resid;  // [M, total] or null
-    Q4RopeTail rope;     // kRope only
-    // kSwiGLU only: if set, the results go to act_out in the fixed-point form the next product
-    // reads (row m at act_out + m * act_out_row_bytes) instead of y. A workgroup then owns exactly
-    // the 32 results of one block, so rows_per_wg is 32 and total a multiple of 32.
-    uint8_t* act_out;
-    int64_t act_out_row_bytes;
-    // HEAD 1: the product's x is RMSNorm(norm_x[m, :]) * norm_w, normalized and converted by
-    // every workgroup for itself as its first phase instead of read from act. HEAD 2: x is
-    // norm_x[m, :] itself (rows x_row_stride floats apart), converted likewise.
-    const float* norm_x;
-    const float* norm_w;
-    float norm_inv_d, norm_eps;
-    int64_t x_row_stride;
-};
-
-constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
 static std::atomic<int> g_q4_batch_off{0};  // measurement aid: 1 keeps products of several rows of x on the one-row kernel, 2 puts all on the batch kernel
 void set_q4_batch_off(int v) { g_q4_batch_off = v; }
 
@@ -809,6 +718,10 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     if constexpr (MODE != kMulti) {
         hipError_t e;
         if (M >= 2 && tune[0] == 0 && tune[1] == 0 && tune[2] == 0 && dispatch_q4_0_i4_batch<MODE>(job, act, y, M, K, st, &e)) return e;
+    }
+    if (tune[0] == 0 && tune[1] == 0 && tune[2] == 0) {  // no launch plan forced: the kernel shaped for the whole chip where it takes the shape
+        hipError_t e;
+        if (q4_0_stream_dispatch(MODE, job, act, y, M, K, st, &e)) return e;
     }
     int nb = (int)(K / 32);
     int npc = (nb / 2 + 63) / 64;  // steps of 64 pairs of blocks that cover a row

@@ -7,13 +7,24 @@
 
 namespace mimir {
 
-// Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even.
-__device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int m, int row, float a, float b, float* yr) {
+// Whether rows (row, row + 1) are a pair that turns, and if so its cosine and sine at position pos: requested apart
+// from the store below by kernels that want the two loads under way before their weights'.
+__device__ __forceinline__ bool q4_rope_coeffs(const Q4RopeTail& t, int pos, int row, float* c, float* sn) {
+    const int head = row / t.dim, f = row - head * t.dim;
+    *c = 1.f;
+    *sn = 0.f;
+    if (head >= t.H + t.HK || f >= t.rope_dim) return false;
+    const int half = t.rope_dim >> 1, i = f >> 1;
+    *c = t.cosv[(int64_t)pos * half + i];
+    *sn = t.sinv[(int64_t)pos * half + i];
+    return true;
+}
+
+// Rows (row, row + 1) of sequence m: features (f, f + 1) of one head, f even; turns says whether they rotate, by (c, sn).
+__device__ __forceinline__ void q4_rope_store_with(const Q4RopeTail& t, int pos, int m, int row, float a, float b, bool turns, float c, float sn, float* yr) {
     const int head = row / t.dim, f = row - head * t.dim;
     float va = a, vb = b;
-    if (head < t.H + t.HK && f < t.rope_dim) {
-        const int half = t.rope_dim >> 1, i = f >> 1;
-        const float c = t.cosv[(int64_t)pos * half + i], sn = t.sinv[(int64_t)pos * half + i];
+    if (turns) {
         const float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;  // four products, then one subtraction and one addition
         va = ac - bs;
         vb = as + bc;
@@ -34,6 +45,12 @@ __device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int 
         ((uint16_t*)cache)[at] = f32_to_f16_bits(va);
         ((uint16_t*)cache)[at + 1] = f32_to_f16_bits(vb);
     }
+}
+
+__device__ __forceinline__ void q4_rope_store(const Q4RopeTail& t, int pos, int m, int row, float a, float b, float* yr) {
+    float c, sn;
+    const bool turns = q4_rope_coeffs(t, pos, row, &c, &sn);
+    q4_rope_store_with(t, pos, m, row, a, b, turns, c, sn, yr);
 }
 
 }  // namespace mimir
