@@ -526,7 +526,7 @@ def main():
                    "N": n, "K": k, "M": 1, "wall_ms_per_step": round(step_wall_ms, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "qgemv_q4_0_stream_kernel<0, 2, 4>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
+                     "kernel": "qgemv_q4_0_stream_kernel<0, 2, 7>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
                      "us_min": round(kern_min, 3), "us_max": round(kern_max, 3),
                      # the product over activations converted beforehand (as a decoding step's launches take them),
                      # back to back in a graph, the wait between dependent kernels included

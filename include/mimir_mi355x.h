@@ -237,7 +237,13 @@ MI355X_API mi355x_status mi355x_llama_destroy(void* model);
  * quantized dtypes). Names are llama.cpp's, as llm.Load reads them
  * (llm/model.go:268-310): token_embd.weight, output_norm.weight, output.weight
  * (absent: tied to the embeddings), blk.N.{attn_norm,attn_q,attn_k,attn_v,
- * attn_output,ffn_norm,ffn_gate,ffn_up,ffn_down}.weight. */
+ * attn_output,ffn_norm,ffn_gate,ffn_up,ffn_down}.weight, and the float32 biases
+ * blk.N.{attn_q,attn_k,attn_v}.bias that qwen2 gives its queries, keys and
+ * values (llm/model.go:251-258; Linear.Forward adds them behind the product,
+ * before the rotation: nn/layers.go:49-55). A block carries all three or none
+ * (mi355x_llama_finalize returns MI355X_ERR_SHAPE otherwise). A model with biases
+ * decodes with one launch per operator: the fused decoding launches are built
+ * for models without them. */
 MI355X_API mi355x_status mi355x_llama_set_tensor(void* model, const char* name, int dtype, const void* host_data, int64_t n_elems);
 /* rope_freqs.weight: divisors of each pair's frequency (llm/model.go:318-346). */
 MI355X_API mi355x_status mi355x_llama_set_rope_factors(void* model, const float* factors, int32_t n);

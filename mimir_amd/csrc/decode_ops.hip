@@ -307,6 +307,20 @@ __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, c
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) out[i] = a[i] + b[i];
 }
 
+// y[r, j] += bias[j]: Linear.Forward's bias (nn/layers.go:49-55), one float32 addition per element behind the product.
+__global__ __launch_bounds__(256) void add_bias_kernel(float* __restrict__ y, const float* __restrict__ bias, int64_t rows, int64_t n) {
+    const int64_t total = rows * n;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) y[i] = y[i] + bias[i % n];
+}
+
+hipError_t add_bias(float* y, const float* bias, int64_t rows, int64_t n, hipStream_t st) {
+    if (rows * n == 0) return hipSuccess;
+    int64_t groups = (rows * n + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    hipLaunchKernelGGL(add_bias_kernel, dim3((unsigned)groups), dim3(256), 0, st, y, bias, rows, n);
+    return hipGetLastError();
+}
+
 hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st) {
     if (n == 0) return hipSuccess;
     int64_t groups = (n + 255) / 256;

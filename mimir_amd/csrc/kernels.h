@@ -174,6 +174,7 @@ hipError_t advance(int32_t* state, const int32_t* next_tok, int32_t* record, int
 hipError_t set_state(int32_t* state, int pos, int step, hipStream_t st);
 hipError_t swiglu(const float* g, const float* u, float* out, int64_t rows, int64_t n, int64_t stride, hipStream_t st);
 hipError_t add(const float* a, const float* b, float* out, int64_t n, hipStream_t st);
+hipError_t add_bias(float* y, const float* bias, int64_t rows, int64_t n, hipStream_t st);  // y[r, :] += bias
 // workspace: argmax_workspace_bytes(rows) bytes, the first kArgmaxTicketBytes zero
 // before the first launch (they restore themselves), or null for one workgroup a row.
 constexpr size_t kArgmaxTicketBytes = 4096;

@@ -80,6 +80,8 @@ enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4 }; 
 // not need them (its kernels read the three matrices where they are).
 struct Block {
     Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down, qkv, gate_up;
+    Weight q_bias, k_bias, v_bias;  // qwen2's (llm/model.go:251-258): float32 [n], all three or none
+    bool biased() const { return q_bias.set(); }
 };
 
 struct Model {
@@ -218,6 +220,11 @@ static mi355x_status forward(Model& m, int64_t s) {
         if (mi355x_status st = linear(m, b.q, h, q, rows)) return st;
         if (mi355x_status st = linear(m, b.k, h, k, rows)) return st;
         if (mi355x_status st = linear(m, b.v, h, v, rows)) return st;
+        if (b.biased()) {  // Linear.Forward: the bias behind the product, before the rotation (nn/layers.go:49-55)
+            LLM_HIP(add_bias(q, b.q_bias.buf.as<float>(), rows, qd, m.stream), "q bias");
+            LLM_HIP(add_bias(k, b.k_bias.buf.as<float>(), rows, kvd, m.stream), "k bias");
+            LLM_HIP(add_bias(v, b.v_bias.buf.as<float>(), rows, kvd, m.stream), "v bias");
+        }
         // q and k are [B, s, heads, dim]. One position: every head of every
         // sequence is a row `dim` apart. More: per sequence, heads are rows
         // `dim` apart and positions heads * dim apart.
@@ -484,6 +491,11 @@ static mi355x_status step_any(Model& m) {
             if (mi355x_status st = linear(m, b.q, h, q, B)) return st;
             if (mi355x_status st = linear(m, b.k, h, k, B)) return st;
             if (mi355x_status st = linear(m, b.v, h, v, B)) return st;
+            if (b.biased()) {
+                LLM_HIP(add_bias(q, b.q_bias.buf.as<float>(), B, qd, m.stream), "q bias");
+                LLM_HIP(add_bias(k, b.k_bias.buf.as<float>(), B, kvd, m.stream), "k bias");
+                LLM_HIP(add_bias(v, b.v_bias.buf.as<float>(), B, kvd, m.stream), "v bias");
+            }
             LLM_HIP(rope_kv_split(q, k, v, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim,
                                   c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
             at.q = q; at.q_strides[0] = qd;
@@ -618,12 +630,15 @@ mi355x_status mi355x_llama_set_tensor(void* model, const char* name, int dtype, 
         else if (leaf == "ffn_gate.weight") { w = &b.gate; n = c.hidden; k = c.embed; }
         else if (leaf == "ffn_up.weight") { w = &b.up; n = c.hidden; k = c.embed; }
         else if (leaf == "ffn_down.weight") { w = &b.down; n = c.embed; k = c.hidden; }
+        else if (leaf == "attn_q.bias") { w = &b.q_bias; n = 1; k = qd; }
+        else if (leaf == "attn_k.bias") { w = &b.k_bias; n = 1; k = kvd; }
+        else if (leaf == "attn_v.bias") { w = &b.v_bias; n = 1; k = kvd; }
     }
     if (!w) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: unknown tensor %s", name);
     if (n * k != n_elems) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: %s of %lld elements, want [%lld, %lld]", name, (long long)n_elems, (long long)n, (long long)k);
     int bs = block_size(dtype), bb = block_bytes(dtype);
     if (bb == 0 || k % bs != 0) return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: %s of dtype %d", name, dtype);
-    if ((w == &m->norm || s.find("_norm.weight") != std::string::npos) && dtype != kF32)
+    if ((w == &m->norm || s.find("_norm.weight") != std::string::npos || s.find(".bias") != std::string::npos) && dtype != kF32)
         return capi_fail(MI355X_ERR_DTYPE, "mi355x: llama: %s of dtype %d, want float32", name, dtype);
     size_t bytes = (size_t)(n_elems / bs) * bb;
     LLM_HIP(w->buf.alloc(bytes), "hipMalloc(weight)");
@@ -660,6 +675,8 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         Block& b = m->blocks[i];
         for (const Weight* w : {&b.attn_norm, &b.ffn_norm, &b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down})
             if (!w->set()) return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: block %d is missing a tensor", i);
+        if (b.q_bias.set() != b.k_bias.set() || b.q_bias.set() != b.v_bias.set())
+            return capi_fail(MI355X_ERR_SHAPE, "mi355x: llama: block %d has some of attn_{q,k,v}.bias, want all three or none", i);
     }
     // nn/transformer.go:146-164 with llm/model.go:332-346: float64 angles, rounded to float32
     const int half = c.rope_dim / 2;
@@ -737,6 +754,9 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     LLM_HIP(m->record.alloc(((size_t)c.context + 1) * c.batch * 4), "hipMalloc");  // a graph keeps its address
     LLM_HIP(m->qkv.alloc((size_t)c.batch * (qd + 2 * kvd) * 4), "hipMalloc");
     m->fast = rmsnorm_q4act_ok(c.embed) && c.head_dim % 2 == 0;
+    bool biased = false;  // q, k, v with biases: separate products with the additions behind them, no fused tails
+    for (int i = 0; i < c.layers; i++) biased = biased || m->blocks[i].biased();
+    if (biased) m->fast = false;
     for (int i = 0; i < c.layers && m->fast; i++) {
         Block& b = m->blocks[i];
         for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down})
@@ -766,7 +786,8 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
             into.dtype = first->dtype; into.n = n; into.k = first->k;
             return MI355X_OK;
         };
-        if (mi355x_status st = fuse({&b.q, &b.k, &b.v}, b.qkv)) return st;
+        if (!biased)
+            if (mi355x_status st = fuse({&b.q, &b.k, &b.v}, b.qkv)) return st;
         if (mi355x_status st = fuse({&b.gate, &b.up}, b.gate_up)) return st;
     }
     LLM_HIP(m->gu.alloc((size_t)c.batch * 2 * c.hidden * 4), "hipMalloc");

@@ -115,15 +115,31 @@ def config_from_metadata(md: dict, vocab: int, context: int | None = None, batch
 
 
 def load_mim(path: str, max_tokens: int = 64, **kw) -> Llama:
+    """llm.Load (llm/model.go:224-316): every tensor the reference reads, the biases that
+    qwen2 gives its queries, keys and values among them (:251-258); a qwen2 file without
+    them is an error, as it is there."""
     f = MimFile(path)
     emb = f["token_embd.weight"]
-    m = Llama(config_from_metadata(f.metadata, emb.shape[0], **kw))
+    c = config_from_metadata(f.metadata, emb.shape[0], **kw)
+    m = Llama(c)
+    biased = f.metadata.get("general.architecture") == "qwen2"
     for name, t in f.tensors.items():
         if name == "rope_freqs.weight":
             m.set_rope_factors(t.data)
+        elif name.startswith("blk.") and name.rsplit(".", 2)[-2:] in (["attn_q", "bias"], ["attn_k", "bias"], ["attn_v", "bias"]):
+            if not biased:
+                continue  # the reference reads them for qwen2 only
+            if t.dtype_name != "f32":
+                raise ValueError(f"{name}: dtype {t.dtype_name}, want f32")
+            m.set_tensor(name, capi.F32, np.ascontiguousarray(t.data, np.float32), int(np.prod(t.shape)))
         elif name.endswith(".weight") and (name.startswith("blk.") or name in ("token_embd.weight", "output_norm.weight", "output.weight")):
             if t.dtype not in _MIM_TO_ABI:
                 raise ValueError(f"{name}: dtype {t.dtype_name}")
             m.set_tensor(name, _MIM_TO_ABI[t.dtype], t.data, int(np.prod(t.shape)))
+    if biased:
+        for i in range(c.layers):
+            for leaf in ("attn_q", "attn_k", "attn_v"):
+                if f"blk.{i}.{leaf}.bias" not in f:
+                    raise KeyError(f"blk.{i}.{leaf}.bias: a qwen2 model has biases on its queries, keys and values")
     m.finalize(max_tokens)
     return m

@@ -70,6 +70,9 @@ class Block:
     gate: Weight = None
     up: Weight = None
     down: Weight = None
+    q_bias: np.ndarray | None = None  # qwen2's (llm/model.go:251-258), float32 [n]
+    k_bias: np.ndarray | None = None
+    v_bias: np.ndarray | None = None
 
 
 @dataclass
@@ -143,7 +146,9 @@ class Model:
         m.output = weight("output.weight") if "output.weight" in f else m.embed  # tied (llm/model.go:283-288)
         for i in range(c.layers):
             p = f"blk.{i}."
+            bias = (lambda leaf: f[p + leaf + ".bias"].data.astype(np.float32)) if arch == "qwen2" else (lambda leaf: None)
             m.blocks.append(Block(
+                q_bias=bias("attn_q"), k_bias=bias("attn_k"), v_bias=bias("attn_v"),
                 attn_norm=f[p + "attn_norm.weight"].data.astype(np.float32),
                 ffn_norm=f[p + "ffn_norm.weight"].data.astype(np.float32),
                 q=weight(p + "attn_q.weight"), k=weight(p + "attn_k.weight"), v=weight(p + "attn_v.weight"),
@@ -160,11 +165,13 @@ class Model:
         return [KVCache(np.zeros((c.kv_heads, capacity, c.head_dim), dt), np.zeros((c.kv_heads, capacity, c.head_dim), dt), dtype)
                 for _ in range(c.layers)]
 
-    def linear(self, x: np.ndarray, w: Weight) -> np.ndarray:
-        """x [..., k] . w^T (nn/layers.go:49-55 -> tensor/quant.go:35-56)."""
+    def linear(self, x: np.ndarray, w: Weight, bias: np.ndarray | None = None) -> np.ndarray:
+        """x [..., k] . w^T, then + bias in float32 if the layer has one (nn/layers.go:49-55 -> tensor/quant.go:35-56)."""
         if w.dtype == O.F32:
-            return O.sgemv(w.data, x, self.threads)
-        return O.qmatmul(w.dtype, w.data, x, w.n, w.k, simd=True, threads=self.threads)
+            y = O.sgemv(w.data, x, self.threads)
+        else:
+            y = O.qmatmul(w.dtype, w.data, x, w.n, w.k, simd=True, threads=self.threads)
+        return y if bias is None else (y + bias.astype(np.float32)).astype(np.float32)
 
     def embed_tokens(self, tokens) -> np.ndarray:
         w = self.embed
@@ -190,9 +197,9 @@ class Model:
         for blk, cache in zip(self.blocks, caches):
             past = cache.n
             h = O.rmsnorm(x, blk.attn_norm, c.eps)
-            q = self.linear(h, blk.q).reshape(s, c.heads, c.head_dim).transpose(1, 0, 2)
-            k = self.linear(h, blk.k).reshape(s, c.kv_heads, c.head_dim).transpose(1, 0, 2)
-            v = self.linear(h, blk.v).reshape(s, c.kv_heads, c.head_dim).transpose(1, 0, 2)
+            q = self.linear(h, blk.q, blk.q_bias).reshape(s, c.heads, c.head_dim).transpose(1, 0, 2)
+            k = self.linear(h, blk.k, blk.k_bias).reshape(s, c.kv_heads, c.head_dim).transpose(1, 0, 2)
+            v = self.linear(h, blk.v, blk.v_bias).reshape(s, c.kv_heads, c.head_dim).transpose(1, 0, 2)
             q, k = self.rope(np.ascontiguousarray(q), past), self.rope(np.ascontiguousarray(k), past)
             if past + s > cache.keys.shape[1]:
                 raise ValueError(f"append {s} positions to a cache holding {past} of {cache.keys.shape[1]}")

@@ -71,6 +71,48 @@ def test_tiny_q4km_known_answers_with_f16_cache(golden_dir):
         assert a == b or margins[i] < 1e-3, (i, a, b, margins[i])
 
 
+@pytest.mark.parametrize("cache", [capi.F32, capi.F16])
+def test_qwen2_biases_on_queries_keys_and_values(golden_dir, cache):
+    """The reference's qwen2 fixture (llm/llm_test.go:36-39): biases on q, k and v added behind the products and
+    before the rotation (llm/model.go:251-258, nn/layers.go:49-55), rotation over halves. Every position of the
+    prompt at once, then token by token through the caches, then greedy tokens: against the oracle's model, which
+    multiplies with int8 activations as the device does."""
+    path = os.path.join(golden_dir, "qwen2-exact.mim")
+    prompt = [1, 79, 110, 99, 101, 363, 264, 315, 307, 280]
+    gpu.lib()
+    gpu.say(f"qwen2, cache dtype {cache}")
+    m = load_mim(path, max_tokens=16, context=64, cache_dtype=cache)
+    om = OL.Model.from_mim(MimFile(path))
+    ocache = O.F32 if cache == capi.F32 else O.F16
+    want = om.logits(prompt, om.new_caches(64, ocache), all=True)
+    got = m.logits(prompt, all=True)[0]
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-4 * scale
+    m.reset()
+    caches = om.new_caches(64, ocache)
+    for t in prompt:
+        assert np.abs(m.logits([t])[0] - om.logits([t], caches)).max() <= 1e-4 * scale
+    m.reset()
+    toks, _ = m.generate(prompt, 12)
+    owant, margins = om.generate(prompt, 12, capacity=64, cache_dtype=ocache)
+    assert toks[0].tolist() == owant, (toks[0].tolist(), owant, min(margins))
+
+
+def test_some_but_not_all_biases_is_an_error(golden_dir):
+    gpu.lib()
+    path = os.path.join(golden_dir, "qwen2-exact.mim")
+    f = MimFile(path)
+    from mimir_amd.llama import config_from_metadata, _MIM_TO_ABI
+    m = Llama(config_from_metadata(f.metadata, f["token_embd.weight"].shape[0], context=16))
+    for name, t in f.tensors.items():
+        if name.endswith(".weight"):
+            m.set_tensor(name, _MIM_TO_ABI[t.dtype], t.data, int(np.prod(t.shape)))
+    m.set_tensor("blk.0.attn_q.bias", capi.F32, f["blk.0.attn_q.bias"].data, int(np.prod(f["blk.0.attn_q.bias"].shape)))
+    with pytest.raises(capi.Mi355xError) as ei:
+        m.finalize(8)
+    assert ei.value.status == capi.ERR_SHAPE
+
+
 def test_errors_before_anything_is_queued(golden_dir):
     gpu.lib()
     m = load_mim(os.path.join(golden_dir, "spm.mim"), max_tokens=8, context=8)

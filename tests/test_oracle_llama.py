@@ -85,3 +85,83 @@ def test_generate_is_the_argmax_of_a_full_pass(golden_dir):
     for i, t in enumerate(out):
         row = full[len(prompt) - 1 + i]
         assert O.argmax(row) == t or margins[i] < 1e-3
+
+
+# ---- qwen2: biases on the queries, keys and values, rotation over halves -------------------------
+# The reference's only expectation for this model is the graph inside qwen2-exact.mim
+# (llm/llm_test.go:36-39,131-160 compares Model with that graph), and the graph section's
+# encoding lives in the mimir-model module, which the reference does not vendor. So this path
+# has no reference-held vector; it is held by what the mathematics fixes instead.
+
+QWEN_PROMPT = [1, 79, 110, 99, 101, 363, 264, 315, 307, 280]  # llm/llm_test.go:41
+
+
+def _float64_forward(m: Model, tokens):
+    """A second formulation of the same function: every position at once in float64, an explicit causal
+    mask, softmax by its definition, the rotation written from RoPE's formula for the halves layout
+    (feature i pairs with i + rope_dim/2), the bias added where Linear adds it. Shares no code with
+    Model.logits beyond the weights' decoding."""
+    c = m.config
+    deq = lambda w: np.asarray(w.dequantized().data, np.float64).reshape(w.n, w.k)
+    x = deq(m.embed)[np.asarray(tokens)]
+    s = len(tokens)
+    half = c.rope_dim // 2
+    ang = np.arange(s)[:, None] * (c.rope_base ** (-2.0 * np.arange(half) / c.rope_dim))[None, :] / c.rope_scale
+    cos, sin = np.cos(ang), np.sin(ang)
+
+    def norm(v, w):
+        return v / np.sqrt((v * v).mean(-1, keepdims=True) + c.eps) * w
+
+    def rope(t):  # [s, heads, dim]
+        a, b = t[..., :half].copy(), t[..., half:c.rope_dim].copy()
+        out = t.copy()
+        out[..., :half] = a * cos[:, None, :] - b * sin[:, None, :]
+        out[..., half:c.rope_dim] = a * sin[:, None, :] + b * cos[:, None, :]
+        return out
+
+    for blk in m.blocks:
+        h = norm(x, blk.attn_norm)
+        q = (h @ deq(blk.q).T + blk.q_bias).reshape(s, c.heads, c.head_dim)
+        k = (h @ deq(blk.k).T + blk.k_bias).reshape(s, c.kv_heads, c.head_dim)
+        v = (h @ deq(blk.v).T + blk.v_bias).reshape(s, c.kv_heads, c.head_dim)
+        q, k = rope(q), rope(k)
+        g = c.heads // c.kv_heads
+        att = np.empty((s, c.heads, c.head_dim))
+        mask = np.where(np.arange(s)[None, :] <= np.arange(s)[:, None], 0.0, -np.inf)
+        for hh in range(c.heads):
+            sc = q[:, hh] @ k[:, hh // g].T / np.sqrt(c.head_dim) + mask
+            p = np.exp(sc - sc.max(-1, keepdims=True))
+            att[:, hh] = (p / p.sum(-1, keepdims=True)) @ v[:, hh // g]
+        x = x + att.reshape(s, -1) @ deq(blk.o).T
+        h = norm(x, blk.ffn_norm)
+        gate, up = h @ deq(blk.gate).T, h @ deq(blk.up).T
+        x = x + (gate / (1 + np.exp(-gate)) * up) @ deq(blk.down).T
+    return norm(x, m.norm) @ deq(m.output).T
+
+
+def test_qwen2_biases_and_halves_rotation(golden_dir):
+    f = MimFile(os.path.join(golden_dir, "qwen2-exact.mim"))
+    m = Model.from_mim(f, dequantized=True)
+    assert m.config.arch == "qwen2" and not m.config.interleaved
+    assert all(b.q_bias is not None and b.k_bias is not None and b.v_bias is not None for b in m.blocks)
+    assert max(float(np.abs(b.q_bias).max()) for b in m.blocks) > 0  # the file's biases are not zeros: dropping them would show
+    want = _float64_forward(m, QWEN_PROMPT)
+    got = m.logits(QWEN_PROMPT, m.new_caches(64), all=True)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-5 * scale
+    # a dropped bias, one added behind the rotation, or the pairs layout in place of the halves: each is far outside that bound
+    for wrong in ("no_bias", "pairs"):
+        m2 = Model.from_mim(f, dequantized=True)
+        if wrong == "no_bias":
+            for b in m2.blocks:
+                b.k_bias = np.zeros_like(b.k_bias)
+        else:
+            m2.config.arch = "llama"
+        bad = m2.logits(QWEN_PROMPT, m2.new_caches(64), all=True)
+        assert np.abs(bad - want).max() > 1e-3 * scale, wrong
+    # one token at a time through the caches (llm/llm_test.go:146-160), and int8 activations stay near
+    caches = m.new_caches(64)
+    stepped = np.stack([m.logits([t], caches) for t in QWEN_PROMPT])
+    assert np.abs(stepped - got).max() <= 1e-4 * scale
+    a8 = Model.from_mim(f).logits(QWEN_PROMPT, Model.from_mim(f).new_caches(64), all=True)
+    assert np.abs(a8 - want).max() <= 0.05 * scale
