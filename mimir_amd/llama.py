@@ -14,7 +14,8 @@ from . import capi
 from .mimfile import MimFile
 
 # container dtype codes (mimfile) -> C-ABI dtype codes
-_MIM_TO_ABI = {1: capi.F32, 2: capi.F16, 3: capi.BF16, 64: capi.Q8_0, 66: capi.Q4_K, 67: capi.Q6_K}
+# dtype names of mimir_amd.mimfile -> dtype codes of the C ABI
+_MIM_TO_ABI = {"f32": capi.F32, "f16": capi.F16, "bf16": capi.BF16, "q8_0": capi.Q8_0, "q4_K": capi.Q4_K, "q6_K": capi.Q6_K, "q4_0": capi.Q4_0}
 
 
 class Llama:
@@ -114,11 +115,11 @@ def config_from_metadata(md: dict, vocab: int, context: int | None = None, batch
     return c
 
 
-def load_mim(path: str, max_tokens: int = 64, **kw) -> Llama:
+def load_mim(path: str, max_tokens: int = 64, q4_0_code: int | None = None, **kw) -> Llama:
     """llm.Load (llm/model.go:224-316): every tensor the reference reads, the biases that
     qwen2 gives its queries, keys and values among them (:251-258); a qwen2 file without
     them is an error, as it is there."""
-    f = MimFile(path)
+    f = MimFile(path, q4_0_code=q4_0_code)  # the container's code for Q4_0 blocks, if the caller knows it
     emb = f["token_embd.weight"]
     c = config_from_metadata(f.metadata, emb.shape[0], **kw)
     m = Llama(c)
@@ -133,9 +134,9 @@ def load_mim(path: str, max_tokens: int = 64, **kw) -> Llama:
                 raise ValueError(f"{name}: dtype {t.dtype_name}, want f32")
             m.set_tensor(name, capi.F32, np.ascontiguousarray(t.data, np.float32), int(np.prod(t.shape)))
         elif name.endswith(".weight") and (name.startswith("blk.") or name in ("token_embd.weight", "output_norm.weight", "output.weight")):
-            if t.dtype not in _MIM_TO_ABI:
+            if t.dtype_name not in _MIM_TO_ABI:
                 raise ValueError(f"{name}: dtype {t.dtype_name}")
-            m.set_tensor(name, _MIM_TO_ABI[t.dtype], t.data, int(np.prod(t.shape)))
+            m.set_tensor(name, _MIM_TO_ABI[t.dtype_name], t.data, int(np.prod(t.shape)))
     if biased:
         for i in range(c.layers):
             for leaf in ("attn_q", "attn_k", "attn_v"):

@@ -10,6 +10,13 @@ and hyperparameters alone (llm/llm_test.go:132-154).
 
 Block-quantized tensors are returned as their raw ggml bytes (uint8), with
 the logical element shape alongside, which is what a device upload wants.
+
+Q4_0 has no container code here: the reference's block accounting
+(backend/quant.go:24-48) and every fixture it holds know Q8_0, Q4_K and Q6_K
+only, and the code a converter would write for Q4_0 is defined in the
+mimir-model module, which the reference does not vendor. A caller who knows it
+passes it as `q4_0_code`; tensors of that code are then kept as 18-byte blocks
+of 32 (ggml's block_q4_0) under the dtype name "q4_0".
 """
 from __future__ import annotations
 
@@ -36,6 +43,9 @@ DTYPE_NAMES = {F32: "f32", F16: "f16", BF16: "bf16", U8: "u8", I32: "i32", I64: 
                Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K"}
 
 
+Q4_0_BLOCK = (32, 18)
+
+
 class MimError(ValueError):
     pass
 
@@ -46,23 +56,24 @@ class MimTensor:
     dtype: int          # container dtype code
     shape: tuple        # logical element shape
     data: np.ndarray    # plain dtypes: array of `shape`; block dtypes: uint8 [nbytes]
-
-    @property
-    def dtype_name(self) -> str:
-        return DTYPE_NAMES.get(self.dtype, f"dtype({self.dtype})")
-
-    @property
-    def quantized(self) -> bool:
-        return self.dtype in _BLOCKS
+    dtype_name: str = ""  # "f32", "q8_0", ...; "q4_0" for the code the file was opened with
+    quantized: bool = False
 
 
 class MimFile:
     """The tensors and metadata of one .mim file, read eagerly."""
 
-    def __init__(self, path: str):
+    def __init__(self, path: str, q4_0_code: int | None = None):
         with open(path, "rb") as f:
             raw = f.read()
         self.path = path
+        if q4_0_code is not None and (q4_0_code in _PLAIN or q4_0_code in _BLOCKS):
+            raise MimError(f"{path}: container code {q4_0_code} is {DTYPE_NAMES[q4_0_code]}, not free for q4_0")
+        self._blocks = dict(_BLOCKS)
+        self._names = dict(DTYPE_NAMES)
+        if q4_0_code is not None:
+            self._blocks[q4_0_code] = Q4_0_BLOCK
+            self._names[q4_0_code] = "q4_0"
         self.tensors: dict[str, MimTensor] = {}
         self.metadata: dict[str, object] = {}
         self._parse(raw)
@@ -121,12 +132,12 @@ class MimFile:
             dt = _PLAIN[dtype]
             if len(blob) != n * dt.itemsize:
                 raise MimError(f"{self.path}: {name}: {len(blob)} bytes for {shape} {dt}")
-            return MimTensor(name, dtype, shape, np.frombuffer(blob, dt).reshape(shape).copy())
-        if dtype in _BLOCKS:
-            bs, bb = _BLOCKS[dtype]
+            return MimTensor(name, dtype, shape, np.frombuffer(blob, dt).reshape(shape).copy(), self._names[dtype], False)
+        if dtype in self._blocks:
+            bs, bb = self._blocks[dtype]
             if not shape or shape[-1] % bs or len(blob) != n // bs * bb:
                 raise MimError(f"{self.path}: {name}: {len(blob)} bytes for {shape} blocks of {bs}")
-            return MimTensor(name, dtype, shape, np.frombuffer(blob, np.uint8).copy())
+            return MimTensor(name, dtype, shape, np.frombuffer(blob, np.uint8).copy(), self._names[dtype], True)
         raise MimError(f"{self.path}: {name}: unknown dtype code {dtype}")
 
     def _metadata(self, sec: bytes) -> None:

@@ -36,9 +36,12 @@ _lib = None
 def lib() -> C.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            build()
-        _lib = C.CDLL(_LIB_PATH)
+        path = os.environ.get("MIMIR_ORACLE_LIB")  # another build of the same source, e.g. `make -C oracle asan`
+        if not path:
+            if not os.path.exists(_LIB_PATH):
+                build()
+            path = _LIB_PATH
+        _lib = C.CDLL(path)
         _declare(_lib)
     return _lib
 

@@ -20,8 +20,8 @@ import numpy as np
 
 import oracle as O
 
-# container dtype codes of mimir_amd.mimfile -> oracle dtype codes
-_MIM_TO_ORACLE = {64: O.Q8_0, 66: O.Q4_K, 67: O.Q6_K}
+# dtype names of mimir_amd.mimfile -> oracle dtype codes
+_MIM_TO_ORACLE = {"q8_0": O.Q8_0, "q4_K": O.Q4_K, "q6_K": O.Q6_K, "q4_0": O.Q4_0}
 
 
 @dataclass
@@ -128,7 +128,7 @@ class Model:
             t = f[name]
             n, k = t.shape
             if t.quantized:
-                w = Weight(_MIM_TO_ORACLE[t.dtype], n, k, t.data)
+                w = Weight(_MIM_TO_ORACLE[t.dtype_name], n, k, t.data)
             elif t.dtype_name == "f32":
                 w = Weight(O.F32, n, k, np.ascontiguousarray(t.data, np.float32))
             elif t.dtype_name == "f16":

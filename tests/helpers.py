@@ -153,3 +153,72 @@ def check_close(got, want, tol, what=""):
 def rel_l2(got, want):
     got = np.asarray(got, np.float64).reshape(-1); want = np.asarray(want, np.float64).reshape(-1)
     return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
+
+
+def write_mim(path, tensors, metadata):
+    """A .mim container in the layout mimir_amd.mimfile reads (a preamble, an index of two sections and the
+    tensor rows with their name pool, a "MIMM" metadata section, a weights section): tensors is a list of
+    (name, container dtype code, logical shape, bytes); metadata maps keys to int, float or str."""
+    import struct
+    pool, rows, blob = b"", b"", b""
+    for name, code, shape, data in tensors:
+        nm = name.encode()
+        while len(blob) % 64:
+            blob += b"\0"
+        dims = list(shape) + [0] * (8 - len(shape))
+        rows += struct.pack("<IIIB3x", len(pool), len(nm), code, len(shape)) + struct.pack("<8Q", *dims) + struct.pack("<QQ", len(blob), len(data))
+        pool += nm
+        blob += bytes(data)
+    mpool, ments = b"", b""
+    for key, val in metadata.items():
+        kb = key.encode()
+        koff = len(mpool)
+        mpool += kb
+        if isinstance(val, bool):
+            typ, v8, nbytes = 4, bytes([int(val)]) + b"\0" * 7, 0
+        elif isinstance(val, int):
+            typ, v8, nbytes = 1, struct.pack("<q", val), 0
+        elif isinstance(val, float):
+            typ, v8, nbytes = 3, struct.pack("<d", val), 0
+        else:
+            sb = str(val).encode()
+            typ, v8, nbytes = 5, struct.pack("<Q", len(mpool)), len(sb)
+            mpool += sb
+        ments += struct.pack("<IIB3xI", koff, len(kb), typ, nbytes) + v8 + b"\0" * 8
+    meta = b"MIMM" + struct.pack("<IQ", len(metadata), len(mpool)) + ments + mpool
+    index_off = 64
+    index_len = 16 + 2 * 64 + len(rows) + len(pool)
+    meta_off = (index_off + index_len + 63) // 64 * 64
+    data_off = (meta_off + len(meta) + 63) // 64 * 64
+    file_len = data_off + len(blob)
+    sect = lambda kind, off, length: struct.pack("<IIQQ", kind, 0, off, length) + b"\0" * 40
+    index = struct.pack("<IIQ", 2, len(tensors), len(pool)) + sect(1, data_off, len(blob)) + sect(2, meta_off, len(meta)) + rows + pool
+    head = b"MIM\0" + struct.pack("<HHIIQQQQQ", 0, 1, 0x0A0B0C0D, 64, index_off, index_len, data_off, len(blob), file_len)
+    out = head + b"\0" * (64 - len(head)) + index
+    out += b"\0" * (meta_off - len(out)) + meta
+    out += b"\0" * (data_off - len(out)) + blob
+    with open(path, "wb") as f:
+        f.write(out)
+
+
+def synthetic_llama_mim(path, om, q4_0_code, arch="llama"):
+    """The oracle's synthetic model `om` (oracle.llama.synthetic) as a .mim file whose Q4_0 tensors carry
+    the container code q4_0_code."""
+    codes = {O.Q4_0: q4_0_code, O.Q8_0: 64, O.Q4_K: 66, O.Q6_K: 67}
+    c = om.config
+    tensors = []
+    wt = lambda name, w: tensors.append((name, codes[w.dtype], (w.n, w.k), np.asarray(w.data, np.uint8).tobytes()))
+    f32 = lambda name, v: tensors.append((name, 1, (len(v),), np.asarray(v, "<f4").tobytes()))
+    wt("token_embd.weight", om.embed)
+    wt("output.weight", om.output)
+    f32("output_norm.weight", om.norm)
+    for i, b in enumerate(om.blocks):
+        p = f"blk.{i}."
+        f32(p + "attn_norm.weight", b.attn_norm); f32(p + "ffn_norm.weight", b.ffn_norm)
+        for leaf, w in (("attn_q", b.q), ("attn_k", b.k), ("attn_v", b.v), ("attn_output", b.o), ("ffn_gate", b.gate), ("ffn_up", b.up), ("ffn_down", b.down)):
+            wt(p + leaf + ".weight", w)
+    md = {"general.architecture": arch, f"{arch}.embedding_length": c.embed, f"{arch}.feed_forward_length": c.hidden,
+          f"{arch}.block_count": c.layers, f"{arch}.attention.head_count": c.heads, f"{arch}.attention.head_count_kv": c.kv_heads,
+          f"{arch}.attention.key_length": c.head_dim, f"{arch}.rope.dimension_count": c.rope_dim, f"{arch}.rope.freq_base": float(c.rope_base),
+          f"{arch}.attention.layer_norm_rms_epsilon": float(c.eps), f"{arch}.context_length": c.context}
+    write_mim(path, tensors, md)

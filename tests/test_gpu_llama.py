@@ -106,11 +106,33 @@ def test_some_but_not_all_biases_is_an_error(golden_dir):
     m = Llama(config_from_metadata(f.metadata, f["token_embd.weight"].shape[0], context=16))
     for name, t in f.tensors.items():
         if name.endswith(".weight"):
-            m.set_tensor(name, _MIM_TO_ABI[t.dtype], t.data, int(np.prod(t.shape)))
+            m.set_tensor(name, _MIM_TO_ABI[t.dtype_name], t.data, int(np.prod(t.shape)))
     m.set_tensor("blk.0.attn_q.bias", capi.F32, f["blk.0.attn_q.bias"].data, int(np.prod(f["blk.0.attn_q.bias"].shape)))
     with pytest.raises(capi.Mi355xError) as ei:
         m.finalize(8)
     assert ei.value.status == capi.ERR_SHAPE
+
+
+def test_q4_0_tensors_from_a_file_under_the_callers_code(tmp_path):
+    """A .mim file whose Q4_0 tensors carry a container code that the caller names (the reference's fixtures
+    hold none): load_mim uploads them as Q4_0 and the model decodes as the oracle's copy of it does."""
+    from oracle.llama import Config, synthetic
+    from tests.helpers import synthetic_llama_mim
+    gpu.lib()
+    oc = Config(embed=512, hidden=1024, layers=2, heads=4, kv_heads=2, head_dim=128, rope_dim=128, vocab=320, context=32, rope_base=500000.0)
+    om = synthetic(oc, seed=5)
+    path = str(tmp_path / "q4_0.mim")
+    synthetic_llama_mim(path, om, q4_0_code=65)
+    gpu.say("a .mim file with Q4_0 tensors")
+    m = load_mim(path, max_tokens=8, q4_0_code=65, cache_dtype=capi.F16)
+    prompt = [3, 200, 41, 7, 19]
+    want = om.logits(prompt, om.new_caches(32, O.F16))
+    got = m.logits(prompt)[0]
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    m.reset()
+    toks, _ = m.generate(prompt, 8)
+    owant, margins = om.generate(prompt, 8, capacity=32, cache_dtype=O.F16)
+    assert toks[0].tolist() == owant, (toks[0].tolist(), owant, min(margins))
 
 
 def test_errors_before_anything_is_queued(golden_dir):

@@ -165,3 +165,26 @@ def test_qwen2_biases_and_halves_rotation(golden_dir):
     assert np.abs(stepped - got).max() <= 1e-4 * scale
     a8 = Model.from_mim(f).logits(QWEN_PROMPT, Model.from_mim(f).new_caches(64), all=True)
     assert np.abs(a8 - want).max() <= 0.05 * scale
+
+
+def test_q4_0_container_code_is_the_callers(tmp_path):
+    """The reference's fixtures hold no Q4_0 tensor and its accounting no code for one: MimFile refuses an
+    unknown code, and reads it as 18-byte blocks of 32 when the caller names it as Q4_0's."""
+    from mimir_amd.mimfile import MimError
+    from oracle.llama import Config, synthetic
+    from tests.helpers import synthetic_llama_mim
+    c = Config(embed=128, hidden=256, layers=1, heads=2, kv_heads=1, head_dim=64, rope_dim=64, vocab=96, context=16)
+    om = synthetic(c, seed=3)
+    path = str(tmp_path / "q4_0.mim")
+    synthetic_llama_mim(path, om, q4_0_code=65)
+    with pytest.raises(MimError):
+        MimFile(path)
+    with pytest.raises(MimError):
+        MimFile(path, q4_0_code=64)  # Q8_0's
+    f = MimFile(path, q4_0_code=65)
+    t = f["blk.0.attn_q.weight"]
+    assert t.dtype_name == "q4_0" and t.quantized and t.shape == (128, 128) and t.data.nbytes == 128 * 128 // 32 * 18
+    assert f["token_embd.weight"].dtype_name == "q8_0"
+    m = Model.from_mim(f)
+    toks = [5, 17, 80, 3]
+    assert np.array_equal(m.logits(toks, m.new_caches(16)), om.logits(toks, om.new_caches(16)))
