@@ -240,7 +240,19 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear=
         om = OL.synthetic(OL.Config(arch="llama", embed=c.embed, hidden=c.hidden, layers=c.layers, heads=c.heads, kv_heads=c.kv_heads,
                                     head_dim=c.head_dim, rope_dim=c.rope_dim, rope_base=c.rope_base, rope_scale=1.0, eps=c.eps,
                                     vocab=c.vocab, context=c.context), seed=0)
-        want, margins = om.generate(toks[0].tolist(), check, capacity=c.context, cache_dtype=O.F16)
+        # the oracle's greedy decoding, step by step so that a long check shows it is alive
+        caches = om.new_caches(c.context, O.F16)
+        print(f"bench.py: CPU oracle: prompt of {prompt} tokens", file=sys.stderr, flush=True)
+        logits = om.logits(toks[0].tolist(), caches)
+        want, margins = [], []
+        for i in range(check):
+            want.append(O.argmax(logits))
+            top2 = np.partition(logits, -2)[-2:]
+            margins.append(float(top2[1] - top2[0]))
+            if i % 16 == 15:
+                print(f"bench.py: CPU oracle: {i + 1} of {check} greedy tokens", file=sys.stderr, flush=True)
+            if i + 1 < check:
+                logits = om.logits([want[-1]], caches)
         got = out[0, :check].tolist()
         first = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), None)
         verdict = {"greedy_checked": check, "greedy_identical": sum(a == b for a, b in zip(got, want)), "first_mismatch": first,
@@ -264,7 +276,12 @@ def layer_step_bench(capi, cached=2048, new=33):
             _, (_, t_decode) = m.generate(toks, new)
             ms[layers] = t_decode / (new - 1) * 1e3
             del m
-        out[f"batch{batch}"] = {"us_per_layer": round((ms[6] - ms[2]) / 4 * 1e3, 2), "ms_per_step_2_layers": round(ms[2], 4), "ms_per_step_6_layers": round(ms[6], 4)}
+        us = (ms[6] - ms[2]) / 4 * 1e3
+        # what a layer's step must read: its seven Q4_0 matrices once, and every sequence's cached keys and values (binary16)
+        layer_bytes = 218103808 * 18 // 32 + batch * cached * 8 * 128 * 2 * 2
+        out[f"batch{batch}"] = {"us_per_layer": round(us, 2), "bytes_per_layer": layer_bytes, "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1),
+                                "frac": round(layer_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                "ms_per_step_2_layers": round(ms[2], 4), "ms_per_step_6_layers": round(ms[6], 4)}
     out["cached_positions"] = cached
     return out
 
@@ -342,7 +359,7 @@ def rows_bench(lib, capi, torch, m=8, shapes=((14336, 4096), (4096, 14336), (409
     return out
 
 
-def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096), (2048, 14336)), k=4096, iters=50):
+def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096), (2048, 14336)), k=4096, iters=50, kquants=True):
     """The prompt-sized products with bfloat16 activations and results, mi355x_qgemm_bf16 as a whole
     (for Q4_K and Q6_K that includes the casts and the int8 rounding of x): TFLOP/s (2 M N K) between
     HIP events on its stream, against the dense peak of the matrix instruction used (bfloat16 2.5 PFLOP/s
@@ -379,6 +396,8 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
         del w, x, y
     out["q4_0_f32_x"] = res
     for name, dt, peak, frac_key in kinds:
+        if dt != capi.Q4_0 and not kquants:
+            continue
         res = {}
         capi.check(lib.mi355x_tune(b"qgemm.f16", 1 if name == "q4_0_binary16_weights" else 0))
         for m, n in shapes:
@@ -452,17 +471,19 @@ def main():
     ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
     ap.add_argument("--counters", type=int, default=0, metavar="N",
                     help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
-    ap.add_argument("--gemm", action="store_true", help="also time the prompt-sized Q4_0 product on the matrix cores (M = 512, 2048)")
+    ap.add_argument("--gemm", action="store_true", help="time the prompt-sized products of Q4_K and Q6_K too (the Q4_0 ones are in every run)")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the prompt-sized products")
     ap.add_argument("--rows", action="store_true", help="also time the Q4_0, Q4_K and Q6_K products of eight rows of x (a batch's decoding step) at the model's shapes")
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
                     help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
                          "rows_kernel, rows_kernel_no_lds_pass, one_row_kernel_per_row (Q4_0), q4_K_rows_kernel, q6_K_rows_kernel, ...")
-    ap.add_argument("--layer-step", action="store_true", help="also time one decoder layer's decoding step against 2048 cached positions (batch 1, 8)")
+    ap.add_argument("--layer-step", action="store_true", help="(default; kept for older command lines)")
+    ap.add_argument("--no-layer-step", action="store_true", help="skip one decoder layer's decoding step against 2048 cached positions (batch 1, 8)")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps one by one instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip decoding with the whole random-init 8B-shaped model")
     ap.add_argument("--decode", action="store_true", help="(default; kept for older command lines)")
-    ap.add_argument("--decode-check", type=int, default=0, metavar="N",
-                    help="compare the first N greedy tokens with the CPU oracle's (minutes of CPU time for the 512-token prompt)")
+    ap.add_argument("--decode-check", type=int, default=64, metavar="N",
+                    help="compare the first N greedy tokens of the 512-token prompt with the CPU oracle's (0: skip; about a minute of CPU time for 64)")
     ap.add_argument("--no-decode-batch8", action="store_true", help="skip the second decoding run, with eight sequences")
     ap.add_argument("--decode-layers", type=int, default=32)
     ap.add_argument("--decode-batch", type=int, default=1)
@@ -550,11 +571,11 @@ def main():
         extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
         out["extra"] = extra
     del g
-    if args.gemm:
-        out["prefill_gemm"] = gemm_bench(lib, capi, torch)
+    if not args.no_gemm:
+        out["prefill_gemm"] = gemm_bench(lib, capi, torch, kquants=args.gemm)
     if args.rows:
         out["batch_rows_gemv"] = rows_bench(lib, capi, torch)
-    if args.layer_step:
+    if not args.no_layer_step:
         out["layer_step"] = layer_step_bench(capi)
     if not args.no_decode:
         out["decode"] = decode_bench(capi, layers=args.decode_layers, batch=args.decode_batch, check=args.decode_check if args.decode_linear == "q4_0" else 0,
