@@ -263,6 +263,48 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear=
             "first_tokens": out[0, :8].tolist()}
 
 
+def gemv_stamps(lib, capi, torch, n=14336, k=4096, bufs=16, launches=40):
+    """Where a launch of the whole-chip Q4_0 GEMV spends its time: every workgroup's first thread reads the device's
+    100 MHz clock at entry, once x is staged in LDS, after its first and its last row of W, and at exit
+    (mi355x_gemv_stamps). Microseconds from the first workgroup's entry, medians over `launches` launches, each
+    synchronized on its own; cold: W rotated over `bufs` copies, hot: one copy, which the caches then hold."""
+    rng = np.random.default_rng(0)
+    w0 = torch.from_numpy(bench_blocks_q4_0(rng, n * k)).to("cuda:0")
+    ws = [w0] + [w0.clone() for _ in range(bufs - 1)]
+    x = torch.randn(k, device="cuda:0")
+    y = torch.empty(n, device="cuda:0")
+    stamps = torch.zeros(5 * 1024, dtype=torch.int64, device="cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    call = lambda i: capi.check(lib.mi355x_qgemv(capi.Q4_0, ws[i % bufs].data_ptr(), x.data_ptr(), y.data_ptr(), 1, n, k, k, st))
+    for i in range(50):
+        call(i)
+    torch.cuda.synchronize()
+    capi.check(lib.mi355x_gemv_stamps(stamps.data_ptr()))
+    out = {}
+    try:
+        for name in ("cold", "hot"):
+            rows = []
+            for i in range(launches):
+                stamps.zero_()
+                torch.cuda.synchronize()
+                call(0 if name == "hot" else i + 3)
+                torch.cuda.synchronize()
+                s = stamps.cpu().numpy().reshape(-1, 5)
+                s = s[s[:, 0] != 0]
+                rel = (s - s[:, 0].min()) / 100.0
+                rows.append([rel[:, 0].max(), np.median(rel[:, 1]), rel[:, 1].max(), np.median(rel[:, 2]), rel[:, 2].max(),
+                             np.median(rel[:, 3]), rel[:, 3].max(), rel[:, 4].max(), len(s)])
+            r = np.median(np.array(rows), axis=0)
+            out[name] = {"workgroups": int(r[8]), "last_entry_us": round(float(r[0]), 2),
+                         "x_staged_us": {"median": round(float(r[1]), 2), "last": round(float(r[2]), 2)},
+                         "first_row_done_us": {"median": round(float(r[3]), 2), "last": round(float(r[4]), 2)},
+                         "last_row_done_us": {"median": round(float(r[5]), 2), "last": round(float(r[6]), 2)},
+                         "last_exit_us": round(float(r[7]), 2)}
+    finally:
+        capi.check(lib.mi355x_gemv_stamps(None))
+    return out
+
+
 def layer_step_bench(capi, cached=2048, new=33):
     """One decoder layer's decoding step against caches holding `cached` positions (batch 1 and 8): the whole
     model's step timed with two and with six layers, the difference divided by four, so that embedding, head and
@@ -471,6 +513,7 @@ def main():
     ap.add_argument("--all-shapes", action="store_true", help="also time the other decode shapes and the streaming-read ceiling")
     ap.add_argument("--counters", type=int, default=0, metavar="N",
                     help="only launch the GEMV kernel and a 256 MiB copy N times each (for rocprofv3 --pmc runs)")
+    ap.add_argument("--gemv-stamps", action="store_true", help="only: per-workgroup clock readings of the GEMV's launches (dispatch, x staging, rows, exit)")
     ap.add_argument("--gemm", action="store_true", help="time the prompt-sized products of Q4_K and Q6_K too (the Q4_0 ones are in every run)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prompt-sized products")
     ap.add_argument("--rows", action="store_true", help="also time the Q4_0, Q4_K and Q6_K products of eight rows of x (a batch's decoding step) at the model's shapes")
@@ -511,6 +554,9 @@ def main():
         print(json.dumps({"rows_counters": args.rows_counters, "launches": 4, "W_bytes": int(14336 * 4096 * per_weight)}))
         return
     n, k = 14336, 4096
+    if args.gemv_stamps:
+        print(json.dumps({"gemv_stamps": gemv_stamps(lib, capi, torch, n, k, args.bufs)}))
+        return
     g = Gemv(lib, capi, torch, n, k, args.bufs)
     g.check()
     if args.counters:
