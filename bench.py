@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes of one launch of the GEMV kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
 # reads for a copy kernel of known size (the summaries under profiles/ hold the
-# runs): FETCH_SIZE and WRITE_SIZE in KiB x 1024, scaled by 1.99976 and 1.0.
-TRAFFIC_BYTES_PER_LAUNCH = 33379431
+# runs): FETCH_SIZE 16278.986 KiB x 1024 x 1.99967 + WRITE_SIZE 56 KiB x 1024 x 1.0.
+TRAFFIC_BYTES_PER_LAUNCH = 33391224
 
 
 def gemv_bytes(n: int, k: int, block_bytes: int = 18) -> int:
