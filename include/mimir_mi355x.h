@@ -128,7 +128,14 @@ MI355X_API mi355x_status mi355x_qgemv_noalloc(int dtype, const void* W, const fl
  *   Q4_K, Q6_K: quantizeRow's int8 super-blocks of 256 with their sums.
  *   Q4_0: 24-bit fixed point per block of 32 (K a multiple of 64, W dword
  *         aligned); no counterpart in the reference, whose kernels take
- *         float32 activations only. */
+ *         float32 activations only. Block floating point, not float32: an
+ *         element is held to 2^-23 of its block's largest magnitude amax_b, so
+ *         y[m, n] is within 2^-23 * sum_b amax_b * sum|w_b| of the float32
+ *         product (b over the blocks of row n), beside the float32 sums' own
+ *         2e-6 * sum|x||w|. For activations of even magnitude that is 1e-6 of
+ *         the result; next to an element 1e6 times the rest of its block the
+ *         small ones keep three of their bits. mi355x_tune("q4_0.path", 1)
+ *         keeps every Q4_0 product on the float32 kernel instead. */
 MI355X_API size_t mi355x_act_bytes(int dtype, int64_t K);
 MI355X_API mi355x_status mi355x_convert_act(int dtype, const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, void* stream);
 MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* act, float* y, int64_t M, int64_t N, int64_t K, void* stream);
