@@ -289,7 +289,8 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
         }
         __syncthreads();
         if (!s_last) return;
-        // the last workgroup of these heads to get here combines the shares
+        // the last workgroup of these heads to get here combines the shares: their (max, sum) and the first eight shares'
+        // values are requested together, one trip to memory for both
         float* fs = osl + g * 64;  // factor of share s of head g
         float f = 0.f, ls = 0.f, ms = -__builtin_inff();
         const float* w0 = ws + ((int64_t)b * p.H + h) * nsplit * (D + 2);
@@ -297,6 +298,16 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
             ms = coherent_load(w0 + lane * (D + 2));
             ls = coherent_load(w0 + lane * (D + 2) + 1);
         }
+        float t[8][OPL];
+        auto load_shares = [&](int s0) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;
+#pragma unroll
+                for (int c = 0; c < OPL; c++) t[u][c] = coherent_load(w0 + s * (D + 2) + 2 + lane + 64 * c);
+            }
+        };
+        if (g < ng) load_shares(0);
         M = wave_max(ms);
         if (ls != 0.f && M > -__builtin_inff()) f = __builtin_expf(ms - M);
         L = wave_sum(ls * f);
@@ -306,13 +317,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
         for (int c = 0; c < OPL; c++) r[c] = 0.f;
         if (g < ng) {
             for (int s0 = 0; s0 < nsplit; s0 += 8) {  // eight shares' loads in flight
-                float t[8][OPL];
-#pragma unroll
-                for (int u = 0; u < 8; u++) {
-                    const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;
-#pragma unroll
-                    for (int c = 0; c < OPL; c++) t[u][c] = coherent_load(w0 + s * (D + 2) + 2 + lane + 64 * c);
-                }
+                if (s0 > 0) load_shares(s0);
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
                     const float fsv = s0 + u < nsplit ? fs[s0 + u] : 0.f;
