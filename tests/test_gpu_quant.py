@@ -91,6 +91,58 @@ def test_q4_0_gemv_matches_oracle(n, k):
     assert rel_l2(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (6144, 4096), (257, 4096 + 64), (1000, 128), (7, 8192), (512, 64)])
+def test_q4_0_gemv_both_launch_shapes_agree(n, k):
+    """One row of float32 x goes to the kernel with a workgroup per compute unit (x digits in registers, rows in chunks
+    of 64 pairs of blocks); "q4_0.stream" = 1 keeps it on the finer-grained launch. Same integers and the same float32
+    operation per block in both: each within the oracle's bound, and equal to each other to the order of a row's sums."""
+    rng = np.random.default_rng(n + 7 * k)
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    got = {}
+    try:
+        for off in (0, 1):
+            capi.check(l.mi355x_tune(b"q4_0.stream", off))
+            gpu.say(f"q4_0 gemv N={n} K={k}, whole-chip kernel {'off' if off else 'on'}")
+            got[off] = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+            check_close(got[off], want, TOL, f"q4_0 {n}x{k} stream off={off}")
+    finally:
+        capi.check(l.mi355x_tune(b"q4_0.stream", 0))
+    scale = np.abs(want).max()
+    assert np.abs(got[0] - got[1]).max() <= 4e-6 * scale
+
+
+def test_q4_0_gemv_clock_readings():
+    """mi355x_gemv_stamps: five readings of the 100 MHz clock per workgroup of the whole-chip kernel, in order, the launch
+    a few microseconds long; NULL stops it (the buffer is then left alone)."""
+    rng = np.random.default_rng(2)
+    n, k = 14336, 4096
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    stamps = torch.zeros(5 * 1024, dtype=torch.int64, device="cuda:0")
+    gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    try:
+        capi.check(l.mi355x_gemv_stamps(stamps.data_ptr()))
+        gpu.say("q4_0 gemv with clock readings")
+        got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    finally:
+        capi.check(l.mi355x_gemv_stamps(None))
+    check_close(got, O.qmatmul(O.Q4_0, raw, x, n, k), TOL)
+    s = stamps.cpu().numpy().reshape(-1, 5)
+    s = s[s[:, 0] != 0]
+    assert 64 <= len(s) <= 512
+    assert np.all(np.diff(s, axis=1) >= 0)
+    assert 100 <= s[:, 4].max() - s[:, 0].min() <= 10000  # 1 us to 100 us in ticks of 10 ns
+    stamps.zero_()
+    gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    assert int(stamps.abs().sum()) == 0
+
+
 def test_q4_0_gemv_random_scales_and_unaligned_start():
     """Weights that start a row into a buffer, 18 bytes past a 256-byte
     boundary (kerneltest/quant.go:89-92), with scales of either sign,
