@@ -102,7 +102,7 @@ struct Q4Job {
 
 constexpr int kHeadAct = 0, kHeadNorm = 1, kHeadConvert = 2;
 
-// ---- one pair of blocks a lane, the digits of x in registers (qgemv_q4_0_stream.hip, llm_step.hip) ----
+// ---- one pair of blocks a lane, the digits of x in registers (qgemv_q4_0_stream.hip) ----
 struct PairRegs {
     u32x4 a, b;
     uint32_t c;

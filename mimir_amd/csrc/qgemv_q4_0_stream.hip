@@ -1,6 +1,6 @@
 // The fixed-point Q4_0 product of one row of x (or a few, each on its own) shaped for the
-// whole chip: one workgroup per compute unit, every load of the matrix requested in the first
-// microsecond, and the arithmetic done row by row as the rows arrive.
+// whole chip: one workgroup per compute unit, up to four rows of the matrix in flight per
+// wavefront from the moment x is staged, and the arithmetic done row by row as the rows arrive.
 //
 // The arithmetic is that of qgemv_q4_0_i4_kernel (qgemv_q4_0.hip; what the reference's CPU
 // computes for a Q4_0 linear is the float32 product with the dequantized weights,
