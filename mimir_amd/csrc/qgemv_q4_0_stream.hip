@@ -36,6 +36,8 @@ namespace mimir {
 
 namespace {
 
+constexpr size_t kStreamLdsMost = 64 * 1024;  // dynamic LDS of a launch
+
 struct StreamShape {
     int items_per_wg;  // items a workgroup owns
     int nchunks;       // chunks a row is cut into (wavefronts per row)
@@ -324,12 +326,7 @@ hipError_t launch_stream(const Q4Job& job, const void* act, float* y, int64_t M,
     const size_t act_bytes = q4_0_act_bytes(K);
     const size_t part_bytes = pl.sh.nchunks > 1 ? (size_t)pl.sh.items_per_wg * RR * pl.sh.nchunks * 4 : 0;
     const size_t lds_bytes = act_bytes + part_bytes;
-    static std::atomic<bool> raised{false};
-    if (lds_bytes > 64 * 1024 && !raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemv_q4_0_stream_kernel<MODE, HEAD, NIT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        raised = true;
-    }
+    if (lds_bytes > kStreamLdsMost) return hipErrorInvalidValue;  // the dispatch keeps such products off this kernel
     dim3 grid((unsigned)pl.grid, (unsigned)M);
     long long* stamps = g_stamps.load(std::memory_order_relaxed);
     hipEvent_t t0, t1;
@@ -368,13 +365,16 @@ bool q4_0_stream_dispatch(int mode, const Q4Job& job, const void* act, float* y,
     if (g_stream_off.load(std::memory_order_relaxed) == 1 || M < 1 || M > 4 || K % 64 != 0) return false;
     const int npairs = (int)(K / 64);
     const int head = job.norm_w ? kHeadNorm : job.norm_x ? kHeadConvert : kHeadAct;
-    if (q4_0_act_bytes(K) > 120 * 1024) return false;
     const int nitems = mode == kRope ? job.total / 2 : job.total;
     if (mode == kRope && (job.total % 2 != 0 || job.n[0] % 2 != 0 || job.n[1] % 2 != 0)) return false;
     if (mode != kPlain && mode != kRope) return false;
     if (head == kHeadNorm && !q4_0_norm_head_ok(K)) return false;
     const StreamPlan pl = plan_stream(nitems, npairs, head == kHeadNorm ? 4 : 1);
     if (!pl.ok) return false;
+    // x and the chunks' sums within what a launch gets of LDS without asking for more (rows of x up to some 20 000
+    // elements): longer rows and very tall matrices stay on the finer-grained launch
+    const size_t rr = mode == kRope ? 2 : 1;
+    if (q4_0_act_bytes(K) + (pl.sh.nchunks > 1 ? (size_t)pl.sh.items_per_wg * rr * pl.sh.nchunks * 4 : 0) > kStreamLdsMost) return false;
 #define STREAM_CASE(MM, HH) \
     if (mode == MM && head == HH) { *err = launch_stream_nit<MM, HH>(job, act, y, M, K, pl, st); return true; }
     // The products this shape was measured faster on than the finer-grained launch: x in float32 converted here, and the

@@ -91,7 +91,8 @@ def test_q4_0_gemv_matches_oracle(n, k):
     assert rel_l2(got, want) < 1e-5
 
 
-@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (6144, 4096), (257, 4096 + 64), (1000, 128), (7, 8192), (512, 64)])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (6144, 4096), (257, 4096 + 64), (1000, 128), (7, 8192), (512, 64),
+                                 (40, 24576), (3, 65536), (70000, 256)])  # rows past what the whole-chip kernel stages; very many rows
 def test_q4_0_gemv_both_launch_shapes_agree(n, k):
     """One row of float32 x goes to the kernel with a workgroup per compute unit (x digits in registers, rows in chunks
     of 64 pairs of blocks); "q4_0.stream" = 1 keeps it on the finer-grained launch. Same integers and the same float32
