@@ -757,8 +757,21 @@ mi355x_status mi355x_tune(const char* key, int value) {
         mimir::set_q4_rows_waves(value);
         return MI355X_OK;
     }
-    if (key && strcmp(key, "q4_0.stream") == 0) {  // 1: off
-        mimir::set_q4_stream_off(value);
+    if (key && strcmp(key, "q4_0.stream") == 0) {  // 1: the whole-chip kernel off; 3: its variant that feeds W through LDS (slower, measured) where it takes the shape
+        mimir::set_q4_stream_off(value == 1);
+        mimir::set_q4_dma_off(value != 3);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.stream_waves") == 0) {
+        mimir::set_q4_stream_waves(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.feeders") == 0) {
+        mimir::set_q4_dma_feed(value, 0);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.feed_window") == 0) {
+        mimir::set_q4_dma_feed(0, value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.batch_off") == 0) {
@@ -811,6 +824,7 @@ mi355x_status mi355x_timed_end(float* ms_each, int* n_launches) {
 // (qgemv_q4_0_stream.hip), or null to stop.
 mi355x_status mi355x_gemv_stamps(void* stamps) {
     mimir::set_q4_stream_stamps((long long*)stamps);
+    HIP_TRY(mimir::set_q4_dma_stamps((long long*)stamps), "gemv_stamps");
     return MI355X_OK;
 }
 

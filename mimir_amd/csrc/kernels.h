@@ -70,6 +70,13 @@ void set_q4_batch_off(int v);  // 1: products of several rows of x stay on the o
 struct Q4Job;
 bool q4_0_stream_dispatch(int mode, const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st, hipError_t* err);
 void set_q4_stream_off(int v);             // measurement aid: 1 keeps every product off that kernel
+// The same products with a compute unit's whole share of W requested at entry by loads that write LDS directly
+// (qgemv_q4_0_dma.hip): one row of x, 16-byte aligned W and x. Tried before q4_0_stream_dispatch; same contract, same bits.
+bool q4_0_dma_dispatch(int mode, const Q4Job& job, const void* act, float* y, int64_t M, int64_t K, hipStream_t st, hipError_t* err);
+void set_q4_dma_off(int v);                // measurement aid: not 0 keeps every product off that kernel
+void set_q4_dma_feed(int feeders, int window);  // its feeding wavefronts (1..4) and the rows each keeps under way; 0 leaves a value as it is
+hipError_t set_q4_dma_stamps(long long* p);  // measurement aid: five timestamps per workgroup of its float32-x launches (null: none)
+void set_q4_stream_waves(int v);           // measurement aid: wavefronts a workgroup of that kernel (0: its own choice)
 void set_q4_stream_stamps(long long* p);   // measurement aid: device memory for five timestamps per workgroup of its launches (null: none)
 bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,

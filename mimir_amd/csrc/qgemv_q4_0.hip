@@ -721,6 +721,7 @@ static hipError_t dispatch_q4_0_i4(const Q4Job& job, const void* act, float* y, 
     }
     if (tune[0] == 0 && tune[1] == 0 && tune[2] == 0) {  // no launch plan forced: the kernel shaped for the whole chip where it takes the shape
         hipError_t e;
+        if (q4_0_dma_dispatch(MODE, job, act, y, M, K, st, &e)) return e;
         if (q4_0_stream_dispatch(MODE, job, act, y, M, K, st, &e)) return e;
     }
     int nb = (int)(K / 32);

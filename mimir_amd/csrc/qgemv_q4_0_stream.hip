@@ -280,6 +280,7 @@ int compute_units() {
 }
 
 std::atomic<int> g_stream_off{0};         // "q4_0.stream": 1 keeps every product off this kernel
+std::atomic<int> g_stream_waves{0};       // "q4_0.stream_waves": wavefronts a workgroup, where the shape allows (0: by the cost below)
 std::atomic<long long*> g_stamps{nullptr};  // where the next launches leave their workgroups' timestamps, if anywhere
 
 struct StreamPlan {
@@ -304,10 +305,12 @@ StreamPlan plan_stream(int nitems, int npairs, int min_waves) {
     const int max_waves = grid > cus ? 8 : 16;
     if (grid > 2 * cus) return pl;
     int best_cost = 1 << 30, best_waves = 0, best_nit = 0;
+    const int forced = g_stream_waves.load(std::memory_order_relaxed);
     for (int w = nchunks; w <= max_waves; w += nchunks) {
         if (w < min_waves) continue;
         const int nrl = w / nchunks, nit = (ipw + nrl - 1) / nrl;
         if (nit > 8) continue;
+        if (forced > 0 && w != forced) continue;
         const int cost = nit * ((w + 3) / 4);  // rows the busiest SIMD multiplies
         if (cost < best_cost || (cost == best_cost && w > best_waves)) best_cost = cost, best_waves = w, best_nit = nit;
     }
@@ -357,6 +360,7 @@ hipError_t launch_stream_nit(const Q4Job& job, const void* act, float* y, int64_
 }  // namespace
 
 void set_q4_stream_off(int v) { g_stream_off = v; }
+void set_q4_stream_waves(int v) { g_stream_waves = v; }
 void set_q4_stream_stamps(long long* p) { g_stamps = p; }
 
 // Whether this kernel takes the product (then *err is the launch's status). mode: a Q4Mode; head: kHeadAct, kHeadNorm or

@@ -116,6 +116,39 @@ def test_q4_0_gemv_both_launch_shapes_agree(n, k):
     assert np.abs(got[0] - got[1]).max() <= 4e-6 * scale
 
 
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (4096, 4096), (1024, 4096), (6144, 4096), (1000, 4096), (300, 8192), (50, 2048)])
+def test_q4_0_gemv_fed_through_lds_gives_the_same_bits(n, k):
+    """"q4_0.stream" = 3 selects the whole-chip kernel's variant whose weights reach LDS by loads that write it directly,
+    requested by wavefronts that do nothing else (slower on this device, kept for measurement). Same integers, same
+    float32 operations in the same order as the default whole-chip kernel: the same bits from float32 x, and from
+    converted x where the default is that kernel's order too, for any number of feeding wavefronts and rows under way."""
+    rng = np.random.default_rng(3 * n + k)
+    raw = bench_blocks(rng, O.Q4_0, n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    l = gpu.lib()
+    buf, ptr = gpu.dev_bytes_at(raw, 0)
+    want = O.qmatmul(O.Q4_0, raw, x, n, k)
+    base = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    base_act = gpu.qgemv_act(O.Q4_0, ptr, gpu.dev(x), n, k)
+    check_close(base, want, TOL)
+    try:
+        capi.check(l.mi355x_tune(b"q4_0.stream", 3))
+        for feeders, window in ((8, 3), (2, 20), (5, 1)):
+            capi.check(l.mi355x_tune(b"q4_0.feeders", feeders))
+            capi.check(l.mi355x_tune(b"q4_0.feed_window", window))
+            gpu.say(f"q4_0 gemv N={n} K={k} fed through LDS by {feeders} wavefronts, {window} rows under way")
+            assert bits_equal(gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k), base)
+            got_act = gpu.qgemv_act(O.Q4_0, ptr, gpu.dev(x), n, k)
+            if k <= 4096:
+                assert bits_equal(got_act, base_act)
+            else:  # converted x of longer rows is otherwise multiplied by the finer-grained launch, which adds a row's blocks in another order
+                assert np.abs(got_act - base_act).max() <= 4e-6 * np.abs(want).max()
+    finally:
+        capi.check(l.mi355x_tune(b"q4_0.stream", 0))
+        capi.check(l.mi355x_tune(b"q4_0.feeders", 8))
+        capi.check(l.mi355x_tune(b"q4_0.feed_window", 3))
+
+
 def test_q4_0_gemv_clock_readings():
     """mi355x_gemv_stamps: five readings of the 100 MHz clock per workgroup of the whole-chip kernel, in order, the launch
     a few microseconds long; NULL stops it (the buffer is then left alone)."""
