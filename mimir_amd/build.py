@@ -36,6 +36,24 @@ def _compile(src: str) -> str:
     return obj
 
 
+PROBE_SRC = os.path.join(HERE, "probe", "launch_cost.hip")
+PROBE_BIN = os.path.join(LIB_DIR, "launch_cost")
+
+
+def build_probe() -> list[str]:
+    """The stand-alone launch-cost probe (no part of the library): once as it is, once with its kernels' arguments
+    preloaded into scalar registers."""
+    outs = []
+    for suffix, extra in (("", []), ("_preload", ["-mllvm", "-amdgpu-kernarg-preload-count=16", '-DPRELOAD_NOTE="16 SGPRs"'])):
+        out = PROBE_BIN + suffix
+        cmd = ["hipcc", "-O3", "-std=c++17", f"--offload-arch={ARCH}", *DEVICE_FLAGS, *extra, PROBE_SRC, "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {PROBE_SRC}:\n{r.stderr[-4000:]}")
+        outs.append(out)
+    return outs
+
+
 def build(verbose: bool = False) -> str:
     """Compiles every .hip source for gfx950 and links the shared library."""
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -48,6 +66,7 @@ def build(verbose: bool = False) -> str:
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, LIB_PATH)
+    build_probe()
     if verbose:
         print(f"built {LIB_PATH} from {len(srcs)} sources", file=sys.stderr)
     return LIB_PATH
