@@ -30,6 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # reads for a copy kernel of known size (the summaries under profiles/ hold the
 # runs): FETCH_SIZE 16278.986 KiB x 1024 x 1.99967 + WRITE_SIZE 56 KiB x 1024 x 1.0.
 TRAFFIC_BYTES_PER_LAUNCH = 33391224
+TRAFFIC_KERNEL = "qgemv_q4_0_stream_kernel<0, 2, 7>"  # the kernel those counter runs launched
 
 
 def gemv_bytes(n: int, k: int, block_bytes: int = 18) -> int:
@@ -48,38 +49,49 @@ def bench_blocks_q4_0(rng, n_elems):
 
 
 class Gemv:
-    """One Q4_0 product y = x . W^T with n_bufs HBM-resident copies of W."""
+    """One product y = x . W^T (Q4_0 unless kind says "q8_0") with n_bufs HBM-resident copies of W."""
 
-    def __init__(self, lib, capi, torch, n, k, n_bufs, seed=0):
+    def __init__(self, lib, capi, torch, n, k, n_bufs, seed=0, kind="q4_0"):
         self.lib, self.capi, self.torch, self.n, self.k, self.n_bufs = lib, capi, torch, n, k, n_bufs
+        self.kind, self.dt, self.block_bytes = kind, (capi.Q4_0 if kind == "q4_0" else capi.Q8_0), (18 if kind == "q4_0" else 34)
         rng = np.random.default_rng(seed)
-        self.raw = bench_blocks_q4_0(rng, n * k)
+        self.raw = bench_blocks_q4_0(rng, n * k) if kind == "q4_0" else q_blocks(rng, "q8_0", n * k)
         self.x = rng.normal(size=k).astype(np.float32)
         w0 = torch.from_numpy(self.raw).to("cuda:0")
         self.bufs = [w0] + [w0.clone() for _ in range(n_bufs - 1)]
         self.xd = torch.from_numpy(self.x).to("cuda:0")
         self.y = torch.empty(n, dtype=torch.float32, device="cuda:0")
-        self.act = torch.empty(lib.mi355x_act_bytes(capi.Q4_0, k) + 64, dtype=torch.uint8, device="cuda:0")
+        self.act = torch.empty(lib.mi355x_act_bytes(self.dt, k) + 64, dtype=torch.uint8, device="cuda:0")
         self.stream = torch.cuda.Stream()
+
+    def bytes(self):
+        return gemv_bytes(self.n, self.k, self.block_bytes)
 
     def step(self, i):
         """The boundary's product, float32 x in and float32 y out: one launch, whose workgroups
         convert x to the kernel's fixed-point form for themselves before they multiply."""
-        self.capi.check(self.lib.mi355x_qgemv(self.capi.Q4_0, self.bufs[i % self.n_bufs].data_ptr(), self.xd.data_ptr(), self.y.data_ptr(),
+        self.capi.check(self.lib.mi355x_qgemv(self.dt, self.bufs[i % self.n_bufs].data_ptr(), self.xd.data_ptr(), self.y.data_ptr(),
                                               1, self.n, self.k, self.k, self.stream.cuda_stream))
+
+    def kernel_name(self):
+        """Which kernel the library's dispatch launched for the latest step of this thread."""
+        import ctypes as C
+        buf = C.create_string_buffer(200)
+        self.capi.check(self.lib.mi355x_last_kernel(buf, 200))
+        return buf.value.decode()
 
     kernel = step  # the step is its dominant kernel and nothing else
 
     def from_converted(self, i):
         """The same product over activations converted beforehand (what a decoding step's fused launches use)."""
-        self.capi.check(self.lib.mi355x_qgemv_act(self.capi.Q4_0, self.bufs[i % self.n_bufs].data_ptr(), self.act.data_ptr(), self.y.data_ptr(),
+        self.capi.check(self.lib.mi355x_qgemv_act(self.dt, self.bufs[i % self.n_bufs].data_ptr(), self.act.data_ptr(), self.y.data_ptr(),
                                                   1, self.n, self.k, self.stream.cuda_stream))
 
     def check(self):
         """Both routes against the oracle, before anything is timed."""
         import oracle as O
-        want = O.qmatmul(O.Q4_0, self.raw, self.x, self.n, self.k)
-        self.capi.check(self.lib.mi355x_convert_act(self.capi.Q4_0, self.xd.data_ptr(), 1, self.k, self.k, self.act.data_ptr(), self.stream.cuda_stream))
+        want = O.qmatmul(O.Q4_0 if self.kind == "q4_0" else O.Q8_0, self.raw, self.x, self.n, self.k)
+        self.capi.check(self.lib.mi355x_convert_act(self.dt, self.xd.data_ptr(), 1, self.k, self.k, self.act.data_ptr(), self.stream.cuda_stream))
         for name, fn in (("qgemv", self.step), ("qgemv_act", self.from_converted)):
             self.y.zero_()
             self.torch.cuda.synchronize()
@@ -109,6 +121,46 @@ class Gemv:
             raise SystemExit(f"bench: {n.value} timed launches, want {steps}")
         us = np.array(ms[:steps], np.float64) * 1e3
         return float(us.mean()), float(us.min()), float(us.max())
+
+    def time_independent(self, width, rounds=64):
+        """Microseconds per product when `width` chains of them run side by side with no edges between the chains:
+        each chain is a graph of `rounds` products on a stream of its own (its own copies of W, its own y), all
+        launched together. What of a launch's ramp and tail another chain's launches can fill."""
+        torch = self.torch
+        sides = [torch.cuda.Stream() for _ in range(width)]
+        ys = [torch.empty_like(self.y) for _ in range(width)]
+        def call(i, w):
+            self.capi.check(self.lib.mi355x_qgemv(self.dt, self.bufs[i % self.n_bufs].data_ptr(), self.xd.data_ptr(), ys[w].data_ptr(),
+                                                  1, self.n, self.k, self.k, sides[w].cuda_stream))
+        graphs = []
+        for w in range(width):
+            with torch.cuda.stream(sides[w]):
+                call(w, w)
+                sides[w].synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=sides[w]):
+                    for r in range(rounds):
+                        call(r * width + w, w)
+                g.replay()
+                sides[w].synchronize()
+            graphs.append(g)
+        main = self.stream
+        reps = 4
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(main)
+        for w in range(width):
+            sides[w].wait_event(e0)
+        for _ in range(reps):
+            for w in range(width):
+                with torch.cuda.stream(sides[w]):
+                    graphs[w].replay()
+        for w in range(width):
+            done = torch.cuda.Event()
+            done.record(sides[w])
+            main.wait_event(done)
+        e1.record(main)
+        main.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * rounds * width)
 
     def time(self, fn, steps, warmup, graph=True):
         """Milliseconds per call of fn over exactly `steps` calls after `warmup`,
@@ -221,7 +273,7 @@ def build_llama(capi, layers=32, batch=1, context=1024, max_tokens=512, seed=0, 
     return m
 
 
-def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear="q4_0"):
+def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear="q4_0", want_tokens=None):
     """Whole-model greedy decoding: a prompt of uniform-random token ids, then
     `new` tokens a sequence. Returns tokens/s of the decoding steps. With
     check, the first `check` tokens of sequence 0 are compared with the CPU
@@ -233,6 +285,12 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear=
     out, (t_prompt, t_decode) = m.generate(toks, new)
     per_tok_bytes = layers * 218103808 * {"q4_0": 0.5625, "q4_K": 0.5625, "q6_K": 0.8203125}[linear] + 128256 * 4096 * 1.0625
     verdict = {}
+    if want_tokens:
+        # sequence 0 of a batch has the prompt of the one-sequence run: its tokens against the oracle's of that run
+        got = out[0, :len(want_tokens)].tolist()
+        first = next((i for i, (a, b) in enumerate(zip(got, want_tokens)) if a != b), None)
+        verdict = {"greedy_checked": len(want_tokens), "greedy_identical": sum(a == b for a, b in zip(got, want_tokens)), "first_mismatch": first,
+                   "checked": "sequence 0 against the CPU oracle's tokens for the same prompt"}
     if check:
         import oracle as O
         from oracle import llama as OL
@@ -256,11 +314,11 @@ def decode_bench(capi, layers=32, batch=1, prompt=512, new=256, check=0, linear=
         got = out[0, :check].tolist()
         first = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), None)
         verdict = {"greedy_checked": check, "greedy_identical": sum(a == b for a, b in zip(got, want)), "first_mismatch": first,
-                   "oracle_min_margin": round(min(margins), 4)}
+                   "oracle_min_margin": round(min(margins), 4), "oracle_tokens": want}
     return {**verdict, "linear_dtype": linear, "layers": layers, "batch": batch, "prompt": prompt, "new": new, "prompt_s": round(t_prompt, 4), "decode_s": round(t_decode, 4),
             "decode_tok_per_s": round(batch * (new - 1) / t_decode, 1), "ms_per_step": round(t_decode / (new - 1) * 1e3, 4),
             "weight_GBps": round(per_tok_bytes / (t_decode / (new - 1)) / 1e9, 1), "build_s": round(build_s, 1),
-            "first_tokens": out[0, :8].tolist()}
+            "first_tokens": out[0, :8].tolist(), "distinct_tokens": len(set(out[0].tolist()))}
 
 
 def gemv_stamps(lib, capi, torch, n=14336, k=4096, bufs=16, launches=40):
@@ -471,6 +529,51 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
     return out
 
 
+def shapes_bench(lib, capi, torch, launches=1024):
+    """The one-row products of the other configurations, each as the boundary takes it (float32 x in, one
+    mi355x_qgemv call, graph-replayed over rotating copies of W that together exceed the last-level cache):
+    the Q8_0 4096 x 4096 product and the Q4_0 down, q/o and k/v shapes. Checked against the oracle before timing."""
+    out = {}
+    for name, kind, n, k in (("q8_0_4096x4096", "q8_0", 4096, 4096), ("q4_0_down_14336->4096", "q4_0", 4096, 14336),
+                             ("q4_0_qo_4096->4096", "q4_0", 4096, 4096), ("q4_0_kv_4096->1024", "q4_0", 1024, 4096)):
+        bb = 18 if kind == "q4_0" else 34
+        nb = int(min(256, max(16, 600e6 // gemv_bytes(n, k, bb) + 1)))
+        g = Gemv(lib, capi, torch, n, k, nb, kind=kind)
+        g.check()
+        ms, _ = g.time(g.step, max(launches, 2 * nb) // nb * nb, 2 * nb)
+        gbps = g.bytes() / (ms * 1e-3) / 1e9
+        out[name] = {"N": n, "K": k, "us_per_step": round(ms * 1e3, 3), "bytes": g.bytes(), "GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBS, 4),
+                     "copies_of_W": nb}
+        if kind == "q4_0":
+            g.step(0)
+            out[name]["kernel"] = g.kernel_name()
+        del g
+    return out
+
+
+def cpu_baseline_q8_0(n=4096, k=4096, seconds=5.0):
+    """The reference's CPU route for a Q8_0 linear, restated by the oracle: x rounded to int8 per block of 32
+    (quantizeRow, backend/cpu/qmatmul.go:208-254), then the AVX2 integer dot products
+    (tools/asmgen/qamd64/main.go:173-226) over rows of W shared among all host cores (qmatmul.go:285-302)."""
+    import oracle as O
+    rng = np.random.default_rng(0)
+    raw = q_blocks(rng, "q8_0", n * k)
+    x = rng.normal(size=k).astype(np.float32)
+    threads = O.lib().mo_num_threads()
+    simd = bool(O.lib().mo_has_simd())
+    O.qmatmul(O.Q8_0, raw, x, n, k, simd=simd)  # warm
+    iters, t0 = 0, time.perf_counter()
+    while True:
+        O.qmatmul(O.Q8_0, raw, x, n, k, simd=simd)
+        iters += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds and iters >= 5:
+            break
+    per = dt / iters
+    return {"value": round(gemv_bytes(n, k, 34) / per / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port", "avx2": simd,
+            "sample": f"{iters} Q8_0 products {n}x{k} (quantizeRow of x, then int8 dot products, {per * 1e6:.1f} us each), {dt:.1f} s wall"}
+
+
 def cpu_baseline(n, k, seconds=2.0):
     """The reference's CPU route for a Q4_0 linear, restated by the oracle:
     weights decoded to float32 once (untimed), then the float32 GEMV over all
@@ -516,6 +619,7 @@ def main():
     ap.add_argument("--gemv-stamps", action="store_true", help="only: per-workgroup clock readings of the GEMV's launches (dispatch, x staging, rows, exit)")
     ap.add_argument("--gemm", action="store_true", help="time the prompt-sized products of Q4_K and Q6_K too (the Q4_0 ones are in every run)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prompt-sized products")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the one-row products of the other shapes (Q8_0 4096x4096; Q4_0 down, q/o, k/v)")
     ap.add_argument("--rows", action="store_true", help="also time the Q4_0, Q4_K and Q6_K products of eight rows of x (a batch's decoding step) at the model's shapes")
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
                     help="only launch that variant of the eight-row product a few times at 14336x4096 (for rocprofv3 --pmc runs): "
@@ -579,6 +683,9 @@ def main():
     hot_ms, _ = g.time(lambda i: g.step(0), args.steps, args.warmup, graph=True)  # one copy of W: the last-level cache serves it
     kern_us, kern_min, kern_max = g.kernel_durations(args.steps, args.warmup)
     bytes_ = gemv_bytes(n, k)
+    g.step(0)
+    kernel = g.kernel_name()  # what the library's dispatch launched for this shape
+    g.stream.synchronize()
     value = bytes_ / (step_ms * 1e-3) / 1e9
     achieved = bytes_ / (kern_us * 1e-6) / 1e9
     out = {
@@ -592,8 +699,8 @@ def main():
                                + ("launched one by one" if args.eager else "replayed from a HIP graph"),
                    "N": n, "K": k, "M": 1, "wall_ms_per_step": round(step_wall_ms, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "qgemv_q4_0_stream_kernel<0, 2, 7>", "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH if kernel == TRAFFIC_KERNEL else None,
+                     "kernel": kernel, "bytes_per_launch": bytes_, "us_per_launch": round(kern_us, 3),
                      "us_min": round(kern_min, 3), "us_max": round(kern_max, 3),
                      # the product over activations converted beforehand (as a decoding step's launches take them),
                      # back to back in a graph, the wait between dependent kernels included
@@ -603,6 +710,8 @@ def main():
     }
     # what a plain 128-bit streaming read of the same bytes, over as many rotating buffers, reaches on this device
     out["roofline"]["stream_read_same_bytes_GBps"] = round(stream_ceiling(lib, capi, torch, 33030144, args.bufs, args.steps), 1)
+    # the same product as one, two and four chains side by side on streams of their own, no edges between the chains
+    out["roofline"]["us_per_launch_in_parallel_chains"] = {str(w): round(g.time_independent(w), 3) for w in (1, 2, 4)}
     extra = {}
     if args.all_shapes:
         for name, (nn, kk) in {"down_14336->4096": (4096, 14336), "qo_4096->4096": (4096, 4096), "kv_4096->1024": (1024, 4096)}.items():
@@ -617,6 +726,8 @@ def main():
         extra["stream_read_1GB_GBps"] = round(stream_ceiling(lib, capi, torch, 1 << 30, 2, 50), 1)
         out["extra"] = extra
     del g
+    if not args.no_shapes:
+        out["gemv_shapes"] = shapes_bench(lib, capi, torch)
     if not args.no_gemm:
         out["prefill_gemm"] = gemm_bench(lib, capi, torch, kquants=args.gemm)
     if args.rows:
@@ -628,9 +739,11 @@ def main():
                                      linear=args.decode_linear)
         if args.decode_batch == 1 and args.decode_linear == "q4_0" and args.decode_layers == 32 and not args.no_decode_batch8:
             # the same model with eight sequences: every weight read once a step for all of them
-            out["decode_batch8"] = decode_bench(capi, layers=32, batch=8)
+            out["decode_batch8"] = decode_bench(capi, layers=32, batch=8, want_tokens=out["decode"].get("oracle_tokens"))
+        out["decode"].pop("oracle_tokens", None)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n, k, seconds=10.0)
+        out["cpu_baseline_q8_0"] = cpu_baseline_q8_0(seconds=5.0)
     print(json.dumps(out), flush=True)
 
 

@@ -82,6 +82,14 @@ MI355X_API mi355x_status mi355x_download(void* dst, const void* src, size_t byte
 /* Waits for the stream, then reports and clears the device error word:
  * MI355X_ERR_INDEX if a gather read an index out of range. */
 MI355X_API mi355x_status mi355x_sync(void* stream);
+/* Frees the scratch memory the library keeps for `stream` on the current device: converted activations,
+ * attention's and argmax's partial results and tickets, qgemm_bf16's float32 copies, and the blocks kept aside
+ * when one of them grew. Waits for the stream first. For hosts that create and destroy streams (the library
+ * otherwise keeps a stream's scratch, some 5 MiB and up, for the life of the process). After it, no HIP graph
+ * recorded over this library's calls on that stream may be replayed: such a graph points into these blocks.
+ * No counterpart in the reference, whose backend owns one stream for its whole life
+ * (backend/rocm/rocm_linux.go:34-40). */
+MI355X_API mi355x_status mi355x_stream_release(void* stream);
 
 /* ---- the hot path: OpQMatMul ------------------------------------------------
  * y[m, :] = x[m, :] . W^T for m < M. W is [N, K] of a block-quantized dtype,
@@ -330,7 +338,11 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * the float32 kernel, 2 the fixed-point one); 0 restores the built-in choice.
  * "q4_0.stream" = 1 keeps Q4_0 products of one to four rows of x off the kernel
  * that runs one workgroup per compute unit (the older, finer-grained launch shape
- * then takes them).
+ * then takes them); 3 sends products of one row of x to that kernel's variant whose
+ * weights reach LDS by loads that write it directly, requested by "q4_0.feeders"
+ * (1 to 8) wavefronts of their own that keep "q4_0.feed_window" rows each under way
+ * (same bits; slower on this device, kept to be measured). "q4_0.stream_waves" = n
+ * fixes the wavefronts a workgroup of the whole-chip kernel where the shape allows.
  * "q4_0.batch_off" = 1 keeps products of several rows of x on the one-row
  * kernel, 2 puts them all on the kernel that shares W among rows of x.
  * "q4_0.rows_path" = 1 keeps Q4_0 and Q8_0 products of a few rows of x off the
@@ -368,23 +380,6 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * every weight once for all of them, 2 keeps that step but runs the rotation
  * and SwiGLU as launches of their own (3, 4: only SwiGLU, only the rotation). */
 MI355X_API mi355x_status mi355x_tune(const char* key, int value);
-/* Between timed_begin and timed_end, each launch of the fixed-point Q4_0 GEMV
- * kernel made by the calling thread (at most max_launches of them; not under
- * stream capture) is bracketed by its own pair of HIP events. timed_end waits
- * for the device and writes the milliseconds of each launch, in order. */
-MI355X_API mi355x_status mi355x_timed_begin(int max_launches);
-MI355X_API mi355x_status mi355x_timed_end(float* ms_each, int* n_launches);
-/* While stamps is not NULL, every launch of the whole-chip Q4_0 decode kernel (one to four rows of x by a Q4_0
- * matrix) writes five int64 readings of the device's 100 MHz clock per workgroup to stamps[5 * workgroup ..]: at
- * entry, once x is staged in LDS, after its first row of W, after its last, and at exit. The caller provides
- * 40 bytes per workgroup of the largest launch (at most two workgroups per compute unit) and reads them back
- * after the launch; NULL stops it. Process-wide. */
-MI355X_API mi355x_status mi355x_gemv_stamps(void* stamps);
-/* Reads `bytes` bytes at p with 128-bit loads from `grid` workgroups of
- * `threads` threads and folds them into scratch (at least grid*threads/64
- * floats): the practical ceiling of a streaming read on this device. */
-MI355X_API mi355x_status mi355x_stream_read(const void* p, size_t bytes, float* scratch, int grid, int threads, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

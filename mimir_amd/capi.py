@@ -74,6 +74,8 @@ SYMBOLS = {
     "mi355x_backend_run_batch": (C.c_uint32, [_vp, _vp]),
     "mi355x_backend_graph_replays": (_i64, [_vp]),
     "mi355x_qgemm_bf16": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "mi355x_stream_release": (C.c_uint32, [_vp]),
+    "mi355x_last_kernel": (C.c_uint32, [_vp, _sz]),
     "mi355x_timed_begin": (C.c_uint32, [_int]),
     "mi355x_timed_end": (C.c_uint32, [_vp, _vp]),
     "mi355x_gemv_stamps": (C.c_uint32, [_vp]),

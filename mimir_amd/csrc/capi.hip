@@ -2,6 +2,7 @@
 // (so that a launch never sees a shape its kernel does not expect), the
 // per-device state, and the mapping of failures onto status codes.
 #include "../../include/mimir_mi355x.h"
+#include "../../include/mimir_mi355x_measure.h"
 
 #include <hip/hip_runtime.h>
 
@@ -51,16 +52,18 @@ static __device__ __align__(256) unsigned char g_noalloc_scratch[kNoallocScratch
 // Scratch memory of the entry points that need some beyond their arguments (converted activations,
 // partial results and tickets of split attention and argmax, float32 copies of qgemm_bf16's general
 // route). One set per device and stream: calls on different streams never share a block, calls on one
-// stream are ordered by it. A block that has become too small is replaced by a larger one and is never
-// freed: work already queued, and HIP graphs a caller has instantiated over an entry point, may still
+// stream are ordered by it. A block that has become too small is replaced by a larger one and kept
+// aside: work already queued, and HIP graphs a caller has instantiated over an entry point, may still
 // read and write it, tickets included (a graph keeps the block it was recorded with and stays valid).
 // Growth at least doubles a block, so what is kept aside stays below the size of the live block.
+// mi355x_stream_release frees everything a stream holds, live and kept aside.
 struct ScratchBlock {
     void* p = nullptr;
     size_t bytes = 0;
 };
 struct StreamScratch {
     ScratchBlock act, attn, gemm, argmax;
+    std::vector<void*> retired;  // outgrown blocks
 };
 
 // Per-device state: the error word kernels OR bits into, read back at sync.
@@ -69,8 +72,7 @@ struct DeviceState {
     uint32_t* err_dev = nullptr;
     uint32_t* err_host = nullptr;  // pinned
     std::map<void*, StreamScratch> scratch;  // by stream handle
-    std::vector<void*> retired;              // outgrown blocks, kept until the process ends
-    void* fixed = nullptr;                   // this device's copy of g_fixed_scratch
+    void* fixed = nullptr;                   // this device's copy of g_noalloc_scratch
 };
 
 std::mutex g_mu;
@@ -95,11 +97,18 @@ std::atomic<int> g_tune_gemm{0};  // 1: qgemm_bf16 always takes its general rout
 std::atomic<int> g_tune_gemm_f16{0};  // 1: the Q4_0 matrix-core product with weights rounded to binary16
 std::atomic<int> g_tune_attn{0};  // 1: the general kernels also for one query position
 }
+thread_local char t_last_kernel[160] = "";
 thread_local std::vector<hipEvent_t> t_events;
 thread_local size_t t_events_used = 0;
 namespace mimir {
 void set_llama_step_mode(int mode);  // llm.hip
 void set_llama_rows_off(int v);      // llm.hip
+void note_kernel(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_last_kernel, sizeof t_last_kernel, fmt, ap);
+    va_end(ap);
+}
 bool next_timing_events(hipEvent_t* start, hipEvent_t* stop) {
     if (t_events_used + 2 > t_events.size()) return false;
     *start = t_events[t_events_used];
@@ -121,10 +130,13 @@ mi355x_status current_state(DeviceState** out) {
         HIP_TRY(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
         if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
             return fail(MI355X_ERR_INTERNAL, "mi355x: device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
-        HIP_TRY(hipMalloc((void**)&s.err_dev, 256), "hipMalloc(error word)");
-        HIP_TRY(hipMemset(s.err_dev, 0, 256), "hipMemset(error word)");
-        HIP_TRY(hipHostMalloc((void**)&s.err_host, 256, hipHostMallocDefault), "hipHostMalloc(error word)");
+        // the lookup first: if it fails nothing has been allocated that a later call would allocate again
         HIP_TRY(hipGetSymbolAddress(&s.fixed, HIP_SYMBOL(g_noalloc_scratch)), "hipGetSymbolAddress(fixed scratch)");
+        if (!s.err_dev) {
+            HIP_TRY(hipMalloc((void**)&s.err_dev, 256), "hipMalloc(error word)");
+            HIP_TRY(hipMemset(s.err_dev, 0, 256), "hipMemset(error word)");
+        }
+        if (!s.err_host) HIP_TRY(hipHostMalloc((void**)&s.err_host, 256, hipHostMallocDefault), "hipHostMalloc(error word)");
         s.ready = true;
     }
     *out = &s;
@@ -140,7 +152,8 @@ mi355x_status stream_scratch(void* stream, ScratchBlock StreamScratch::*which, s
     DeviceState* s;
     if (mi355x_status st = current_state(&s)) return st;
     std::lock_guard<std::mutex> lock(g_mu);
-    ScratchBlock& b = s->scratch[stream].*which;
+    StreamScratch& mine = s->scratch[stream];
+    ScratchBlock& b = mine.*which;
     if (b.bytes < bytes) {
         size_t want = bytes < floor ? floor : bytes;
         if (want < 2 * b.bytes) want = 2 * b.bytes;
@@ -148,13 +161,15 @@ mi355x_status stream_scratch(void* stream, ScratchBlock StreamScratch::*which, s
         hipError_t e = hipMalloc(&p, want);
         if (e != hipSuccess) return fail((mi355x_status)e, "mi355x: hipMalloc(%s scratch, %zu bytes): %s", what, want, hipGetErrorName(e));
         if (zero_prefix) {
-            e = hipMemset(p, 0, zero_prefix);
+            // on the calling stream, so that the zeros are in place before the first kernel that takes a ticket there
+            // (never under capture: the allocation above fails first)
+            e = hipMemsetAsync(p, 0, zero_prefix, (hipStream_t)stream);
             if (e != hipSuccess) {
                 (void)hipFree(p);  // nothing has seen it yet
                 return fail((mi355x_status)e, "mi355x: hipMemset(%s tickets): %s", what, hipGetErrorName(e));
             }
         }
-        if (b.p) s->retired.push_back(b.p);
+        if (b.p) mine.retired.push_back(b.p);
         b.p = p;
         b.bytes = want;
     }
@@ -709,6 +724,27 @@ mi355x_status mi355x_argmax(const float* logits, int64_t rows, int64_t n, int32_
     return MI355X_OK;
 }
 
+// Frees the scratch memory the library holds for `stream` on the current device (converted activations, attention's
+// and argmax's partial results and tickets, qgemm_bf16's float32 copies), blocks kept aside after growth included.
+// Waits for the stream first. The caller promises that no HIP graph recorded over this library's calls on that
+// stream will be replayed afterwards: such a graph points into these blocks.
+mi355x_status mi355x_stream_release(void* stream) {
+    DeviceState* s;
+    if (mi355x_status st = current_state(&s)) return st;
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = s->scratch.find(stream);
+    if (it == s->scratch.end()) return MI355X_OK;
+    StreamScratch& m = it->second;
+    hipError_t first = hipSuccess;
+    for (void* p : {m.act.p, m.attn.p, m.gemm.p, m.argmax.p})
+        if (p) { hipError_t e = hipFree(p); if (first == hipSuccess) first = e; }
+    for (void* p : m.retired) { hipError_t e = hipFree(p); if (first == hipSuccess) first = e; }
+    s->scratch.erase(it);
+    HIP_TRY(first, "hipFree(stream scratch)");
+    return MI355X_OK;
+}
+
 mi355x_status mi355x_tune(const char* key, int value) {
     static const char* keys[5] = {"q4_0.rows", "q4_0.cols", "q4_0.waves", "q4_0.no_lds", "q4_0.path"};
     for (int i = 0; i < 5; i++)
@@ -823,8 +859,15 @@ mi355x_status mi355x_timed_end(float* ms_each, int* n_launches) {
 // Where the launches of the Q4_0 product's whole-chip kernel leave five timestamps per workgroup
 // (qgemv_q4_0_stream.hip), or null to stop.
 mi355x_status mi355x_gemv_stamps(void* stamps) {
-    mimir::set_q4_stream_stamps((long long*)stamps);
+    HIP_TRY(mimir::set_q4_stream_stamps((long long*)stamps), "gemv_stamps");
     HIP_TRY(mimir::set_q4_dma_stamps((long long*)stamps), "gemv_stamps");
+    return MI355X_OK;
+}
+
+// The kernel (name and template arguments) that the calling thread's latest Q4_0 product of one row of x launched.
+mi355x_status mi355x_last_kernel(char* buf, size_t n) {
+    if (!buf || n == 0) return fail(MI355X_ERR_INTERNAL, "mi355x: last_kernel: no buffer");
+    snprintf(buf, n, "%s", t_last_kernel);
     return MI355X_OK;
 }
 

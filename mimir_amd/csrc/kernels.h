@@ -77,7 +77,7 @@ void set_q4_dma_off(int v);                // measurement aid: not 0 keeps every
 void set_q4_dma_feed(int feeders, int window);  // its feeding wavefronts (1..4) and the rows each keeps under way; 0 leaves a value as it is
 hipError_t set_q4_dma_stamps(long long* p);  // measurement aid: five timestamps per workgroup of its float32-x launches (null: none)
 void set_q4_stream_waves(int v);           // measurement aid: wavefronts a workgroup of that kernel (0: its own choice)
-void set_q4_stream_stamps(long long* p);   // measurement aid: device memory for five timestamps per workgroup of its launches (null: none)
+hipError_t set_q4_stream_stamps(long long* p);   // measurement aid: device memory for five timestamps per workgroup of its launches (null: none)
 bool q4_0_swiglu_convert_ok(int64_t N, int64_t K);
 hipError_t qgemv_q4_0_act_swiglu_convert(const void* gate, const void* up, const void* act, void* act_out, int64_t M, int64_t N,
                                          int64_t K, const Q4NormHead& norm, const int* tune, hipStream_t st);
@@ -289,6 +289,8 @@ hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 // While a measurement is on (capi.hip), hands out the next pair of events for a
 // launch to be bracketed by; false otherwise.
 bool next_timing_events(hipEvent_t* start, hipEvent_t* stop);
+// Records which kernel the calling thread's latest Q4_0 one-row product launched (printf-style), for mi355x_last_kernel.
+void note_kernel(const char* fmt, ...);
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);
 int stream_read_out_len(int grid, int threads);
 

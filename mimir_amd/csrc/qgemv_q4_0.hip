@@ -663,6 +663,7 @@ static hipError_t launch_q4_0_i4(const Q4Job& job, const void* act, float* y, in
     dim3 grid((unsigned)((job.total + rows_per_wg - 1) / rows_per_wg), (unsigned)M);
     size_t act_bytes = q4_0_act_bytes(K);
     const size_t lds_bytes = act_bytes + (MODE == kSwiGLU ? 128 : 0);  // kSwiGLU: room for a block of results
+    note_kernel("qgemv_q4_0_i4_kernel<%d, %d, %d, %d>", R, PC, MODE, HEAD);
     hipEvent_t t0, t1;
     if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
         hipExtLaunchKernelGGL((qgemv_q4_0_i4_kernel<R, PC, MODE, HEAD>), grid, dim3(64 * waves), lds_bytes, st, t0, t1, 0, job,

@@ -464,6 +464,7 @@ template <int MODE, int HEAD, int NIT, int P>
 hipError_t launch_dma(const Q4Job& job, const void* act, float* y, int64_t K, const DmaPlan& pl, hipStream_t st) {
     const size_t act_bytes = q4_0_act_bytes(K);
     dim3 grid((unsigned)pl.grid), block((unsigned)(64 * (pl.sh.nc + pl.sh.nl)));
+    note_kernel("qgemv_q4_0_dma_kernel<%d, %d, %d, %d>", MODE, HEAD, NIT, P);
     if constexpr (MODE == kPlain && HEAD == kHeadConvert) {
         if (g_dma_stamps.load(std::memory_order_relaxed)) {
             if (hipError_t e = dma_kernel_ready<MODE, HEAD, NIT, P, true>()) return e;

@@ -49,9 +49,14 @@ struct StreamShape {
 // requested ahead: up to four rows of W (sixteen wavefronts of 128 registers a lane). Measured and dropped:
 // workgroups of eight wavefronts with 256 registers and a wavefront's whole share under way from its first
 // instructions (x then arrives later, behind the other workgroups' weights); stores that bypass the cache.
-template <int MODE, int HEAD, int NIT>
+// Where the instantiation that takes clock readings leaves them (null: nowhere).
+__device__ long long* g_stream_stamps_dev = nullptr;
+
+// STAMPS: the build that reads the clock at five points per workgroup (a measurement aid, launched only on request).
+template <int MODE, int HEAD, int NIT, bool STAMPS = false>
 __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, const uint8_t* __restrict__ act, float* __restrict__ y, int nb,
-                                                                       int64_t act_row_bytes, StreamShape sh, long long* __restrict__ stamps) {
+                                                                       int64_t act_row_bytes, StreamShape sh) {
+    long long* const stamps = STAMPS ? g_stream_stamps_dev : nullptr;
     static_assert(MODE == kPlain || MODE == kRope, "the modes this launch shape is faster on");
     constexpr int RR = MODE == kRope ? 2 : 1;  // rows of W an item reads
     constexpr int kMaxRows = 4;
@@ -72,7 +77,7 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
     const int item_end = item0 + sh.items_per_wg < nitems ? item0 + sh.items_per_wg : nitems;
     const int rope_pos = MODE == kRope ? *job.rope.pos : 0;
     long long t_entry = 0;
-    if (stamps && tid == 0) t_entry = wall_clock64();
+    if (STAMPS && tid == 0) t_entry = wall_clock64();
 
     // the lane's pair of blocks; lanes beyond the chunk (or the row) re-read its first pair and add nothing
     const int p_own = chunk * sh.ppc + lane;
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
         for (int t = 0; t < RR; t++) load_pair(tile[u][t], row_ptr(it, t), p);
     }
     long long t_staged = 0;
-    if (stamps && tid == 0) t_staged = wall_clock64();
+    if (STAMPS && tid == 0) t_staged = wall_clock64();
 
     // the lane's digits and scales, for every row of the launch
     u32x4 d0[kDigits], d1[kDigits];
@@ -214,10 +219,10 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
         }
 #pragma unroll
         for (int t = 0; t < RR; t++) res[i][t] = wave_sum(res[i][t]);
-        if (stamps && tid == 0 && i == 0) t_first = wall_clock64();
+        if (STAMPS && tid == 0 && i == 0) t_first = wall_clock64();
     }
     long long t_last = 0;
-    if (stamps && tid == 0) t_last = wall_clock64();
+    if (STAMPS && tid == 0) t_last = wall_clock64();
 
     // ---- the tails ----
 #pragma unroll
@@ -263,7 +268,7 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
             yr[it] = s;
         }
     }
-    if (stamps && tid == 0) {
+    if (STAMPS && stamps && tid == 0) {
         long long* s = stamps + 5 * ((int64_t)blockIdx.y * gridDim.x + blockIdx.x);
         s[0] = t_entry; s[1] = t_staged; s[2] = t_first; s[3] = t_last; s[4] = wall_clock64();
     }
@@ -331,14 +336,21 @@ hipError_t launch_stream(const Q4Job& job, const void* act, float* y, int64_t M,
     const size_t lds_bytes = act_bytes + part_bytes;
     if (lds_bytes > kStreamLdsMost) return hipErrorInvalidValue;  // the dispatch keeps such products off this kernel
     dim3 grid((unsigned)pl.grid, (unsigned)M);
-    long long* stamps = g_stamps.load(std::memory_order_relaxed);
+    note_kernel("qgemv_q4_0_stream_kernel<%d, %d, %d>", MODE, HEAD, NIT);
+    if constexpr (MODE == kPlain && HEAD == kHeadConvert) {
+        if (g_stamps.load(std::memory_order_relaxed)) {  // clock readings asked for: the build that takes them
+            hipLaunchKernelGGL((qgemv_q4_0_stream_kernel<MODE, HEAD, NIT, true>), grid, dim3(64 * pl.waves), lds_bytes, st, job, (const uint8_t*)act, y,
+                               (int)(K / 32), (int64_t)act_bytes, pl.sh);
+            return hipGetLastError();
+        }
+    }
     hipEvent_t t0, t1;
     if (next_timing_events(&t0, &t1))  // a measurement is on: this launch's own begin and end
         hipExtLaunchKernelGGL((qgemv_q4_0_stream_kernel<MODE, HEAD, NIT>), grid, dim3(64 * pl.waves), lds_bytes, st, t0, t1, 0, job, (const uint8_t*)act, y,
-                              (int)(K / 32), (int64_t)act_bytes, pl.sh, stamps);
+                              (int)(K / 32), (int64_t)act_bytes, pl.sh);
     else
         hipLaunchKernelGGL((qgemv_q4_0_stream_kernel<MODE, HEAD, NIT>), grid, dim3(64 * pl.waves), lds_bytes, st, job, (const uint8_t*)act, y, (int)(K / 32),
-                           (int64_t)act_bytes, pl.sh, stamps);
+                           (int64_t)act_bytes, pl.sh);
     return hipGetLastError();
 }
 
@@ -361,7 +373,10 @@ hipError_t launch_stream_nit(const Q4Job& job, const void* act, float* y, int64_
 
 void set_q4_stream_off(int v) { g_stream_off = v; }
 void set_q4_stream_waves(int v) { g_stream_waves = v; }
-void set_q4_stream_stamps(long long* p) { g_stamps = p; }
+hipError_t set_q4_stream_stamps(long long* p) {  // synchronous
+    g_stamps = p;
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_stream_stamps_dev), &p, sizeof(p));
+}
 
 // Whether this kernel takes the product (then *err is the launch's status). mode: a Q4Mode; head: kHeadAct, kHeadNorm or
 // kHeadConvert, as the job's fields say. Few rows of x only: each is a pass over W of its own.

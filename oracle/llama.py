@@ -241,9 +241,11 @@ class Model:
 
 # ---- synthetic models in the shapes the benchmark configurations name -----
 
-def _q_blocks(rng, dt, n, k):
+def _q_blocks(rng, dt, n, k, centered=False):
     """Random blocks of dtype dt for an [n, k] weight: quants uniform over their range, binary16 scales
-    |N(0, 0.02)| (divided by 32 for the K-quants, whose sub-block scales multiply them)."""
+    |N(0, 0.02)| (divided by 32 for the K-quants, whose sub-block scales multiply them). centered (Q4_0): nibbles
+    1..15 only, so that the weights -7..7 have no mean (uniform nibbles 0..15 average -0.5, which gives every
+    linear a common-mode term that swamps what depends on the token)."""
     def half(count, scale):
         d = np.abs(rng.normal(0, scale, count)).astype(np.float32).astype(np.float16).view(np.uint16)
         return np.stack([d & 0xff, d >> 8], 1).astype(np.uint8)
@@ -262,7 +264,11 @@ def _q_blocks(rng, dt, n, k):
     b = np.empty((nb, bb), np.uint8)
     b[:, 0:2] = half(nb, 0.02)
     if dt == O.Q4_0:
-        b[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
+        if centered:
+            nib = rng.integers(1, 16, (nb, 32), dtype=np.uint8)
+            b[:, 2:] = nib[:, :16] | (nib[:, 16:] << 4)
+        else:
+            b[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
     else:
         b[:, 2:] = rng.integers(-127, 128, (nb, 32)).astype(np.int8).view(np.uint8)
     return Weight(dt, n, k, b.reshape(-1))
@@ -277,10 +283,12 @@ def tensor_seed(seed: int, name: str) -> int:
     return h
 
 
-def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: int = O.Q8_0, output_dt: int | None = None) -> Model:
+def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: int = O.Q8_0, output_dt: int | None = None,
+              centered: bool = False) -> Model:
     """A random-init Llama: linear weights of linear_dt, embeddings and the
     output projection of table_dt, norm weights N(1, 0.02); block scales
-    |N(0, 0.02)| as binary16, quants uniform over their range."""
+    |N(0, 0.02)| as binary16, quants uniform over their range (centered: Q4_0
+    linears drawn without a mean, see _q_blocks)."""
     c = config
     m = Model(c)
 
@@ -296,8 +304,8 @@ def synthetic(config: Config, seed: int = 0, linear_dt: int = O.Q4_0, table_dt: 
         m.blocks.append(Block(
             attn_norm=rng(p + "attn_norm.weight").normal(1, 0.02, c.embed).astype(np.float32),
             ffn_norm=rng(p + "ffn_norm.weight").normal(1, 0.02, c.embed).astype(np.float32),
-            q=_q_blocks(rng(p + "attn_q.weight"), linear_dt, qd, c.embed), k=_q_blocks(rng(p + "attn_k.weight"), linear_dt, kvd, c.embed),
-            v=_q_blocks(rng(p + "attn_v.weight"), linear_dt, kvd, c.embed), o=_q_blocks(rng(p + "attn_output.weight"), linear_dt, c.embed, qd),
-            gate=_q_blocks(rng(p + "ffn_gate.weight"), linear_dt, c.hidden, c.embed), up=_q_blocks(rng(p + "ffn_up.weight"), linear_dt, c.hidden, c.embed),
-            down=_q_blocks(rng(p + "ffn_down.weight"), linear_dt, c.embed, c.hidden)))
+            q=_q_blocks(rng(p + "attn_q.weight"), linear_dt, qd, c.embed, centered), k=_q_blocks(rng(p + "attn_k.weight"), linear_dt, kvd, c.embed, centered),
+            v=_q_blocks(rng(p + "attn_v.weight"), linear_dt, kvd, c.embed, centered), o=_q_blocks(rng(p + "attn_output.weight"), linear_dt, c.embed, qd, centered),
+            gate=_q_blocks(rng(p + "ffn_gate.weight"), linear_dt, c.hidden, c.embed, centered), up=_q_blocks(rng(p + "ffn_up.weight"), linear_dt, c.hidden, c.embed, centered),
+            down=_q_blocks(rng(p + "ffn_down.weight"), linear_dt, c.embed, c.hidden, centered)))
     return m

@@ -1,5 +1,5 @@
-"""The C-ABI library loads and exports every symbol include/mimir_mi355x.h
-declares. No compute call is made: this runs without a GPU."""
+"""The C-ABI library loads and exports every symbol that the headers under include/ declare (the boundary in
+mimir_mi355x.h, the measurement aids in mimir_mi355x_measure.h). No compute call is made: this runs without a GPU."""
 import os
 import re
 
@@ -9,7 +9,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared():
-    text = open(os.path.join(ROOT, "include", "mimir_mi355x.h")).read()
+    inc = os.path.join(ROOT, "include")
+    text = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     return set(re.findall(r"MI355X_API\s+[\w\s\*]+?\b(mi355x_\w+)\s*\(", text))
 
 

@@ -84,7 +84,7 @@ def test_generate_is_the_argmax_of_a_full_pass(golden_dir):
     full = m.logits(seq[:-1], m.new_caches(len(seq)), all=True)
     for i, t in enumerate(out):
         row = full[len(prompt) - 1 + i]
-        assert O.argmax(row) == t or margins[i] < 1e-3
+        assert O.argmax(row) == t, f"token {i}: a full pass picks {O.argmax(row)}, cached steps picked {t}, margin there {margins[i]:.4g}"
 
 
 # ---- qwen2: biases on the queries, keys and values, rotation over halves -------------------------
