@@ -10,9 +10,15 @@
 // one Go function variable per entry point it uses, with the parameter list of
 // the header's declaration.
 //
+// This package has not been compiled: the image it was written in has no Go
+// toolchain. Its table of entry points is held to the header by a test of the
+// library's repository (parameter counts and kinds), nothing more.
+//
 // The backend shares the rocm backend's buffers and stream, so both sides see
 // the same memory in the same order. That needs two accessors from
-// backend/rocm, one line each beside the unexported fields they read:
+// backend/rocm, one line each beside the unexported fields they read (the
+// only symbols this package uses that the reference does not export today:
+// DevicePointer, Stream):
 //
 //	// DevicePointer returns the device address of a buffer of b.
 //	func (b *Backend) DevicePointer(buf backend.Buffer) (uint64, error) { rb, err := b.own(buf); if err != nil { return 0, err }; return rb.ptr, nil }

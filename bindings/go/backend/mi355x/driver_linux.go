@@ -3,6 +3,7 @@
 package mi355x
 
 import (
+	"errors"
 	"fmt"
 	"os"
 	"strings"
@@ -54,9 +55,8 @@ var (
 	miQGemmBF16  func(dtype int32, w, x, y uint64, m, n, k, xRowStride int64, outDType int32, stream uintptr) status
 	miDequant    func(dtype int32, w uint64, first, n int64, out uint64, outDType int32, stream uintptr) status
 	miGatherRows func(dtype int32, table uint64, rows, k int64, idx uint64, n int64, out uint64, stream uintptr) status
-	miAttention  func(q uint64, qStrides *int64, k uint64, kStrides *int64, v uint64, vStrides *int64, kvDType int32,
-		mask uint64, maskStrides *int64, out uint64, outStrides *int64, lse uint64,
-		b int64, h, hk int32, nq, nk int64, d, dv int32, scale float64, causal int32, causalOffset int64, stream uintptr) status
+	miAttention  func(desc *attentionDesc, stream uintptr) status
+	miStreamFree func(stream uintptr) status
 	miTune func(key string, value int32) status
 )
 
@@ -72,42 +72,55 @@ var (
 
 const captureModeThreadLocal = 1 // hipStreamCaptureModeThreadLocal
 
-// symbol is a function pointer to bind and the name of its symbol.
-type symbol struct {
-	fptr any
-	name string
+// attentionDesc is mi355x_attention_desc, field for field: six device addresses, the strides of queries, keys,
+// values and result ({batch, head, position}) and of the mask ({batch, head, query, key}), the sizes, the scale and
+// the 32-bit fields. One pointer to it keeps the call within what purego.RegisterFunc takes as parameters.
+type attentionDesc struct {
+	q, k, v, mask, out, lse                              uint64
+	qStrides, kStrides, vStrides, outStrides             [3]int64
+	maskStrides                                          [4]int64
+	b, nq, nk, causalOffset                              int64
+	scale                                                float64
+	kvDType, heads, kvHeads, d, dv, causal               int32
 }
 
-// libraries returns the names to try for a library: the one the environment
-// variable env names, if it is set, otherwise names.
-func libraries(env string, names ...string) []string {
-	if path := os.Getenv(env); path != "" {
-		return []string{path}
+// binding is one row of a table that load fills in: where the function goes and what the library calls it.
+type binding struct {
+	target any
+	symbol string
+}
+
+// dlopenFirst opens the library a host names in the environment variable override, or else the first of
+// candidates that the dynamic loader can open, and says why each one failed when none does.
+func dlopenFirst(override string, candidates ...string) (uintptr, error) {
+	if forced, ok := os.LookupEnv(override); ok && forced != "" {
+		candidates = []string{forced}
 	}
-	return names
-}
-
-// open loads the first of names the dynamic loader finds.
-func open(names []string) (uintptr, error) {
-	var err error
-	for _, name := range names {
-		var lib uintptr
-		if lib, err = purego.Dlopen(name, purego.RTLD_GLOBAL|purego.RTLD_NOW); err == nil {
-			return lib, nil
+	var why []string
+	for _, path := range candidates {
+		handle, err := purego.Dlopen(path, purego.RTLD_NOW|purego.RTLD_GLOBAL)
+		if err == nil {
+			return handle, nil
 		}
+		why = append(why, path+": "+err.Error())
 	}
-	return 0, fmt.Errorf("none of %s loads: %w", strings.Join(names, ", "), err)
+	return 0, errors.New("no library could be opened (" + strings.Join(why, "; ") + ")")
 }
 
-// register binds each function pointer to the symbol of lib it names, or
-// reports the first that is missing.
-func register(lib uintptr, fns []symbol) error {
-	for _, f := range fns {
-		sym, err := purego.Dlsym(lib, f.name)
+// bindAll resolves every row of table in handle. All rows are tried, so that the error names every symbol the
+// library lacks at once (a library older than this package shows up as such a list).
+func bindAll(handle uintptr, table []binding) error {
+	var absent []string
+	for _, row := range table {
+		addr, err := purego.Dlsym(handle, row.symbol)
 		if err != nil {
-			return err
+			absent = append(absent, row.symbol)
+			continue
 		}
-		purego.RegisterFunc(f.fptr, sym)
+		purego.RegisterFunc(row.target, addr)
+	}
+	if len(absent) != 0 {
+		return fmt.Errorf("symbols not found: %s", strings.Join(absent, ", "))
 	}
 	return nil
 }
@@ -115,12 +128,12 @@ func register(lib uintptr, fns []symbol) error {
 // load loads the library and the HIP graph API once.
 func load() error {
 	libOnce.Do(func() {
-		lib, err := open(libraries("MIMIR_MI355X_LIB", "libmimir_mi355x.so"))
+		lib, err := dlopenFirst("MIMIR_MI355X_LIB", "libmimir_mi355x.so")
 		if err != nil {
 			libErr = err
 			return
 		}
-		if libErr = register(lib, []symbol{
+		if libErr = bindAll(lib, []binding{
 			{&miInit, "mi355x_init"},
 			{&miLastError, "mi355x_last_error"},
 			{&miSync, "mi355x_sync"},
@@ -128,17 +141,18 @@ func load() error {
 			{&miQGemmBF16, "mi355x_qgemm_bf16"},
 			{&miDequant, "mi355x_dequant"},
 			{&miGatherRows, "mi355x_gather_rows"},
-			{&miAttention, "mi355x_attention"},
+			{&miAttention, "mi355x_attention_d"},
+			{&miStreamFree, "mi355x_stream_release"},
 			{&miTune, "mi355x_tune"},
 		}); libErr != nil {
 			return
 		}
-		hip, err := open(libraries("MIMIR_HIP", "libamdhip64.so.7", "libamdhip64.so.6", "libamdhip64.so"))
+		hip, err := dlopenFirst("MIMIR_HIP", "libamdhip64.so.7", "libamdhip64.so.6", "libamdhip64.so")
 		if err != nil {
 			libErr = err
 			return
 		}
-		libErr = register(hip, []symbol{
+		libErr = bindAll(hip, []binding{
 			{&hipStreamBeginCapture, "hipStreamBeginCapture"},
 			{&hipStreamEndCapture, "hipStreamEndCapture"},
 			{&hipGraphInstantiate, "hipGraphInstantiateWithFlags"},

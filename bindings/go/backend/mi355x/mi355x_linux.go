@@ -28,19 +28,28 @@ type Backend struct {
 
 var _ backend.Backend = (*Backend)(nil)
 
-// New returns the backend of device dev.
-func New(dev int) (*Backend, error) {
+// New returns the backend of the first ROCm device, the one rocm.New opens
+// (backend/rocm/rocm_linux.go:86-97).
+func New() (*Backend, error) {
 	if err := load(); err != nil {
 		return nil, fmt.Errorf("mi355x: %w", err)
 	}
-	rb, err := rocm.New(dev)
+	rb, err := rocm.New()
 	if err != nil {
 		return nil, err
 	}
-	if err := check(miInit(int32(dev)), "init"); err != nil {
+	if err := check(miInit(0), "init"); err != nil {
 		return nil, err
 	}
 	return &Backend{Backend: rb, stream: rb.Stream()}, nil
+}
+
+// Close gives back the scratch memory the library keeps for this backend's stream; graphs recorded
+// over it (a Batch's State) must not be replayed afterwards.
+func (b *Backend) Close() error {
+	b.mu.Lock()
+	defer b.mu.Unlock()
+	return check(miStreamFree(b.stream), "release stream scratch")
 }
 
 // Name identifies the device.
@@ -131,10 +140,11 @@ func (b *Backend) plan(k *backend.Kernel, outs, ins []backend.Buffer) call {
 		n, kk := w.Shape[0], w.Shape[1]
 		rows, stride, ok := rowsOf(x, kk)
 		// W from a block boundary, rows one after another (backend/cpu/qmatmul.go:323-332)
-		if !ok || w.Strides[1] != 1 || w.Strides[0] != kk || w.Offset%backend.BlockSize(ins[1].DType()) != 0 {
+		if !ok || w.Strides[1] != 1 || w.Strides[0] != kk || w.Offset%ins[1].DType().BlockSize() != 0 {
 			break
 		}
-		woff := uint64(backend.Bytes(ins[1].DType(), w.Offset))
+		wbytes, _ := ins[1].DType().Bytes(w.Offset) // whole blocks: the offset was just checked
+		woff := uint64(wbytes)
 		xoff := 4 * uint64(x.Offset)
 		return call{what: "qmatmul", issue: func(p []uint64) status {
 			return miQGemv(wc, p[2]+woff, p[1]+xoff, p[0], int64(rows), int64(n), int64(kk), int64(stride), stream)
@@ -242,14 +252,20 @@ func (b *Backend) planAttention(k *backend.Kernel, ins []backend.Buffer) (call, 
 		causal = 1
 	}
 	scale, coff, stream := k.Attrs.Scale, int64(k.Attrs.CausalOffset), b.stream
+	desc := attentionDesc{b: bsz, nq: int64(s.Q), nk: int64(s.K), causalOffset: coff, scale: scale, kvDType: kv,
+		heads: int32(s.Heads), kvHeads: int32(s.KVHeads), d: int32(s.D), dv: int32(s.DV), causal: causal}
+	copy(desc.qStrides[:], qs)
+	copy(desc.kStrides[:], ks)
+	copy(desc.vStrides[:], vs)
+	copy(desc.outStrides[:], os)
+	copy(desc.maskStrides[:], ms)
 	return call{what: "attention", issue: func(p []uint64) status {
-		var mask uint64
-		var msp *int64
+		d := desc // the descriptor of this issue: the same shape, this run's buffers
+		d.q, d.k, d.v, d.out, d.lse = p[1]+offs[0], p[2]+offs[1], p[3]+offs[2], p[0], p[0]+lseOff
 		if ms != nil {
-			mask, msp = p[4]+offs[3], &ms[0]
+			d.mask = p[4] + offs[3]
 		}
-		return miAttention(p[1]+offs[0], &qs[0], p[2]+offs[1], &ks[0], p[3]+offs[2], &vs[0], kv, mask, msp, p[0], &os[0], p[0]+lseOff,
-			bsz, int32(s.Heads), int32(s.KVHeads), int64(s.Q), int64(s.K), int32(s.D), int32(s.DV), scale, causal, coff, stream)
+		return miAttention(&d, stream)
 	}}, true
 }
 

@@ -223,6 +223,22 @@ MI355X_API mi355x_status mi355x_attention(const float* q, const int64_t* q_strid
                                const int64_t* v_strides, int kv_dtype, const float* mask, const int64_t* mask_strides, float* out,
                                const int64_t* out_strides, float* lse, int64_t B, int H, int HK, int64_t Q, int64_t K, int D, int DV, double scale,
                                int causal, int64_t causal_offset, void* stream);
+/* mi355x_attention with its arguments in one structure, for hosts whose foreign-function layer limits the number of
+ * parameters of a call (purego's RegisterFunc in Go): the same operation, checks and results. Strides as above;
+ * mask_strides is read only when mask is not NULL. */
+typedef struct mi355x_attention_desc {
+    const float* q;
+    const void* k;
+    const void* v;
+    const float* mask;
+    float* out;
+    float* lse;
+    int64_t q_strides[3], k_strides[3], v_strides[3], out_strides[3], mask_strides[4];
+    int64_t B, Q, K, causal_offset;
+    double scale;
+    int32_t kv_dtype, H, HK, D, DV, causal;
+} mi355x_attention_desc;
+MI355X_API mi355x_status mi355x_attention_d(const mi355x_attention_desc* desc, void* stream);
 /* Block.mlp's activation (llm/model.go:446-448): out = SiLU(gate) * up, rows of
  * gate and up in_row_stride floats apart, out contiguous. */
 MI355X_API mi355x_status mi355x_swiglu(const float* gate, const float* up, float* out, int64_t rows, int64_t n, int64_t in_row_stride, void* stream);

@@ -74,6 +74,7 @@ SYMBOLS = {
     "mi355x_backend_run_batch": (C.c_uint32, [_vp, _vp]),
     "mi355x_backend_graph_replays": (_i64, [_vp]),
     "mi355x_qgemm_bf16": (C.c_uint32, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "mi355x_attention_d": (C.c_uint32, [_vp, _vp]),
     "mi355x_stream_release": (C.c_uint32, [_vp]),
     "mi355x_last_kernel": (C.c_uint32, [_vp, _sz]),
     "mi355x_timed_begin": (C.c_uint32, [_int]),
@@ -87,6 +88,14 @@ class LlamaConfig(C.Structure):
     """mi355x_llama_config."""
     _fields_ = [(n, C.c_int32) for n in ("embed", "hidden", "layers", "heads", "kv_heads", "head_dim", "rope_dim", "vocab", "context",
                                           "interleaved", "cache_dtype", "batch")] + [(n, C.c_double) for n in ("rope_base", "rope_scale", "eps")]
+
+
+class AttentionDesc(C.Structure):
+    """mi355x_attention_desc."""
+    _fields_ = [(n, C.c_void_p) for n in ("q", "k", "v", "mask", "out", "lse")] + \
+               [("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3), ("out_strides", C.c_int64 * 3),
+                ("mask_strides", C.c_int64 * 4)] + [(n, C.c_int64) for n in ("B", "Q", "K", "causal_offset")] + [("scale", C.c_double)] + \
+               [(n, C.c_int32) for n in ("kv_dtype", "H", "HK", "D", "DV", "causal")]
 
 
 class Mi355xError(RuntimeError):

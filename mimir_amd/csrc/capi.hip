@@ -697,6 +697,12 @@ mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const v
     return MI355X_OK;
 }
 
+mi355x_status mi355x_attention_d(const mi355x_attention_desc* d, void* stream) {
+    if (!d) return fail(MI355X_ERR_INTERNAL, "mi355x: attention_d: null descriptor");
+    return mi355x_attention(d->q, d->q_strides, d->k, d->k_strides, d->v, d->v_strides, d->kv_dtype, d->mask, d->mask_strides, d->out, d->out_strides, d->lse,
+                            d->B, d->H, d->HK, d->Q, d->K, d->D, d->DV, d->scale, d->causal, d->causal_offset, stream);
+}
+
 mi355x_status mi355x_swiglu(const float* gate, const float* up, float* out, int64_t rows, int64_t n, int64_t in_row_stride, void* stream) {
     if (rows < 0 || n < 0) return fail(MI355X_ERR_SHAPE, "mi355x: swiglu of [%lld, %lld]", (long long)rows, (long long)n);
     if (rows == 0 || n == 0) return MI355X_OK;

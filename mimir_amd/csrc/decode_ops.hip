@@ -170,7 +170,10 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ q, con
                                                       int64_t q_row, int64_t k_row, int64_t v_row, void* __restrict__ kcache,
                                                       void* __restrict__ vcache, int cache_dt, int B, int H, int HK, int dim, int rope_dim,
                                                       int interleaved, int64_t cap, const float* __restrict__ cosv,
-                                                      const float* __restrict__ sinv, const int32_t* __restrict__ pos_dev) {
+                                                      const float* __restrict__ sinv, const int32_t* __restrict__ pos_dev,
+                                                      const float* __restrict__ bias) {
+    // bias: null, or [(H + 2 HK) dim] added to every sequence's heads before anything else happens to them: Linear.Forward's
+    // bias behind the product (nn/layers.go:49-55), for models whose q, k and v have one (llm/model.go:251-258)
     const int pos = *pos_dev;
     const int half = rope_dim >> 1, hd2 = dim >> 1;  // work items: pairs of features
     const int64_t total = (int64_t)B * (H + 2 * HK) * hd2;
@@ -182,12 +185,17 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ q, con
         // sequence b's heads: H of queries at q, HK of keys at k, HK of values at v, rows q_row, k_row, v_row floats apart
         const float* hp = head < H ? q + b * q_row + (int64_t)head * dim
                                    : head < H + HK ? k + b * k_row + (int64_t)(head - H) * dim : v + b * v_row + (int64_t)(head - H - HK) * dim;
+        const float* bp = bias ? bias + (int64_t)head * dim : nullptr;
         int ia, ib;
         float va, vb;
         if (head < H + HK && i < half) {
             ia = interleaved ? 2 * i : i;
             ib = interleaved ? 2 * i + 1 : i + half;
             float a = hp[ia], c2 = hp[ib];
+            if (bp) {
+                a = a + bp[ia];
+                c2 = c2 + bp[ib];
+            }
             float c = cosv[(int64_t)pos * half + i], sn = sinv[(int64_t)pos * half + i];
             float ac = a * c, bs = c2 * sn, as = a * sn, bc = c2 * c;
             va = ac - bs;
@@ -198,6 +206,10 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ q, con
             ib = ia + 1;
             va = hp[ia];
             vb = hp[ib];
+            if (bp) {
+                va = va + bp[ia];
+                vb = vb + bp[ib];
+            }
         }
         if (head < H) {
             float* qp = q + b * q_row + (int64_t)head * dim;
@@ -221,30 +233,30 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float* __restrict__ q, con
 
 static hipError_t rope_kv_launch(float* q, const float* k, const float* v, int64_t q_row, int64_t k_row, int64_t v_row, void* kcache,
                                  void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim, int interleaved, int64_t cap,
-                                 const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
+                                 const float* cosv, const float* sinv, const int32_t* pos_dev, const float* bias, hipStream_t st) {
     int64_t total = B * (H + 2 * HK) * (dim / 2);
     if (total == 0) return hipSuccess;
     int64_t groups = (total + 255) / 256;
     if (groups > 65536) groups = 65536;
     hipLaunchKernelGGL(rope_kv_kernel, dim3((unsigned)groups), dim3(256), 0, st, q, k, v, q_row, k_row, v_row, kcache, vcache, cache_dt,
-                       (int)B, H, HK, dim, rope_dim, interleaved, cap, cosv, sinv, pos_dev);
+                       (int)B, H, HK, dim, rope_dim, interleaved, cap, cosv, sinv, pos_dev, bias);
     return hipGetLastError();
 }
 
-// qkv [B, (H + 2 HK) dim]: each sequence's query, key and value heads in one row.
+// qkv [B, (H + 2 HK) dim]: each sequence's query, key and value heads in one row. bias: null, or [(H + 2 HK) dim] added first.
 hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
-                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st) {
+                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st, const float* bias) {
     const int64_t row = (int64_t)(H + 2 * HK) * dim;
     return rope_kv_launch(qkv, qkv + (int64_t)H * dim, qkv + (int64_t)(H + HK) * dim, row, row, row, kcache, vcache, cache_dt, B, H, HK, dim,
-                          rope_dim, interleaved, cap, cosv, sinv, pos_dev, st);
+                          rope_dim, interleaved, cap, cosv, sinv, pos_dev, bias, st);
 }
 
 // q [B, H dim], k and v [B, HK dim], each contiguous.
 hipError_t rope_kv_split(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim,
                          int rope_dim, int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev,
-                         hipStream_t st) {
+                         hipStream_t st, const float* bias) {
     return rope_kv_launch(q, k, v, (int64_t)H * dim, (int64_t)HK * dim, (int64_t)HK * dim, kcache, vcache, cache_dt, B, H, HK, dim, rope_dim,
-                          interleaved, cap, cosv, sinv, pos_dev, st);
+                          interleaved, cap, cosv, sinv, pos_dev, bias, st);
 }
 
 // After a step: appends the chosen tokens to the record and moves on one

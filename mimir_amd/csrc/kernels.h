@@ -169,12 +169,14 @@ bool rmsnorm_q4act_ok(int64_t d);
 hipError_t rmsnorm_q4act(const float* x, const float* w, float* y, void* act, int64_t rows, int64_t d, double eps, hipStream_t st);
 // One decoding position: rotates the queries of qkv [B, (H + 2 HK) * dim] in
 // place, rotates and caches its keys, caches its values, at position *pos_dev.
+// bias, if not null: [(H + 2 HK) * dim] float32 added to every row before that (the q, k, v biases of qwen2, concatenated).
 hipError_t rope_kv(float* qkv, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim, int rope_dim,
-                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st);
+                   int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev, hipStream_t st,
+                   const float* bias = nullptr);
 // The same for q [B, H dim], k and v [B, HK dim] in buffers of their own.
 hipError_t rope_kv_split(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dt, int64_t B, int H, int HK, int dim,
                          int rope_dim, int interleaved, int64_t cap, const float* cosv, const float* sinv, const int32_t* pos_dev,
-                         hipStream_t st);
+                         hipStream_t st, const float* bias = nullptr);
 // state = {position, steps}: record[steps] = next_tok [B], then steps += 1 and
 // position += pos_inc.
 hipError_t advance(int32_t* state, const int32_t* next_tok, int32_t* record, int B, int pos_inc, hipStream_t st);

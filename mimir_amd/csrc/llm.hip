@@ -81,6 +81,7 @@ enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4 }; 
 struct Block {
     Weight attn_norm, ffn_norm, q, k, v, o, gate, up, down, qkv, gate_up;
     Weight q_bias, k_bias, v_bias;  // qwen2's (llm/model.go:251-258): float32 [n], all three or none
+    DevBuf qkv_bias;                // the three in one row, beside qkv
     bool biased() const { return q_bias.set(); }
 };
 
@@ -472,7 +473,7 @@ static mi355x_status step_any(Model& m) {
             const bool read_once = B >= 3 && qkv_kq && qgemv_kquant_rows_pays(b.qkv.dtype, qa);
             const bool pairs = c.interleaved && c.head_dim % 2 == 0 && c.rope_dim % 2 == 0;
             const bool once_rope = read_once && pairs && qgemv_kquant_rows_rope_ok(b.qkv.dtype, qa);
-            if (once_rope || (qkv_kq && !read_once && pairs && qgemv_kquant_rope_ok(b.qkv.dtype, qa))) {
+            if (!b.biased() && (once_rope || (qkv_kq && !read_once && pairs && qgemv_kquant_rope_ok(b.qkv.dtype, qa)))) {
                 Q4RopeTail tail;  // the rotation and the cache writes ride on the product
                 tail.cosv = m.cos_t.as<float>(); tail.sinv = m.sin_t.as<float>(); tail.pos = pos;
                 tail.kcache = m.keys[i].p; tail.vcache = m.values[i].p;
@@ -481,9 +482,11 @@ static mi355x_status step_any(Model& m) {
                 if (once_rope) LLM_HIP(qgemv_kquant_rows_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
                 else LLM_HIP(qgemv_kquant_act_rope(b.qkv.dtype, qa, tail, m.stream), "q|k|v, rope and cache");
             } else {
+                // with biases (qwen2): one product, then the biases, the rotation and the cache writes in one launch
                 if (mi355x_status st = linear(m, b.qkv, h, qkv, B)) return st;
                 LLM_HIP(rope_kv(qkv, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim, c.interleaved,
-                                c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+                                c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream,
+                                b.biased() ? b.qkv_bias.as<float>() : nullptr), "biases, rope and cache");
             }
             at.q = qkv; at.q_strides[0] = qd + 2 * kvd;
         } else {
@@ -491,13 +494,10 @@ static mi355x_status step_any(Model& m) {
             if (mi355x_status st = linear(m, b.q, h, q, B)) return st;
             if (mi355x_status st = linear(m, b.k, h, k, B)) return st;
             if (mi355x_status st = linear(m, b.v, h, v, B)) return st;
-            if (b.biased()) {
-                LLM_HIP(add_bias(q, b.q_bias.buf.as<float>(), B, qd, m.stream), "q bias");
-                LLM_HIP(add_bias(k, b.k_bias.buf.as<float>(), B, kvd, m.stream), "k bias");
-                LLM_HIP(add_bias(v, b.v_bias.buf.as<float>(), B, kvd, m.stream), "v bias");
-            }
+            // biases (qwen2), rotation and cache writes in one launch
             LLM_HIP(rope_kv_split(q, k, v, m.keys[i].p, m.values[i].p, c.cache_dtype, B, c.heads, c.kv_heads, c.head_dim, c.rope_dim,
-                                  c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
+                                  c.interleaved, c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream,
+                                  b.biased() ? b.qkv_bias.as<float>() : nullptr), "biases, rope and cache");
             at.q = q; at.q_strides[0] = qd;
         }
         at.k = m.keys[i].p; at.v = m.values[i].p;
@@ -754,7 +754,7 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     LLM_HIP(m->record.alloc(((size_t)c.context + 1) * c.batch * 4), "hipMalloc");  // a graph keeps its address
     LLM_HIP(m->qkv.alloc((size_t)c.batch * (qd + 2 * kvd) * 4), "hipMalloc");
     m->fast = rmsnorm_q4act_ok(c.embed) && c.head_dim % 2 == 0;
-    bool biased = false;  // q, k, v with biases: separate products with the additions behind them, no fused tails
+    bool biased = false;  // q, k, v with biases: the generic step, whose rotation launch adds them first
     for (int i = 0; i < c.layers; i++) biased = biased || m->blocks[i].biased();
     if (biased) m->fast = false;
     for (int i = 0; i < c.layers && m->fast; i++) {
@@ -786,8 +786,15 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
             into.dtype = first->dtype; into.n = n; into.k = first->k;
             return MI355X_OK;
         };
-        if (!biased)
-            if (mi355x_status st = fuse({&b.q, &b.k, &b.v}, b.qkv)) return st;
+        if (mi355x_status st = fuse({&b.q, &b.k, &b.v}, b.qkv)) return st;
+        if (b.biased()) {  // the three biases in one row, as the three matrices are where they share a block dtype
+            LLM_HIP(b.qkv_bias.alloc((size_t)(qd + 2 * kvd) * 4), "hipMalloc(fused biases)");
+            size_t off = 0;
+            for (const Weight* p : {&b.q_bias, &b.k_bias, &b.v_bias}) {
+                LLM_HIP(hipMemcpy((uint8_t*)b.qkv_bias.p + off, p->buf.p, p->buf.bytes, hipMemcpyDeviceToDevice), "hipMemcpy(fused biases)");
+                off += p->buf.bytes;
+            }
+        }
         if (mi355x_status st = fuse({&b.gate, &b.up}, b.gate_up)) return st;
     }
     LLM_HIP(m->gu.alloc((size_t)c.batch * 2 * c.hidden * 4), "hipMalloc");

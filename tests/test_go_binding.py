@@ -110,3 +110,47 @@ def test_the_sources_call_only_what_the_table_binds():
         c = re.search(rf"\b{c_name}\s*=\s*(\w+)", text)
         g = re.search(rf"\b{go_name}\s+status\s*=\s*(\w+)", src)
         assert c and g and int(c.group(1), 0) == int(g.group(1), 0), (go_name, c_name)
+
+
+REFERENCE = "/root/reference"
+
+
+def _go_sources():
+    return {name: re.sub(r"//[^\n]*", "", open(os.path.join(GO, name)).read()) for name in os.listdir(GO) if name.endswith(".go")}
+
+
+def test_every_symbol_of_the_reference_that_the_binding_uses_exists_there_or_is_a_listed_patch():
+    """The package cannot be compiled here, so what it takes from github.com/gsoultan/mimir is checked by name:
+    every rocm.X, every method called on the embedded rocm backend and every backend.X must be defined in the
+    reference's backend/rocm or backend packages, or be one of the additions doc.go asks a maintainer for."""
+    import pytest
+    if not os.path.isdir(REFERENCE):
+        pytest.skip("the reference tree is not here")
+    doc = open(os.path.join(GO, "doc.go")).read()
+    patches = set(re.findall(r"func \(b \*Backend\) (\w+)\(", doc))
+    assert patches == {"DevicePointer", "Stream"}, patches
+
+    def defined(pkg_dir, name, method_of=None):
+        for fn in os.listdir(pkg_dir):
+            if not fn.endswith(".go") or fn.endswith("_test.go"):
+                continue
+            text = open(os.path.join(pkg_dir, fn)).read()
+            if method_of and re.search(rf"^func \(\w+ \*?{method_of}\) {name}\(", text, flags=re.M):
+                return True
+            if not method_of and re.search(rf"^(func {name}\(|type {name}\b|var {name}\b|const {name}\b|\t{name}(\s|$))", text, flags=re.M):
+                return True
+        return False
+
+    rocm_dir, backend_dir = os.path.join(REFERENCE, "backend", "rocm"), os.path.join(REFERENCE, "backend")
+    srcs = _go_sources()
+    for name, src in srcs.items():
+        for sym in set(re.findall(r"\brocm\.(\w+)", src)):
+            assert defined(rocm_dir, sym), f"{name}: rocm.{sym} is not in the reference"
+        for sym in set(re.findall(r"\b(?:b\.Backend|rb)\.(\w+)\(", src)):
+            assert sym in patches or defined(rocm_dir, sym, "Backend"), f"{name}: (*rocm.Backend).{sym} is neither in the reference nor a listed patch"
+        for sym in set(re.findall(r"\bbackend\.(\w+)", src)):
+            assert defined(backend_dir, sym), f"{name}: backend.{sym} is not in the reference"
+    # and the constructor is called the way the reference declares it
+    new = re.search(r"^func New\(([^)]*)\)", open(os.path.join(rocm_dir, "rocm_linux.go")).read(), flags=re.M)
+    assert new and new.group(1).strip() == ""
+    assert re.search(r"rocm\.New\(\)", srcs["mi355x_linux.go"])

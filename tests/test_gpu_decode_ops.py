@@ -150,6 +150,24 @@ def attention(q, k, v, scale, causal=False, offset=0, kv_dt=capi.F32, k_len=None
                                   out.data_ptr(), arr(H * Q * DV, Q * DV, DV), lse.data_ptr() if want_lse else None, B, H, HK, Q, K, D, DV,
                                   scale, int(causal), offset, gpu.stream()))
     gpu.sync()
+    # the same call with its arguments in one structure (mi355x_attention_d) gives the same bits
+    out2, lse2 = torch.full_like(out, float("nan")), torch.full_like(lse, float("nan"))
+    d = capi.AttentionDesc()
+    d.q, d.k, d.v, d.out, d.lse = qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out2.data_ptr(), (lse2.data_ptr() if want_lse else None)
+    d.mask = md.data_ptr() if md is not None else None
+    d.q_strides[:] = [H * Q * D, Q * D, D]
+    d.k_strides[:] = [HK * cap * D, cap * D, D]
+    d.v_strides[:] = [HK * cap * DV, cap * DV, DV]
+    d.out_strides[:] = [H * Q * DV, Q * DV, DV]
+    if ms is not None:
+        d.mask_strides[:] = list(ms)
+    d.B, d.Q, d.K, d.causal_offset, d.scale = B, Q, K, offset, scale
+    d.kv_dtype, d.H, d.HK, d.D, d.DV, d.causal = kv_dt, H, HK, D, DV, int(causal)
+    capi.check(l.mi355x_attention_d(C.byref(d), gpu.stream()))
+    gpu.sync()
+    assert torch.equal(out.view(torch.int32), out2.view(torch.int32))
+    if want_lse:
+        assert torch.equal(lse.view(torch.int32), lse2.view(torch.int32))
     return out.cpu().numpy(), lse.cpu().numpy()
 
 

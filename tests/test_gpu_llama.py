@@ -92,10 +92,19 @@ def test_qwen2_biases_on_queries_keys_and_values(golden_dir, cache):
     caches = om.new_caches(64, ocache)
     for t in prompt:
         assert np.abs(m.logits([t])[0] - om.logits([t], caches)).max() <= 1e-4 * scale
-    m.reset()
-    toks, _ = m.generate(prompt, 12)
     owant, margins = om.generate(prompt, 12, capacity=64, cache_dtype=ocache)
-    assert toks[0].tolist() == owant, (toks[0].tolist(), owant, min(margins))
+    # the decoding step three ways: launched operator by operator with the position from the host (2), its device-resident
+    # form, where one launch adds the biases, rotates and writes the caches (1), and that form replayed from a graph (0, twice)
+    lib = gpu.lib()
+    try:
+        for mode in (2, 1, 0, 0):
+            gpu.say(f"qwen2, cache dtype {cache}: step mode {mode}")
+            capi.check(lib.mi355x_tune(b"llama.step", mode))
+            m.reset()
+            toks, _ = m.generate(prompt, 12)
+            assert toks[0].tolist() == owant, (mode, toks[0].tolist(), owant, min(margins))
+    finally:
+        capi.check(lib.mi355x_tune(b"llama.step", 0))
 
 
 def test_some_but_not_all_biases_is_an_error(golden_dir):
