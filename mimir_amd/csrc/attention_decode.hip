@@ -45,6 +45,7 @@ struct DecParams {
     int64_t act_row_bytes;
     int act_rows;  // the converted result in the form for a few rows of x (q4_rows_act.h), all sequences in one buffer
     int act_kq;    // the converted result as int8 super-blocks for Q4_K / Q6_K products (kq_act.h), rows act_row_bytes apart
+    int fence;     // 1: the ticket is a release-acquire operation at device scope (the default); 0, 2: measurement aids, see the ticket
 };
 
 __device__ __forceinline__ float group16_sum(float v) {
@@ -125,17 +126,11 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     const int ng = G - g0 < kHeads ? G - g0 : kHeads;
     const int b = blockIdx.z;
 
-    int64_t seen = (int64_t)p.K + (p.dyn_k ? *p.dyn_k : 0);
-    if (p.causal) {
-        int64_t c = p.causal_offset + 1;
-        seen = c < seen ? c : seen;
-    }
-    seen = seen < 0 ? 0 : seen > p.kmax ? p.kmax : seen;
-    const int per = (int)((seen + nsplit - 1) / nsplit);  // <= cmax
-    const int j0 = split * per;
-    const int j1 = j0 + per < (int)seen ? j0 + per : (int)seen;
-    const int nj = j1 > j0 ? j1 - j0 : 0;
-
+    // The shares are cmax keys each, fixed for the launch: share `split` takes keys [split cmax, (split + 1) cmax) of
+    // those the step sees. How many it sees may come from device memory (p.dyn_k); nothing below waits for that
+    // number before the queries, keys and values of the first batch have been requested (rows past the last key
+    // seen are requested too, from within the caches, and ignored).
+    const int j0 = split * cmax;
     float qr[kHeads][FPL];
 #pragma unroll
     for (int g = 0; g < kHeads; g++) {
@@ -159,16 +154,25 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     // that a share of up to 16 U keys costs one trip to memory for both.
     constexpr int U = sizeof(KV) == 2 ? 8 : 4;
     RawRow<KV, FPL> kraw[U], vraw[U];
+    const int last_row = p.kmax - 1;  // the caches hold kmax rows
 #pragma unroll
     for (int u = 0; u < U; u++) {
-        const int jj = kKeyGroups * u + kg;
-        load_raw<KV, FPL>(kbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), kp), kraw[u]);
+        const int jj = kKeyGroups * u + kg, row = j0 + (jj < cmax ? jj : 0);
+        load_raw<KV, FPL>(kbase + (uint32_t)__mul24(row < last_row ? row : last_row, kp), kraw[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; u++) {
-        const int jj = kKeyGroups * u + kg;
-        load_raw<KV, FPL>(vbase + (uint32_t)__mul24(j0 + (jj < nj ? jj : 0), vp), vraw[u]);
+        const int jj = kKeyGroups * u + kg, row = j0 + (jj < cmax ? jj : 0);
+        load_raw<KV, FPL>(vbase + (uint32_t)__mul24(row < last_row ? row : last_row, vp), vraw[u]);
     }
+    __builtin_amdgcn_sched_barrier(0);  // the requests above go out before the number of keys is waited for
+    int64_t seen = (int64_t)p.K + (p.dyn_k ? *p.dyn_k : 0);
+    if (p.causal) {
+        int64_t c = p.causal_offset + 1;
+        seen = c < seen ? c : seen;
+    }
+    seen = seen < 0 ? 0 : seen > p.kmax ? p.kmax : seen;
+    const int nj = seen > j0 ? (int)(seen - j0 < cmax ? seen - j0 : cmax) : 0;
     for (int jj0 = 0; jj0 < nj; jj0 += U * kKeyGroups) {
         if (jj0 > 0) {
 #pragma unroll
@@ -265,25 +269,39 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     if (nsplit > 1) {
         // The shares travel between workgroups (and so between the L2 caches of
         // the chip's dies) through stores and loads that are coherent at device
-        // scope by themselves (relaxed atomics: write-through stores, loads that
-        // bypass stale lines), so no cache-wide write-back or invalidation is
-        // needed. Ordering: every thread's stores have completed (the counters
-        // are waited on, then the barrier) before thread 0 takes the ticket, and
-        // the combining loads are issued only after the last ticket is known.
+        // scope by themselves (write-through stores, loads that bypass stale
+        // lines). Ordering: every thread's stores have completed (the counters
+        // are waited on, then the barrier) before thread 0 takes the ticket, a
+        // release-acquire operation at device scope, and the combining loads are
+        // issued only after the last ticket is known.
         if (g < ng) {
             float* w = ws + (((int64_t)b * p.H + h) * nsplit + split) * (D + 2);
-            if (lane == 0) {
-                coherent_store(w, M);
-                coherent_store(w + 1, L);
-            }
+            if (p.fence == 2) {  // measurement aid: plain stores, made visible by the ticket's release
+                if (lane == 0) {
+                    w[0] = M;
+                    w[1] = L;
+                }
 #pragma unroll
-            for (int c = 0; c < OPL; c++) coherent_store(w + 2 + lane + 64 * c, r[c]);
+                for (int c = 0; c < OPL; c++) w[2 + lane + 64 * c] = r[c];
+            } else {
+                if (lane == 0) {
+                    coherent_store(w, M);
+                    coherent_store(w + 1, L);
+                }
+#pragma unroll
+                for (int c = 0; c < OPL; c++) coherent_store(w + 2 + lane + 64 * c, r[c]);
+            }
         }
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (tid == 0) {
             uint32_t* ctr = counters + (int64_t)b * gridDim.y + blockIdx.y;
-            uint32_t ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // Release-acquire at device scope: the shares stored above (by operations that are coherent at that scope on their
+            // own, and complete: the wait above counts them) happen before the ticket, and the combining loads below after it.
+            // Measured against a relaxed ticket: no difference within the run-to-run spread of a decoding step (0.5 %).
+            // p.fence 0: the relaxed ticket; 2: plain stores and loads of the shares under the same ticket (both to be measured).
+            uint32_t ticket = p.fence != 0 ? __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                           : __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = ticket == (uint32_t)(nsplit - 1);
             if (s_last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
         }
@@ -295,8 +313,8 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
         float f = 0.f, ls = 0.f, ms = -__builtin_inff();
         const float* w0 = ws + ((int64_t)b * p.H + h) * nsplit * (D + 2);
         if (g < ng && lane < nsplit) {
-            ms = coherent_load(w0 + lane * (D + 2));
-            ls = coherent_load(w0 + lane * (D + 2) + 1);
+            ms = p.fence == 2 ? w0[lane * (D + 2)] : coherent_load(w0 + lane * (D + 2));
+            ls = p.fence == 2 ? w0[lane * (D + 2) + 1] : coherent_load(w0 + lane * (D + 2) + 1);
         }
         float t[8][OPL];
         auto load_shares = [&](int s0) {
@@ -304,7 +322,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
             for (int u = 0; u < 8; u++) {
                 const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;
 #pragma unroll
-                for (int c = 0; c < OPL; c++) t[u][c] = coherent_load(w0 + s * (D + 2) + 2 + lane + 64 * c);
+                for (int c = 0; c < OPL; c++) t[u][c] = p.fence == 2 ? w0[s * (D + 2) + 2 + lane + 64 * c] : coherent_load(w0 + s * (D + 2) + 2 + lane + 64 * c);
             }
         };
         if (g < ng) load_shares(0);
@@ -375,7 +393,9 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 }  // namespace
 
 static std::atomic<int> g_force_splits{0};  // measurement aid: a fixed number of shares
+static std::atomic<int> g_fence{1};         // "attention.fence"
 void set_attention_decode_splits(int n) { g_force_splits = n; }
+void set_attention_decode_fence(int v) { g_fence = v; }
 
 // Shares of the keys and the most keys a share can hold, for at most kmax keys.
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax) {
@@ -445,6 +465,7 @@ hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, vo
     p.act_row_bytes = act_row_bytes;
     p.act_rows = act_form == kAttnActRows ? 1 : 0;
     p.act_kq = act_form == kAttnActKQ ? 1 : 0;
+    p.fence = g_fence.load(std::memory_order_relaxed);
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
     dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
     size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);

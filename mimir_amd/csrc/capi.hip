@@ -824,6 +824,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
         mimir::set_attention_decode_splits(value);
         return MI355X_OK;
     }
+    if (key && strcmp(key, "attention.fence") == 0) {
+        mimir::set_attention_decode_fence(value);
+        return MI355X_OK;
+    }
     if (key && strcmp(key, "attention.path") == 0) {
         g_tune_attn = value;
         return MI355X_OK;

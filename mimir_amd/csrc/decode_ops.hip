@@ -436,7 +436,8 @@ __global__ __launch_bounds__(256) void argmax_split_kernel(const float* __restri
         __hip_atomic_store(&cand_v[r * kArgmaxBlocks + blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&cand_i[r * kArgmaxBlocks + blockIdx.x], at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __builtin_amdgcn_s_waitcnt(0);
-        uint32_t ticket = __hip_atomic_fetch_add(&tickets[r], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // release-acquire at device scope: the candidates stored above happen before it, the loads of the last workgroup after it
+        uint32_t ticket = __hip_atomic_fetch_add(&tickets[r], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         s_last = ticket == (uint32_t)(nblk - 1);
         if (s_last) __hip_atomic_store(&tickets[r], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }

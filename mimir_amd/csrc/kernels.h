@@ -226,6 +226,7 @@ hipError_t attention_empty(const AttnArgs& a, hipStream_t st);
 constexpr size_t kAttnTicketBytes = 4096;
 bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
 void set_attention_decode_splits(int n);
+void set_attention_decode_fence(int v);  // 1 (default): the hand-over's ticket is a release-acquire operation at device scope; 0 relaxed, 2 plain share accesses (measurement)
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 enum { kAttnActQ4 = 0, kAttnActRows = 1, kAttnActKQ = 2 };

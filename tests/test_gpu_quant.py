@@ -294,6 +294,16 @@ def test_q4_0_fixed_point_outliers_inside_a_block(m):
             # what a float32 product keeps and this one loses: the neighbours' low bits, at most the bound above,
             # which here is about 1e-1 of the result (the neighbours are 1e-6 of their block's scale)
             print(f"[outliers m={m}] worst error {err.max():.3e}, bound {float((fixed + f32).max()):.3e}, largest |want| {np.abs(want).max():.3e}")
+        # "q4_0.path" = 1, the float32 kernel (every weight decoded and multiplied in float32 as the reference does), meets
+        # the conformance rule on all three cases: the route for a caller whose activations hold such outliers
+        try:
+            capi.check(gpu.lib().mi355x_tune(b"q4_0.path", 1))
+            gpu.say(f"q4_0 float32 kernel on the same case, m={m}: {name}")
+            got32 = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+        finally:
+            capi.check(gpu.lib().mi355x_tune(b"q4_0.path", 0))
+        err32 = np.abs(got32.astype(np.float64) - want)
+        assert np.all(err32 <= np.maximum(1e-3 * np.maximum(1, np.abs(want)), f32)), (name, float(err32.max()))
 
 
 def test_q4_0_gemv_without_lds_staging():
