@@ -368,7 +368,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * it (0: up to where the tiled kernel's cost model undercuts its own).
  * "q8_0.mfma" = 1 sends every Q8_0 product of two to eight rows of x that the
  * matrix-core kernel takes to it, 2 none (0: matrices of 64 M weights or more).
- * "attention.splits" = n fixes the shares of the keys in decode attention;
+ * "attention.splits" = n fixes the shares of the keys in decode attention; "attention.share" = 128 makes it aim at
+ * shares of 128 keys whatever their number (otherwise 64 while there are at most sixteen shares);
+ * "attention.handover" = 1 makes its shares travel through a ticket per head instead of as (value, flag) pairs;
  * "attention.fence" = 0 makes the ticket that hands its shares over a relaxed operation instead of a
  * release-acquire one at device scope, 2 also stores and loads the shares plainly (both to be measured; 1 restores).
  * "q4_0.fx_rows" = n sends Q4_0 products of at least n rows of float32 x to the

@@ -46,6 +46,8 @@ struct DecParams {
     int act_rows;  // the converted result in the form for a few rows of x (q4_rows_act.h), all sequences in one buffer
     int act_kq;    // the converted result as int8 super-blocks for Q4_K / Q6_K products (kq_act.h), rows act_row_bytes apart
     int fence;     // 1: the ticket is a release-acquire operation at device scope (the default); 0, 2: measurement aids, see the ticket
+    unsigned long long* flagged;  // not null: shares travel as (value, flag) pairs and the first share's workgroup collects them (no ticket)
+    uint32_t* err;                // the device's error word (a hand-over that never completes sets kErrInternal)
 };
 
 __device__ __forceinline__ float group16_sum(float v) {
@@ -59,6 +61,18 @@ __device__ __forceinline__ float group16_sum(float v) {
 // Stores and loads that are coherent across the device on their own.
 __device__ __forceinline__ void coherent_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float coherent_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// A value and the flag that says it is there, in one 8-byte store: whoever loads the pair sees both or neither.
+constexpr uint32_t kShareReady = 1u;
+constexpr int kGather = 16;           // shares whose values the collecting workgroup requests together
+constexpr int kShareSpins = 1 << 18;  // polls of a slot before the collecting workgroup gives up (some tenths of a second)
+__device__ __forceinline__ void flagged_store(unsigned long long* p, float v) {
+    __hip_atomic_store(p, ((unsigned long long)kShareReady << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long flagged_load(const unsigned long long* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void flagged_clear(unsigned long long* p) { __hip_atomic_store(p, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // FPL consecutive elements of a cache row as floats.
 template <typename KV, int FPL>
@@ -106,7 +120,8 @@ __device__ __forceinline__ void raw_values(const RawRow<KV, FPL>& r, float out[F
     }
 }
 
-template <typename KV, int FPL>
+// UU: rows of keys (and of values) a thread has under way at a time: a batch is 16 UU keys.
+template <typename KV, int FPL, int UU>
 __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __restrict__ q, const KV* __restrict__ k,
                                                                const KV* __restrict__ v, float* __restrict__ ws,
                                                                uint32_t* __restrict__ counters, float* __restrict__ out,
@@ -120,9 +135,13 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     __shared__ int s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int part = tid & 15, kg = tid >> 4;
-    const int split = blockIdx.x, nsplit = p.nsplit, cmax = p.cmax;
+    // The grid's first dimension runs over the key heads (times the groups of four query heads), the second over the shares
+    // of the keys: workgroups are handed to the chip's dies round robin by their linear index, so with eight key heads
+    // every share of a head runs on the same die, whose L2 alone then holds the head's keys and values.
+    const int split = blockIdx.y, nsplit = p.nsplit, cmax = p.cmax;
+    const int group = blockIdx.x;
     const int G = p.H / p.HK, ngq = (G + kHeads - 1) / kHeads;
-    const int hk = blockIdx.y / ngq, g0 = (blockIdx.y % ngq) * kHeads;
+    const int hk = group / ngq, g0 = (group % ngq) * kHeads;
     const int ng = G - g0 < kHeads ? G - g0 : kHeads;
     const int b = blockIdx.z;
 
@@ -152,7 +171,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     // Rows in flight per thread: key j0 + jj with jj = jj0 + 16 u + kg. The first
     // batch of keys and of values is requested before anything is computed, so
     // that a share of up to 16 U keys costs one trip to memory for both.
-    constexpr int U = sizeof(KV) == 2 ? 8 : 4;
+    constexpr int U = UU;
     RawRow<KV, FPL> kraw[U], vraw[U];
     const int last_row = p.kmax - 1;  // the caches hold kmax rows
 #pragma unroll
@@ -266,7 +285,94 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
     }
     float M = red[g], L = red[kHeads + g];
 
-    if (nsplit > 1) {
+    if (nsplit > 1 && p.flagged) {
+        // The shares travel as (value, flag) pairs, each one 8-byte store that is coherent at device scope on its own:
+        // a pair is seen whole or not at all, so nothing has to be waited for between the data and a signal that it
+        // is there. The workgroups of shares 1.. store theirs and are done; the workgroup of share 0 keeps its own in
+        // registers, polls the others' slots until every pair shows its flag (a bounded number of times: all
+        // workgroups of a launch are resident together, the grid being far smaller than the chip), combines them in
+        // the shares' order and clears the slots for the next launch on the stream.
+        unsigned long long* slots = p.flagged + ((int64_t)b * p.H + h) * nsplit * (D + 2);
+        if (split != 0) {
+            if (g < ng) {
+                unsigned long long* w = slots + (int64_t)split * (D + 2);
+                if (lane == 0) {
+                    flagged_store(w, M);
+                    flagged_store(w + 1, L);
+                }
+#pragma unroll
+                for (int c = 0; c < OPL; c++) flagged_store(w + 2 + lane + 64 * c, r[c]);
+            }
+            return;
+        }
+        bool late = false;
+        float* fs = osl + g * 64;  // factor of share s of head g
+        float own[OPL];
+#pragma unroll
+        for (int c = 0; c < OPL; c++) own[c] = r[c];
+        const unsigned long long ready = (unsigned long long)kShareReady << 32;
+        // Sixteen shares' values at a time, asked for again while any pair lacks its flag; with the first sixteen go the
+        // (max, sum) of every share, so that one trip to memory brings all a short context needs.
+        unsigned long long raw[kGather][OPL], mraw = ready | __float_as_uint(M), lraw = ready | __float_as_uint(L);
+        auto gather = [&](int s0, bool with_sums) {
+            bool all = g >= ng;  // a wavefront without a head has nothing to wait for
+            for (int spin = 0; !all && spin < kShareSpins; spin++) {
+                if (spin) __builtin_amdgcn_s_sleep(2);
+                all = true;
+                if (with_sums && lane < nsplit && lane > 0) {
+                    mraw = flagged_load(slots + lane * (D + 2));
+                    lraw = flagged_load(slots + lane * (D + 2) + 1);
+                }
+#pragma unroll
+                for (int u = 0; u < kGather; u++) {
+                    const int sidx = s0 + u < nsplit ? s0 + u : nsplit - 1;
+#pragma unroll
+                    for (int c = 0; c < OPL; c++)
+                        raw[u][c] = sidx == 0 ? ready | __float_as_uint(own[c]) : flagged_load(slots + (int64_t)sidx * (D + 2) + 2 + lane + 64 * c);
+                }
+                all = (uint32_t)(mraw >> 32) == kShareReady && (uint32_t)(lraw >> 32) == kShareReady;
+#pragma unroll
+                for (int u = 0; u < kGather; u++)
+#pragma unroll
+                    for (int c = 0; c < OPL; c++) all = all && (uint32_t)(raw[u][c] >> 32) == kShareReady;
+            }
+            if (!all) late = true;
+        };
+        gather(0, true);
+        float f = 0.f, ls = 0.f, ms = -__builtin_inff();
+        if (g < ng && lane < nsplit) {
+            ms = __uint_as_float((uint32_t)mraw);
+            ls = __uint_as_float((uint32_t)lraw);
+        }
+        M = wave_max(ms);
+        if (ls != 0.f && M > -__builtin_inff()) f = __builtin_expf(ms - M);
+        L = wave_sum(ls * f);
+        fs[lane] = f;
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < OPL; c++) r[c] = 0.f;
+        if (g < ng) {
+            for (int s0 = 0; s0 < nsplit; s0 += kGather) {
+                if (s0 > 0) gather(s0, false);
+#pragma unroll
+                for (int u = 0; u < kGather; u++) {
+                    const float fsv = s0 + u < nsplit ? fs[s0 + u] : 0.f;
+#pragma unroll
+                    for (int c = 0; c < OPL; c++) r[c] = fmaf(__uint_as_float((uint32_t)raw[u][c]), fsv, r[c]);
+                }
+            }
+            // the slots are read: empty again for the next launch
+            if (lane < nsplit && lane > 0) {
+                flagged_clear(slots + lane * (D + 2));
+                flagged_clear(slots + lane * (D + 2) + 1);
+            }
+            for (int sidx = 1; sidx < nsplit; sidx++)
+#pragma unroll
+                for (int c = 0; c < OPL; c++) flagged_clear(slots + (int64_t)sidx * (D + 2) + 2 + lane + 64 * c);
+        }
+        if (late && p.err) atomicOr(p.err, kErrInternal);
+        __syncthreads();  // fs is read; the results go over it
+    } else if (nsplit > 1) {
         // The shares travel between workgroups (and so between the L2 caches of
         // the chip's dies) through stores and loads that are coherent at device
         // scope by themselves (write-through stores, loads that bypass stale
@@ -295,7 +401,7 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (tid == 0) {
-            uint32_t* ctr = counters + (int64_t)b * gridDim.y + blockIdx.y;
+            uint32_t* ctr = counters + (int64_t)b * gridDim.x + group;
             // Release-acquire at device scope: the shares stored above (by operations that are coherent at that scope on their
             // own, and complete: the wait above counts them) happen before the ticket, and the combining loads below after it.
             // Measured against a relaxed ticket: no difference within the run-to-run spread of a decoding step (0.5 %).
@@ -392,6 +498,8 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(const float* __re
 
 }  // namespace
 
+static std::atomic<int> g_share_keys{64};  // "attention.share": keys a share aims at (64 or 128)
+void set_attention_decode_share(int n) { g_share_keys = n == 128 ? 128 : 64; }
 static std::atomic<int> g_force_splits{0};  // measurement aid: a fixed number of shares
 static std::atomic<int> g_fence{1};         // "attention.fence"
 void set_attention_decode_splits(int n) { g_force_splits = n; }
@@ -403,7 +511,12 @@ void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, 
     int64_t rows = B * HK * ngq;
     int64_t ns = 512 / (rows > 0 ? rows : 1);
     ns = ns > 64 ? 64 : ns;
-    int64_t by_keys = kmax / 128;  // a share of 128 keys is one batch of loads per thread
+    // A share is one batch of loads per thread: 64 keys while that makes no more shares than the collecting workgroup
+    // gathers in one trip to memory, 128 beyond ("attention.share" = 128: always). Measured at 768 keys against 128:
+    // the scores and the weighted values of a share take half as long, the hand-over a little longer.
+    const int64_t aim = g_share_keys.load(std::memory_order_relaxed);
+    int64_t by_keys = (kmax + aim - 1) / aim;
+    if (by_keys > kGather) by_keys = (kmax + 127) / 128;
     ns = ns > by_keys ? by_keys : ns;
     ns = ns < 1 ? 1 : ns;
     if (g_force_splits > 0 && g_force_splits <= 64) ns = g_force_splits;
@@ -450,7 +563,13 @@ bool attention_decode_kq_ok(const AttnArgs& a) {
 // fixed-point form, act_row_bytes apart; out may then be null.
 // act_form: kAttnActQ4 that form; kAttnActRows the form for eight sequences together (q4_rows_act.h), a buffer per group of eight: row b's
 // result as row b % 8 of group b / 8; kAttnActKQ int8 super-blocks for the K-quant products (where attention_decode_kq_ok).
-hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, int act_form) {
+size_t attention_decode_flagged_bytes(int64_t B, int H, int D, int nsplit) { return nsplit <= 1 ? 0 : (size_t)(B * H * nsplit * (D + 2)) * 8; }
+
+static std::atomic<int> g_handover{0};  // "attention.handover": 1 keeps the ticket protocol although flagged slots are there
+void set_attention_decode_handover(int v) { g_handover = v; }
+
+hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, int act_form,
+                            void* flagged, size_t flagged_bytes, uint32_t* err) {
     DecParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];
@@ -466,18 +585,24 @@ hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, vo
     p.act_rows = act_form == kAttnActRows ? 1 : 0;
     p.act_kq = act_form == kAttnActKQ ? 1 : 0;
     p.fence = g_fence.load(std::memory_order_relaxed);
+    const bool flags_fit = flagged && attention_decode_flagged_bytes(a.B, a.H, a.D, p.nsplit) <= flagged_bytes;  // else the tickets
+    p.flagged = g_handover.load(std::memory_order_relaxed) == 1 || !flags_fit ? nullptr : (unsigned long long*)flagged;
+    p.err = err;
     int G = a.H / a.HK, ngq = (G + kHeads - 1) / kHeads;
-    dim3 grid((unsigned)p.nsplit, (unsigned)(a.HK * ngq), (unsigned)a.B);
+    dim3 grid((unsigned)(a.HK * ngq), (unsigned)p.nsplit, (unsigned)a.B);
     size_t lds = (size_t)(kHeads * p.cmax + kKeyGroups * kHeads * a.D) * sizeof(float);
     uint32_t* counters = (uint32_t*)workspace;
     float* ws = (float*)((uint8_t*)workspace + kCounterBytes);
-#define DEC_LAUNCH(KV, FPL)                                                                                                   \
-    hipLaunchKernelGGL((attn_decode_kernel<KV, FPL>), grid, dim3(kThreads), lds, st, a.q, (const KV*)a.k, (const KV*)a.v, ws, \
+    // a thread keeps eight rows of binary16 keys (four of float32) under way, or half as many where a share is that short
+#define DEC_LAUNCH(KV, FPL, UU)                                                                                                   \
+    hipLaunchKernelGGL((attn_decode_kernel<KV, FPL, UU>), grid, dim3(kThreads), lds, st, a.q, (const KV*)a.k, (const KV*)a.v, ws, \
                        counters, a.out, a.lse, (uint8_t*)act, p)
+    const bool short_share = p.cmax <= kKeyGroups * 4;
     if (a.kv_dtype == kF16) {
-        if (a.D == 128) DEC_LAUNCH(uint16_t, 8); else DEC_LAUNCH(uint16_t, 4);
+        if (a.D == 128) { if (short_share) DEC_LAUNCH(uint16_t, 8, 4); else DEC_LAUNCH(uint16_t, 8, 8); }
+        else { if (short_share) DEC_LAUNCH(uint16_t, 4, 4); else DEC_LAUNCH(uint16_t, 4, 8); }
     } else {
-        if (a.D == 128) DEC_LAUNCH(float, 8); else DEC_LAUNCH(float, 4);
+        if (a.D == 128) DEC_LAUNCH(float, 8, 4); else DEC_LAUNCH(float, 4, 4);
     }
 #undef DEC_LAUNCH
     return hipGetLastError();

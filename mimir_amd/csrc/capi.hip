@@ -62,7 +62,7 @@ struct ScratchBlock {
     size_t bytes = 0;
 };
 struct StreamScratch {
-    ScratchBlock act, attn, gemm, argmax;
+    ScratchBlock act, attn, attn_flags, gemm, argmax;
     std::vector<void*> retired;  // outgrown blocks
 };
 
@@ -163,7 +163,7 @@ mi355x_status stream_scratch(void* stream, ScratchBlock StreamScratch::*which, s
         if (zero_prefix) {
             // on the calling stream, so that the zeros are in place before the first kernel that takes a ticket there
             // (never under capture: the allocation above fails first)
-            e = hipMemsetAsync(p, 0, zero_prefix, (hipStream_t)stream);
+            e = hipMemsetAsync(p, 0, zero_prefix < want ? zero_prefix : want, (hipStream_t)stream);
             if (e != hipSuccess) {
                 (void)hipFree(p);  // nothing has seen it yet
                 return fail((mi355x_status)e, "mi355x: hipMemset(%s tickets): %s", what, hipGetErrorName(e));
@@ -196,6 +196,10 @@ mi355x_status act_for(const ActSource& src, size_t bytes, void** out) {
 }
 mi355x_status attn_scratch(void* stream, size_t bytes, void** out) {
     return stream_scratch(stream, &StreamScratch::attn, bytes, 4u << 20, mimir::kAttnTicketBytes, "attention", out);
+}
+// The (value, flag) slots of decode attention's hand-over: all zero when handed out, and nobody else's.
+mi355x_status attn_flags_scratch(void* stream, size_t bytes, void** out) {
+    return stream_scratch(stream, &StreamScratch::attn_flags, bytes, 1u << 20, (size_t)-1 /* all of it */, "attention hand-over", out);
 }
 mi355x_status gemm_scratch(void* stream, size_t bytes, void** out) {
     return stream_scratch(stream, &StreamScratch::gemm, bytes, 0, 0, "gemm", out);
@@ -687,7 +691,11 @@ mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const v
         int cmax;
         mimir::attention_decode_plan(B, H, HK, K, &a.nsplit, &cmax);
         if (mi355x_status st = attn_scratch(stream, mimir::attention_decode_workspace_bytes(B, H, D, a.nsplit), &ws)) return st;
-        HIP_TRY(mimir::attention_decode(a, K, ws, nullptr, 0, (hipStream_t)stream), "launch attention_decode");
+        void* flags = nullptr;
+        const size_t flag_bytes = mimir::attention_decode_flagged_bytes(B, H, D, a.nsplit);
+        if (a.nsplit > 1)
+            if (mi355x_status st = attn_flags_scratch(stream, flag_bytes, &flags)) return st;
+        HIP_TRY(mimir::attention_decode(a, K, ws, nullptr, 0, (hipStream_t)stream, mimir::kAttnActQ4, flags, flag_bytes, mimir::device_error_word()), "launch attention_decode");
         return MI355X_OK;
     }
     mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
@@ -743,7 +751,7 @@ mi355x_status mi355x_stream_release(void* stream) {
     if (it == s->scratch.end()) return MI355X_OK;
     StreamScratch& m = it->second;
     hipError_t first = hipSuccess;
-    for (void* p : {m.act.p, m.attn.p, m.gemm.p, m.argmax.p})
+    for (void* p : {m.act.p, m.attn.p, m.attn_flags.p, m.gemm.p, m.argmax.p})
         if (p) { hipError_t e = hipFree(p); if (first == hipSuccess) first = e; }
     for (void* p : m.retired) { hipError_t e = hipFree(p); if (first == hipSuccess) first = e; }
     s->scratch.erase(it);
@@ -822,6 +830,14 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "attention.splits") == 0) {
         mimir::set_attention_decode_splits(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "attention.share") == 0) {
+        mimir::set_attention_decode_share(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "attention.handover") == 0) {
+        mimir::set_attention_decode_handover(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "attention.fence") == 0) {

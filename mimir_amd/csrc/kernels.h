@@ -226,12 +226,18 @@ hipError_t attention_empty(const AttnArgs& a, hipStream_t st);
 constexpr size_t kAttnTicketBytes = 4096;
 bool attention_decode_ok(const AttnArgs& a, int64_t kmax);
 void set_attention_decode_splits(int n);
+void set_attention_decode_share(int n);  // keys a share of decode attention aims at: 64 or 128
 void set_attention_decode_fence(int v);  // 1 (default): the hand-over's ticket is a release-acquire operation at device scope; 0 relaxed, 2 plain share accesses (measurement)
 void attention_decode_plan(int64_t B, int H, int HK, int64_t kmax, int* nsplit, int* cmax);
 size_t attention_decode_workspace_bytes(int64_t B, int H, int D, int nsplit);
 enum { kAttnActQ4 = 0, kAttnActRows = 1, kAttnActKQ = 2 };
+// flagged, if not null: flagged_bytes bytes (at least attention_decode_flagged_bytes, else the tickets are used), zero before the first launch and left zero by every launch, that no
+// other kernel writes: the shares of the keys then travel as (value, flag) pairs to the first share's workgroup, which polls for
+// them (a bounded number of times; a pair that never arrives sets kErrInternal in *err), instead of through tickets.
+size_t attention_decode_flagged_bytes(int64_t B, int H, int D, int nsplit);
+void set_attention_decode_handover(int v);  // measurement aid: 1 keeps the ticket protocol
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st,
-                            int act_form = kAttnActQ4);
+                            int act_form = kAttnActQ4, void* flagged = nullptr, size_t flagged_bytes = 0, uint32_t* err = nullptr);
 bool attention_decode_kq_ok(const AttnArgs& a);
 
 // The fixed-point Q4_0 product of a few rows of float32 x that reads W once per eight of them (qgemv_q4_0_rows.hip,

@@ -94,6 +94,7 @@ struct Model {
     bool ready = false;
 
     DevBuf cos_t, sin_t;                 // [context, rope_dim/2]
+    DevBuf attn_flags;                   // decode attention's (value, flag) slots: zero between launches
     std::vector<DevBuf> keys, values;    // per block: [batch, kv_heads, context, head_dim]
     int64_t cache_len = 0;
 
@@ -332,7 +333,7 @@ static mi355x_status step_fast(Model& m) {
         at.k = m.keys[i].p; at.v = m.values[i].p;
         if (one_launch) {  // leaves its result converted for the output projection
             at.out = nullptr;
-            LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, (int64_t)q4_0_act_bytes(qd), m.stream), "attention");
+            LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, (int64_t)q4_0_act_bytes(qd), m.stream, kAttnActQ4, m.attn_flags.p, m.attn_flags.bytes, device_error_word()), "attention");
         } else {
             LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
             LLM_HIP(q4_0_convert_act(a, B, qd, qd, act, m.stream), "convert");
@@ -411,7 +412,7 @@ static mi355x_status step_rows(Model& m) {
                             c.context, m.cos_t.as<float>(), m.sin_t.as<float>(), pos, m.stream), "rope and cache");
         }
         at.k = m.keys[i].p; at.v = m.values[i].p;
-        LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, kAttnActRows), "attention");
+        LLM_HIP(attention_decode(at, c.context, m.act[0].p, act, 0, m.stream, kAttnActRows, m.attn_flags.p, m.attn_flags.bytes, device_error_word()), "attention");
         LLM_HIP(qgemv_q4_0_rows(b.o.buf.p, act, parts, nullptr, B, c.embed, qd, shares, m.stream), "attn_output");
         LLM_HIP(rows_norm_act(x, parts, shares, b.ffn_norm.buf.as<float>(), act, B, c.embed, c.eps, m.stream), "ffn_norm");
         if (g_llama_rows_plain != 2 && g_llama_rows_plain != 3) {  // SiLU * up and the conversion ride on the product, into a buffer of their own
@@ -504,9 +505,9 @@ static mi355x_status step_any(Model& m) {
         // K-quant output projection: attention leaves its result as the int8 super-blocks that product reads
         const bool a_kq = one_launch && act_class(b.o, B) == kActKQ && attention_decode_kq_ok(at);
         if (a_kq) {
-            LLM_HIP(attention_decode(at, c.context, m.act[0].p, m.act[kActKQ].p, (int64_t)kq_act_bytes(qd), m.stream, kAttnActKQ), "attention");
+            LLM_HIP(attention_decode(at, c.context, m.act[0].p, m.act[kActKQ].p, (int64_t)kq_act_bytes(qd), m.stream, kAttnActKQ, m.attn_flags.p, m.attn_flags.bytes, device_error_word()), "attention");
         } else {
-            if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream), "attention");
+            if (one_launch) LLM_HIP(attention_decode(at, c.context, m.act[0].p, nullptr, 0, m.stream, kAttnActQ4, m.attn_flags.p, m.attn_flags.bytes, device_error_word()), "attention");
             else LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
             if (mi355x_status st = convert_for(m, a, B, qd, {&b.o}, done)) return st;
         }
@@ -741,6 +742,13 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     }
     LLM_HIP(m->act[0].alloc(attn_ws + 64), "hipMalloc(attention scratch)");
     LLM_HIP(hipMemset(m->act[0].p, 0, kAttnTicketBytes), "hipMemset(attention tickets)");
+    {
+        int ns = 1, cm = 1;
+        attention_decode_plan(c.batch, c.heads, c.kv_heads, c.context, &ns, &cm);
+        const size_t fb = attention_decode_flagged_bytes(c.batch, c.heads, c.head_dim, ns);
+        LLM_HIP(m->attn_flags.alloc(fb + 64), "hipMalloc(attention hand-over)");
+        LLM_HIP(hipMemset(m->attn_flags.p, 0, fb + 64), "hipMemset(attention hand-over)");
+    }
     if (!m->stream) LLM_HIP(hipStreamCreate(&m->stream), "hipStreamCreate");
     if (m->step_graph) {
         (void)hipGraphExecDestroy(m->step_graph);
