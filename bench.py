@@ -111,6 +111,11 @@ class Gemv:
             for i in range(max(warmup, 3)):
                 self.kernel(i)
             self.stream.synchronize()
+            t_warm = time.perf_counter()
+            while time.perf_counter() - t_warm < 0.25:  # untimed: the device's clocks up, as in time()
+                for i in range(64):
+                    self.kernel(i)
+                self.stream.synchronize()
             self.capi.check(self.lib.mi355x_timed_begin(steps))
             for i in range(steps):
                 self.kernel(i)
@@ -165,9 +170,10 @@ class Gemv:
     def time(self, fn, steps, warmup, graph=True):
         """Milliseconds per call of fn over exactly `steps` calls after `warmup`,
         between HIP events on the stream that carries the launches. With graph,
-        the calls are captured n_bufs at a time (plus one graph for the
-        remainder) and replayed, as the decoder replays its step, so the host's
-        launch cost stays off the device's timeline. Also returns wall ms/call."""
+        the calls are captured into one graph (very many steps: n_bufs at a time,
+        plus one graph for the remainder) and replayed, as the decoder replays its
+        step, so the host's launch cost stays off the device's timeline. Also
+        returns wall ms/call."""
         torch, s = self.torch, self.stream
         with torch.cuda.stream(s):
             for i in range(max(warmup, 3)):
@@ -175,7 +181,10 @@ class Gemv:
             s.synchronize()
             graphs = []
             if graph:
-                for count in (self.n_bufs, steps % self.n_bufs):
+                # the timed region is one graph of exactly `steps` launches where that is a graph of reasonable size (one
+                # graph launch to pay for), else a graph of n_bufs launches replayed plus one for the remainder
+                counts = (steps, 0) if steps <= 4096 else (self.n_bufs, steps % self.n_bufs)
+                for count in counts:
                     g = None
                     if count:
                         g = torch.cuda.CUDAGraph()
@@ -185,11 +194,22 @@ class Gemv:
                     graphs.append(g)
                 graphs[0].replay()
                 s.synchronize()
+            # untimed, beyond the warm-up steps asked for: a quarter of a second of the same work, so that the device's
+            # clocks are where a decoding loop holds them (a timed region of a few hundred microseconds from idle otherwise
+            # reads 10 % slow)
+            t_warm = time.perf_counter()
+            while time.perf_counter() - t_warm < 0.25:
+                for _ in range(32):
+                    if graph:
+                        graphs[0].replay()
+                    else:
+                        fn(0)
+                s.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
             e0.record(s)
             if graph:
-                for _ in range(steps // self.n_bufs):
+                for _ in range(1 if steps <= 4096 else steps // self.n_bufs):
                     graphs[0].replay()
                 if graphs[1] is not None:
                     graphs[1].replay()
