@@ -191,6 +191,7 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
     }
     long long t_staged = 0;
     if (STAMPS && tid == 0) t_staged = wall_clock64();
+    __builtin_amdgcn_sched_barrier(0);  // the schedule below is written in program order: nothing moves across these points
 
     // the lane's digits and scales, for every row of the launch
     u32x4 d0[kDigits], d1[kDigits];
@@ -220,6 +221,7 @@ __global__ __launch_bounds__(1024) void qgemv_q4_0_stream_kernel(Q4Job job, cons
 #pragma unroll
         for (int t = 0; t < RR; t++) res[i][t] = wave_sum(res[i][t]);
         if (STAMPS && tid == 0 && i == 0) t_first = wall_clock64();
+        __builtin_amdgcn_sched_barrier(0);  // a row's multiply, refill and reduction stay together
     }
     long long t_last = 0;
     if (STAMPS && tid == 0) t_last = wall_clock64();
