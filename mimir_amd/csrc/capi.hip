@@ -324,9 +324,10 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     void* ws;
     if (dtype == MI355X_Q4_0 && g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
         void* half_ws = nullptr;
-        if (g_tune_gemm_f16 == 1)
-            if (mi355x_status s2 = gemm_scratch(stream, mimir::qgemm_q4_0_half_ws_bytes(M, K), &half_ws)) return s2;
-        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, half_ws, st), "launch qgemm_q4_0");
+        const bool panel = g_tune_gemm_f16 == 1;  // 2: the binary16 form without the panel route
+        if (g_tune_gemm_f16 == 1 || g_tune_gemm_f16 == 2)
+            if (mi355x_status s2 = gemm_scratch(stream, mimir::qgemm_q4_0_half_ws_bytes(M, N, K, panel), &half_ws)) return s2;
+        HIP_TRY(mimir::qgemm_q4_0_bf16(W, X, Y, M, N, K, x_row_stride, f32, half_ws, panel, st), "launch qgemm_q4_0");
         return MI355X_OK;
     }
     if ((dtype == MI355X_Q4_K || dtype == MI355X_Q6_K) && g_tune_gemm != 1 && ((uintptr_t)X & 7) == 0 && x_row_stride % 4 == 0) {
@@ -775,7 +776,7 @@ mi355x_status mi355x_tune(const char* key, int value) {
         return MI355X_OK;
     }
     if (key && strcmp(key, "qgemm.f16") == 0) {
-        g_tune_gemm_f16 = value == 1 ? 1 : 0;
+        g_tune_gemm_f16 = value == 1 || value == 2 ? value : 0;
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.fx_rows") == 0) {

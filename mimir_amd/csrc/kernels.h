@@ -284,12 +284,19 @@ hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* 
 
 // Prompt-sized Q4_0 product on the matrix cores (qgemm_q4_0.hip): X [M, K]
 // bfloat16, Y [M, N] bfloat16 or float32. Exact up to the order of the float32 sums when half_ws is null; with
-// half_ws (qgemm_q4_0_half_ws_bytes(M, K) bytes of device memory, 256-byte aligned) the weights are rounded to
-// binary16 (2^-11 of each) and X goes through half_ws as row-scaled binary16.
+// half_ws (qgemm_q4_0_half_ws_bytes(M, N, K, panel) bytes of device memory, 256-byte aligned) the weights are rounded to
+// binary16 (2^-11 of each) and X goes through half_ws as row-scaled binary16. With `panel` (the same value in both
+// calls) the products that qgemm_f16_panel_pays names write W to half_ws once as a binary16 panel and multiply from it.
 bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K, int64_t x_row_stride);
-size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t K);
+size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t N, int64_t K, bool panel);
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
-                           void* half_ws, hipStream_t st);
+                           void* half_ws, bool panel, hipStream_t st);
+// The panel route (qgemm_f16_panel.hip): X16 [M, K] binary16 with row_scale[m] to multiply row m's results by, W Q4_0,
+// `panel` qgemm_f16_panel_bytes(N, K) bytes of device memory, 256-byte aligned.
+size_t qgemm_f16_panel_bytes(int64_t N, int64_t K);
+bool qgemm_f16_panel_pays(int64_t M, int64_t N, int64_t K);
+hipError_t qgemm_f16_panel(const void* W, const void* X16, const float* row_scale, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32,
+                           void* panel, hipStream_t st);
 hipError_t bf16_rows_to_f32(const void* x, float* y, int64_t M, int64_t K, int64_t x_row_stride, hipStream_t st);
 hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 

@@ -463,19 +463,27 @@ bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K
 // finite scales, Y [M, N] bfloat16, or float32 if out_f32.
 // With half_ws (qgemm_q4_0_half_ws_bytes(M, K) bytes, 16-byte aligned) the product takes its approximate form:
 // X converted into half_ws first, weights rounded to binary16.
-size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t K) { return (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * 4; }
+// With `panel` the workspace also holds W as a binary16 panel, and products for which qgemm_f16_panel_pays take the
+// two launches of qgemm_f16_panel.hip (the same weights, bit for bit; the sums in another order).
+static size_t half_x_bytes(int64_t M, int64_t K) { return ((size_t)M * K * 2 + 255) & ~(size_t)255; }
+static size_t half_scale_bytes(int64_t M) { return ((size_t)M * 4 + 255) & ~(size_t)255; }
+size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t N, int64_t K, bool panel) {
+    return half_x_bytes(M, K) + half_scale_bytes(M) + (panel && qgemm_f16_panel_pays(M, N, K) ? qgemm_f16_panel_bytes(N, K) : 0);
+}
 
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
-                           void* half_ws, hipStream_t st) {
+                           void* half_ws, bool panel, hipStream_t st) {
     const bool half = half_ws != nullptr;
     const float* row_scale = nullptr;
     if (half) {
-        float* sb = (float*)((uint8_t*)half_ws + (((size_t)M * K * 2 + 255) & ~(size_t)255));
+        float* sb = (float*)((uint8_t*)half_ws + half_x_bytes(M, K));
         hipLaunchKernelGGL(bf16_rows_to_f16_scaled_kernel, dim3((unsigned)M), dim3(256), 0, st, (const uint16_t*)X, (uint16_t*)half_ws, sb, K,
                            x_row_stride);
         X = half_ws;
         x_row_stride = K;
         row_scale = sb;
+        if (panel && qgemm_f16_panel_pays(M, N, K))
+            return qgemm_f16_panel(W, X, row_scale, Y, M, N, K, out_f32, (uint8_t*)half_ws + half_x_bytes(M, K) + half_scale_bytes(M), st);
     }
     // the tallest tiles that still give three quarters of the compute units work: a taller tile reads less from
     // LDS per MFMA (a wavefront multiplies 32 MT x 64 of it), which is worth more than the idle quarter (measured at

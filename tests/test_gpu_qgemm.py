@@ -289,6 +289,44 @@ def test_binary16_form_small_and_ragged_shapes(m, n, k):
     assert np.array_equal(got, O.f32_to_bf16(got32))  # one rounding of the same float32 sums
 
 
+class binary16_weights_in_tiles:
+    """The binary16 form kept on the one launch whose tiles convert W for themselves, whatever the shape."""
+
+    def __enter__(self):
+        capi.check(gpu.lib().mi355x_tune(b"qgemm.f16", 2))
+
+    def __exit__(self, *exc):
+        capi.check(gpu.lib().mi355x_tune(b"qgemm.f16", 0))
+
+
+@pytest.mark.parametrize("m,n,k", [(1024, 12288, 256), (1100, 9800, 512), (2047, 6200, 768), (1300, 10241, 256)])
+def test_binary16_form_through_the_panel(m, n, k):
+    """From 1024 rows of x on, with at least 192 tiles of 256 x 256, W is first written once as a binary16 panel
+    and the product is a plain one from LDS (two launches). Shapes that fill their tiles and shapes whose last
+    tiles are ragged both ways; scales over binary16's range; rows of x apart and W at an offset. The same weights
+    as the tile kernel's, bit for bit, so the two routes differ by the order of the float32 sums only."""
+    rng = np.random.default_rng(m + 3 * n + k)
+    w = scales_within_binary16(rng, n * k)
+    xf = rng.normal(size=(m, k)).astype(np.float32)
+    xf[5] *= 2.0 ** 90
+    xf[6] *= 2.0 ** -90
+    xf[7] = 0
+    x = bf16_bits(xf)
+    gpu.say(f"qgemm_bf16, binary16 weights through the panel, {m}x{k} by {n}x{k}")
+    with binary16_weights():
+        got32 = qgemm(w, x, n, k, capi.F32)
+        got = qgemm(w, x, n, k)
+        got2 = qgemm(w, x, n, k, capi.F32, x_stride=k + 24, w_offset=32)
+    check_binary16_form(w, x, n, k, got32)
+    assert np.array_equal(got2, got32)
+    assert np.array_equal(got, O.f32_to_bf16(got32))  # one rounding of the same float32 sums
+    assert np.all(got32[7] == 0)
+    gpu.say(f"qgemm_bf16, binary16 weights in tiles, {m}x{k} by {n}x{k}")
+    with binary16_weights_in_tiles():
+        tiles32 = qgemm(w, x, n, k, capi.F32)
+    check_f32(got32, tiles32.astype(np.float64), 2 * f32_bound(w, x, n, k), "panel route against the tile kernel")
+
+
 def test_binary16_form_rows_of_any_range():
     """Each row of x is scaled by a power of two of its own before it becomes binary16:
     rows near float32's largest and smallest magnitudes, a row of zeros, a row with one
