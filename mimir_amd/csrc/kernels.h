@@ -291,12 +291,12 @@ bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K
 size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t N, int64_t K, bool panel);
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
                            void* half_ws, bool panel, hipStream_t st);
-// The panel route (qgemm_f16_panel.hip): X16 [M, K] binary16 with row_scale[m] to multiply row m's results by, W Q4_0,
-// `panel` qgemm_f16_panel_bytes(N, K) bytes of device memory, 256-byte aligned.
+// The panel route (qgemm_f16_panel.hip): X [M, K] bfloat16 goes to X16 [M, K] binary16 with row_scale[m] to multiply row
+// m's results by (both written here), W Q4_0 to `panel` (qgemm_f16_panel_bytes(N, K) bytes of device memory, 256-byte aligned).
 size_t qgemm_f16_panel_bytes(int64_t N, int64_t K);
 bool qgemm_f16_panel_pays(int64_t M, int64_t N, int64_t K);
-hipError_t qgemm_f16_panel(const void* W, const void* X16, const float* row_scale, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32,
-                           void* panel, hipStream_t st);
+hipError_t qgemm_f16_panel(const void* W, const void* X, int64_t x_row_stride, void* X16, float* row_scale, void* Y, int64_t M, int64_t N, int64_t K,
+                           bool out_f32, void* panel, hipStream_t st);
 hipError_t bf16_rows_to_f32(const void* x, float* y, int64_t M, int64_t K, int64_t x_row_stride, hipStream_t st);
 hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 

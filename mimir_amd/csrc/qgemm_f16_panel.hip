@@ -2,18 +2,25 @@
 // first: the approximate form of the prompt-sized product (weights rounded once to binary16, as qgemm_q4_0.hip's
 // template argument HALF does inside its tiles), split into two launches.
 //
-//   1. q4_0_f16_panel_kernel writes W once as a plain binary16 panel P [N, K]: weight (n - 8) d rounded to nearest,
+//   1. panel_prepare_kernel writes W once as a plain binary16 panel P [N, K]: weight (n - 8) d rounded to nearest,
 //      the same instruction sequence as the tile kernel's, so the same bits. A weight is converted once here instead
-//      of once per 256 rows of X there.
-//   2. hgemm_f16_nt_kernel multiplies X16 [M, K] (binary16, rows scaled by a power of two beforehand,
-//      bf16_rows_to_f16_scaled in qgemm_q4_0.hip) by P: 256 x 256 tiles of Y, eight wavefronts of 128 x 64 each,
+//      of once per 256 rows of X there. The same launch brings X to binary16 (X16, rows scaled by a power of two each,
+//      half_rows.h), in workgroups of its own that run beside the panel's.
+//   2. hgemm_f16_nt_kernel multiplies X16 [M, K] by P: 256 x 256 tiles of Y, eight wavefronts of 128 x 64 each,
 //      steps of 64 along K through two stages of LDS. Both operands go from global memory straight into LDS
 //      (global_load_lds_dwordx4: no registers, no vector arithmetic in the wavefronts that share a SIMD with the MFMAs);
 //      a row of a stage is 128 bytes and its eight 16-byte pieces are placed at piece ^ (row / 2 mod 8), which the
 //      loading lane undoes in the address it reads from, so that the fragment reads of v_mfma_f32_32x32x16_f16
-//      (32 rows, the same piece) spread over all banks. The loads of the next step are issued in four parts between
-//      the four groups of MFMAs of a step, and the fragments of the next group are read while the current group
+//      (32 rows, the same piece) spread over all banks. The loads of the next step are issued in two parts with
+//      the first two of a step's four groups of MFMAs (issued later they had not landed by the step's end, issued all
+//      at once they hold the wavefront up), and the fragments of the next group are read while the current group
 //      multiplies.
+//
+// A compute unit holds one workgroup (128 KB of LDS), so a product takes as long as the unit with the most tiles. Where
+// 256 x 256 tiles would leave the last round partly empty (2048 x 14336: 448 tiles on 256 units), the right-hand
+// columns of Y are cut into tiles of 256 x 192 instead, handed out after the wide ones (32 + 32 column tiles there: one
+// wide and one narrow tile a unit); products with too few wide tiles for the device take 128 x 256 tiles. The cut is
+// chosen on the host by the time the last tile ends (plan_panel).
 //
 // Workgroups go round-robin over the eight dies; a die takes a contiguous range of tiles with the tile's row of X
 // varying fastest, so the 32 workgroups a die runs together share 4 column panels of P and the 8 row panels of X
@@ -21,6 +28,7 @@
 //
 // Reference semantics: Tensor.MatMulT for a half-precision x and block-quantized w, tensor/quant.go:45-48.
 #include "device_util.h"
+#include "half_rows.h"
 #include "kernels.h"
 
 namespace mimir {
@@ -30,36 +38,61 @@ namespace {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kTile = 256;                        // rows of X and rows of W a workgroup multiplies
-constexpr int kStep = 64;                         // of K a step
-constexpr int kRowBytes = kStep * 2;              // a row of a stage in LDS
-constexpr int kStageBytes = 2 * kTile * kRowBytes;  // X's 256 rows, then P's 256 rows
-constexpr int kLoads = 8;                         // 1 KB loads a wavefront issues per step: 64 of the stage's 512 rows, 8 rows a load
-constexpr size_t kLdsBytes = 2 * (size_t)kStageBytes;
+constexpr int kStep = 64;              // of K a step
+constexpr int kRowBytes = kStep * 2;   // a row of a stage in LDS
+constexpr int kUnits = 256;            // compute units; one workgroup each at a time (LDS)
 
-// Eight weights a thread: the low or high nibbles of eight bytes of a block, as the binary16 values (n - 8) d.
-__global__ __launch_bounds__(256) void q4_0_f16_panel_kernel(const uint8_t* __restrict__ W, uint16_t* __restrict__ P, int64_t pieces) {
-    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < pieces; t += (int64_t)gridDim.x * 256) {
-        const int q = (int)(t & 3);
-        const uint8_t* blk = W + (t >> 2) * 18;
+// A workgroup's tile of Y: WM x (8 / WM) wavefronts of (32 MT) x (32 NT) each.
+template <int WM, int MT, int NT>
+struct Tile {
+    static constexpr int WN = 8 / WM, kMT = MT, kNT = NT;
+    static constexpr int BM = WM * 32 * MT, BN = WN * 32 * NT;
+    static constexpr int kRows = BM + BN;                // rows of a stage: X's, then P's
+    static constexpr int kLoads = kRows / 64;            // 1 KB loads (8 rows) a wavefront issues per step
+    static constexpr int kStageBytes = kRows * kRowBytes;
+    static_assert(kRows % 64 == 0 && BM % 8 == 0, "whole loads, none across the two operands");
+};
+using Wide = Tile<2, 4, 2>;    // 256 x 256: the most MFMAs per byte read from LDS (0.75 fragment reads an MFMA)
+using Narrow = Tile<4, 2, 3>;  // 256 x 192: three quarters of a Wide tile, to fill a last round that Wide tiles would leave a quarter empty
+using Low = Tile<2, 2, 2>;     // 128 x 256: for products with too few Wide tiles for the device
+constexpr size_t kLdsBytes = 2 * (size_t)Wide::kStageBytes;
+
+// The pass before the product, one launch: workgroups [0, M) bring a row of X each to binary16 (half_rows.h), the
+// others write the panel. Sixteen weights a thread there: the low and the high nibbles of eight bytes of a block, as
+// the binary16 values (n - 8) d.
+__global__ __launch_bounds__(256) void panel_prepare_kernel(const uint16_t* __restrict__ X, uint16_t* __restrict__ X16, float* __restrict__ scale_back,
+                                                            int M, int64_t K, int64_t x_row_stride, const uint8_t* __restrict__ W,
+                                                            uint16_t* __restrict__ P, int64_t halves) {
+    if ((int)blockIdx.x < M) {
+        bf16_row_to_f16_scaled(X, X16, scale_back, K, x_row_stride, blockIdx.x);
+        return;
+    }
+    const int64_t first = (int64_t)((int)blockIdx.x - M) * 256 + threadIdx.x, stride = (int64_t)((int)gridDim.x - M) * 256;
+    for (int64_t t = first; t < halves; t += stride) {
+        const int q = (int)(t & 1);
+        const uint8_t* blk = W + (t >> 1) * 18;
         const uint16_t rd = *(const uint16_t*)blk;  // blocks are 2-byte aligned, no more
-        const uint16_t* src = (const uint16_t*)(blk + 2 + 8 * (q & 1));
+        const uint16_t* src = (const uint16_t*)(blk + 2 + 8 * q);
         const uint32_t raw[2] = {(uint32_t)src[0] | (uint32_t)src[1] << 16, (uint32_t)src[2] | (uint32_t)src[3] << 16};
         const _Float16 dh = __builtin_bit_cast(_Float16, rd);
         const f16x2 d2 = {dh, dh}, off = {(_Float16)1032.f, (_Float16)1032.f};
-        u32x4 out;
+        uint16_t* out = P + (t >> 1) * 32 + 8 * q;  // elements 8 q .. 8 q + 7 (low nibbles) and 16 more on (high nibbles)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            // the nibble into the mantissa of binary16's 1024, minus 1032 is n - 8, times d rounds once
-            const uint32_t nib = (raw[i] >> (4 * (q >> 1))) & 0x0f0f0f0fu;
-            const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
-            const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
-            const f16x2 w0 = (__builtin_bit_cast(f16x2, p0) - off) * d2;
-            const f16x2 w1 = (__builtin_bit_cast(f16x2, p1) - off) * d2;
-            out[2 * i] = __builtin_bit_cast(uint32_t, w0);
-            out[2 * i + 1] = __builtin_bit_cast(uint32_t, w1);
+        for (int half = 0; half < 2; half++) {
+            u32x4 v;
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                // the nibble into the mantissa of binary16's 1024, minus 1032 is n - 8, times d rounds once
+                const uint32_t nib = (raw[i] >> (4 * half)) & 0x0f0f0f0fu;
+                const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
+                const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
+                const f16x2 w0 = (__builtin_bit_cast(f16x2, p0) - off) * d2;
+                const f16x2 w1 = (__builtin_bit_cast(f16x2, p1) - off) * d2;
+                v[2 * i] = __builtin_bit_cast(uint32_t, w0);
+                v[2 * i + 1] = __builtin_bit_cast(uint32_t, w1);
+            }
+            *(u32x4*)(out + 16 * half) = v;
         }
-        *(u32x4*)(P + 8 * t) = out;
     }
 }
 
@@ -71,52 +104,50 @@ __device__ __forceinline__ void load_to_lds(const void* g, uint32_t lds_base) {
 __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Y [M, N] = (X16 [M, K] . P [N, K]^T) row_scale[m], float32 sums, Y bfloat16 or float32. K a multiple of 64.
-template <bool OUT_F32>
-__global__ __launch_bounds__(512, 2) void hgemm_f16_nt_kernel(const uint16_t* __restrict__ X16, const uint16_t* __restrict__ P, void* __restrict__ Yv,
-                                                              const float* __restrict__ row_scale, int M, int N, int K, int tiles_m, int ntiles) {
-    extern __shared__ __align__(1024) char lds_gemm[];
+// One tile: Y [m0 .. m0 + BM) x [n0 .. n0 + BN) = (X16 . P^T) row_scale[m], float32 sums, Y bfloat16 or float32.
+template <class T, bool OUT_F32>
+__device__ __forceinline__ void tile_body(const uint16_t* __restrict__ X16, const uint16_t* __restrict__ P, void* __restrict__ Yv,
+                                          const float* __restrict__ row_scale, int M, int N, int K, int m0, int n0, char* lds) {
+    constexpr int MT = T::kMT, NT = T::kNT;
+    constexpr int kLoads = T::kLoads;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;
-    const int per_die = (ntiles + 7) >> 3;
-    const int t = ((int)blockIdx.x & 7) * per_die + ((int)blockIdx.x >> 3);
-    if (t >= ntiles) return;  // the whole workgroup
-    const int m0 = (t % tiles_m) * kTile, n0 = (t / tiles_m) * kTile;
+    const int wm = wave / T::WN, wn = wave % T::WN;
 
-    // This wavefront's loads: rows [64 wave, 64 wave + 64) of the stage, X's for wavefronts 0-3 and P's for 4-7.
-    // Rows past the matrix re-read its last row (their results are not stored).
+    // This wavefront's loads: load g = kLoads wave + j brings rows [8 g, 8 g + 8) of the stage, X's below BM and P's
+    // from there. Rows past the matrix re-read its last row (their results are not stored).
     const char* from[kLoads];
     uint32_t into[kLoads];
 #pragma unroll
     for (int j = 0; j < kLoads; j++) {
-        const int row = 64 * wave + 8 * j + (lane >> 3);
+        const int first = 8 * (kLoads * wave + j);
+        const int row = first + (lane >> 3);
         const int piece = (lane & 7) ^ ((row >> 1) & 7);
         const uint16_t* base;
-        if (wave < 4) {
+        if (first < T::BM) {
             const int m = m0 + row < M ? m0 + row : M - 1;
             base = X16 + (size_t)m * K;
         } else {
-            const int n = n0 + row - kTile < N ? n0 + row - kTile : N - 1;
+            const int n = n0 + row - T::BM < N ? n0 + row - T::BM : N - 1;
             base = P + (size_t)n * K;
         }
         from[j] = (const char*)(base + 8 * piece);
-        into[j] = (uint32_t)((64 * wave + 8 * j) * kRowBytes);
+        into[j] = (uint32_t)(first * kRowBytes);
     }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_gemm;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
 
     const int r32 = lane & 31, hi = lane >> 5;
     const int swz = (r32 >> 1) & 7;
     int piece_off[4];
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) piece_off[kk] = ((2 * kk + hi) ^ swz) * 16;
-    const int a_row = (wm * 128 + r32) * kRowBytes, b_row = (kTile + wn * 64 + r32) * kRowBytes;
+    const int a_row = (wm * 32 * MT + r32) * kRowBytes, b_row = (T::BM + wn * 32 * NT + r32) * kRowBytes;
 
-    f32x16 acc[4][2];
+    f32x16 acc[MT][NT];
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
+        for (int nt = 0; nt < NT; nt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mt][nt][i] = 0.f;
 
@@ -130,55 +161,55 @@ __global__ __launch_bounds__(512, 2) void hgemm_f16_nt_kernel(const uint16_t* __
         wait_loads();   // this wavefront's part of step i has landed
         lds_barrier();  // everyone's has, and everyone has read the other stage for the last time
         const bool more = i + 1 < nk;
-        const uint32_t next = lds0 + ((i + 1) & 1) * kStageBytes;
-        const char* st = lds_gemm + (i & 1) * kStageBytes;
-        f16x8 a[2][4], b[2][2];
+        const uint32_t next = lds0 + ((i + 1) & 1) * T::kStageBytes;
+        const char* st = lds + (i & 1) * T::kStageBytes;
+        f16x8 a[2][MT], b[2][NT];
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) a[0][mt] = *(const f16x8*)(st + a_row + mt * 32 * kRowBytes + piece_off[0]);
+        for (int mt = 0; mt < MT; mt++) a[0][mt] = *(const f16x8*)(st + a_row + mt * 32 * kRowBytes + piece_off[0]);
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) b[0][nt] = *(const f16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[0]);
+        for (int nt = 0; nt < NT; nt++) b[0][nt] = *(const f16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[0]);
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             const int c = kk & 1, n = c ^ 1;
-            if (more) {  // a quarter of the next step's loads
+            if (more && kk < 2) {  // half of the next step's loads: all of them early in the step, so that they have landed by its end
 #pragma unroll
-                for (int j = 2 * kk; j < 2 * kk + 2; j++) {
+                for (int j = kk * kLoads / 2; j < (kk + 1) * kLoads / 2; j++) {
                     load_to_lds(from[j], __builtin_amdgcn_readfirstlane(next + into[j]));
                     from[j] += kRowBytes;
                 }
             }
             if (kk + 1 < 4) {
 #pragma unroll
-                for (int mt = 0; mt < 4; mt++) a[n][mt] = *(const f16x8*)(st + a_row + mt * 32 * kRowBytes + piece_off[kk + 1]);
+                for (int mt = 0; mt < MT; mt++) a[n][mt] = *(const f16x8*)(st + a_row + mt * 32 * kRowBytes + piece_off[kk + 1]);
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++) b[n][nt] = *(const f16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[kk + 1]);
+                for (int nt = 0; nt < NT; nt++) b[n][nt] = *(const f16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[kk + 1]);
             }
 #pragma unroll
-            for (int mt = 0; mt < 4; mt++)
+            for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++) acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[c][mt], b[c][nt], acc[mt][nt], 0, 0, 0);
+                for (int nt = 0; nt < NT; nt++) acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[c][mt], b[c][nt], acc[mt][nt], 0, 0, 0);
             if (kk + 1 < 4) {  // one fragment read between two MFMAs
 #pragma unroll
-                for (int q = 0; q < 6; q++) {
+                for (int q = 0; q < MT + NT; q++) {
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 }
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                if (MT * NT > MT + NT) __builtin_amdgcn_sched_group_barrier(0x008, MT * NT - MT - NT, 0);
             }
         }
     }
 
     // the row's scale undone (a power of two: exact), then one rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51)
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const int m = m0 + wm * 128 + mt * 32 + (i >> 2) * 8 + hi * 4 + (i & 3);
+            const int m = m0 + wm * 32 * MT + mt * 32 + (i >> 2) * 8 + hi * 4 + (i & 3);
             if (m >= M) continue;
             const float back = row_scale[m];
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++) {
-                const int n = n0 + wn * 64 + nt * 32 + r32;
+            for (int nt = 0; nt < NT; nt++) {
+                const int n = n0 + wn * 32 * NT + nt * 32 + r32;
                 if (n >= N) continue;
                 const float v = acc[mt][nt][i] * back;
                 if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n] = v;
@@ -187,20 +218,127 @@ __global__ __launch_bounds__(512, 2) void hgemm_f16_nt_kernel(const uint16_t* __
         }
 }
 
+// How Y is cut into tiles. Columns [0, 256 wide_cols) in Wide tiles, then narrow_cols Narrow tiles; or, with `low`,
+// every tile Low. Workgroups take the Wide tiles first (the dispatcher hands them out in the order of their index).
+struct PanelPlan {
+    int tiles_m;      // tiles along M (256 rows, or 128 with low)
+    int wide_cols, narrow_cols;
+    int low;
+};
+
+// A die's workgroups (every eighth, round-robin) take a contiguous range of the tiles, the tile's row of X varying
+// fastest: the 32 that run together share 4 column panels of P and the 8 row panels of X through the die's L2.
+__device__ __forceinline__ int tile_of(int b, int ntiles) {
+    const int per_die = (ntiles + 7) >> 3;
+    return (b & 7) * per_die + (b >> 3);
+}
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(512, 2) void hgemm_f16_nt_kernel(const uint16_t* __restrict__ X16, const uint16_t* __restrict__ P, void* __restrict__ Yv,
+                                                              const float* __restrict__ row_scale, int M, int N, int K, PanelPlan plan) {
+    extern __shared__ __align__(1024) char lds_gemm[];
+    int b = (int)blockIdx.x;
+    if (plan.low) {
+        const int ntiles = plan.tiles_m * plan.wide_cols;
+        const int t = tile_of(b, ntiles);
+        if (t >= ntiles) return;  // the whole workgroup
+        tile_body<Low, OUT_F32>(X16, P, Yv, row_scale, M, N, K, (t % plan.tiles_m) * Low::BM, (t / plan.tiles_m) * Low::BN, lds_gemm);
+        return;
+    }
+    const int nwide = plan.tiles_m * plan.wide_cols;
+    const int wide_wgs = ((nwide + 7) >> 3) << 3;
+    if (b < wide_wgs) {
+        const int t = tile_of(b, nwide);
+        if (t >= nwide) return;
+        tile_body<Wide, OUT_F32>(X16, P, Yv, row_scale, M, N, K, (t % plan.tiles_m) * Wide::BM, (t / plan.tiles_m) * Wide::BN, lds_gemm);
+        return;
+    }
+    b -= wide_wgs;
+    const int nnarrow = plan.tiles_m * plan.narrow_cols;
+    const int t = tile_of(b, nnarrow);
+    if (t >= nnarrow) return;
+    tile_body<Narrow, OUT_F32>(X16, P, Yv, row_scale, M, N, K, (t % plan.tiles_m) * Narrow::BM, plan.wide_cols * Wide::BN + (t / plan.tiles_m) * Narrow::BN,
+                               lds_gemm);
+}
+
+// When the last of n_first jobs of cost c_first, then n_then jobs of cost c_then, ends on kUnits units that each
+// take the next job as soon as they are free.
+double makespan(int n_first, double c_first, int n_then, double c_then) {
+    struct Level { double at; int units; };
+    Level lv[64];
+    int n = 0;
+    const int q = n_first / kUnits, r = n_first % kUnits;
+    if (kUnits - r > 0) lv[n++] = {q * c_first, kUnits - r};
+    if (r > 0) lv[n++] = {(q + 1) * c_first, r};
+    while (n_then > 0) {
+        const int k = lv[0].units < n_then ? lv[0].units : n_then;  // lv is kept in ascending order
+        n_then -= k;
+        const double to = lv[0].at + c_then;
+        lv[0].units -= k;
+        if (lv[0].units == 0) {
+            for (int i = 1; i < n; i++) lv[i - 1] = lv[i];
+            n--;
+        }
+        int at = 0;
+        while (at < n && lv[at].at < to) at++;
+        if (at < n && lv[at].at == to) {
+            lv[at].units += k;
+        } else if (n < 64) {
+            for (int i = n; i > at; i--) lv[i] = lv[i - 1];
+            lv[at] = {to, k};
+            n++;
+        } else {
+            lv[n - 1].units += k;  // more levels than this holds: counted at the latest
+        }
+    }
+    return n > 0 ? lv[n - 1].at : 0.0;
+}
+
+// Costs in Wide tiles' time: a Narrow tile has three quarters of the MFMAs and reads a little more from LDS for each,
+// a Low tile half of them and a third more.
+constexpr double kNarrowCost = 0.78, kLowCost = 0.56;
+
+// The cut with the earliest end, and that end (in Wide tiles' time).
+double plan_panel(int64_t M, int64_t N, PanelPlan* out) {
+    const int tm = (int)((M + 255) / 256);
+    PanelPlan best{tm, (int)((N + 255) / 256), 0, 0};
+    double best_end = makespan(best.tiles_m * best.wide_cols, 1.0, 0, 0.0);
+    for (int cn = 1; (int64_t)192 * (cn - 1) < N; cn++) {
+        const int64_t left = N - (int64_t)192 * cn;
+        const int cw = left > 0 ? (int)((left + 255) / 256) : 0;
+        const double end = makespan(tm * cw, 1.0, tm * cn, kNarrowCost);
+        if (end < best_end - 1e-9) {
+            best_end = end;
+            best = PanelPlan{tm, cw, cn, 0};
+        }
+    }
+    const int tl = (int)((M + 127) / 128), cl = (int)((N + 255) / 256);
+    const double low_end = makespan(tl * cl, kLowCost, 0, 0.0);
+    if (low_end < best_end - 1e-9) {
+        best_end = low_end;
+        best = PanelPlan{tl, cl, 0, 1};
+    }
+    *out = best;
+    return best_end;
+}
+
 }  // namespace
 
 size_t qgemm_f16_panel_bytes(int64_t N, int64_t K) { return ((size_t)N * K * 2 + 255) & ~(size_t)255; }
 
 // Whether the two launches beat the one whose tiles convert W for themselves: the panel costs a pass over W
-// (N K (0.5625 + 2) bytes), which 256 rows of X a tile and at least 1024 rows in all repay, and the 256 x 256 tiles
-// must keep three quarters of the compute units busy.
+// (N K (0.5625 + 2) bytes), which at least 1024 rows of X repay when the tiles keep 70 % of the device busy
+// until the last one ends.
 bool qgemm_f16_panel_pays(int64_t M, int64_t N, int64_t K) {
-    const int64_t tiles = ((M + kTile - 1) / kTile) * ((N + kTile - 1) / kTile);
-    return M >= 1024 && K % kStep == 0 && K >= kStep && tiles >= 192 && M < (1 << 24) && N < (1 << 24) && K < (1 << 24);
+    if (!(M >= 1024 && K % kStep == 0 && K >= kStep && M < (1 << 24) && N < (1 << 24) && K < (1 << 24) && N > 0)) return false;
+    PanelPlan plan;
+    const double end = plan_panel(M, N, &plan);
+    const double work = (double)M * (double)N / (256.0 * 256.0);
+    return work >= 0.70 * kUnits * end;
 }
 
-hipError_t qgemm_f16_panel(const void* W, const void* X16, const float* row_scale, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32,
-                           void* panel, hipStream_t st) {
+hipError_t qgemm_f16_panel(const void* W, const void* X, int64_t x_row_stride, void* X16, float* row_scale, void* Y, int64_t M, int64_t N, int64_t K,
+                           bool out_f32, void* panel, hipStream_t st) {
     {
         static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
         if (!raised) {
@@ -210,18 +348,22 @@ hipError_t qgemm_f16_panel(const void* W, const void* X16, const float* row_scal
             raised = true;
         }
     }
-    const int64_t pieces = N * K / 8;
-    const int64_t want = (pieces + 255) / 256;
-    hipLaunchKernelGGL(q4_0_f16_panel_kernel, dim3((unsigned)(want > 8192 ? 8192 : want)), dim3(256), 0, st, (const uint8_t*)W, (uint16_t*)panel, pieces);
-    const int tiles_m = (int)((M + kTile - 1) / kTile);
-    const int ntiles = tiles_m * (int)((N + kTile - 1) / kTile);
-    const dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
+    const int64_t halves = N * K / 16;
+    const int64_t want = (halves + 255) / 256;
+    hipLaunchKernelGGL(panel_prepare_kernel, dim3((unsigned)(M + (want > 8192 ? 8192 : want))), dim3(256), 0, st, (const uint16_t*)X, (uint16_t*)X16, row_scale,
+                       (int)M, K, x_row_stride, (const uint8_t*)W, (uint16_t*)panel, halves);
+    PanelPlan plan;
+    plan_panel(M, N, &plan);
+    const int first = plan.tiles_m * plan.wide_cols, then = plan.tiles_m * plan.narrow_cols;
+    note_kernel("hgemm_f16_nt_kernel: %d x %d tiles of %s, %d x %d tiles of 256 x 192", plan.tiles_m, plan.wide_cols, plan.low ? "128 x 256" : "256 x 256",
+                plan.tiles_m, plan.narrow_cols);
+    const dim3 grid((unsigned)(((first + 7) / 8) * 8 + ((then + 7) / 8) * 8));
     if (out_f32)
         hipLaunchKernelGGL(hgemm_f16_nt_kernel<true>, grid, dim3(512), kLdsBytes, st, (const uint16_t*)X16, (const uint16_t*)panel, Y, row_scale, (int)M,
-                           (int)N, (int)K, tiles_m, ntiles);
+                           (int)N, (int)K, plan);
     else
         hipLaunchKernelGGL(hgemm_f16_nt_kernel<false>, grid, dim3(512), kLdsBytes, st, (const uint16_t*)X16, (const uint16_t*)panel, Y, row_scale, (int)M,
-                           (int)N, (int)K, tiles_m, ntiles);
+                           (int)N, (int)K, plan);
     return hipGetLastError();
 }
 

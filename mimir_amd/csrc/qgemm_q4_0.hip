@@ -47,6 +47,7 @@
 // row's largest, whatever the row's range, and the results are scaled back
 // (exactly) when they are written.
 #include "device_util.h"
+#include "half_rows.h"
 #include "kernels.h"
 
 namespace mimir {
@@ -382,55 +383,9 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f32_kernel(const uint16_t* _
         y[t] = bf16_bits_to_f32(x[(t / K) * x_row_stride + t % K]);
 }
 
-// A row of bfloat16 to binary16, scaled by the power of two that brings the row's largest finite magnitude into
-// [2^14, 2^15) (clamped to what float32 can hold both ways); scale_back[m] undoes it. One workgroup a row; K in
-// pieces of eight elements.
 __global__ __launch_bounds__(256) void bf16_rows_to_f16_scaled_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                                       float* __restrict__ scale_back, int64_t K, int64_t x_row_stride) {
-    __shared__ uint32_t part[4];
-    const int64_t m = blockIdx.x;
-    const uint16_t* row = x + m * x_row_stride;
-    const int pieces = (int)(K >> 3);
-    uint32_t top = 0;  // the largest finite magnitude's bits (bfloat16 magnitudes order as integers)
-    for (int p = threadIdx.x; p < pieces; p += 256) {
-        u32x4 v;
-        __builtin_memcpy(&v, __builtin_assume_aligned(row + 8 * (int64_t)p, 16), 16);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t a = v[i] & 0x7fffu, b = (v[i] >> 16) & 0x7fffu;
-            if (a < 0x7f80u && a > top) top = a;
-            if (b < 0x7f80u && b > top) top = b;
-        }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint32_t other = (uint32_t)__shfl_xor((int)top, o, 64);
-        top = other > top ? other : top;
-    }
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = top;
-    __syncthreads();
-    top = part[0];
-#pragma unroll
-    for (int i = 1; i < 4; i++) top = part[i] > top ? part[i] : top;
-    int e = 0;
-    if (top != 0) {
-        const int ex = (int)(top >> 7) - 127;  // floor(log2) of a normal magnitude; subnormals count as 2^-117
-        e = 14 - ex;
-        e = e > 126 ? 126 : e < -126 ? -126 : e;
-    }
-    const float up = __uint_as_float((uint32_t)(e + 127) << 23);
-    if (threadIdx.x == 0) scale_back[m] = __uint_as_float((uint32_t)(127 - e) << 23);
-    uint16_t* out = y + m * K;
-    for (int p = threadIdx.x; p < pieces; p += 256) {
-        u32x4 v, r;
-        __builtin_memcpy(&v, __builtin_assume_aligned(row + 8 * (int64_t)p, 16), 16);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const f16x2 h = {(_Float16)(__uint_as_float(v[i] << 16) * up), (_Float16)(__uint_as_float(v[i] & 0xffff0000u) * up)};
-            r[i] = __builtin_bit_cast(uint32_t, h);
-        }
-        *(u32x4*)(out + 8 * (int64_t)p) = r;
-    }
+    bf16_row_to_f16_scaled(x, y, scale_back, K, x_row_stride, blockIdx.x);
 }
 
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n) {
@@ -477,13 +432,13 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
     const float* row_scale = nullptr;
     if (half) {
         float* sb = (float*)((uint8_t*)half_ws + half_x_bytes(M, K));
+        if (panel && qgemm_f16_panel_pays(M, N, K))
+            return qgemm_f16_panel(W, X, x_row_stride, half_ws, sb, Y, M, N, K, out_f32, (uint8_t*)half_ws + half_x_bytes(M, K) + half_scale_bytes(M), st);
         hipLaunchKernelGGL(bf16_rows_to_f16_scaled_kernel, dim3((unsigned)M), dim3(256), 0, st, (const uint16_t*)X, (uint16_t*)half_ws, sb, K,
                            x_row_stride);
         X = half_ws;
         x_row_stride = K;
         row_scale = sb;
-        if (panel && qgemm_f16_panel_pays(M, N, K))
-            return qgemm_f16_panel(W, X, row_scale, Y, M, N, K, out_f32, (uint8_t*)half_ws + half_x_bytes(M, K) + half_scale_bytes(M), st);
     }
     // the tallest tiles that still give three quarters of the compute units work: a taller tile reads less from
     // LDS per MFMA (a wavefront multiplies 32 MT x 64 of it), which is worth more than the idle quarter (measured at

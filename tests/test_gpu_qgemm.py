@@ -8,6 +8,8 @@ matrix cores), so its float32 result differs from the oracle's in the last bits,
 rounding boundary: by one unit in the last place of bfloat16, at a small share of
 the outputs. The float32 output is held to 1e-4 of max(1, |want|) at K = 4096 (the
 bound asked for is 1e-3)."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -299,12 +301,24 @@ class binary16_weights_in_tiles:
         capi.check(gpu.lib().mi355x_tune(b"qgemm.f16", 0))
 
 
-@pytest.mark.parametrize("m,n,k", [(1024, 12288, 256), (1100, 9800, 512), (2047, 6200, 768), (1300, 10241, 256)])
-def test_binary16_form_through_the_panel(m, n, k):
-    """From 1024 rows of x on, with at least 192 tiles of 256 x 256, W is first written once as a binary16 panel
-    and the product is a plain one from LDS (two launches). Shapes that fill their tiles and shapes whose last
-    tiles are ragged both ways; scales over binary16's range; rows of x apart and W at an offset. The same weights
-    as the tile kernel's, bit for bit, so the two routes differ by the order of the float32 sums only."""
+def last_kernel():
+    buf = ctypes.create_string_buffer(200)
+    capi.check(gpu.lib().mi355x_last_kernel(buf, 200))
+    return buf.value.decode()
+
+
+@pytest.mark.parametrize("m,n,k,tiles", [
+    (2048, 14336, 256, "8 x 32 tiles of 256 x 256, 8 x 32 tiles of 256 x 192"),  # the quoted shape's cut: a wide and a narrow tile a compute unit
+    (1024, 12288, 256, "4 x 0 tiles of 256 x 256, 4 x 64 tiles of 256 x 192"),
+    (2047, 6200, 768, "8 x 25 tiles of 256 x 256, 8 x 0 tiles of 256 x 192"),   # ragged both ways
+    (1300, 10241, 256, "6 x 41 tiles of 256 x 256, 6 x 0 tiles of 256 x 192"),
+    (1024, 8100, 512, "8 x 32 tiles of 128 x 256, 8 x 0 tiles of 256 x 192"),   # too few wide tiles for the device
+])
+def test_binary16_form_through_the_panel(m, n, k, tiles):
+    """From 1024 rows of x on, where its tiles keep the device busy, W is first written once as a binary16 panel
+    and the product is a plain one from LDS (two launches). Every kind of tile; shapes that fill their tiles and
+    shapes whose last tiles are ragged both ways; scales over binary16's range; rows of x apart and W at an offset.
+    The same weights as the tile kernel's, bit for bit, so the two routes differ by the order of the float32 sums only."""
     rng = np.random.default_rng(m + 3 * n + k)
     w = scales_within_binary16(rng, n * k)
     xf = rng.normal(size=(m, k)).astype(np.float32)
@@ -317,6 +331,7 @@ def test_binary16_form_through_the_panel(m, n, k):
         got32 = qgemm(w, x, n, k, capi.F32)
         got = qgemm(w, x, n, k)
         got2 = qgemm(w, x, n, k, capi.F32, x_stride=k + 24, w_offset=32)
+        assert last_kernel() == "hgemm_f16_nt_kernel: " + tiles
     check_binary16_form(w, x, n, k, got32)
     assert np.array_equal(got2, got32)
     assert np.array_equal(got, O.f32_to_bf16(got32))  # one rounding of the same float32 sums
