@@ -649,6 +649,8 @@ def main():
     ap.add_argument("--gemv-stamps", action="store_true", help="only: per-workgroup clock readings of the GEMV's launches (dispatch, x staging, rows, exit)")
     ap.add_argument("--gemm", action="store_true", help="time the prompt-sized products of Q4_K and Q6_K too (the Q4_0 ones are in every run)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prompt-sized products")
+    ap.add_argument("--gemm-shapes", default=None, metavar="MxN[,MxN...]", help="the prompt-sized products of these shapes only (K = 4096), e.g. 2048x14336")
+    ap.add_argument("--gemm-iters", type=int, default=50, help="timed calls per prompt-sized product")
     ap.add_argument("--no-shapes", action="store_true", help="skip the one-row products of the other shapes (Q8_0 4096x4096; Q4_0 down, q/o, k/v)")
     ap.add_argument("--rows", action="store_true", help="also time the Q4_0, Q4_K and Q6_K products of eight rows of x (a batch's decoding step) at the model's shapes")
     ap.add_argument("--rows-counters", metavar="VARIANT", default=None,
@@ -759,7 +761,11 @@ def main():
     if not args.no_shapes:
         out["gemv_shapes"] = shapes_bench(lib, capi, torch)
     if not args.no_gemm:
-        out["prefill_gemm"] = gemm_bench(lib, capi, torch, kquants=args.gemm)
+        if args.gemm_shapes:
+            shapes = tuple(tuple(int(v) for v in sh.split("x")) for sh in args.gemm_shapes.split(","))
+            out["prefill_gemm"] = gemm_bench(lib, capi, torch, shapes=shapes, kquants=args.gemm, iters=args.gemm_iters)
+        else:
+            out["prefill_gemm"] = gemm_bench(lib, capi, torch, kquants=args.gemm, iters=args.gemm_iters)
     if args.rows:
         out["batch_rows_gemv"] = rows_bench(lib, capi, torch)
     if not args.no_layer_step:
