@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
 # reads for a copy kernel of known size (the summaries under profiles/ hold the
 # runs): FETCH_SIZE 16278.986 KiB x 1024 x 1.99967 + WRITE_SIZE 56 KiB x 1024 x 1.0.
-TRAFFIC_BYTES_PER_LAUNCH = 33391224
+TRAFFIC_BYTES_PER_LAUNCH = 33398365
 TRAFFIC_KERNEL = "qgemv_q4_0_stream_kernel<0, 2, 7>"  # the kernel those counter runs launched
 
 

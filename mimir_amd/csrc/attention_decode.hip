@@ -11,12 +11,25 @@
 // Sixteen lanes share a key row, 16 or 32 bytes each, so a wavefront's load
 // covers four whole rows; the sixteen key groups of the workgroup take
 // consecutive keys. Scores go through LDS for the softmax, values are
-// accumulated per key group and summed through LDS. Each workgroup writes its
-// share's (max, sum, weighted values) and takes a ticket; the one that draws
-// the last ticket of its heads combines the shares, so no workgroup ever waits
-// for another. It can also leave the result in the fixed-point form the Q4_0
-// product reads (q4_act.h), which saves the conversion launch before the
-// output projection.
+// accumulated per key group and summed through LDS. The rows of a share are
+// requested before the number of keys is read (shares are fixed ranges of the
+// cache, rows past the end clamped), so that load's round trip runs beside the
+// keys'. A share's (max, sum, weighted values) reach the combining workgroup one
+// of two ways. With flag slots (the decoder's steps): every float travels as an
+// 8-byte (value, flag) pair, stored and loaded as one word, so a pair that
+// reads as flagged is complete without any fence; the first share's workgroup
+// polls the other shares' slots (all of them requested in one trip, a bounded
+// number of polls, the device's error word on a time-out), combines, and clears
+// the slots for the next launch. The workgroups it waits for never wait
+// themselves, and its own share is done before it polls. Without slots (the
+// boundary's call with its own workspace): each workgroup takes a ticket
+// (release-acquire at device scope) and the one that draws the last ticket of
+// its heads combines, so no workgroup waits at all. Either can leave the
+// result in the fixed-point form the Q4_0 product reads (q4_act.h), which
+// saves the conversion launch before the output projection. The grid is
+// (key head x query group, share, sequence): with eight key heads a head's
+// shares have workgroup indices congruent modulo eight, i.e. they run on one
+// die, and the head's rows and slots stay in that die's L2.
 #include "device_util.h"
 #include "kernels.h"
 #include "kq_act.h"
