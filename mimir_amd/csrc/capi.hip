@@ -891,7 +891,7 @@ mi355x_status mi355x_gemv_stamps(void* stamps) {
     return MI355X_OK;
 }
 
-// The kernel (name and template arguments) that the calling thread's latest Q4_0 product of one row of x launched.
+// The kernel (name and template arguments) that the calling thread's latest Q4_0 product (one row of x, or prompt-sized) launched.
 mi355x_status mi355x_last_kernel(char* buf, size_t n) {
     if (!buf || n == 0) return fail(MI355X_ERR_INTERNAL, "mi355x: last_kernel: no buffer");
     snprintf(buf, n, "%s", t_last_kernel);

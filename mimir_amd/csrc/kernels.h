@@ -305,7 +305,7 @@ hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 // While a measurement is on (capi.hip), hands out the next pair of events for a
 // launch to be bracketed by; false otherwise.
 bool next_timing_events(hipEvent_t* start, hipEvent_t* stop);
-// Records which kernel the calling thread's latest Q4_0 one-row product launched (printf-style), for mi355x_last_kernel.
+// Records which kernel the calling thread's latest Q4_0 product (of one row of x, or prompt-sized with bfloat16 x) launched (printf-style), for mi355x_last_kernel.
 void note_kernel(const char* fmt, ...);
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);
 int stream_read_out_len(int grid, int threads);

@@ -473,6 +473,7 @@ hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int
             hipLaunchKernelGGL((qgemm_q4_0_kernel<MT_, F32_, false>), grid, dim3(512), lds, st, (const uint16_t*)X, (const uint8_t*)W, Y,    \
                                (int)M, (int)N, (int)K, x_row_stride, tiles_m, ntiles, row_scale);                                            \
     } while (0)
+    note_kernel("qgemm_q4_0_kernel<%d, %s, %s>", MT, out_f32 ? "true" : "false", half ? "true" : "false");
     if (MT == 4) {
         if (out_f32) QGEMM_LAUNCH(4, true); else QGEMM_LAUNCH(4, false);
     } else if (MT == 2) {

@@ -342,14 +342,14 @@ def test_binary16_form_through_the_panel(m, n, k, tiles):
     check_f32(got32, tiles32.astype(np.float64), 2 * f32_bound(w, x, n, k), "panel route against the tile kernel")
 
 
-def test_binary16_form_rows_of_any_range():
+@pytest.mark.parametrize("m,n,k,panel", [(64, 256, 512, False), (1024, 8192, 256, True)])
+def test_binary16_form_rows_of_any_range(m, n, k, panel):
     """Each row of x is scaled by a power of two of its own before it becomes binary16:
     rows near float32's largest and smallest magnitudes, a row of zeros, a row with one
     element 2^20 above the others and a row of bfloat16 subnormals come out as exactly
     as rows of ordinary size; a row holding an infinity or a NaN has no finite results
-    and leaves the other rows alone."""
+    and leaves the other rows alone. In the tile kernel and through the panel."""
     rng = np.random.default_rng(5)
-    m, n, k = 64, 256, 512
     w = bench_blocks(rng, O.Q4_0, n * k)
     xf = rng.normal(size=(m, k)).astype(np.float32)
     xf[1] *= 2.0 ** 100
@@ -366,6 +366,7 @@ def test_binary16_form_rows_of_any_range():
     gpu.say("qgemm_bf16, binary16 weights, rows of extreme ranges")
     with binary16_weights():
         got32 = qgemm(w, x, n, k, capi.F32)
+        assert last_kernel().startswith("hgemm_f16_nt_kernel") == panel
         got_bad = qgemm(w, bad, n, k, capi.F32)
     check_binary16_form(w, x, n, k, got32)
     assert np.all(got32[3] == 0)
