@@ -101,6 +101,25 @@ __global__ void k_write(Stamp* slot, int* out, int n4) {
     }
 }
 
+// a kernel that reads n bytes with 16-byte loads (NT: non-temporal ones) from every workgroup before the next one
+// starts; its slot gets the first workgroup's entry and the last workgroup's exit
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+template <bool NT>
+__global__ void k_read(Stamp* slot, const u32x4_t* src, long long n16, int* sink) {
+    const long long t = wall_clock64();
+    u32x4_t acc = {0, 0, 0, 0};
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long long)gridDim.x * blockDim.x) {
+        const u32x4_t v = NT ? __builtin_nontemporal_load(src + i) : src[i];
+        acc ^= v;
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[threadIdx.x] = 1;  // keeps the loads
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (blockIdx.x == 0) slot->t_in = t;
+        atomicMax((unsigned long long*)&slot->t_out, (unsigned long long)wall_clock64());
+    }
+}
+
 // a kernel with dynamic LDS
 __global__ void k_lds(Stamp* slot) {
     extern __shared__ int lds[];
@@ -115,15 +134,16 @@ __global__ void k_lds(Stamp* slot) {
 
 struct Launch {
     const char* name;
-    int kind;  // 0 none, 1 none_1024, 2 stamp, 3 stamp_1024, 4 load, 5 fat, 6 fat_ptr, 7 write, 8 lds
+    int kind;  // 0 none, 1 none_1024, 2 stamp, 3 stamp_1024, 4 load, 5 fat, 6 fat_ptr, 7 write, 8 lds, 9 read, 10 read non-temporal
     int grid, block;
-    int bytes;  // kind 7: bytes written; kind 8: dynamic LDS
+    int bytes;  // kind 7: bytes written; kind 8: dynamic LDS; kinds 9, 10: bytes read
 };
 
 struct Ctx {
     Stamp* stamps;
     int* word;
     int* sink;
+    u32x4_t* big;  // 64 MB to read
     Fat* fat_dev;
     Fat fat_host;
 };
@@ -145,6 +165,8 @@ static void launch(const Launch& l, Ctx& c, int node, hipStream_t st) {
     case 6: hipLaunchKernelGGL(k_fat_ptr, dim3(l.grid), dim3(l.block), 0, st, (const Fat*)(c.fat_dev + node)); break;
     case 7: hipLaunchKernelGGL(k_write, dim3((l.bytes / 4 + l.block - 1) / l.block), dim3(l.block), 0, st, slot, c.sink, l.bytes / 4); break;
     case 8: hipLaunchKernelGGL(k_lds, dim3(l.grid), dim3(l.block), l.bytes, st, slot); break;
+    case 9: hipLaunchKernelGGL(k_read<false>, dim3(l.grid), dim3(l.block), 0, st, slot, (const u32x4_t*)c.big, (long long)l.bytes / 16, c.sink); break;
+    case 10: hipLaunchKernelGGL(k_read<true>, dim3(l.grid), dim3(l.block), 0, st, slot, (const u32x4_t*)c.big, (long long)l.bytes / 16, c.sink); break;
     }
     CHECK(hipGetLastError());
 }
@@ -229,6 +251,8 @@ int main(int argc, char** argv) {
     CHECK(hipMalloc(&c.word, 256));
     CHECK(hipMemset(c.word, 0, 256));
     CHECK(hipMalloc(&c.sink, 4 << 20));
+    CHECK(hipMalloc(&c.big, 64 << 20));
+    CHECK(hipMemset(c.big, 1, 64 << 20));
     CHECK(hipMalloc(&c.fat_dev, sizeof(Fat) * nodes));
     for (int i = 0; i < 26; i++) c.fat_host.p[i] = c.word;
     c.fat_host.tail = 1;
@@ -272,6 +296,10 @@ int main(int argc, char** argv) {
         {"pair: a kernel that stores 1 MB, then 1 x 64", {{"write", 7, 0, 256, 1 << 20}, stamp1}},
         {"pair: a kernel that stores 4 MB, then 1 x 64", {{"write", 7, 0, 256, 4 << 20}, stamp1}},
         {"pair: 256 x 1024 stamps, then 1 x 64", {{"stamp", 3, 256, 1024, 0}, stamp1}},
+        {"pair: 256 x 512 read 1 MB, then 1 x 64", {{"read", 9, 256, 512, 1 << 20}, stamp1}},
+        {"pair: 256 x 512 read 33 MB, then 1 x 64", {{"read", 9, 256, 512, 33 << 20}, stamp1}},
+        {"pair: the same 33 MB with non-temporal loads, then 1 x 64", {{"readnt", 10, 256, 512, 33 << 20}, stamp1}},
+        {"pair: 256 x 512 read 33 MB, then 256 x 512 stamps", {{"read", 9, 256, 512, 33 << 20}, {"stamp", 2, 256, 512, 0}}},
     };
     for (const Case& cs : cases) {
         const Result r = run(cs.pattern, c, nodes, replays, st);
