@@ -104,6 +104,19 @@ __device__ __forceinline__ void load_to_lds(const void* g, uint32_t lds_base) {
 __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// A 4 x 4 transposition within every quad of lanes: lane j's register k and lane k's register j change places.
+__device__ __forceinline__ void quad_transpose(float v[4], int lane) {
+    const bool odd = lane & 1, upper = lane & 2;
+    float got = dpp_f32<0xb1>(odd ? v[0] : v[1]);  // quad_perm [1,0,3,2]: the neighbour in the pair
+    if (odd) v[0] = got; else v[1] = got;
+    got = dpp_f32<0xb1>(odd ? v[2] : v[3]);
+    if (odd) v[2] = got; else v[3] = got;
+    got = dpp_f32<0x4e>(upper ? v[0] : v[2]);      // quad_perm [2,3,0,1]: the other pair
+    if (upper) v[0] = got; else v[2] = got;
+    got = dpp_f32<0x4e>(upper ? v[1] : v[3]);
+    if (upper) v[1] = got; else v[3] = got;
+}
+
 // One tile: Y [m0 .. m0 + BM) x [n0 .. n0 + BN) = (X16 . P^T) row_scale[m], float32 sums, Y bfloat16 or float32.
 template <class T, bool OUT_F32>
 __device__ __forceinline__ void tile_body(const uint16_t* __restrict__ X16, const uint16_t* __restrict__ P, void* __restrict__ Yv,
@@ -199,21 +212,43 @@ __device__ __forceinline__ void tile_body(const uint16_t* __restrict__ X16, cons
         }
     }
 
-    // the row's scale undone (a power of two: exact), then one rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51)
+    // The row's scale undone (a power of two: exact), then one rounding to the output's dtype (f32ToBF16,
+    // backend/cpu/half.go:42-51). An MFMA leaves a lane one column of Y and four consecutive rows per group of four
+    // registers; a 4 x 4 transposition within each quad of lanes turns that into one row and four consecutive columns a
+    // lane, so that a group is stored with one 8-byte (bfloat16) or 16-byte (float32) store a lane instead of four
+    // narrow ones (the stores of the untransposed form took 5 % of the launch).
+    const bool wide_ok = (N & 3) == 0 && ((uintptr_t)Yv & 15) == 0;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int m = m0 + wm * 32 * MT + mt * 32 + (i >> 2) * 8 + hi * 4 + (i & 3);
-            if (m >= M) continue;
-            const float back = row_scale[m];
+        for (int q = 0; q < 4; q++) {
+            const int m = m0 + wm * 32 * MT + mt * 32 + q * 8 + hi * 4 + (lane & 3);
+            const float back = m < M ? row_scale[m] : 0.f;
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) {
-                const int n = n0 + wn * 32 * NT + nt * 32 + r32;
-                if (n >= N) continue;
-                const float v = acc[mt][nt][i] * back;
-                if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n] = v;
-                else ((uint16_t*)Yv)[(int64_t)m * N + n] = f32_to_bf16_bits(v);
+                float v[4] = {acc[mt][nt][4 * q], acc[mt][nt][4 * q + 1], acc[mt][nt][4 * q + 2], acc[mt][nt][4 * q + 3]};
+                quad_transpose(v, lane);
+                const int n = n0 + wn * 32 * NT + nt * 32 + (r32 & ~3);
+                if (m >= M || n >= N) continue;
+#pragma unroll
+                for (int k = 0; k < 4; k++) v[k] = v[k] * back;
+                if (wide_ok && n + 3 < N) {
+                    if (OUT_F32) {
+                        const f32x4 o = {v[0], v[1], v[2], v[3]};
+                        *(f32x4*)((float*)Yv + (int64_t)m * N + n) = o;
+                    } else {
+                        const u32x2 o = {(uint32_t)f32_to_bf16_bits(v[0]) | (uint32_t)f32_to_bf16_bits(v[1]) << 16,
+                                         (uint32_t)f32_to_bf16_bits(v[2]) | (uint32_t)f32_to_bf16_bits(v[3]) << 16};
+                        *(u32x2*)((uint16_t*)Yv + (int64_t)m * N + n) = o;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        if (n + k >= N) continue;
+                        if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n + k] = v[k];
+                        else ((uint16_t*)Yv)[(int64_t)m * N + n + k] = f32_to_bf16_bits(v[k]);
+                    }
+                }
             }
         }
 }
