@@ -25,6 +25,19 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __builtin_bit_cast(float, r);
 }
 
+// A 4 x 4 transposition within every quad of lanes: lane j's register k and lane k's register j change places.
+__device__ __forceinline__ void quad_transpose(float v[4], int lane) {
+    const bool odd = lane & 1, upper = lane & 2;
+    float got = dpp_f32<0xb1>(odd ? v[0] : v[1]);  // quad_perm [1,0,3,2]: the neighbour in the pair
+    if (odd) v[0] = got; else v[1] = got;
+    got = dpp_f32<0xb1>(odd ? v[2] : v[3]);
+    if (odd) v[2] = got; else v[3] = got;
+    got = dpp_f32<0x4e>(upper ? v[0] : v[2]);      // quad_perm [2,3,0,1]: the other pair
+    if (upper) v[0] = got; else v[2] = got;
+    got = dpp_f32<0x4e>(upper ? v[1] : v[3]);
+    if (upper) v[1] = got; else v[3] = got;
+}
+
 // Sum of v over the 64 lanes, the same in every call order: an inclusive scan
 // of each row of 16 (row_shr 1, 2, 4, 8), then row_bcast:15 and row_bcast:31
 // carry the row totals up; lane 63 holds the total, returned to every lane.

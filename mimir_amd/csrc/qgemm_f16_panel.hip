@@ -104,19 +104,6 @@ __device__ __forceinline__ void load_to_lds(const void* g, uint32_t lds_base) {
 __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// A 4 x 4 transposition within every quad of lanes: lane j's register k and lane k's register j change places.
-__device__ __forceinline__ void quad_transpose(float v[4], int lane) {
-    const bool odd = lane & 1, upper = lane & 2;
-    float got = dpp_f32<0xb1>(odd ? v[0] : v[1]);  // quad_perm [1,0,3,2]: the neighbour in the pair
-    if (odd) v[0] = got; else v[1] = got;
-    got = dpp_f32<0xb1>(odd ? v[2] : v[3]);
-    if (odd) v[2] = got; else v[3] = got;
-    got = dpp_f32<0x4e>(upper ? v[0] : v[2]);      // quad_perm [2,3,0,1]: the other pair
-    if (upper) v[0] = got; else v[2] = got;
-    got = dpp_f32<0x4e>(upper ? v[1] : v[3]);
-    if (upper) v[1] = got; else v[3] = got;
-}
-
 // One tile: Y [m0 .. m0 + BM) x [n0 .. n0 + BN) = (X16 . P^T) row_scale[m], float32 sums, Y bfloat16 or float32.
 template <class T, bool OUT_F32>
 __device__ __forceinline__ void tile_body(const uint16_t* __restrict__ X16, const uint16_t* __restrict__ P, void* __restrict__ Yv,

@@ -358,20 +358,43 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_kernel(const uint16_t* __restr
         lds_barrier();
     }
 
-    // one rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51)
+    // One rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51). An MFMA leaves a lane one column of Y and
+    // four consecutive rows per group of four registers: transposed within each quad of lanes (quad_transpose) a group is
+    // one row and four consecutive columns a lane, stored with one 8-byte (bfloat16) or 16-byte (float32) store.
+    const bool wide_ok = (N & 3) == 0 && ((uintptr_t)Yv & 15) == 0;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            const int n = n0 + wn * 64 + nt * 32 + l32;
+        for (int q = 0; q < 4; q++) {
+            const int m = m0 + wm * (32 * MT) + mt * 32 + q * 8 + lh * 4 + (l32 & 3);
+            float back = 1.f;
+            if (HALF) back = m < M ? row_scale[m] : 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int m = m0 + wm * (32 * MT) + mt * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
-                if (m < M && n < N) {
-                    float v = total[mt][nt][i];
-                    if (HALF) v *= row_scale[m];
-                    if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n] = v;
-                    else ((uint16_t*)Yv)[(int64_t)m * N + n] = f32_to_bf16_bits(v);
+            for (int nt = 0; nt < 2; nt++) {
+                float v[4] = {total[mt][nt][4 * q], total[mt][nt][4 * q + 1], total[mt][nt][4 * q + 2], total[mt][nt][4 * q + 3]};
+                quad_transpose(v, l32);
+                const int n = n0 + wn * 64 + nt * 32 + (l32 & ~3);
+                if (m >= M || n >= N) continue;
+                if (HALF) {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) v[k] *= back;
+                }
+                if (wide_ok && n + 3 < N) {
+                    if (OUT_F32) {
+                        const f32x4 o = {v[0], v[1], v[2], v[3]};
+                        *(f32x4*)((float*)Yv + (int64_t)m * N + n) = o;
+                    } else {
+                        const u32x2 o = {(uint32_t)f32_to_bf16_bits(v[0]) | (uint32_t)f32_to_bf16_bits(v[1]) << 16,
+                                         (uint32_t)f32_to_bf16_bits(v[2]) | (uint32_t)f32_to_bf16_bits(v[3]) << 16};
+                        *(u32x2*)((uint16_t*)Yv + (int64_t)m * N + n) = o;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        if (n + k >= N) continue;
+                        if (OUT_F32) ((float*)Yv)[(int64_t)m * N + n + k] = v[k];
+                        else ((uint16_t*)Yv)[(int64_t)m * N + n + k] = f32_to_bf16_bits(v[k]);
+                    }
                 }
             }
         }
