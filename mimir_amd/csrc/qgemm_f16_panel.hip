@@ -98,6 +98,8 @@ __global__ __launch_bounds__(256) void panel_prepare_kernel(const uint16_t* __re
 
 // 16 bytes a lane from global memory into LDS: lane l's piece lands at lds_base + 16 l. Written out because the
 // compiler, given the builtin, waits for every load under way before any LDS access; these loads are counted by hand.
+// The instruction takes its LDS base from M0, which the compiler does not let an asm statement name as clobbered: nothing
+// else in this kernel uses M0 (no dynamically indexed registers, no LDS-direct reads), and it is set anew before every load.
 __device__ __forceinline__ void load_to_lds(const void* g, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g) : "memory");
 }
