@@ -45,13 +45,15 @@ __global__ __launch_bounds__(64 * kWaves) void qgemv_q8_0_mfma_kernel(const uint
     extern __shared__ __align__(16) uint8_t smem[];  // a slab per wavefront; later the wavefronts' sums
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n0 = blockIdx.x * 32, n = n0 + l32;
+    // The grid runs over the groups of eight rows of x first: the workgroups that read the same 32 rows of W are handed
+    // out together, so the rows come from HBM once and from the memory-side cache for the other groups.
+    const int ngroups = (M + 7) >> 3, group = (int)(blockIdx.x % (unsigned)ngroups);
+    const int n0 = (int)(blockIdx.x / (unsigned)ngroups) * 32, n = n0 + l32;
     const int nruns = nb / kRunBlocks, nbp = nb | 1;
     uint8_t* slab = smem + wave * kSlabBytes;
-    // blockIdx.y: the group of eight rows of x
-    act += (int64_t)8 * blockIdx.y * act_row_bytes;
-    y += (int64_t)8 * blockIdx.y * N;
-    M = M - 8 * (int)blockIdx.y < 8 ? M - 8 * (int)blockIdx.y : 8;
+    act += (int64_t)8 * group * act_row_bytes;
+    y += (int64_t)8 * group * N;
+    M = M - 8 * group < 8 ? M - 8 * group : 8;
 
     // piece p = 64 i + lane of a run: row p / 17 of the 32, bytes 16 (p % 17).. of its 272
     uint32_t goff[kLoads], loff[kLoads];
@@ -196,7 +198,9 @@ bool qgemv_q8_0_mfma_pays(const QGemvArgs& a) {
 
 hipError_t qgemv_q8_0_mfma(const QGemvArgs& a, hipStream_t st) {
     const size_t lds = (size_t)kWaves * kSlabBytes + kWaves * 64 * 4;
-    hipLaunchKernelGGL(qgemv_q8_0_mfma_kernel, dim3((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 7) / 8)), dim3(64 * kWaves), lds, st, (const uint8_t*)a.W,
+    const int64_t wgs = ((a.N + 31) / 32) * ((a.M + 7) / 8);
+    if (wgs > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(qgemv_q8_0_mfma_kernel, dim3((unsigned)wgs), dim3(64 * kWaves), lds, st, (const uint8_t*)a.W,
                        (const uint8_t*)a.act, a.y, (int)a.M, (int)a.N, (int)(a.K / 32), (int64_t)q8_act_bytes(a.K));
     return hipGetLastError();
 }
