@@ -29,6 +29,8 @@
 // through LDS, and each lane reads its block back as dwords. Shapes that do not
 // allow this (K not a multiple of 256, W not 16-byte aligned) take a kernel that
 // loads each lane's block where it lies.
+#include <type_traits>
+
 #include "device_util.h"
 #include "kernels.h"
 #include "q4_rows_act.h"
@@ -356,8 +358,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
     const uint8_t* mine = slab + l32 * kSlabStride + 20 * lh;
     const uint8_t* mine_d = slab + l32 * kSlabStride + 16 * lh;
     const uint32_t shift = lh ? 0u : 16u;
-    // One run of `cur` into acc, with the run (wn, nrun) requested for afterwards.
-    auto one_run = [&](float (&acc)[4], const uint8_t* wn, int nrun) {
+    // One run of `cur` into acc, with the run (wn, nrun) requested for afterwards; x_too: also the operands of x
+    // for run nrun (not when the run after has the same, as up's after gate's).
+    auto one_run = [&](auto x_too, float (&acc)[4], const uint8_t* wn, int nrun) {
         fetch_w(nxt, wn, nrun);
         // slab and tail are this wavefront's alone: every lane's reads of the last run were waited for before
         // its last MFMAs and FMAs, and a wavefront's LDS operations complete in order
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const XPair xp = xs[j];
-            fetch_x(xs[j], 4 * nrun + j);
+            if constexpr (decltype(x_too)::value) fetch_x(xs[j], 4 * nrun + j);
             i32x4 wa, wb;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -404,22 +407,18 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
         cur = nxt;
     };
 
-    // this wavefront's runs one after the other; with the SwiGLU tail, the same runs of up after those of gate
+    // this wavefront's runs one after the other; with the SwiGLU tail, each run of gate is followed by the same
+    // run of up, which meets the same operands of x
     float acc[4] = {0.f, 0.f, 0.f, 0.f}, gate_acc[4] = {0.f, 0.f, 0.f, 0.f};
     const int mine_runs = run0 < run_end ? (run_end - run0 + WAVES - 1) / WAVES : 0;
-    const int items = TAIL == kRowsSwiGLU ? 2 * mine_runs : mine_runs;
-    for (int it = 0; it < items; it++) {
-        if (TAIL == kRowsSwiGLU && it == mine_runs) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                gate_acc[j] = acc[j];
-                acc[j] = 0.f;
-            }
+    for (int it = 0; it < mine_runs; it++) {
+        const int nx = it + 1 < mine_runs ? it + 1 : it;  // the run requested ahead
+        if (TAIL == kRowsSwiGLU) {
+            one_run(std::false_type{}, gate_acc, job.W[1], run0 + it * WAVES);
+            one_run(std::true_type{}, acc, W, run0 + nx * WAVES);
+        } else {
+            one_run(std::true_type{}, acc, W, run0 + nx * WAVES);
         }
-        int nx = it + 1 < items ? it + 1 : it;  // the item requested ahead
-        const uint8_t* wn = TAIL == kRowsSwiGLU && nx >= mine_runs ? job.W[1] : W;
-        if (nx >= mine_runs) nx -= mine_runs;
-        one_run(acc, wn, run0 + nx * WAVES);
     }
 
     __syncthreads();  // every wavefront is done with its slab
