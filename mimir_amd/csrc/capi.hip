@@ -418,9 +418,14 @@ static mi355x_status qgemv_impl(int dtype, const void* W, const float* x, float*
                 ((uintptr_t)x & 15) == 0 && x_row_stride % 4 == 0) {
                 // many rows: the same fixed-point arithmetic on the int8 matrix cores
                 void* act;
-                if (mi355x_status st = act_for(src, mimir::q4_0_fx_act_bytes(K) * (size_t)M, &act)) return st;
-                HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, (hipStream_t)stream), "launch q4_0_fx_convert_act");
-                HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, (hipStream_t)stream), "launch qgemm_q4_0_fx");
+                // from some hundreds of rows on as pairs of 12-bit digits on the binary16 matrix cores, which want a
+                // workspace behind the activations (not from a fixed scratch, which is too small for it)
+                const bool pairs = !src.fixed && mimir::q4_0_fx16_form(M, K);
+                const size_t act_bytes = (mimir::q4_0_fx_act_bytes(K) * (size_t)M + 255) / 256 * 256;
+                if (mi355x_status st = act_for(src, act_bytes + (pairs ? mimir::qgemm_q4_0_fx16_ws_bytes(N, K) : 0), &act)) return st;
+                HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, pairs, (hipStream_t)stream), "launch q4_0_fx_convert_act");
+                HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, pairs ? (uint8_t*)act + act_bytes : nullptr, (hipStream_t)stream),
+                        "launch qgemm_q4_0_fx");
                 return MI355X_OK;
             }
             if (M == 1 && ((uintptr_t)x & 15) == 0) {
@@ -777,6 +782,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "qgemm.f16") == 0) {
         g_tune_gemm_f16 = value == 1 || value == 2 ? value : 0;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "q4_0.fx_pairs") == 0) {  // 0: every product of many rows on the int8 form
+        mimir::set_q4_0_fx16(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "q4_0.fx_rows") == 0) {

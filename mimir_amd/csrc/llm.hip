@@ -101,6 +101,7 @@ struct Model {
     // activations of up to max_rows rows (batch x tokens of one call)
     int64_t max_rows = 0;
     DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[5], act2, tokens_dev, next_tok;
+    DevBuf fx_panel;  // the workspace of the fixed-point Q4_0 product of a prompt's rows in its binary16 form: the largest matrix's
     hipStream_t stream = nullptr;
 
     // The decoding step as a fixed run of launches that read the position from
@@ -146,6 +147,9 @@ size_t act_row_bytes(int cls, int64_t K) {
 
 const int kNoTune[5] = {0, 0, 0, 0, 0};
 
+// Whether a prompt's fixed-point Q4_0 products of `rows` rows take the binary16 form (the model holds its workspace).
+bool fx_pairs(const Model& m, int64_t rows, int64_t K) { return m.fx_panel.p != nullptr && q4_0_fx16_form(rows, K); }
+
 // Converts rows of x once for every activation form that `ws` need.
 mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[5]) {
     for (int i = 0; i < 5; i++) done[i] = false;
@@ -156,7 +160,7 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
         if (m.act[cls].bytes < need) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: activation scratch of %zu bytes, need %zu", m.act[cls].bytes, need);
         hipError_t e = cls == kActQ4   ? q4_0_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
                        : cls == kActQ8 ? q8_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
-                       : cls == kActFx ? q4_0_fx_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
+                       : cls == kActFx ? q4_0_fx_convert_act(x, rows, K, K, m.act[cls].p, fx_pairs(m, rows, K), m.stream)
                                        : kq_convert_act(x, rows, K, K, m.act[cls].p, m.stream);
         LLM_HIP(e, "convert activations");
         done[cls] = true;
@@ -174,7 +178,7 @@ mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_
     hipError_t e;
     switch (w.dtype) {
     case kQ4_0:
-        e = cls == kActFx   ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, m.stream)
+        e = cls == kActFx   ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, fx_pairs(m, rows, w.k) ? m.fx_panel.p : nullptr, m.stream)
             : cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream)
                             : qgemv_q4_0(a, kNoTune, m.stream);
         break;
@@ -727,6 +731,15 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
         LLM_HIP(m->act[cls].alloc(act_row_bytes(cls, kk) * rows + 64), "hipMalloc(activations)");
     }
     LLM_HIP(m->act2.alloc(q4_0_act_bytes((c.hidden + 63) / 64 * 64) * c.batch + 64), "hipMalloc(activations)");
+    {
+        size_t panel = 0;  // calls of enough rows for the binary16 form of the fixed-point product: its workspace
+        for (const Block& b : m->blocks)
+            for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down, &b.qkv, &b.gate_up})
+                if (w->set() && w->dtype == kQ4_0 && q4_0_fx16_form(rows, w->k) && qgemm_q4_0_fx16_ws_bytes(w->n, w->k) > panel)
+                    panel = qgemm_q4_0_fx16_ws_bytes(w->n, w->k);
+        m->fx_panel.release();
+        if (panel) LLM_HIP(m->fx_panel.alloc(panel), "hipMalloc(fixed-point product workspace)");
+    }
     int chunk, nsplit;
     attention_plan(c.batch, c.heads, c.kv_heads, max_tokens, c.context, &chunk, &nsplit);
     size_t attn_ws = 0;  // the most splits come from the smallest chunk

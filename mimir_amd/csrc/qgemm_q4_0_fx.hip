@@ -66,7 +66,10 @@ __device__ __forceinline__ uint32_t nibbles_to_i8(uint32_t v) { return ((v | 0x8
 // One row of x with nb blocks, converted for this kernel (K = 32 nb):
 //   int8 plane[3][K]   digit j of element e at plane[j][e]; x[e] ~ scale * (d0 + 256 d1 + 65536 d2)
 //   float scale[nb]
-size_t q4_0_fx_act_bytes(int64_t K) { return (size_t)((3 * K + K / 8 + 15) / 16 * 16); }
+static size_t fx_i8_act_bytes(int64_t K) { return (size_t)((3 * K + K / 8 + 15) / 16 * 16); }
+
+// Room for either form.
+size_t q4_0_fx_act_bytes(int64_t K) { return fx_i8_act_bytes(K) > q4_0_fx16_act_bytes(K) ? fx_i8_act_bytes(K) : q4_0_fx16_act_bytes(K); }
 
 // Thread t takes elements 4t..4t+3; a block's eight threads are consecutive lanes. The integers and
 // scales are those of q4_convert_item: the block's largest magnitude maps to kFixMax.
@@ -120,10 +123,11 @@ __global__ __launch_bounds__(256) void fx_convert_kernel(const float* __restrict
     }
 }
 
-hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st) {
+hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, bool pairs, hipStream_t st) {
+    if (pairs) return q4_0_fx16_convert_act(x, M, K, x_row_stride, act, st);
     int gx = (int)((K / 4 + 255) / 256);
     hipLaunchKernelGGL(fx_convert_kernel, dim3((unsigned)gx, (unsigned)M), dim3(256), 0, st, x, x_row_stride, (int)K, (uint8_t*)act,
-                       (int64_t)q4_0_fx_act_bytes(K));
+                       (int64_t)fx_i8_act_bytes(K));
     return hipGetLastError();
 }
 
@@ -301,8 +305,9 @@ bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K) {
     return qgemm_q4_0_fx_cost_us(M, N, K) < rows_us;
 }
 
-// act: q4_0_fx_convert_act's rows. y = x . W^T (+ resid, which may be y itself).
-hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+// act: q4_0_fx_convert_act's rows, as pairs if ws is given. y = x . W^T (+ resid, which may be y itself).
+hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, void* ws, hipStream_t st) {
+    if (ws) return qgemm_q4_0_fx16(W, act, y, resid, M, N, K, ws, st);
     static std::atomic<bool> raised{false};  // threads may race here: both then set the same attribute
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void*)qgemm_q4_0_fx_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Layout::total);
@@ -312,7 +317,8 @@ hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* 
     const int tiles_m = (int)((M + kTM - 1) / kTM), ntiles = (int)((N + kTN - 1) / kTN);
     const int per_xcd = (ntiles + 7) / 8;
     hipLaunchKernelGGL(qgemm_q4_0_fx_kernel, dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), Layout::total, st, (const uint8_t*)W,
-                       (const uint8_t*)act, y, resid, (int)M, (int)N, (int)K, (int64_t)q4_0_fx_act_bytes(K), tiles_m, ntiles);
+                       (const uint8_t*)act, y, resid, (int)M, (int)N, (int)K, (int64_t)fx_i8_act_bytes(K), tiles_m, ntiles);
+    note_kernel("qgemm_q4_0_fx_kernel");
     return hipGetLastError();
 }
 
