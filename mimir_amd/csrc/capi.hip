@@ -420,8 +420,8 @@ static mi355x_status qgemv_impl(int dtype, const void* W, const float* x, float*
                 void* act;
                 // from some hundreds of rows on as pairs of 12-bit digits on the binary16 matrix cores, which want a
                 // workspace behind the activations (not from a fixed scratch, which is too small for it)
-                const bool pairs = !src.fixed && mimir::q4_0_fx16_form(M, K);
-                const size_t act_bytes = (mimir::q4_0_fx_act_bytes(K) * (size_t)M + 255) / 256 * 256;
+                const bool pairs = !src.fixed && mimir::qgemm_q4_0_fx16_pays(M, N, K);
+                const size_t act_bytes = ((pairs ? mimir::q4_0_fx16_act_bytes(K) : mimir::q4_0_fx_act_bytes(K)) * (size_t)M + 255) / 256 * 256;
                 if (mi355x_status st = act_for(src, act_bytes + (pairs ? mimir::qgemm_q4_0_fx16_ws_bytes(N, K) : 0), &act)) return st;
                 HIP_TRY(mimir::q4_0_fx_convert_act(x, M, K, x_row_stride, act, pairs, (hipStream_t)stream), "launch q4_0_fx_convert_act");
                 HIP_TRY(mimir::qgemm_q4_0_fx(W, act, y, nullptr, M, N, K, pairs ? (uint8_t*)act + act_bytes : nullptr, (hipStream_t)stream),
@@ -784,7 +784,7 @@ mi355x_status mi355x_tune(const char* key, int value) {
         g_tune_gemm_f16 = value == 1 || value == 2 ? value : 0;
         return MI355X_OK;
     }
-    if (key && strcmp(key, "q4_0.fx_pairs") == 0) {  // 0: every product of many rows on the int8 form
+    if (key && strcmp(key, "q4_0.fx_pairs") == 0) {  // 0: every product of many rows on the int8 form; 2: on the binary16 form; 1: by cost
         mimir::set_q4_0_fx16(value);
         return MI355X_OK;
     }

@@ -275,16 +275,16 @@ void set_q4_rows_waves(int v);   // measurement aid: 4 or 8 wavefronts a workgro
 void set_q4_rows_direct(int v);  // measurement aid: 1 = its kernel that loads each lane's block where it lies
 // The fixed-point Q4_0 product for many rows of float32 x on the matrix cores: x converted by q4_0_fx_convert_act
 // (q4_0_fx_act_bytes(K) bytes a row), K a multiple of 128. On the int8 matrix cores (qgemm_q4_0_fx.hip), or, with
-// `pairs` and a workspace (some hundreds of rows and more: q4_0_fx16_form says whether it pays), x converted into pairs
-// of 12-bit digits and the product on the binary16 matrix cores with the same bits (qgemm_q4_0_fx16.hip): ws
-// qgemm_q4_0_fx16_ws_bytes(N, K) bytes, 16-byte aligned; ws null: act holds the int8 form.
+// `pairs` and a workspace (some hundreds of rows and more: qgemm_q4_0_fx16_pays says when), x converted into pairs
+// of 12-bit digits (q4_0_fx16_act_bytes(K) bytes a row) and the product on the binary16 matrix cores with the same
+// bits (qgemm_q4_0_fx16.hip): ws qgemm_q4_0_fx16_ws_bytes(N, K) bytes, 16-byte aligned; ws null: act holds the int8 form.
 size_t q4_0_fx_act_bytes(int64_t K);
 hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, bool pairs, hipStream_t st);
 bool qgemm_q4_0_fx_ok(const void* W, int64_t M, int64_t N, int64_t K);
 bool qgemm_q4_0_fx_pays(const void* W, int64_t M, int64_t N, int64_t K);  // and is the faster choice against the one-row kernels
 double qgemm_q4_0_fx_cost_us(int64_t M, int64_t N, int64_t K);           // about what it takes, conversion aside
 hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* resid, int64_t M, int64_t N, int64_t K, void* ws, hipStream_t st);
-bool q4_0_fx16_form(int64_t M, int64_t K);
+bool qgemm_q4_0_fx16_pays(int64_t M, int64_t N, int64_t K);  // against the int8 form, its pass over W included
 size_t q4_0_fx16_act_bytes(int64_t K);
 hipError_t q4_0_fx16_convert_act(const float* x, int64_t M, int64_t K, int64_t x_row_stride, void* act, hipStream_t st);
 size_t qgemm_q4_0_fx16_ws_bytes(int64_t N, int64_t K);

@@ -72,7 +72,8 @@ struct Weight {
 };
 
 // The form of converted activations a weight's product reads.
-enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4 };  // kActFx: Q4_0 by many rows of x, on the matrix cores
+// kActFx: Q4_0 by many rows of x, on the int8 matrix cores; kActFxPairs: the same product through the binary16 ones
+enum ActClass { kActNone = 0, kActQ4 = 1, kActQ8 = 2, kActKQ = 3, kActFx = 4, kActFxPairs = 5, kActClasses = 6 };
 
 // qkv and gate_up: where q, k, v (gate, up) share a block dtype, finalize also keeps their rows in one
 // buffer, which a decoding step multiplies in one product (the reference concatenates the same
@@ -100,7 +101,7 @@ struct Model {
 
     // activations of up to max_rows rows (batch x tokens of one call)
     int64_t max_rows = 0;
-    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[5], act2, tokens_dev, next_tok;
+    DevBuf x, h, q, k, v, a, o, gate, up, s, xlast, hlast, logits, act[kActClasses], act2, tokens_dev, next_tok;
     DevBuf fx_panel;  // the workspace of the fixed-point Q4_0 product of a prompt's rows in its binary16 form: the largest matrix's
     hipStream_t stream = nullptr;
 
@@ -127,7 +128,7 @@ struct Model {
 int act_class(const Weight& w, int64_t rows = 1) {
     switch (w.dtype) {
     case kQ4_0:
-        if (qgemm_q4_0_fx_pays(w.buf.p, rows, w.n, w.k)) return kActFx;
+        if (qgemm_q4_0_fx_pays(w.buf.p, rows, w.n, w.k)) return qgemm_q4_0_fx16_pays(rows, w.n, w.k) ? kActFxPairs : kActFx;
         return q4_0_fixed_point_ok(w.buf.p, w.k) ? kActQ4 : kActNone;
     case kQ8_0: return q8_act_fits(w.k) ? kActQ8 : kActNone;
     case kQ4_K: case kQ6_K: return kActKQ;
@@ -141,18 +142,16 @@ size_t act_row_bytes(int cls, int64_t K) {
     case kActQ8: return q8_act_bytes(K);
     case kActKQ: return kq_act_bytes(K);
     case kActFx: return q4_0_fx_act_bytes(K);
+    case kActFxPairs: return q4_0_fx16_act_bytes(K);
     default: return 0;
     }
 }
 
 const int kNoTune[5] = {0, 0, 0, 0, 0};
 
-// Whether a prompt's fixed-point Q4_0 products of `rows` rows take the binary16 form (the model holds its workspace).
-bool fx_pairs(const Model& m, int64_t rows, int64_t K) { return m.fx_panel.p != nullptr && q4_0_fx16_form(rows, K); }
-
 // Converts rows of x once for every activation form that `ws` need.
-mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[5]) {
-    for (int i = 0; i < 5; i++) done[i] = false;
+mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[kActClasses]) {
+    for (int i = 0; i < kActClasses; i++) done[i] = false;
     for (const Weight* w : ws) {
         int cls = act_class(*w, rows);
         if (cls == kActNone || done[cls]) continue;
@@ -160,7 +159,7 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
         if (m.act[cls].bytes < need) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: activation scratch of %zu bytes, need %zu", m.act[cls].bytes, need);
         hipError_t e = cls == kActQ4   ? q4_0_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
                        : cls == kActQ8 ? q8_convert_act(x, rows, K, K, m.act[cls].p, m.stream)
-                       : cls == kActFx ? q4_0_fx_convert_act(x, rows, K, K, m.act[cls].p, fx_pairs(m, rows, K), m.stream)
+                       : cls == kActFx || cls == kActFxPairs ? q4_0_fx_convert_act(x, rows, K, K, m.act[cls].p, cls == kActFxPairs, m.stream)
                                        : kq_convert_act(x, rows, K, K, m.act[cls].p, m.stream);
         LLM_HIP(e, "convert activations");
         done[cls] = true;
@@ -172,13 +171,16 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
 // With resid, y = product + resid (which may be y); only the row kernels of the quantized dtypes add it.
 mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows, const float* resid = nullptr) {
     int cls = act_class(w, rows);
-    if (resid && (cls == kActFx || cls == kActNone)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
+    if (resid && (cls == kActFx || cls == kActFxPairs || cls == kActNone)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
     QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
     a.resid = resid;
     hipError_t e;
     switch (w.dtype) {
     case kQ4_0:
-        e = cls == kActFx   ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, fx_pairs(m, rows, w.k) ? m.fx_panel.p : nullptr, m.stream)
+        if (cls == kActFxPairs && m.fx_panel.bytes < qgemm_q4_0_fx16_ws_bytes(w.n, w.k))
+            return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: fixed-point product workspace of %zu bytes, need %zu", m.fx_panel.bytes, qgemm_q4_0_fx16_ws_bytes(w.n, w.k));
+        e = cls == kActFx || cls == kActFxPairs
+                ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, cls == kActFxPairs ? m.fx_panel.p : nullptr, m.stream)
             : cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream)
                             : qgemv_q4_0(a, kNoTune, m.stream);
         break;
@@ -217,7 +219,7 @@ static mi355x_status forward(Model& m, int64_t s) {
     const int64_t qd = (int64_t)c.heads * c.head_dim, kvd = (int64_t)c.kv_heads * c.head_dim;
     float *x = m.x.as<float>(), *h = m.h.as<float>(), *q = m.q.as<float>(), *k = m.k.as<float>(), *v = m.v.as<float>();
     float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
-    bool done[5];
+    bool done[kActClasses];
     if (mi355x_status st = embed_rows(m, m.tokens_dev.as<int32_t>(), rows, x, device_error_word())) return st;
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
@@ -446,7 +448,7 @@ static mi355x_status step_any(Model& m) {
     float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
     float *qkv = m.qkv.as<float>(), *gu = m.gu.as<float>();
     const int32_t* pos = m.state.as<int32_t>();
-    bool done[5];
+    bool done[kActClasses];
     if (mi355x_status st = embed_rows(m, m.next_tok.as<int32_t>(), B, x, device_error_word())) return st;
     AttnArgs at;
     at.q = q; at.kv_dtype = c.cache_dtype; at.out = a; at.lse = nullptr;
@@ -565,7 +567,7 @@ static mi355x_status head(Model& m, const float* xin, int64_t rows, int64_t row_
             LLM_HIP(rmsnorm(xin + r * row_stride, m.norm.buf.as<float>(), hl + r * c.embed, 1, c.embed, c.eps, m.stream), "output_norm");
     }
     const Weight& w = m.tied ? m.embed : m.output;
-    bool done[5];
+    bool done[kActClasses];
     if (mi355x_status st = convert_for(m, hl, rows, c.embed, {&w}, done)) return st;
     return linear(m, w, hl, m.logits.as<float>(), rows);
 }
@@ -726,17 +728,16 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     LLM_HIP(m->logits.alloc((size_t)rows * c.vocab * 4), "hipMalloc(logits)");
     LLM_HIP(m->tokens_dev.alloc(rows * 4), "hipMalloc"); LLM_HIP(m->next_tok.alloc(c.batch * 4), "hipMalloc");
     const int64_t kmax = c.hidden > qd ? (c.hidden > c.embed ? c.hidden : c.embed) : (qd > c.embed ? qd : c.embed);
-    for (int cls = 1; cls < 5; cls++) {
-        int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : cls == kActFx ? (kmax + 127) / 128 * 128 : (kmax + 63) / 64 * 64;
+    for (int cls = 1; cls < kActClasses; cls++) {
+        int64_t kk = cls == kActKQ ? (kmax + 255) / 256 * 256 : cls == kActFx || cls == kActFxPairs ? (kmax + 127) / 128 * 128 : (kmax + 63) / 64 * 64;
         LLM_HIP(m->act[cls].alloc(act_row_bytes(cls, kk) * rows + 64), "hipMalloc(activations)");
     }
     LLM_HIP(m->act2.alloc(q4_0_act_bytes((c.hidden + 63) / 64 * 64) * c.batch + 64), "hipMalloc(activations)");
     {
-        size_t panel = 0;  // calls of enough rows for the binary16 form of the fixed-point product: its workspace
+        size_t panel = 0;  // the workspace of the fixed-point product's binary16 form, for whichever calls take it
         for (const Block& b : m->blocks)
             for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down, &b.qkv, &b.gate_up})
-                if (w->set() && w->dtype == kQ4_0 && q4_0_fx16_form(rows, w->k) && qgemm_q4_0_fx16_ws_bytes(w->n, w->k) > panel)
-                    panel = qgemm_q4_0_fx16_ws_bytes(w->n, w->k);
+                if (w->set() && w->dtype == kQ4_0 && qgemm_q4_0_fx16_ws_bytes(w->n, w->k) > panel) panel = qgemm_q4_0_fx16_ws_bytes(w->n, w->k);
         m->fx_panel.release();
         if (panel) LLM_HIP(m->fx_panel.alloc(panel), "hipMalloc(fixed-point product workspace)");
     }

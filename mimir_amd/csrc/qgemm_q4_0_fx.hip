@@ -66,10 +66,7 @@ __device__ __forceinline__ uint32_t nibbles_to_i8(uint32_t v) { return ((v | 0x8
 // One row of x with nb blocks, converted for this kernel (K = 32 nb):
 //   int8 plane[3][K]   digit j of element e at plane[j][e]; x[e] ~ scale * (d0 + 256 d1 + 65536 d2)
 //   float scale[nb]
-static size_t fx_i8_act_bytes(int64_t K) { return (size_t)((3 * K + K / 8 + 15) / 16 * 16); }
-
-// Room for either form.
-size_t q4_0_fx_act_bytes(int64_t K) { return fx_i8_act_bytes(K) > q4_0_fx16_act_bytes(K) ? fx_i8_act_bytes(K) : q4_0_fx16_act_bytes(K); }
+size_t q4_0_fx_act_bytes(int64_t K) { return (size_t)((3 * K + K / 8 + 15) / 16 * 16); }
 
 // Thread t takes elements 4t..4t+3; a block's eight threads are consecutive lanes. The integers and
 // scales are those of q4_convert_item: the block's largest magnitude maps to kFixMax.
@@ -127,7 +124,7 @@ hipError_t q4_0_fx_convert_act(const float* x, int64_t M, int64_t K, int64_t x_r
     if (pairs) return q4_0_fx16_convert_act(x, M, K, x_row_stride, act, st);
     int gx = (int)((K / 4 + 255) / 256);
     hipLaunchKernelGGL(fx_convert_kernel, dim3((unsigned)gx, (unsigned)M), dim3(256), 0, st, x, x_row_stride, (int)K, (uint8_t*)act,
-                       (int64_t)fx_i8_act_bytes(K));
+                       (int64_t)q4_0_fx_act_bytes(K));
     return hipGetLastError();
 }
 
@@ -317,7 +314,7 @@ hipError_t qgemm_q4_0_fx(const void* W, const void* act, float* y, const float* 
     const int tiles_m = (int)((M + kTM - 1) / kTM), ntiles = (int)((N + kTN - 1) / kTN);
     const int per_xcd = (ntiles + 7) / 8;
     hipLaunchKernelGGL(qgemm_q4_0_fx_kernel, dim3((unsigned)(8 * per_xcd * tiles_m)), dim3(512), Layout::total, st, (const uint8_t*)W,
-                       (const uint8_t*)act, y, resid, (int)M, (int)N, (int)K, (int64_t)fx_i8_act_bytes(K), tiles_m, ntiles);
+                       (const uint8_t*)act, y, resid, (int)M, (int)N, (int)K, (int64_t)q4_0_fx_act_bytes(K), tiles_m, ntiles);
     note_kernel("qgemm_q4_0_fx_kernel");
     return hipGetLastError();
 }

@@ -43,7 +43,7 @@ typedef float f32x32 __attribute__((ext_vector_type(32)));
 
 constexpr int kBM = 128;        // rows of x a workgroup
 constexpr int kBN = 128;        // rows of W a workgroup
-constexpr int kMinRows = 256;   // from here on x is converted for this kernel
+constexpr int kMinRows = 256;   // fewer rows stay with the int8 form
 constexpr int kStages = 3;
 
 // A stage in LDS: the rows of x for the block, the rows of P, then the scales of both.
@@ -352,14 +352,27 @@ __global__ __launch_bounds__(256, 2) void qgemm_q4_0_fx16_kernel(const uint8_t* 
         }
 }
 
-std::atomic<int> g_fx16{1};  // measurement aid: 0 keeps every product on the int8 form
+std::atomic<int> g_fx16{1};  // measurement aid: 0 keeps every product on the int8 form, 2 takes this one whatever the shape
 
 }  // namespace
 
 void set_q4_0_fx16(int v) { g_fx16 = v; }
 
-// Whether rows of x for a product of M rows are converted for this kernel (and the product runs here).
-bool q4_0_fx16_form(int64_t M, int64_t K) { return g_fx16 != 0 && M >= kMinRows && K > 0 && K % 64 == 0; }
+// Whether the product is the faster here than in the int8 form (qgemm_q4_0_fx_cost_us), the pass over W included:
+// that pass reads the blocks and writes the panel at about 4.4 TB/s; a workgroup takes 0.82 us a block when it has its
+// compute unit to itself, and two that share one 0.74 us a block each (measured at 4096 x 4096, 14336 x 4096 and
+// 4096 x 14336 weights, 512 to 4096 rows: 512 x 4096 x 4096 stays with the int8 form, 512 x 14336 x 4096 comes here).
+bool qgemm_q4_0_fx16_pays(int64_t M, int64_t N, int64_t K) {
+    if (g_fx16 == 0 || M <= 0 || N <= 0 || K <= 0 || K % 64 != 0) return false;
+    if (g_fx16 == 2) return true;
+    if (M < kMinRows) return false;
+    const double tiles = (double)((M + kBM - 1) / kBM) * (double)((N + kBN - 1) / kBN);
+    const double per_unit = tiles / 256.0, blocks = (double)(K / 32);
+    const double rounds = (double)(int64_t)(per_unit + 0.999999);
+    const double product_us = per_unit <= 1.0 ? 0.82 * blocks : 0.74 * blocks * rounds;
+    const double panel_us = (double)N * (double)K * (18.0 / 32.0 + 2.0) / 4.4e6;
+    return panel_us + product_us < qgemm_q4_0_fx_cost_us(M, N, K);
+}
 
 // X16 [M, K / 32, 64] binary16, then XS [M, K / 32] float32: 4 K + K / 8 bytes a row.
 size_t q4_0_fx16_act_bytes(int64_t K) { return (size_t)((4 * K + K / 8 + 15) / 16 * 16); }

@@ -83,15 +83,18 @@ def test_rows_with_nan_and_inf():
     assert np.all(np.abs(got - rows)[ok] <= 1e-6 * magnitude(raw, x, n, k)[ok] + 1e-30)
 
 
-def test_prompt_shapes_pick_the_matrix_cores_by_themselves():
-    """512 rows of x by 4096 x 4096 weights: the library's own choice, within 1e-4 of max(1, |want|)."""
-    m, n, k = 512, 4096, 4096
+@pytest.mark.parametrize("m,kernel", [(512, "qgemm_q4_0_fx_kernel"), (1024, "qgemm_q4_0_fx16_kernel: 8 x 32 tiles of 128 x 128")])
+def test_prompt_shapes_pick_the_matrix_cores_by_themselves(m, kernel):
+    """512 and 1024 rows of x by 4096 x 4096 weights: the library's own choice (the int8 form, and from where its
+    pass over W pays the binary16 one), within 1e-4 of max(1, |want|)."""
+    n, k = 4096, 4096
     rng = np.random.default_rng(2)
     raw = bench_blocks(rng, O.Q4_0, n * k)
     x = rng.normal(size=(m, k)).astype(np.float32)
     buf, ptr = gpu.dev_bytes_at(raw, 0)
-    gpu.say("q4_0 fx gemm 512 x 4096 x 4096")
+    gpu.say(f"q4_0 fx gemm {m} x 4096 x 4096")
     got = gpu.qgemv(O.Q4_0, ptr, gpu.dev(x), n, k)
+    assert last_kernel() == kernel
     lo, hi = 1000, 1256
     want = O.qmatmul(O.Q4_0, raw.reshape(n, -1)[lo:hi].reshape(-1), x, hi - lo, k)
     assert np.all(np.abs(got[:, lo:hi] - want) <= 1e-4 * np.maximum(1, np.abs(want)))
@@ -105,13 +108,14 @@ def last_kernel():
 
 def pairs_and_int8(raw, x_dev, n, k):
     """The same product from 256 rows on in its two forms: 12-bit digit pairs on the binary16 matrix cores (the
-    library's choice there), and the int8 form ("q4_0.fx_pairs" = 0). Returns both and the kernels that ran."""
+    library's choice for large products; "q4_0.fx_pairs" = 2 asks for it whatever the shape), and the int8 form
+    ("q4_0.fx_pairs" = 0). Returns both and the kernels that ran."""
     l = gpu.lib()
     buf, ptr = gpu.dev_bytes_at(raw, 0)
     out, ran = [], []
     try:
         capi.check(l.mi355x_tune(b"q4_0.fx_rows", 1))
-        for pairs in (1, 0):
+        for pairs in (2, 0):
             capi.check(l.mi355x_tune(b"q4_0.fx_pairs", pairs))
             out.append(gpu.qgemv(O.Q4_0, ptr, x_dev, n, k))
             ran.append(last_kernel())
@@ -121,7 +125,7 @@ def pairs_and_int8(raw, x_dev, n, k):
     return out[0], out[1], ran
 
 
-@pytest.mark.parametrize("m,n,k,tiles", [(256, 64, 128, "2 x 1"), (300, 520, 256, "3 x 5"), (1000, 1030, 1152, "8 x 9"), (2047, 700, 768, "16 x 6"),
+@pytest.mark.parametrize("m,n,k,tiles", [(40, 100, 256, "1 x 1"), (256, 64, 128, "2 x 1"), (300, 520, 256, "3 x 5"), (1000, 1030, 1152, "8 x 9"), (2047, 700, 768, "16 x 6"),
                                          (512, 4096, 4096, "4 x 32"), (257, 129, 14336, "3 x 2")])
 def test_digit_pairs_on_the_binary16_matrix_cores_give_the_int8_form_its_bits(m, n, k, tiles):
     """Rows and columns that do not fill the last tiles, one and many blocks of K; scales of either sign, zero and
