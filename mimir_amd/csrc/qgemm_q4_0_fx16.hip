@@ -15,14 +15,22 @@
 //
 // Two launches. fx16_panel_kernel writes W's integers once as a binary16 panel P [N, K] (the pass the approximate
 // form's panel takes too, qgemm_f16_panel.hip, without the scales). qgemm_q4_0_fx16_kernel multiplies: a workgroup
-// of four wavefronts owns 128 rows of x by 128 rows of W, a wavefront 64 by 64, and a compute unit runs two such
-// workgroups, so that one computes while the other waits at its barrier or for its operands. A stage is one block (32
-// of K): the rows of x (128 bytes a row: 32 digits d0, then 32 digits d1), the rows of P (64 bytes) and the scales of
-// both (W's binary16 bits as they lie in the blocks). Everything goes from global memory straight into LDS
-// (global_load_lds_*), operands with the 16-byte pieces of a row placed so that the 16 rows a quarter wavefront reads
-// fall on all banks (piece ^ (row / 2 mod 8) in the 128-byte rows, piece ^ (row / 4 mod 4) in the 64-byte ones, which
-// the loading lane undoes in the address it reads from). Three stages in a ring, requested two blocks ahead, one
-// barrier a block.
+// of eight wavefronts owns 128 rows of x by 256 rows of W, a wavefront 64 by 64; a stage is a pair of blocks (64 of K):
+// the rows of x (128 bytes a row and block: 32 digits d0, then 32 digits d1), the rows of P (128 bytes a row: the two
+// blocks) and the scales. Operands go from global memory straight into LDS (global_load_lds_dwordx4) with the 16-byte
+// pieces of a row placed at piece ^ (row / 2 mod 8), so that the 32 rows of a fragment read fall on all banks; the
+// scales pass through registers (W's are read from the blocks themselves). Two stages, one barrier a stage.
+//
+// The products of the two scales come from the matrix cores as well: dw dx over a sub-tile is an outer product, an
+// MFMA with K = 1 on float32 operands (one exact product per output, nothing added: the rounding of a multiplication).
+// That leaves the vector unit two instructions per output and block.
+//
+// What was measured on the way (2048 and 4096 rows by 14336 x 4096): tiles of 128 x 128 in workgroups of four
+// wavefronts, two a compute unit, with everything loaded straight into LDS and three stages, 335 to 340 TFLOP/s against
+// 350 to 360 here (half as many bytes again from L2 per product); the barrier moved to the middle of a block with the
+// next block's fragments read under the last vector work, and the order of MFMAs and vector instructions inside a
+// group imposed: no change. Under this kernel the device clock settles near 1.6 GHz, lower the fewer cycles a variant
+// needs: the time did not follow the cycle counts.
 //
 // x converted by fx16_convert_kernel: X16 [M, K / 32, 64] binary16 digits, then XS [M, K / 32] float32 scales; the
 // integers and scales are those of fx_convert_kernel and q4_convert_item.
@@ -42,20 +50,21 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x32 __attribute__((ext_vector_type(32)));
 
 constexpr int kBM = 128;        // rows of x a workgroup
-constexpr int kBN = 128;        // rows of W a workgroup
+constexpr int kBN = 256;        // rows of W a workgroup
+constexpr int kRowBytes = 128;  // a row of a stage: 64 binary16
+constexpr int kLoads = 8;       // 1 KB loads (8 rows) a wavefront issues per stage: 512 rows
 constexpr int kMinRows = 256;   // fewer rows stay with the int8 form
-constexpr int kStages = 3;
 
-// A stage in LDS: the rows of x for the block, the rows of P, then the scales of both.
+// A stage in LDS: the rows of x for the even block, for the odd block, the rows of P, then the scales.
 struct Stage {
-    static constexpr int a = 0;                      // [kBM] rows of 128 bytes
-    static constexpr int b = kBM * 128;              // [kBN] rows of 64 bytes
-    static constexpr int sx = b + kBN * 64;          // float [kBM]
-    static constexpr int sw = sx + kBM * 4;          // uint32 [kBN]: binary16 bits
-    static constexpr int bytes = sw + kBN * 4;
+    static constexpr int a = 0;                          // [2][kBM] rows
+    static constexpr int b = 2 * kBM * kRowBytes;        // [kBN] rows
+    static constexpr int sx = b + kBN * kRowBytes;       // float [2][kBN]: x's in the first kBM of each, the rest so that every thread stores
+    static constexpr int sw = sx + 2 * kBN * 4;          // float [2][kBN]
+    static constexpr int bytes = sw + 2 * kBN * 4;
 };
-static_assert(Stage::bytes % 1024 == 0, "stages start on a boundary the loads' layout can assume");
-constexpr size_t kLdsBytes = kStages * (size_t)Stage::bytes;  // 75 KB: two workgroups a compute unit
+static_assert(Stage::bytes % 1024 == 0, "stages start on the boundary the loads assume");
+constexpr size_t kLdsBytes = 2 * (size_t)Stage::bytes;
 
 // Thread t takes elements 4t..4t+3 of row blockIdx.y; a block's eight threads are consecutive lanes.
 __global__ __launch_bounds__(256) void fx16_convert_kernel(const float* __restrict__ x, int64_t x_row_stride, int K, uint16_t* __restrict__ X16,
@@ -141,15 +150,7 @@ __global__ __launch_bounds__(256) void fx16_panel_kernel(const uint8_t* __restri
 __device__ __forceinline__ void load_to_lds(const void* g, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g) : "memory");
 }
-// 4 bytes a lane (lane l's lands at lds_base + 4 l), and 2 bytes a lane, which LDS receives as a zero-extended dword.
-__device__ __forceinline__ void load_dword_to_lds(const void* g, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(g) : "memory");
-}
-__device__ __forceinline__ void load_ushort_to_lds(const void* g, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_ushort %1, off" ::"s"(lds_base), "v"(g) : "memory");
-}
-constexpr int kLoads = 7;  // a wavefront's loads per stage: four of x's rows, two of P's, one of scales
-__device__ __forceinline__ void wait_all_but_last_stage() { asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); }
+__device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // A die's workgroups (every eighth, round-robin) take a contiguous range of the tiles, the tile's rows of x varying
@@ -159,77 +160,57 @@ __device__ __forceinline__ int tile_of(int b, int ntiles) {
     return (b & 7) * per_die + (b >> 3);
 }
 
-__global__ __launch_bounds__(256, 2) void qgemm_q4_0_fx16_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ P,
-                                                                 const uint16_t* __restrict__ X16, const float* __restrict__ XS, float* y,
-                                                                 const float* resid,  // may be y
-                                                                 int M, int N, int K, int tiles_m, int ntiles) {
+__global__ __launch_bounds__(512) void qgemm_q4_0_fx16_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ P,
+                                                              const uint16_t* __restrict__ X16, const float* __restrict__ XS, float* y,
+                                                              const float* resid,  // may be y
+                                                              int M, int N, int K, int tiles_m, int ntiles) {
     extern __shared__ __align__(1024) char lds[];
     const int t = tile_of((int)blockIdx.x, ntiles);
     if (t >= ntiles) return;  // the whole workgroup
     const int m0 = (t % tiles_m) * kBM, n0 = (t / tiles_m) * kBN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 2, wn = wave & 3;
     const int nb = K >> 5;
 
-    // This wavefront's loads of a stage. Rows past the matrix re-read its last row (their results are not stored).
-    //   j = 0..3: rows [8 (4 wave + j), + 8) of x: a lane one 16-byte piece of a 128-byte row
-    //   j = 4, 5: rows [16 (2 wave + j - 4), + 16) of P: a lane one piece of a 64-byte row
-    //   j = 6:    wavefronts 0 and 1 the scales of x's rows [64 wave, + 64), 2 and 3 those of W's rows [64 (wave - 2), + 64)
+    // This wavefront's loads: load g = kLoads wave + j brings rows [8 g, 8 g + 8) of the stage: x's rows for the even
+    // block, for the odd block, then P's. Rows past the matrix re-read its last row (their results are not stored).
     const char* from[kLoads];
     uint32_t into[kLoads];
+    int advance[kLoads];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int first = 8 * (4 * wave + j), row = first + (lane >> 3);
+    for (int j = 0; j < kLoads; j++) {
+        const int first = 8 * (kLoads * wave + j);
+        const int row = first + (lane >> 3);
         const int piece = (lane & 7) ^ ((row >> 1) & 7);
-        const int m = m0 + row < M ? m0 + row : M - 1;
-        from[j] = (const char*)(X16 + (size_t)m * nb * 64 + 8 * piece);
-        into[j] = (uint32_t)(Stage::a + first * 128);
+        const uint16_t* base;
+        if (first < 2 * kBM) {
+            const int r = row & (kBM - 1), odd = row >> 7;
+            const int m = m0 + r < M ? m0 + r : M - 1;
+            base = X16 + ((size_t)m * nb + odd) * 64;
+            advance[j] = 2 * kRowBytes;
+        } else {
+            const int r = row - 2 * kBM;
+            const int n = n0 + r < N ? n0 + r : N - 1;
+            base = P + (size_t)n * K;
+            advance[j] = kRowBytes;
+        }
+        from[j] = (const char*)(base + 8 * piece);
+        into[j] = (uint32_t)(first * kRowBytes);
     }
-#pragma unroll
-    for (int j = 4; j < 6; j++) {
-        const int first = 16 * (2 * wave + j - 4), row = first + (lane >> 2);
-        const int piece = (lane & 3) ^ ((row >> 2) & 3);
-        const int n = n0 + row < N ? n0 + row : N - 1;
-        from[j] = (const char*)(P + (size_t)n * K + 8 * piece);
-        into[j] = (uint32_t)(Stage::b + first * 64);
-    }
-    const bool x_scales = wave < 2;  // uniform
-    if (x_scales) {
-        const int row = 64 * wave + lane;
-        from[6] = (const char*)(XS + (size_t)(m0 + row < M ? m0 + row : M - 1) * nb);
-        into[6] = (uint32_t)(Stage::sx + 4 * 64 * wave);
-    } else {
-        const int row = 64 * (wave - 2) + lane;
-        from[6] = (const char*)(W + (size_t)(n0 + row < N ? n0 + row : N - 1) * nb * 18);
-        into[6] = (uint32_t)(Stage::sw + 4 * 64 * (wave - 2));
-    }
-    const int scale_step = x_scales ? 4 : 18;
+    // the scales: thread t takes block t % 2 of the stage for row t / 2 of W and of x (x's rows beyond kBM: loaded and
+    // stored like the others, so that no branch is needed, and never read)
+    const int srow = tid >> 1, sodd = tid & 1;
+    const uint8_t* wscale = W + ((size_t)(n0 + srow < N ? n0 + srow : N - 1) * nb + sodd) * 18;
+    const float* xscale = XS + (size_t)(m0 + srow < M ? m0 + srow : M - 1) * nb + sodd;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
-    // Every load into the stage at stage_base, `ahead` (0 or 1) blocks on from the last request.
-    auto request = [&](uint32_t stage_base, int ahead) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            from[j] += 128 * ahead;
-            load_to_lds(from[j], __builtin_amdgcn_readfirstlane(stage_base + into[j]));
-        }
-#pragma unroll
-        for (int j = 4; j < 6; j++) {
-            from[j] += 64 * ahead;
-            load_to_lds(from[j], __builtin_amdgcn_readfirstlane(stage_base + into[j]));
-        }
-        from[6] += scale_step * ahead;
-        if (x_scales) load_dword_to_lds(from[6], __builtin_amdgcn_readfirstlane(stage_base + into[6]));
-        else load_ushort_to_lds(from[6], __builtin_amdgcn_readfirstlane(stage_base + into[6]));
-    };
 
     const int r32 = lane & 31, hi = lane >> 5;
-    int a_off[4], b_off[2];  // x: piece 2 p + hi is half p % 2 of digit p / 2; P: piece 2 h + hi is half h
+    const int swz = (r32 >> 1) & 7;
+    int piece_off[4];  // of a row's pieces 2 p + hi: of x, half p % 2 of digit p / 2; of P, half p % 2 of the stage's block p / 2
 #pragma unroll
-    for (int p = 0; p < 4; p++) a_off[p] = ((2 * p + hi) ^ ((r32 >> 1) & 7)) * 16;
-#pragma unroll
-    for (int h = 0; h < 2; h++) b_off[h] = ((2 * h + hi) ^ ((r32 >> 2) & 3)) * 16;
-    const int a_row = Stage::a + (wm * 64 + r32) * 128, b_row = Stage::b + (wn * 64 + r32) * 64;
+    for (int p = 0; p < 4; p++) piece_off[p] = ((2 * p + hi) ^ swz) * 16;
+    const int a_row = (wm * 64 + r32) * kRowBytes, b_row = Stage::b + (wn * 64 + r32) * kRowBytes;
 
     f32x16 acc[2][2];
 #pragma unroll
@@ -239,82 +220,100 @@ __global__ __launch_bounds__(256, 2) void qgemm_q4_0_fx16_kernel(const uint8_t* 
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mt][nt][i] = 0.f;
 
-    // Blocks 0 and 1 are requested before the loop, block i + 2 during block i. No branches around the loads, and
-    // always seven a stage, so that the count the wait leaves under way is right: past the end the last block is
-    // requested again, into a stage that is not read any more.
-    request(lds0, 0);
-    request(lds0 + Stage::bytes, 1);  // K has at least two blocks
-    int cur = 0;  // the stage of block i
-    for (int i = 0; i < nb; i++) {
-        wait_all_but_last_stage();  // this wavefront's part of block i has landed (the seven loads after it may be under way)
-        lds_barrier();              // everyone's has, and everyone has read block i - 1's stage for the last time
-        const int nxt2 = cur == 0 ? 2 : cur - 1;  // (cur + 2) % 3: block i - 1's stage
-        const char* st = lds + cur * Stage::bytes;
-        request(lds0 + nxt2 * Stage::bytes, i + 2 < nb ? 1 : 0);
-        cur = cur == 2 ? 0 : cur + 1;
-
-        f16x8 a[2][2][2], b[2][2];  // a[mt][digit][half], b[nt][half]
-        auto read_a = [&](int mt) {
+    const int nstages = K / 64;
+    {
+        const float dw = f16_bits_to_f32(load_u16(wscale));
+        const float dx = *xscale;
 #pragma unroll
-            for (int p = 0; p < 4; p++) a[mt][p >> 1][p & 1] = *(const f16x8*)(st + a_row + mt * 32 * 128 + a_off[p]);
-        };
+        for (int j = 0; j < kLoads; j++) load_to_lds(from[j], __builtin_amdgcn_readfirstlane(lds0 + into[j]));
+        ((float*)(lds + Stage::sw))[sodd * kBN + srow] = dw;
+        ((float*)(lds + Stage::sx))[sodd * kBN + srow] = dx;
+    }
+    // No branches around the loads and stores: past the end the last stage is requested and stored again, into the
+    // buffer that is not being read.
+    for (int i = 0; i < nstages; i++) {
+        wait_loads();   // this wavefront's part of stage i has landed
+        lds_barrier();  // everyone's has, with the scales, and everyone has read the other stage for the last time
+        const int step = i + 1 < nstages ? 1 : 0;
+        const uint32_t next = lds0 + ((i + 1) & 1) * Stage::bytes;
+        char* next_p = lds + ((i + 1) & 1) * Stage::bytes;
+        const char* st = lds + (i & 1) * Stage::bytes;
+        wscale += 36 * step;
+        xscale += 2 * step;
+        const float next_dw = f16_bits_to_f32(load_u16(wscale));
+        const float next_dx = *xscale;
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
+        for (int odd = 0; odd < 2; odd++) {
+            // half of the next stage's loads with each block
 #pragma unroll
-            for (int h = 0; h < 2; h++) b[nt][h] = *(const f16x8*)(st + b_row + nt * 32 * 64 + b_off[h]);
-        read_a(0);
-        // The products of the two scales, dw dx rounded to float32, come from the matrix cores as well: an outer
-        // product is an MFMA with K = 1 (float32 operands, one exact product per output and nothing added to it, so
-        // the same rounding as a multiplication). v_mfma_f32_32x32x1_2b_f32 makes two of them: its first 32 lanes give
-        // x's rows and W's rows for the first, the other 32 for the second; here the 32 rows of x of sub-tiles
-        // (mt, 0) and (mt, 1) and the 64 rows of W of both.
-        const float dwv = f16_bits_to_f32((uint16_t)((const uint32_t*)(st + Stage::sw))[wn * 64 + lane]);
-        float dxv[2];
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++) dxv[mt] = ((const float*)(st + Stage::sx))[wm * 64 + mt * 32 + r32];
-        auto scales = [&](int mt, f32x32& w) {
-            f32x32 zero;
-#pragma unroll
-            for (int e = 0; e < 32; e++) zero[e] = 0.f;
-            w = __builtin_amdgcn_mfma_f32_32x32x1f32(dxv[mt], dwv, zero, 0, 0, 0);
-        };
-        // Sub-tile s = 2 mt + nt: its four MFMAs are issued with the finish of the sub-tile before it, so that the
-        // vector unit works while the matrix cores do (two pairs of sums live at a time; more, and registers spill).
-        auto multiply = [&](int sub, f32x16& c0, f32x16& c1) {
-            const int mt = sub >> 1, nt = sub & 1;
-            f32x16 zero;
-#pragma unroll
-            for (int e = 0; e < 16; e++) zero[e] = 0.f;
-            c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][0][0], b[nt][0], zero, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][1][0], b[nt][0], zero, 0, 0, 0);
-            c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][0][1], b[nt][1], c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][1][1], b[nt][1], c1, 0, 0, 0);
-        };
-        auto finish = [&](int sub, const f32x16& c0, const f32x16& c1, const f32x32& w) {
-            const int mt = sub >> 1, nt = sub & 1;
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const float isum = fmaf(c1[e], 4096.f, c0[e]);  // the exact integer, rounded once
-                acc[mt][nt][e] = fmaf(w[16 * nt + e], isum, acc[mt][nt][e]);
+            for (int j = odd * kLoads / 2; j < (odd + 1) * kLoads / 2; j++) {
+                from[j] += advance[j] * step;
+                load_to_lds(from[j], __builtin_amdgcn_readfirstlane(next + into[j]));
             }
-        };
-        f32x16 p0, p1, q0, q1;
-        f32x32 w;
-        multiply(0, p0, p1);
-        scales(0, w);
+            f16x8 a[2][2][2], b[2][2];  // a[mt][digit][half], b[nt][half]
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int p = 0; p < 4; p++)
+                    a[mt][p >> 1][p & 1] = *(const f16x8*)(st + Stage::a + odd * kBM * kRowBytes + a_row + mt * 32 * kRowBytes + piece_off[p]);
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) b[nt][h] = *(const f16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[2 * odd + h]);
+            // The operands of the outer products that give dw dx: v_mfma_f32_32x32x1_2b_f32 makes two, its first 32
+            // lanes giving x's rows and W's rows of the first, the other 32 of the second; here the 32 rows of x of
+            // sub-tiles (mt, 0) and (mt, 1), and the 64 rows of W of both (a lane each).
+            const float dwv = ((const float*)(st + Stage::sw))[odd * kBN + wn * 64 + lane];
+            float dxv[2];
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++) dxv[mt] = ((const float*)(st + Stage::sx))[odd * kBN + wm * 64 + mt * 32 + r32];
+            auto scales = [&](int mt, f32x32& w) {
+                f32x32 zero;
+#pragma unroll
+                for (int e = 0; e < 32; e++) zero[e] = 0.f;
+                w = __builtin_amdgcn_mfma_f32_32x32x1f32(dxv[mt], dwv, zero, 0, 0, 0);
+            };
+            // Sub-tile s = 2 mt + nt: its four MFMAs are issued with the finish of the sub-tile before it, so that the
+            // vector unit works while the matrix cores do (two pairs of sums live at a time; more, and registers spill).
+            auto multiply = [&](int sub, f32x16& c0, f32x16& c1) {
+                const int mt = sub >> 1, nt = sub & 1;
+                f32x16 zero;
+#pragma unroll
+                for (int e = 0; e < 16; e++) zero[e] = 0.f;
+                c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][0][0], b[nt][0], zero, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][1][0], b[nt][0], zero, 0, 0, 0);
+                c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][0][1], b[nt][1], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][1][1], b[nt][1], c1, 0, 0, 0);
+            };
+            auto finish = [&](int sub, const f32x16& c0, const f32x16& c1, const f32x32& w) {
+                const int mt = sub >> 1, nt = sub & 1;
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const float isum = fmaf(c1[e], 4096.f, c0[e]);  // the exact integer, rounded once
+                    acc[mt][nt][e] = fmaf(w[16 * nt + e], isum, acc[mt][nt][e]);
+                }
+            };
+            f32x16 p0, p1, q0, q1;
+            f32x32 w;
+            multiply(0, p0, p1);
+            scales(0, w);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(1, q0, q1);
+            finish(0, p0, p1, w);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(2, p0, p1);
+            finish(1, q0, q1, w);
+            __builtin_amdgcn_sched_barrier(0);
+            scales(1, w);
+            multiply(3, q0, q1);
+            finish(2, p0, p1, w);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(3, q0, q1, w);
+        }
+        // the next stage's scales, at the end: by now their loads have landed with everything requested before them
         __builtin_amdgcn_sched_barrier(0);
-        multiply(1, q0, q1);
-        read_a(1);
-        finish(0, p0, p1, w);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(2, p0, p1);
-        finish(1, q0, q1, w);
-        __builtin_amdgcn_sched_barrier(0);
-        scales(1, w);
-        multiply(3, q0, q1);
-        finish(2, p0, p1, w);
-        __builtin_amdgcn_sched_barrier(0);
-        finish(3, q0, q1, w);
+        ((float*)(next_p + Stage::sw))[sodd * kBN + srow] = next_dw;
+        ((float*)(next_p + Stage::sx))[sodd * kBN + srow] = next_dx;
     }
 
     // An MFMA leaves a lane one column of y and four consecutive rows per group of four registers; a 4 x 4
@@ -359,17 +358,15 @@ std::atomic<int> g_fx16{1};  // measurement aid: 0 keeps every product on the in
 void set_q4_0_fx16(int v) { g_fx16 = v; }
 
 // Whether the product is the faster here than in the int8 form (qgemm_q4_0_fx_cost_us), the pass over W included:
-// that pass reads the blocks and writes the panel at about 4.4 TB/s; a workgroup takes 0.82 us a block when it has its
-// compute unit to itself, and two that share one 0.74 us a block each (measured at 4096 x 4096, 14336 x 4096 and
-// 4096 x 14336 weights, 512 to 4096 rows: 512 x 4096 x 4096 stays with the int8 form, 512 x 14336 x 4096 comes here).
+// that pass reads the blocks and writes the panel at about 4.4 TB/s; a workgroup takes about 2.85 us a stage of 64 of K,
+// one a compute unit at a time (measured at 4096 x 4096, 14336 x 4096 and 4096 x 14336 weights, 512 to 4096 rows:
+// 512 x 4096 x 4096 stays with the int8 form, 512 x 14336 x 4096 comes here).
 bool qgemm_q4_0_fx16_pays(int64_t M, int64_t N, int64_t K) {
     if (g_fx16 == 0 || M <= 0 || N <= 0 || K <= 0 || K % 64 != 0) return false;
     if (g_fx16 == 2) return true;
     if (M < kMinRows) return false;
-    const double tiles = (double)((M + kBM - 1) / kBM) * (double)((N + kBN - 1) / kBN);
-    const double per_unit = tiles / 256.0, blocks = (double)(K / 32);
-    const double rounds = (double)(int64_t)(per_unit + 0.999999);
-    const double product_us = per_unit <= 1.0 ? 0.82 * blocks : 0.74 * blocks * rounds;
+    const int64_t tiles = ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN);
+    const double product_us = (double)((tiles + 255) / 256) * (double)(K / 64) * 2.85;
     const double panel_us = (double)N * (double)K * (18.0 / 32.0 + 2.0) / 4.4e6;
     return panel_us + product_us < qgemm_q4_0_fx_cost_us(M, N, K);
 }
@@ -409,9 +406,9 @@ hipError_t qgemm_q4_0_fx16(const void* W, const void* act, float* y, const float
     const uint16_t* X16 = (const uint16_t*)act;
     const float* XS = (const float*)(X16 + (size_t)M * K * 2);
     const int wgs = (int)(((ntiles + 7) / 8) * 8);
-    hipLaunchKernelGGL(qgemm_q4_0_fx16_kernel, dim3((unsigned)wgs), dim3(256), kLdsBytes, st, (const uint8_t*)W, P, X16, XS, y, resid, (int)M, (int)N,
+    hipLaunchKernelGGL(qgemm_q4_0_fx16_kernel, dim3((unsigned)wgs), dim3(512), kLdsBytes, st, (const uint8_t*)W, P, X16, XS, y, resid, (int)M, (int)N,
                        (int)K, (int)tiles_m, (int)ntiles);
-    note_kernel("qgemm_q4_0_fx16_kernel: %lld x %lld tiles of 128 x 128", (long long)tiles_m, (long long)(ntiles / tiles_m));
+    note_kernel("qgemm_q4_0_fx16_kernel: %lld x %lld tiles of 128 x 256", (long long)tiles_m, (long long)(ntiles / tiles_m));
     return hipGetLastError();
 }
 

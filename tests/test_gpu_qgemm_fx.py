@@ -83,9 +83,9 @@ def test_rows_with_nan_and_inf():
     assert np.all(np.abs(got - rows)[ok] <= 1e-6 * magnitude(raw, x, n, k)[ok] + 1e-30)
 
 
-@pytest.mark.parametrize("m,kernel", [(512, "qgemm_q4_0_fx_kernel"), (1024, "qgemm_q4_0_fx16_kernel: 8 x 32 tiles of 128 x 128")])
+@pytest.mark.parametrize("m,kernel", [(512, "qgemm_q4_0_fx_kernel"), (2048, "qgemm_q4_0_fx16_kernel: 16 x 16 tiles of 128 x 256")])
 def test_prompt_shapes_pick_the_matrix_cores_by_themselves(m, kernel):
-    """512 and 1024 rows of x by 4096 x 4096 weights: the library's own choice (the int8 form, and from where its
+    """512 and 2048 rows of x by 4096 x 4096 weights: the library's own choice (the int8 form, and from where its
     pass over W pays the binary16 one), within 1e-4 of max(1, |want|)."""
     n, k = 4096, 4096
     rng = np.random.default_rng(2)
@@ -125,8 +125,8 @@ def pairs_and_int8(raw, x_dev, n, k):
     return out[0], out[1], ran
 
 
-@pytest.mark.parametrize("m,n,k,tiles", [(40, 100, 256, "1 x 1"), (256, 64, 128, "2 x 1"), (300, 520, 256, "3 x 5"), (1000, 1030, 1152, "8 x 9"), (2047, 700, 768, "16 x 6"),
-                                         (512, 4096, 4096, "4 x 32"), (257, 129, 14336, "3 x 2")])
+@pytest.mark.parametrize("m,n,k,tiles", [(40, 100, 256, "1 x 1"), (256, 64, 128, "2 x 1"), (300, 520, 256, "3 x 3"), (1000, 1030, 1152, "8 x 5"), (2047, 700, 768, "16 x 3"),
+                                         (512, 4096, 4096, "4 x 16"), (257, 129, 14336, "3 x 1")])
 def test_digit_pairs_on_the_binary16_matrix_cores_give_the_int8_form_its_bits(m, n, k, tiles):
     """Rows and columns that do not fill the last tiles, one and many blocks of K; scales of either sign, zero and
     subnormal; rows of x of very different magnitude, a block of zeros, a tiny and a huge block, a NaN and an
@@ -142,7 +142,7 @@ def test_digit_pairs_on_the_binary16_matrix_cores_give_the_int8_form_its_bits(m,
     x[m - 1, 7] = np.inf
     gpu.say(f"q4_0 fx gemm, digit pairs, M={m} N={n} K={k}")
     got, int8, ran = pairs_and_int8(raw, gpu.dev(x), n, k)
-    assert ran == [f"qgemm_q4_0_fx16_kernel: {tiles} tiles of 128 x 128", "qgemm_q4_0_fx_kernel"]
+    assert ran == [f"qgemm_q4_0_fx16_kernel: {tiles} tiles of 128 x 256", "qgemm_q4_0_fx_kernel"]
     assert np.isnan(got[5]).all() and np.isnan(got[m - 1]).all() and not np.isnan(got[:5]).any()
     assert np.array_equal(got.view(np.uint32), int8.view(np.uint32))
     if m * n * k <= 1 << 30:  # the larger ones rest on the int8 form, which the tests above hold to the oracle
