@@ -502,7 +502,8 @@ def gemm_bench(lib, capi, torch, shapes=((512, 4096), (512, 14336), (2048, 4096)
     kinds = (("q4_0", capi.Q4_0, 2500.0, "frac_of_bf16_peak"), ("q4_0_binary16_weights", capi.Q4_0, 2500.0, "frac_of_f16_peak"),
              ("q4_K", capi.Q4_K, 5000.0, "frac_of_int8_peak"), ("q6_K", capi.Q6_K, 5000.0, "frac_of_int8_peak"))
     # float32 activations by Q4_0 (what the decoder's prompt pass multiplies): mi355x_qgemv, whose 24-bit
-    # fixed-point x takes three int8 multiplications a weight
+    # fixed-point x takes three int8 multiplications a weight, or, where the library's cost model says so, two
+    # binary16 ones (the same integers as pairs of 12-bit digits, the same bits); priced against the int8 peak
     res = {}
     for m, n in shapes:
         w = torch.from_numpy(bench_blocks_q4_0(rng, n * k)).to("cuda:0")

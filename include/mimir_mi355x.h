@@ -106,7 +106,10 @@ MI355X_API mi355x_status mi355x_stream_release(void* stream);
  * x by Q4_0 or by a small Q8_0, Q4_K or Q6_K matrix; Q8_0 weights are read
  * once for up to eight rows) or kernels on the int8 matrix cores (Q4_0 from two
  * rows on: up to some tens of rows a kernel that reads W once per eight rows,
- * beyond them a tiled one; two to eight rows by a large Q8_0
+ * beyond them a tiled one, and from some hundreds of rows by a large matrix the
+ * same integers through the binary16 matrix cores, with the tiled one's bits,
+ * which takes a workspace of 2 N K bytes in the stream's scratch; two to eight
+ * rows by a large Q8_0
  * matrix; Q4_K, Q6_K from enough rows on); which one ran changes the results
  * only by the order of float32 additions (Q4_0, Q8_0), or not at all (Q8_0
  * among its row kernels, Q4_K, Q6_K). */
@@ -374,7 +377,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * "attention.fence" = 0 makes the ticket that hands its shares over a relaxed operation instead of a
  * release-acquire one at device scope, 2 also stores and loads the shares plainly (both to be measured; 1 restores).
  * "q4_0.fx_rows" = n sends Q4_0 products of at least n rows of float32 x to the
- * int8 matrix cores whatever the shape (0: the built-in cost model).
+ * int8 matrix cores whatever the shape (0: the built-in cost model);
+ * "q4_0.fx_pairs" = 0 keeps those products off the binary16 form of that
+ * kernel, 2 sends them all there (1: its cost model).
  * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
  * kernels takes; "kquant.path" = 1 forces their variant that reads x from
  * global memory (otherwise used only for rows of x too long for the LDS), 2
