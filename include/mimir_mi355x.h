@@ -157,8 +157,11 @@ MI355X_API mi355x_status mi355x_qgemv_act(int dtype, const void* W, const void* 
  * one rounding to x's dtype): X [M, K] bfloat16 with rows x_row_stride elements
  * apart, W [N, K] of any block dtype, Y [M, N] contiguous of out_dtype
  * MI355X_BF16 (the reference's result) or MI355X_F32 (the same sums before the
- * rounding). Q4_0 runs on the bfloat16 matrix cores, exactly (each weight as two
- * bfloat16 halves), when K is a multiple of 256, X and W are 16-byte aligned
+ * rounding). Q4_0 runs on the bfloat16 matrix cores without rounding any
+ * operand (each weight as two bfloat16 halves; or, for large products, the
+ * weights' integers against x block by block and one float32 FMA per block with
+ * the block's scale, which takes a workspace of 2 N K bytes in the stream's
+ * scratch), when K is a multiple of 256, X and W are 16-byte aligned
  * and rows of X are a multiple of 8 elements apart; otherwise, and for the other
  * dtypes, X goes through mi355x_qgemv as float32. Q4_K and Q6_K then run on
  * the int8 matrix cores from a few rows of X on, with the CPU's results bit for
@@ -380,6 +383,9 @@ MI355X_API int64_t mi355x_backend_graph_replays(void* backend);
  * int8 matrix cores whatever the shape (0: the built-in cost model);
  * "q4_0.fx_pairs" = 0 keeps those products off the binary16 form of that
  * kernel, 2 sends them all there (1: its cost model).
+ * "qgemm.blocks" = 0 keeps the exact Q4_0 products of mi355x_qgemm_bf16 on the
+ * kernel that needs no workspace, 2 sends them all through the panel of the
+ * weights' integers (1: by shape).
  * "kquant.rows" = 1, 2 or 4 fixes the rows of W a wavefront of the Q4_K / Q6_K
  * kernels takes; "kquant.path" = 1 forces their variant that reads x from
  * global memory (otherwise used only for rows of x too long for the LDS), 2

@@ -323,6 +323,12 @@ mi355x_status mi355x_qgemm_bf16(int dtype, const void* W, const void* X, void* Y
     }
     void* ws;
     if (dtype == MI355X_Q4_0 && g_tune_gemm != 1 && mimir::qgemm_q4_0_ok(W, X, M, N, K, x_row_stride)) {
+        if (g_tune_gemm_f16 == 0 && mimir::qgemm_q4_0_blocks_pays(M, N, K)) {
+            // the exact form of a large product: W's integers once as a bfloat16 panel, then one MFMA a weight
+            if (mi355x_status s2 = gemm_scratch(stream, mimir::qgemm_q4_0_blocks_ws_bytes(N, K), &ws)) return s2;
+            HIP_TRY(mimir::qgemm_q4_0_blocks(W, X, x_row_stride, Y, M, N, K, f32, ws, st), "launch qgemm_q4_0_blocks");
+            return MI355X_OK;
+        }
         void* half_ws = nullptr;
         const bool panel = g_tune_gemm_f16 == 1;  // 2: the binary16 form without the panel route
         if (g_tune_gemm_f16 == 1 || g_tune_gemm_f16 == 2)
@@ -778,6 +784,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "qgemm.path") == 0) {
         g_tune_gemm = value;
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "qgemm.blocks") == 0) {  // 0: the exact form always on the tile kernel; 2: always from the panel of integers; 1: by shape
+        mimir::set_q4_0_blocks(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "qgemm.f16") == 0) {

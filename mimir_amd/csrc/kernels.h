@@ -300,6 +300,14 @@ bool qgemm_q4_0_ok(const void* W, const void* X, int64_t M, int64_t N, int64_t K
 size_t qgemm_q4_0_half_ws_bytes(int64_t M, int64_t N, int64_t K, bool panel);
 hipError_t qgemm_q4_0_bf16(const void* W, const void* X, void* Y, int64_t M, int64_t N, int64_t K, int64_t x_row_stride, bool out_f32,
                            void* half_ws, bool panel, hipStream_t st);
+// The exact form from a panel of the weights' integers (qgemm_q4_0_blocks.hip): block sums on the bfloat16 matrix
+// cores, one FMA per output and block with the block's scale; X as for qgemm_q4_0_bf16, ws qgemm_q4_0_blocks_ws_bytes(N, K)
+// bytes of device memory, 16-byte aligned.
+size_t qgemm_q4_0_blocks_ws_bytes(int64_t N, int64_t K);
+bool qgemm_q4_0_blocks_pays(int64_t M, int64_t N, int64_t K);  // against the tile kernel, its pass over W included
+hipError_t qgemm_q4_0_blocks(const void* W, const void* X, int64_t x_row_stride, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32, void* ws,
+                             hipStream_t st);
+void set_q4_0_blocks(int v);  // measurement aid: 0 keeps every product on the tile kernel, 2 takes this route whatever the shape
 // The panel route (qgemm_f16_panel.hip): X [M, K] bfloat16 goes to X16 [M, K] binary16 with row_scale[m] to multiply row
 // m's results by (both written here), W Q4_0 to `panel` (qgemm_f16_panel_bytes(N, K) bytes of device memory, 256-byte aligned).
 size_t qgemm_f16_panel_bytes(int64_t N, int64_t K);

@@ -147,8 +147,9 @@ def test_special_values():
 def test_prefill_shapes(n):
     """M = 512 tokens at the 8B model's shapes, weights and activations as the
     configurations draw them. The oracle takes a band of output columns (rows of
-    W) at N = 14336 to stay within seconds; M = 2048 is checked against the M =
-    512 result row for row, rows being independent."""
+    W) at N = 14336 to stay within seconds; M = 2048 (which takes the exact form's
+    other kernel) is checked against the oracle too, and row for row against
+    itself, rows being independent."""
     rng = np.random.default_rng(0)
     m, k = 512, 4096
     w = bench_blocks(rng, O.Q4_0, n * k)
@@ -167,7 +168,11 @@ def test_prefill_shapes(n):
         gpu.say("qgemm_bf16 2048x4096 by 4096x4096")
         x4 = np.concatenate([x, x[::-1], x, x[::-1]], axis=0)
         got4 = qgemm(w, x4, n, k)
-        assert np.array_equal(got4[:512], got) and np.array_equal(got4[512:1024], got[::-1]) and np.array_equal(got4[1024:1536], got)
+        # rows are independent: the same row of x gives the same bits wherever it stands among the 2048
+        assert np.array_equal(got4[512:1024], got4[:512][::-1]) and np.array_equal(got4[1024:1536], got4[:512]) and np.array_equal(got4[1536:], got4[512:1024])
+        # 2048 rows take the exact form's other kernel (the weights' integers from a panel): the same sums in another order
+        assert last_kernel().startswith("qgemm_q4_0_blocks_kernel")
+        check_bf16(got4[:512], O.q4_0_matmul_bf16(w, x, n, k), 1e-4 * np.maximum(1, np.abs(want_f32)))
 
 
 def test_prefill_shape_2048_by_14336():
@@ -399,3 +404,59 @@ def test_binary16_form_prefill_shapes(n):
     size = np.sqrt(np.mean(want ** 2))
     print(f"binary16 weights, N={n}: rms error {np.sqrt(np.mean(err ** 2)) / size:.2e}, worst {np.abs(err).max() / size:.2e} of the rms result")
     assert np.sqrt(np.mean(err ** 2)) <= 3e-4 * size and np.abs(err).max() <= 2e-3 * size
+
+
+@pytest.mark.parametrize("m,n,k,tiles", [(300, 515, 512, "3 x 3 tiles of 128 x 256"), (1000, 1030, 1280, "8 x 5 tiles of 128 x 256"),
+                                         (2047, 6200, 768, "8 x 25 tiles of 256 x 256"), (512, 14336, 256, "4 x 56 tiles of 128 x 256")])
+def test_exact_form_from_the_panel_of_integers(m, n, k, tiles):
+    """The exact form's second kernel (W's integers n - 8 once as a bfloat16 panel, block sums on the matrix cores, one
+    FMA per block with the block's scale), asked for whatever the shape: against the oracle within the bound of the
+    first, and against the first (the same exact products, other float32 sums); rows of x further apart than K, W at
+    another address, tiles that the edges do not fill; both output dtypes, the bfloat16 one the rounding of
+    the float32 one."""
+    rng = np.random.default_rng(m + n + k)
+    w = random_blocks(rng, O.Q4_0, n * k)
+    x = bf16_bits(rng.normal(size=(m, k)) * np.exp(rng.normal(size=(m, 1)) * 2))
+    l = gpu.lib()
+    try:
+        capi.check(l.mi355x_tune(b"qgemm.blocks", 2))
+        gpu.say(f"qgemm_bf16, exact form from the panel, M={m} N={n} K={k}")
+        got32 = qgemm(w, x, n, k, capi.F32, x_stride=k + 8)
+        assert last_kernel() == "qgemm_q4_0_blocks_kernel: " + tiles
+        got = qgemm(w, x, n, k, x_stride=k + 8)
+        moved = qgemm(w, x, n, k, capi.F32, w_offset=16)
+        capi.check(l.mi355x_tune(b"qgemm.blocks", 0))
+        tile32 = qgemm(w, x, n, k, capi.F32)
+        assert last_kernel().startswith("qgemm_q4_0_kernel")
+    finally:
+        capi.check(l.mi355x_tune(b"qgemm.blocks", 1))
+    bound = f32_bound(w, x, n, k)
+    assert np.array_equal(moved, got32)
+    assert np.array_equal(got, bf16_bits(got32))
+    check_f32(got32, tile32.astype(np.float64), 2 * bound, "against the tile kernel")
+    if m * n * k <= 1 << 30:
+        check_f32(got32, reference_f32(w, x, n, k), bound, "against the oracle")
+    else:
+        lo, hi = n - 300, n  # the last columns, across the edge tile
+        wb = w.reshape(n, -1)[lo:hi].reshape(-1)
+        check_f32(got32[:, lo:hi], reference_f32(wb, x, hi - lo, k), bound[:, lo:hi], "against the oracle")
+
+
+def test_exact_form_from_the_panel_rows_with_nan_and_inf():
+    m, n, k = 300, 260, 512
+    rng = np.random.default_rng(8)
+    w = random_blocks(rng, O.Q4_0, n * k)
+    xf = rng.normal(size=(m, k)).astype(np.float32)
+    clean = bf16_bits(xf)
+    xf[5, 7] = np.inf; xf[6, 9] = np.nan
+    l = gpu.lib()
+    try:
+        capi.check(l.mi355x_tune(b"qgemm.blocks", 2))
+        gpu.say("qgemm_bf16, exact form from the panel, nan and inf")
+        got32 = qgemm(w, bf16_bits(xf), n, k, capi.F32)
+        base = qgemm(w, clean, n, k, capi.F32)
+    finally:
+        capi.check(l.mi355x_tune(b"qgemm.blocks", 1))
+    assert not np.isfinite(got32[5]).any() and np.isnan(got32[6]).all()
+    keep = np.ones(m, bool); keep[[5, 6]] = False
+    assert np.array_equal(got32[keep], base[keep])
