@@ -30,6 +30,7 @@
 #include "device_util.h"
 #include "half_rows.h"
 #include "kernels.h"
+#include "tile_plan.h"
 
 namespace mimir {
 
@@ -40,7 +41,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kStep = 64;              // of K a step
 constexpr int kRowBytes = kStep * 2;   // a row of a stage in LDS
-constexpr int kUnits = 256;            // compute units; one workgroup each at a time (LDS)
 
 // A workgroup's tile of Y: WM x (8 / WM) wavefronts of (32 MT) x (32 NT) each.
 template <int WM, int MT, int NT>
@@ -242,14 +242,6 @@ __device__ __forceinline__ void tile_body(const uint16_t* __restrict__ X16, cons
         }
 }
 
-// How Y is cut into tiles. Columns [0, 256 wide_cols) in Wide tiles, then narrow_cols Narrow tiles; or, with `low`,
-// every tile Low. Workgroups take the Wide tiles first (the dispatcher hands them out in the order of their index).
-struct PanelPlan {
-    int tiles_m;      // tiles along M (256 rows, or 128 with low)
-    int wide_cols, narrow_cols;
-    int low;
-};
-
 // A die's workgroups (every eighth, round-robin) take a contiguous range of the tiles, the tile's row of X varying
 // fastest: the 32 that run together share 4 column panels of P and the 8 row panels of X through the die's L2.
 __device__ __forceinline__ int tile_of(int b, int ntiles) {
@@ -285,66 +277,9 @@ __global__ __launch_bounds__(512, 2) void hgemm_f16_nt_kernel(const uint16_t* __
                                lds_gemm);
 }
 
-// When the last of n_first jobs of cost c_first, then n_then jobs of cost c_then, ends on kUnits units that each
-// take the next job as soon as they are free.
-double makespan(int n_first, double c_first, int n_then, double c_then) {
-    struct Level { double at; int units; };
-    Level lv[64];
-    int n = 0;
-    const int q = n_first / kUnits, r = n_first % kUnits;
-    if (kUnits - r > 0) lv[n++] = {q * c_first, kUnits - r};
-    if (r > 0) lv[n++] = {(q + 1) * c_first, r};
-    while (n_then > 0) {
-        const int k = lv[0].units < n_then ? lv[0].units : n_then;  // lv is kept in ascending order
-        n_then -= k;
-        const double to = lv[0].at + c_then;
-        lv[0].units -= k;
-        if (lv[0].units == 0) {
-            for (int i = 1; i < n; i++) lv[i - 1] = lv[i];
-            n--;
-        }
-        int at = 0;
-        while (at < n && lv[at].at < to) at++;
-        if (at < n && lv[at].at == to) {
-            lv[at].units += k;
-        } else if (n < 64) {
-            for (int i = n; i > at; i--) lv[i] = lv[i - 1];
-            lv[at] = {to, k};
-            n++;
-        } else {
-            lv[n - 1].units += k;  // more levels than this holds: counted at the latest
-        }
-    }
-    return n > 0 ? lv[n - 1].at : 0.0;
-}
-
 // Costs in Wide tiles' time: a Narrow tile has three quarters of the MFMAs and reads a little more from LDS for each,
 // a Low tile half of them and a third more.
 constexpr double kNarrowCost = 0.78, kLowCost = 0.56;
-
-// The cut with the earliest end, and that end (in Wide tiles' time).
-double plan_panel(int64_t M, int64_t N, PanelPlan* out) {
-    const int tm = (int)((M + 255) / 256);
-    PanelPlan best{tm, (int)((N + 255) / 256), 0, 0};
-    double best_end = makespan(best.tiles_m * best.wide_cols, 1.0, 0, 0.0);
-    for (int cn = 1; (int64_t)192 * (cn - 1) < N; cn++) {
-        const int64_t left = N - (int64_t)192 * cn;
-        const int cw = left > 0 ? (int)((left + 255) / 256) : 0;
-        const double end = makespan(tm * cw, 1.0, tm * cn, kNarrowCost);
-        if (end < best_end - 1e-9) {
-            best_end = end;
-            best = PanelPlan{tm, cw, cn, 0};
-        }
-    }
-    const int tl = (int)((M + 127) / 128), cl = (int)((N + 255) / 256);
-    const double low_end = makespan(tl * cl, kLowCost, 0, 0.0);
-    if (low_end < best_end - 1e-9) {
-        best_end = low_end;
-        best = PanelPlan{tl, cl, 0, 1};
-    }
-    *out = best;
-    return best_end;
-}
 
 }  // namespace
 
@@ -356,7 +291,7 @@ size_t qgemm_f16_panel_bytes(int64_t N, int64_t K) { return ((size_t)N * K * 2 +
 bool qgemm_f16_panel_pays(int64_t M, int64_t N, int64_t K) {
     if (!(M >= 1024 && K % kStep == 0 && K >= kStep && M < (1 << 24) && N < (1 << 24) && K < (1 << 24) && N > 0)) return false;
     PanelPlan plan;
-    const double end = plan_panel(M, N, &plan);
+    const double end = plan_panel(M, N, kNarrowCost, kLowCost, &plan);
     const double work = (double)M * (double)N / (256.0 * 256.0);
     return work >= 0.70 * kUnits * end;
 }
@@ -377,7 +312,7 @@ hipError_t qgemm_f16_panel(const void* W, const void* X, int64_t x_row_stride, v
     hipLaunchKernelGGL(panel_prepare_kernel, dim3((unsigned)(M + (want > 8192 ? 8192 : want))), dim3(256), 0, st, (const uint16_t*)X, (uint16_t*)X16, row_scale,
                        (int)M, K, x_row_stride, (const uint8_t*)W, (uint16_t*)panel, halves);
     PanelPlan plan;
-    plan_panel(M, N, &plan);
+    plan_panel(M, N, kNarrowCost, kLowCost, &plan);
     const int first = plan.tiles_m * plan.wide_cols, then = plan.tiles_m * plan.narrow_cols;
     note_kernel("hgemm_f16_nt_kernel: %d x %d tiles of %s, %d x %d tiles of 256 x 192", plan.tiles_m, plan.wide_cols, plan.low ? "128 x 256" : "256 x 256",
                 plan.tiles_m, plan.narrow_cols);

@@ -10,8 +10,9 @@
 // the results differ in the last bits like two orders of addition do (the tests' bound is the same for both).
 //
 // Two launches. blocks_panel_kernel writes W's integers once as a bfloat16 panel P [N, K]. qgemm_q4_0_blocks_kernel
-// multiplies X, read where the caller has it, by P: a workgroup of eight wavefronts owns 32 MT x 2 rows of X by 256 rows
-// of W (MT = 4: 256 x 256, a wavefront 128 x 64; MT = 2: 128 x 256 for products with few tiles), a stage is a pair of
+// multiplies X, read where the caller has it, by P: a workgroup of eight wavefronts owns a tile of Y of 256 x 256 (a
+// wavefront 128 x 64), 256 x 192 (64 x 96) or 128 x 256 (64 x 64), cut as tile_plan.h says so that the last round of
+// tiles leaves few compute units idle; a stage is a pair of
 // blocks (64 of K); both operands go from global memory straight into LDS (global_load_lds_dwordx4), rows of 128 bytes
 // with their 16-byte pieces at piece ^ (row / 2 mod 8), so that the 32 rows of a fragment read fall on all banks; the
 // scales pass through registers, read from the blocks themselves. The two MFMAs of a 32 x 32 sub-tile and block are
@@ -20,6 +21,7 @@
 // Reference semantics: Tensor.MatMulT for a half-precision x and block-quantized w, tensor/quant.go:45-48.
 #include "device_util.h"
 #include "kernels.h"
+#include "tile_plan.h"
 
 namespace mimir {
 
@@ -28,18 +30,24 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kBN = 256;        // rows of W a workgroup
 constexpr int kRowBytes = 128;  // a row of a stage: 64 bfloat16
+constexpr int kScaleRows = 256; // rows of W whose scales a stage holds (every thread stores one: 512 = 2 blocks x 256)
 
-template <int MT>
+// A workgroup's tile of Y: WM x (8 / WM) wavefronts of (32 MT) x (32 NT) each.
+template <int WM, int MT_, int NT_>
 struct Shape {
-    static constexpr int BM = 64 * MT;                   // rows of X a workgroup: two wavefronts of 32 MT
-    static constexpr int kLoads = (BM + kBN) / 64;       // 1 KB loads (8 rows) a wavefront issues per stage
+    static constexpr int WN = 8 / WM, MT = MT_, NT = NT_;
+    static constexpr int BM = WM * 32 * MT, BN = WN * 32 * NT;
+    static constexpr int kLoads = (BM + BN) / 64;        // 1 KB loads (8 rows) a wavefront issues per stage
     static constexpr int b = BM * kRowBytes;             // the stage in LDS: X's rows, P's rows,
-    static constexpr int sw = b + kBN * kRowBytes;       // float [2][kBN]: W's scales of the stage's two blocks
-    static constexpr int bytes = sw + 2 * kBN * 4;
-    static_assert(bytes % 1024 == 0 && (BM + kBN) % 64 == 0, "whole loads, stages on the boundary they assume");
+    static constexpr int sw = b + BN * kRowBytes;        // float [2][kScaleRows]: W's scales of the stage's two blocks
+    static constexpr int bytes = sw + 2 * kScaleRows * 4;
+    static_assert(bytes % 1024 == 0 && (BM + BN) % 64 == 0 && BM % 8 == 0 && BN <= kScaleRows, "whole loads, none across the operands");
 };
+using Wide = Shape<2, 4, 2>;    // 256 x 256
+using Narrow = Shape<4, 2, 3>;  // 256 x 192: to fill a last round that wide tiles would leave partly empty
+using Low = Shape<2, 2, 2>;     // 128 x 256: for products with too few wide tiles for the device
+constexpr size_t kLdsBytes = 2 * (size_t)Wide::bytes;
 
 // Sixteen weights a thread: the low and the high nibbles of eight bytes of a block, as the bfloat16 integers n - 8.
 __global__ __launch_bounds__(256) void blocks_panel_kernel(const uint8_t* __restrict__ W, uint16_t* __restrict__ P, int64_t halves) {
@@ -82,18 +90,14 @@ __device__ __forceinline__ int tile_of(int b, int ntiles) {
     return (b & 7) * per_die + (b >> 3);
 }
 
-template <int MT, bool OUT_F32>
-__global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ P,
-                                                                const uint16_t* __restrict__ X, int64_t x_row_stride, void* __restrict__ Yv,
-                                                                int M, int N, int K, int tiles_m, int ntiles) {
-    typedef Shape<MT> S;
-    extern __shared__ __align__(1024) char lds[];
-    const int t = tile_of((int)blockIdx.x, ntiles);
-    if (t >= ntiles) return;  // the whole workgroup
-    const int m0 = (t % tiles_m) * S::BM, n0 = (t / tiles_m) * kBN;
+// One tile: Y [m0 .. m0 + BM) x [n0 .. n0 + BN).
+template <class S, bool OUT_F32>
+__device__ __forceinline__ void tile_body(const uint8_t* __restrict__ W, const uint16_t* __restrict__ P, const uint16_t* __restrict__ X,
+                                          int64_t x_row_stride, void* __restrict__ Yv, int M, int N, int K, int m0, int n0, char* lds) {
+    constexpr int MT = S::MT, NT = S::NT;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;
+    const int wm = wave / S::WN, wn = wave % S::WN;
     const int nb = K >> 5;
 
     // This wavefront's loads: load g = kLoads wave + j brings rows [8 g, 8 g + 8) of the stage, X's below BM and P's
@@ -126,13 +130,13 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
     int piece_off[4];  // of a row's pieces 2 p + hi: half p % 2 of the stage's block p / 2
 #pragma unroll
     for (int p = 0; p < 4; p++) piece_off[p] = ((2 * p + hi) ^ swz) * 16;
-    const int a_row = (wm * 32 * MT + r32) * kRowBytes, b_row = S::b + (wn * 64 + r32) * kRowBytes;
+    const int a_row = (wm * 32 * MT + r32) * kRowBytes, b_row = S::b + (wn * 32 * NT + r32) * kRowBytes;
 
-    f32x16 acc[MT][2];
+    f32x16 acc[MT][NT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
+        for (int nt = 0; nt < NT; nt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mt][nt][i] = 0.f;
 
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
         const float dw = f16_bits_to_f32(load_u16(wscale));
 #pragma unroll
         for (int j = 0; j < S::kLoads; j++) load_to_lds(from[j], __builtin_amdgcn_readfirstlane(lds0 + into[j]));
-        ((float*)(lds + S::sw))[sodd * kBN + srow] = dw;
+        ((float*)(lds + S::sw))[sodd * kScaleRows + srow] = dw;
     }
     // No branches around the loads and stores: past the end the last stage is requested and stored again, into the
     // buffer that is not being read.
@@ -162,23 +166,23 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
                 from[j] += kRowBytes * step;
                 load_to_lds(from[j], __builtin_amdgcn_readfirstlane(next + into[j]));
             }
-            bf16x8 a[MT][2], b[2][2];  // [sub-tile][half of the block]
+            bf16x8 a[MT][2], b[NT][2];  // [sub-tile][half of the block]
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                 for (int h = 0; h < 2; h++) a[mt][h] = *(const bf16x8*)(st + a_row + mt * 32 * kRowBytes + piece_off[2 * odd + h]);
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
+            for (int nt = 0; nt < NT; nt++)
 #pragma unroll
                 for (int h = 0; h < 2; h++) b[nt][h] = *(const bf16x8*)(st + b_row + nt * 32 * kRowBytes + piece_off[2 * odd + h]);
-            float dw[2];
+            float dw[NT];
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++) dw[nt] = ((const float*)(st + S::sw))[odd * kBN + wn * 64 + nt * 32 + r32];
-            // Sub-tile s = 2 mt + nt: its two MFMAs are issued with the FMAs of the sub-tile before it, so that the
+            for (int nt = 0; nt < NT; nt++) dw[nt] = ((const float*)(st + S::sw))[odd * kScaleRows + wn * 32 * NT + nt * 32 + r32];
+            // Sub-tile s = NT mt + nt: its two MFMAs are issued with the FMAs of the sub-tile before it, so that the
             // vector unit works while the matrix cores do.
             f32x16 c[2];
             auto multiply = [&](int sub) {
-                const int mt = sub >> 1, nt = sub & 1;
+                const int mt = sub / NT, nt = sub % NT;
                 f32x16 zero;
 #pragma unroll
                 for (int e = 0; e < 16; e++) zero[e] = 0.f;
@@ -186,23 +190,23 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
                 c[sub & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mt][1], b[nt][1], c[sub & 1], 0, 0, 0);
             };
             auto finish = [&](int sub) {
-                const int mt = sub >> 1, nt = sub & 1;
+                const int mt = sub / NT, nt = sub % NT;
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[mt][nt][e] = fmaf(dw[nt], c[sub & 1][e], acc[mt][nt][e]);
             };
             multiply(0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int sub = 1; sub < 2 * MT; sub++) {
+            for (int sub = 1; sub < MT * NT; sub++) {
                 multiply(sub);
                 finish(sub - 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            finish(2 * MT - 1);
+            finish(MT * NT - 1);
         }
         // the next stage's scales, at the end: by now their load has landed with everything requested before it
         __builtin_amdgcn_sched_barrier(0);
-        ((float*)(next_p + S::sw))[sodd * kBN + srow] = next_dw;
+        ((float*)(next_p + S::sw))[sodd * kScaleRows + srow] = next_dw;
     }
 
     // One rounding to the output's dtype (f32ToBF16, backend/cpu/half.go:42-51). An MFMA leaves a lane one column of Y
@@ -215,10 +219,10 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
         for (int q = 0; q < 4; q++) {
             const int m = m0 + wm * 32 * MT + mt * 32 + q * 8 + hi * 4 + (lane & 3);
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++) {
+            for (int nt = 0; nt < NT; nt++) {
                 float v[4] = {acc[mt][nt][4 * q], acc[mt][nt][4 * q + 1], acc[mt][nt][4 * q + 2], acc[mt][nt][4 * q + 3]};
                 quad_transpose(v, lane);
-                const int n = n0 + wn * 64 + nt * 32 + (r32 & ~3);
+                const int n = n0 + wn * 32 * NT + nt * 32 + (r32 & ~3);
                 if (m >= M || n >= N) continue;
                 if (wide_ok && n + 3 < N) {
                     if (OUT_F32) {
@@ -241,36 +245,39 @@ __global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* _
         }
 }
 
-std::atomic<int> g_blocks{1};  // measurement aid: 0 keeps every product on the tile kernel, 2 takes this one whatever the shape
-
-template <int MT>
-hipError_t launch(const void* W, const uint16_t* P, const void* X, int64_t x_row_stride, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32,
-                  hipStream_t st) {
-    typedef Shape<MT> S;
-    const size_t lds = 2 * (size_t)S::bytes;
-    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attributes
-    if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)qgemm_q4_0_blocks_kernel<MT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void*)qgemm_q4_0_blocks_kernel<MT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        raised = true;
+template <bool OUT_F32>
+__global__ __launch_bounds__(512) void qgemm_q4_0_blocks_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ P,
+                                                                const uint16_t* __restrict__ X, int64_t x_row_stride, void* __restrict__ Yv,
+                                                                int M, int N, int K, PanelPlan plan) {
+    extern __shared__ __align__(1024) char lds[];
+    int b = (int)blockIdx.x;
+    if (plan.low) {
+        const int ntiles = plan.tiles_m * plan.wide_cols;
+        const int t = tile_of(b, ntiles);
+        if (t >= ntiles) return;  // the whole workgroup
+        tile_body<Low, OUT_F32>(W, P, X, x_row_stride, Yv, M, N, K, (t % plan.tiles_m) * Low::BM, (t / plan.tiles_m) * Low::BN, lds);
+        return;
     }
-    const int64_t tiles_m = (M + S::BM - 1) / S::BM, ntiles = tiles_m * ((N + kBN - 1) / kBN);
-    if (ntiles >= ((int64_t)1 << 28)) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)(((ntiles + 7) / 8) * 8));
-    if (out_f32)
-        hipLaunchKernelGGL((qgemm_q4_0_blocks_kernel<MT, true>), grid, dim3(512), lds, st, (const uint8_t*)W, P, (const uint16_t*)X, x_row_stride, Y,
-                           (int)M, (int)N, (int)K, (int)tiles_m, (int)ntiles);
-    else
-        hipLaunchKernelGGL((qgemm_q4_0_blocks_kernel<MT, false>), grid, dim3(512), lds, st, (const uint8_t*)W, P, (const uint16_t*)X, x_row_stride, Y,
-                           (int)M, (int)N, (int)K, (int)tiles_m, (int)ntiles);
-    note_kernel("qgemm_q4_0_blocks_kernel: %lld x %lld tiles of %d x 256", (long long)tiles_m, (long long)(ntiles / tiles_m), S::BM);
-    return hipGetLastError();
+    const int nwide = plan.tiles_m * plan.wide_cols;
+    const int wide_wgs = ((nwide + 7) >> 3) << 3;
+    if (b < wide_wgs) {
+        const int t = tile_of(b, nwide);
+        if (t >= nwide) return;
+        tile_body<Wide, OUT_F32>(W, P, X, x_row_stride, Yv, M, N, K, (t % plan.tiles_m) * Wide::BM, (t / plan.tiles_m) * Wide::BN, lds);
+        return;
+    }
+    b -= wide_wgs;
+    const int nnarrow = plan.tiles_m * plan.narrow_cols;
+    const int t = tile_of(b, nnarrow);
+    if (t >= nnarrow) return;
+    tile_body<Narrow, OUT_F32>(W, P, X, x_row_stride, Yv, M, N, K, (t % plan.tiles_m) * Narrow::BM,
+                               plan.wide_cols * Wide::BN + (t / plan.tiles_m) * Narrow::BN, lds);
 }
 
-// Tiles of 256 rows where they fill the device, of 128 where those would leave compute units idle.
-bool tall(int64_t M, int64_t N) { return ((M + 255) / 256) * ((N + kBN - 1) / kBN) >= 192; }
+// Costs in wide tiles' time, measured: a tile of 256 x 192 has three quarters of the work, one of 128 x 256 half.
+constexpr double kNarrowCost = 0.78, kLowCost = 0.56;
+
+std::atomic<int> g_blocks{1};  // measurement aid: 0 keeps every product on the tile kernel, 2 takes this one whatever the shape
 
 }  // namespace
 
@@ -285,7 +292,7 @@ size_t qgemm_q4_0_blocks_ws_bytes(int64_t N, int64_t K) { return (size_t)N * (si
 bool qgemm_q4_0_blocks_pays(int64_t M, int64_t N, int64_t K) {
     if (g_blocks == 0 || M <= 0 || N <= 0 || K <= 0 || K % 64 != 0) return false;
     if (g_blocks == 2) return true;
-    return M >= 256 && ((M + 127) / 128) * ((N + kBN - 1) / kBN) >= 192;
+    return M >= 256 && ((M + 127) / 128) * ((N + 255) / 256) >= 192;
 }
 
 // X [M, K] bfloat16 (16-byte aligned, rows x_row_stride elements apart, a multiple of 8), W [N, K] Q4_0, Y [M, N] bfloat16
@@ -293,13 +300,32 @@ bool qgemm_q4_0_blocks_pays(int64_t M, int64_t N, int64_t K) {
 hipError_t qgemm_q4_0_blocks(const void* W, const void* X, int64_t x_row_stride, void* Y, int64_t M, int64_t N, int64_t K, bool out_f32, void* ws,
                              hipStream_t st) {
     if (!ws || ((uintptr_t)ws & 15) != 0 || ((uintptr_t)X & 15) != 0 || x_row_stride % 8 != 0 || x_row_stride < K || ((uintptr_t)W & 1) != 0 ||
-        M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || M >= (1 << 30) || N >= (1 << 30) || K > (1 << 24))
+        M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || M >= (1 << 24) || N >= (1 << 24) || K > (1 << 24))
         return hipErrorInvalidValue;
+    static std::atomic<bool> raised{false};  // threads may race here: both then set the same attributes
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)qgemm_q4_0_blocks_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)qgemm_q4_0_blocks_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
     uint16_t* P = (uint16_t*)ws;
     const int64_t halves = N * (K / 32) * 2;
     const int64_t want = (halves + 255) / 256;
     hipLaunchKernelGGL(blocks_panel_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, st, (const uint8_t*)W, P, halves);
-    return tall(M, N) ? launch<4>(W, P, X, x_row_stride, Y, M, N, K, out_f32, st) : launch<2>(W, P, X, x_row_stride, Y, M, N, K, out_f32, st);
+    PanelPlan plan;
+    plan_panel(M, N, kNarrowCost, kLowCost, &plan);
+    const int first = plan.tiles_m * plan.wide_cols, then = plan.tiles_m * plan.narrow_cols;
+    const dim3 grid((unsigned)(((first + 7) / 8) * 8 + ((then + 7) / 8) * 8));
+    if (out_f32)
+        hipLaunchKernelGGL(qgemm_q4_0_blocks_kernel<true>, grid, dim3(512), kLdsBytes, st, (const uint8_t*)W, P, (const uint16_t*)X, x_row_stride, Y, (int)M,
+                           (int)N, (int)K, plan);
+    else
+        hipLaunchKernelGGL(qgemm_q4_0_blocks_kernel<false>, grid, dim3(512), kLdsBytes, st, (const uint8_t*)W, P, (const uint16_t*)X, x_row_stride, Y, (int)M,
+                           (int)N, (int)K, plan);
+    note_kernel("qgemm_q4_0_blocks_kernel: %d x %d tiles of %s, %d x %d tiles of 256 x 192", plan.tiles_m, plan.wide_cols, plan.low ? "128 x 256" : "256 x 256",
+                plan.tiles_m, plan.narrow_cols);
+    return hipGetLastError();
 }
 
 }  // namespace mimir

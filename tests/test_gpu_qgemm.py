@@ -187,6 +187,8 @@ def test_prefill_shape_2048_by_14336():
     gpu.say("qgemm_bf16 2048x4096 by 14336x4096")
     got = qgemm(w, x, n, k)
     got32 = qgemm(w, x, n, k, capi.F32)
+    # the exact form's cut of this shape: a wide and a narrow tile a compute unit
+    assert last_kernel() == "qgemm_q4_0_blocks_kernel: 8 x 32 tiles of 256 x 256, 8 x 32 tiles of 256 x 192"
     with binary16_weights():
         gpu.say("qgemm_bf16 2048x4096 by 14336x4096, binary16 weights")
         half32 = qgemm(w, x, n, k, capi.F32)
@@ -406,8 +408,12 @@ def test_binary16_form_prefill_shapes(n):
     assert np.sqrt(np.mean(err ** 2)) <= 3e-4 * size and np.abs(err).max() <= 2e-3 * size
 
 
-@pytest.mark.parametrize("m,n,k,tiles", [(300, 515, 512, "3 x 3 tiles of 128 x 256"), (1000, 1030, 1280, "8 x 5 tiles of 128 x 256"),
-                                         (2047, 6200, 768, "8 x 25 tiles of 256 x 256"), (512, 14336, 256, "4 x 56 tiles of 128 x 256")])
+@pytest.mark.parametrize("m,n,k,tiles", [(300, 515, 512, "3 x 3 tiles of 128 x 256, 3 x 0 tiles of 256 x 192"),
+                                         (1000, 1030, 1280, "8 x 5 tiles of 128 x 256, 8 x 0 tiles of 256 x 192"),
+                                         (2047, 6200, 768, "8 x 25 tiles of 256 x 256, 8 x 0 tiles of 256 x 192"),
+                                         (2047, 9000, 256, "8 x 25 tiles of 256 x 256, 8 x 14 tiles of 256 x 192"),  # the last narrow tile ragged
+                                         (1024, 12288, 256, "4 x 0 tiles of 256 x 256, 4 x 64 tiles of 256 x 192"),
+                                         (512, 14336, 256, "4 x 56 tiles of 128 x 256, 4 x 0 tiles of 256 x 192")])
 def test_exact_form_from_the_panel_of_integers(m, n, k, tiles):
     """The exact form's second kernel (W's integers n - 8 once as a bfloat16 panel, block sums on the matrix cores, one
     FMA per block with the block's scale), asked for whatever the shape: against the oracle within the bound of the
