@@ -125,10 +125,12 @@ struct Model {
     }
 };
 
-int act_class(const Weight& w, int64_t rows = 1) {
+// panel_bytes: what the model holds as workspace for the fixed-point product's binary16 form (0: that form is not taken)
+int act_class(const Weight& w, int64_t rows = 1, size_t panel_bytes = 0) {
     switch (w.dtype) {
     case kQ4_0:
-        if (qgemm_q4_0_fx_pays(w.buf.p, rows, w.n, w.k)) return qgemm_q4_0_fx16_pays(rows, w.n, w.k) ? kActFxPairs : kActFx;
+        if (qgemm_q4_0_fx_pays(w.buf.p, rows, w.n, w.k))
+            return panel_bytes >= qgemm_q4_0_fx16_ws_bytes(w.n, w.k) && qgemm_q4_0_fx16_pays(rows, w.n, w.k) ? kActFxPairs : kActFx;
         return q4_0_fixed_point_ok(w.buf.p, w.k) ? kActQ4 : kActNone;
     case kQ8_0: return q8_act_fits(w.k) ? kActQ8 : kActNone;
     case kQ4_K: case kQ6_K: return kActKQ;
@@ -153,7 +155,7 @@ const int kNoTune[5] = {0, 0, 0, 0, 0};
 mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std::initializer_list<const Weight*> ws, bool done[kActClasses]) {
     for (int i = 0; i < kActClasses; i++) done[i] = false;
     for (const Weight* w : ws) {
-        int cls = act_class(*w, rows);
+        int cls = act_class(*w, rows, m.fx_panel.bytes);
         if (cls == kActNone || done[cls]) continue;
         size_t need = act_row_bytes(cls, K) * (size_t)rows;
         if (m.act[cls].bytes < need) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: activation scratch of %zu bytes, need %zu", m.act[cls].bytes, need);
@@ -170,15 +172,13 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
 // y[rows, n] = x[rows, k] . W^T (nn/layers.go:49-55 -> tensor/quant.go:35-56).
 // With resid, y = product + resid (which may be y); only the row kernels of the quantized dtypes add it.
 mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows, const float* resid = nullptr) {
-    int cls = act_class(w, rows);
+    int cls = act_class(w, rows, m.fx_panel.bytes);
     if (resid && (cls == kActFx || cls == kActFxPairs || cls == kActNone)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
     QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
     a.resid = resid;
     hipError_t e;
     switch (w.dtype) {
     case kQ4_0:
-        if (cls == kActFxPairs && m.fx_panel.bytes < qgemm_q4_0_fx16_ws_bytes(w.n, w.k))
-            return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: fixed-point product workspace of %zu bytes, need %zu", m.fx_panel.bytes, qgemm_q4_0_fx16_ws_bytes(w.n, w.k));
         e = cls == kActFx || cls == kActFxPairs
                 ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, cls == kActFxPairs ? m.fx_panel.p : nullptr, m.stream)
             : cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream)
@@ -734,12 +734,14 @@ mi355x_status mi355x_llama_finalize(void* model, int64_t max_tokens) {
     }
     LLM_HIP(m->act2.alloc(q4_0_act_bytes((c.hidden + 63) / 64 * 64) * c.batch + 64), "hipMalloc(activations)");
     {
-        size_t panel = 0;  // the workspace of the fixed-point product's binary16 form, for whichever calls take it
+        // the workspace of the fixed-point product's binary16 form, which calls of some hundreds of rows take: the largest matrix's
+        size_t panel = 0;
         for (const Block& b : m->blocks)
             for (const Weight* w : {&b.q, &b.k, &b.v, &b.o, &b.gate, &b.up, &b.down, &b.qkv, &b.gate_up})
                 if (w->set() && w->dtype == kQ4_0 && qgemm_q4_0_fx16_ws_bytes(w->n, w->k) > panel) panel = qgemm_q4_0_fx16_ws_bytes(w->n, w->k);
         m->fx_panel.release();
-        if (panel) LLM_HIP(m->fx_panel.alloc(panel), "hipMalloc(fixed-point product workspace)");
+        m->fx_panel.bytes = 0;
+        if (panel && rows >= 256) LLM_HIP(m->fx_panel.alloc(panel), "hipMalloc(fixed-point product workspace)");
     }
     int chunk, nsplit;
     attention_plan(c.batch, c.heads, c.kv_heads, max_tokens, c.context, &chunk, &nsplit);
