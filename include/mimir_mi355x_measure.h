@@ -29,8 +29,10 @@ MI355X_API mi355x_status mi355x_gemv_stamps(void* stamps);
 MI355X_API mi355x_status mi355x_stream_read(const void* p, size_t bytes, float* scratch, int grid, int threads, void* stream);
 
 /* The kernel, with its template arguments, that the calling thread's latest Q4_0 product launched: of one row of x,
- * or the prompt-sized one of mi355x_qgemm_bf16 (for its panel route, the cut of Y into tiles). Which of the library's
- * launch shapes the dispatch chose, as a NUL-terminated string of at most n bytes. */
+ * or the prompt-sized one of mi355x_qgemm_bf16 (for its panel route, the cut of Y into tiles); or, if it came later,
+ * the kernel of its latest mi355x_attention call with keys (attn_prompt_kernel, attn_partial_kernel,
+ * attn_decode_kernel). Which of the library's launch shapes the dispatch chose, as a NUL-terminated string of at most
+ * n bytes. */
 MI355X_API mi355x_status mi355x_last_kernel(char* buf, size_t n);
 
 #ifdef __cplusplus

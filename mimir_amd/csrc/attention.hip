@@ -246,6 +246,8 @@ void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, 
 }
 
 hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st) {
+    if (attention_prompt_ok(a)) return attention_prompt(a, st);  // a prompt: tiles of rows on the matrix cores
+    note_kernel("attn_partial_kernel");
     AttnParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1]; p.q_i = a.q_strides[2];
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];

@@ -583,6 +583,7 @@ void set_attention_decode_handover(int v) { g_handover = v; }
 
 hipError_t attention_decode(const AttnArgs& a, int64_t kmax, void* workspace, void* act, int64_t act_row_bytes, hipStream_t st, int act_form,
                             void* flagged, size_t flagged_bytes, uint32_t* err) {
+    note_kernel("attn_decode_kernel");
     DecParams p;
     p.q_b = a.q_strides[0]; p.q_h = a.q_strides[1];
     p.k_b = a.k_strides[0]; p.k_h = a.k_strides[1]; p.k_p = a.k_strides[2];

@@ -710,6 +710,10 @@ mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const v
         HIP_TRY(mimir::attention_decode(a, K, ws, nullptr, 0, (hipStream_t)stream, mimir::kAttnActQ4, flags, flag_bytes, mimir::device_error_word()), "launch attention_decode");
         return MI355X_OK;
     }
+    if (mimir::attention_prompt_ok(a)) {  // many query positions: tiles of rows on the matrix cores, no scratch
+        HIP_TRY(mimir::attention_prompt(a, (hipStream_t)stream), "launch attention_prompt");
+        return MI355X_OK;
+    }
     mimir::attention_plan(B, H, HK, Q, K, &a.chunk, &a.nsplit);
     // the scratch begins with the decode kernel's tickets
     if (mi355x_status st = attn_scratch(stream, mimir::kAttnTicketBytes + mimir::attention_workspace_bytes(B, H, Q, DV, a.nsplit), &ws)) return st;
@@ -862,6 +866,10 @@ mi355x_status mi355x_tune(const char* key, int value) {
     }
     if (key && strcmp(key, "attention.fence") == 0) {
         mimir::set_attention_decode_fence(value);
+        return MI355X_OK;
+    }
+    if (key && strcmp(key, "attention.prompt") == 0) {  // 0: calls of many query positions on the kernel that takes a row a workgroup too
+        mimir::set_attention_prompt(value);
         return MI355X_OK;
     }
     if (key && strcmp(key, "attention.path") == 0) {

@@ -215,6 +215,11 @@ struct AttnArgs {
 void attention_plan(int64_t B, int H, int HK, int64_t Q, int64_t K, int* chunk, int* nsplit);
 size_t attention_workspace_bytes(int64_t B, int H, int64_t Q, int D, int nsplit);
 hipError_t attention(const AttnArgs& a, void* workspace, hipStream_t st);
+// Many query positions at once on the float32 matrix cores (attention_prompt.hip), which attention() takes for the calls
+// attention_prompt_ok names: the same results up to the order of the float32 sums.
+bool attention_prompt_ok(const AttnArgs& a);
+hipError_t attention_prompt(const AttnArgs& a, hipStream_t st);
+void set_attention_prompt(int v);  // measurement aid: 0 keeps every call on the kernel that takes a query row a workgroup
 // K == 0: zeros and a logsumexp of -Inf for every row; reads neither keys nor values.
 hipError_t attention_empty(const AttnArgs& a, hipStream_t st);
 
@@ -322,7 +327,7 @@ hipError_t f32_to_bf16(const float* x, void* y, int64_t n, hipStream_t st);
 // While a measurement is on (capi.hip), hands out the next pair of events for a
 // launch to be bracketed by; false otherwise.
 bool next_timing_events(hipEvent_t* start, hipEvent_t* stop);
-// Records which kernel the calling thread's latest Q4_0 product (of one row of x, or prompt-sized with bfloat16 x) launched (printf-style), for mi355x_last_kernel.
+// Records which kernel the calling thread's latest Q4_0 product (of one row of x, or prompt-sized with bfloat16 x) or attention call launched (printf-style), for mi355x_last_kernel.
 void note_kernel(const char* fmt, ...);
 hipError_t stream_read(const void* p, size_t bytes, float* out, int grid, int threads, hipStream_t st);
 int stream_read_out_len(int grid, int threads);

@@ -299,6 +299,69 @@ def test_prompt_attention_f32_cache_and_empty_rows():
     close(out, wo); close(lse[:, :, 2:], wl[:, :, 2:])
 
 
+def last_kernel():
+    buf = C.create_string_buffer(200)
+    capi.check(gpu.lib().mi355x_last_kernel(buf, 200))
+    return buf.value.decode()
+
+
+@pytest.mark.parametrize("B,H,HK,Q,K,D,kv_dt,causal,off", [
+    (1, 8, 2, 64, 64, 128, capi.F16, True, 0),      # the smallest call the kernel takes: half a workgroup's rows
+    (2, 8, 2, 300, 337, 128, capi.F16, True, 37),   # ragged rows and keys, a past of 37 positions
+    (1, 4, 4, 129, 129, 64, capi.F32, True, 0),     # one row into a second workgroup, 64 features, a float32 cache
+    (2, 6, 3, 200, 90, 64, capi.F16, False, 0),     # every row sees every key; groups of 2
+    (1, 4, 1, 256, 256, 128, capi.F32, True, -40),  # the first 40 rows see no key: zeros and -Inf
+    (1, 2, 1, 100, 400, 128, capi.F16, True, 500),  # the offset beyond the keys: every row sees all 400
+    (1, 32, 8, 512, 512, 128, capi.F16, True, 0),   # a 512-token prompt of the 8B shape
+])
+def test_prompt_attention_on_the_matrix_cores(B, H, HK, Q, K, D, kv_dt, causal, off):
+    """Calls of 64 and more query positions go to the kernel that walks tiles of keys with 32 rows a wavefront: against
+    the oracle to the float32 tolerance of the other attention tests, and against the kernel that takes a query row a
+    workgroup (the same call with the route switched off), which it follows up to the order of the sums."""
+    l = gpu.lib()
+    rng = np.random.default_rng(Q * 1000 + K)
+    q = rng.normal(size=(B, H, Q, D)).astype(np.float32)
+    k = rng.normal(size=(B, HK, K, D)).astype(np.float32); v = rng.normal(size=(B, HK, K, D)).astype(np.float32)
+    odt = O.F32
+    if kv_dt == capi.F16:
+        k, v, odt = O.f32_to_f16(k), O.f32_to_f16(v), O.F16
+    scale = 1 / np.sqrt(D)
+    gpu.say(f"prompt attention B={B} H={H} HK={HK} Q={Q} K={K} D={D} dt={kv_dt} causal={causal} offset={off}")
+    out, lse = attention(q, k, v, scale, causal=causal, offset=off, kv_dt=kv_dt)
+    assert last_kernel() == "attn_prompt_kernel"
+    wo, wl = O.attention(q, k, v, scale, causal=causal, causal_offset=off, kv_dt=odt)
+    close(out, wo); close(lse, wl)
+    try:
+        capi.check(l.mi355x_tune(b"attention.prompt", 0))
+        out2, lse2 = attention(q, k, v, scale, causal=causal, offset=off, kv_dt=kv_dt)
+        assert last_kernel() != "attn_prompt_kernel"
+    finally:
+        capi.check(l.mi355x_tune(b"attention.prompt", 1))
+    close(out, out2); close(lse, lse2)
+    if causal and off < 0:
+        assert not out[:, :, :-off].any() and np.all(lse[:, :, :-off] == -np.inf)
+
+
+def test_prompt_attention_leaves_other_calls_where_they_were():
+    """Fewer than 64 query positions, values of another width than the keys, a mask, and rows of keys that do not start
+    on 16 bytes stay on the other kernels."""
+    rng = np.random.default_rng(77)
+    def call(Q, D, DV, mask=False):
+        q = rng.normal(size=(1, 2, Q, D)).astype(np.float32)
+        k = rng.normal(size=(1, 2, 70, D)).astype(np.float32); v = rng.normal(size=(1, 2, 70, DV)).astype(np.float32)
+        m = rng.normal(size=(1, 2, Q, 70)).astype(np.float32) if mask else None
+        gpu.say(f"attention Q={Q} D={D} DV={DV} mask={mask}")
+        out, lse = attention(q, k, v, 0.2, mask=m)
+        wo, wl = O.attention(q, k, v, 0.2, mask=m)
+        close(out, wo); close(lse, wl)
+        return last_kernel()
+    assert call(64, 64, 64) == "attn_prompt_kernel"
+    assert call(63, 64, 64) != "attn_prompt_kernel"
+    assert call(64, 64, 128) != "attn_prompt_kernel"
+    assert call(64, 64, 64, mask=True) != "attn_prompt_kernel"
+    assert call(64, 32, 32) != "attn_prompt_kernel"
+
+
 def test_swiglu_add_argmax():
     l = gpu.lib()
     rng = np.random.default_rng(6)
