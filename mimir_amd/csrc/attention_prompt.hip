@@ -5,14 +5,17 @@
 // serves one query row a workgroup, re-reading every key and value for every row.
 //
 // Here a wavefront owns 32 query rows of one head and walks the keys in tiles of 32 with a running maximum and sum per
-// row (the rows' results are rescaled when the maximum grows), and both products of a tile are MFMAs on float32
-// operands, so that nothing is rounded that the other kernel does not round: scores = Q . K^T with
-// v_mfma_f32_32x32x2_f32 over the features (Q's rows live in registers for the whole walk, 64 a lane at 128 features),
-// then P . V with the same instruction over the tile's keys, P passing through LDS from the layout an MFMA leaves (a
-// lane holds a key's column for 16 rows) to the one it takes (a lane holds a row). A workgroup is four wavefronts with
-// consecutive rows of one head, which share the tile of keys and values in LDS (converted to float32 as they are
-// loaded; K's rows padded by a float so that 32 keys' equal feature falls on 32 banks). Rows' maxima and sums over a
-// tile are reductions over the 32 lanes that hold a row's columns.
+// row (a row's result is rescaled when its maximum grows), and both products of a tile are MFMAs on float32 operands
+// (v_mfma_f32_32x32x2_f32), so that nothing is rounded that the other kernel does not round. Both are computed
+// transposed, so that everything a row owns lives in one lane (and its partner 32 lanes on): scores^T = K . Q^T over the
+// features, the tile's keys as the first operand from LDS and the lane's own row of Q (scaled, in registers for the
+// whole walk, 64 a lane at 128 features) as the second, which leaves a lane 16 of its row's 32 scores in registers (the
+// partner holds the other 16): maximum and sum are chains over those registers and one exchange with the partner; then
+// result^T = V^T . P^T over the tile's keys, taken in the order the scores' registers hold them, so that p goes from the
+// exponential straight into the MFMA's second operand, and the lane ends with 16 features of every 32 of its row. A
+// workgroup is four wavefronts with consecutive rows of one head, which share the tile of keys and values in LDS
+// (converted to float32 as they are loaded, the next tile's rows requested while this one is used; K's rows padded by a
+// float so that 32 keys' equal feature falls on 32 banks).
 //
 // What differs from the other kernel is the order of the float32 sums (features and keys in pairs as the MFMA takes
 // them, keys in tiles of 32 with rescaling), so results agree to float32 rounding, not bit for bit.
@@ -26,7 +29,7 @@ namespace {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kRows = 32;       // query rows a wavefront
-constexpr int kWaves = 4;       // wavefronts a workgroup: 128 consecutive rows of one head
+// wavefronts a workgroup (WAVES below): four, 128 consecutive rows of one head, or two where four would leave the device short of workgroups
 constexpr int kTile = 32;       // keys a tile
 
 struct PromptParams {
@@ -45,35 +48,26 @@ __device__ __forceinline__ float element<float>(const uint32_t* raw, int e) { re
 template <>
 __device__ __forceinline__ float element<uint16_t>(const uint32_t* raw, int e) { return f16_bits_to_f32((uint16_t)(raw[e >> 1] >> (16 * (e & 1)))); }
 
-// Over the 32 lanes that share lane / 32: every lane gets the result.
-__device__ __forceinline__ float half_max(float v) {
-    v = fmaxf(v, dpp_f32<0xb1>(v));   // quad_perm [1,0,3,2]
-    v = fmaxf(v, dpp_f32<0x4e>(v));   // quad_perm [2,3,0,1]
-    v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
-    v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
-    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));  // lane ^ 16
-}
-__device__ __forceinline__ float half_sum(float v) {
-    v = v + dpp_f32<0xb1>(v);
-    v = v + dpp_f32<0x4e>(v);
-    v = v + dpp_f32<0x141>(v);
-    v = v + dpp_f32<0x140>(v);
-    return v + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+// The other half's value: lane ^ 32.
+__device__ __forceinline__ float other_half(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, v)));
 }
 
-template <typename KV, int D>
-__global__ __launch_bounds__(64 * kWaves) void attn_prompt_kernel(const float* __restrict__ q, const KV* __restrict__ k, const KV* __restrict__ v,
-                                                                  float* __restrict__ out, float* __restrict__ lse, PromptParams p) {
+template <typename KV, int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, (sizeof(KV) == 4 && D == 128 && WAVES == 2) ? 1 : 2) void attn_prompt_kernel(const float* __restrict__ q, const KV* __restrict__ k, const KV* __restrict__ v,
+                                                                     float* __restrict__ out, float* __restrict__ lse, PromptParams p) {
     constexpr int KS = D + 1;            // floats between rows of the keys' tile
-    constexpr int PS = kTile + 1;        // and of a wavefront's tile of p
-    constexpr int NT = D / 32;           // 32-column tiles of the result
+    constexpr int NT = D / 32;           // 32-feature tiles of the result
     constexpr int PER = D / 8;           // elements of a key (value) row a thread loads: eight threads a row
+    constexpr int RP = 8 * WAVES;        // rows of a tile the workgroup loads at once
+    constexpr int NP = kTile / RP;       // and how often
     __shared__ float ks[kTile * KS];
     __shared__ __align__(16) float vs[kTile * D];
-    __shared__ float ps[kWaves * kRows * PS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r32 = lane & 31, hi = lane >> 5;
-    const int b = blockIdx.z, h = blockIdx.y, hk = h / (p.H / p.HK);
-    const int i0 = ((int)blockIdx.x * kWaves + wave) * kRows;  // this wavefront's first row
+    // the grid is (head, sequence, block of rows), the last rows first: under causality they see the most keys, and
+    // workgroups are handed out in this order
+    const int b = blockIdx.y, h = blockIdx.x, hk = h / (p.H / p.HK), bx = (int)(gridDim.z - 1 - blockIdx.z);
+    const int i0 = (bx * WAVES + wave) * kRows;  // this wavefront's first row
     const int64_t Kt = p.K;
     auto seen_of = [&](int i) -> int {  // keys row i sees
         int64_t s = Kt;
@@ -83,62 +77,61 @@ __global__ __launch_bounds__(64 * kWaves) void attn_prompt_kernel(const float* _
         }
         return (int)s;
     };
-    const int last_row_wg = ((int)blockIdx.x + 1) * kWaves * kRows - 1 < p.Q ? ((int)blockIdx.x + 1) * kWaves * kRows - 1 : p.Q - 1;
+    const int last_row_wg = (bx + 1) * WAVES * kRows - 1 < p.Q ? (bx + 1) * WAVES * kRows - 1 : p.Q - 1;
     const int last_row_wave = i0 + kRows - 1 < p.Q ? i0 + kRows - 1 : p.Q - 1;
     const int seen_wg = p.causal ? seen_of(last_row_wg) : (int)Kt;
     const int seen_wave = i0 < p.Q ? (p.causal ? seen_of(last_row_wave) : (int)Kt) : 0;
 
-    // Q's rows, scaled, as the MFMA's first operand: lane (row r32, feature 2 s + hi) for s = 0 .. D / 2
+    // this lane's row, scaled, as the MFMA's second operand: lane (feature 2 s + hi, column r32) for s = 0 .. D / 2
+    const int row = i0 + r32;
     float qreg[D / 2];
     {
-        const int i = i0 + r32 < p.Q ? i0 + r32 : p.Q - 1;
+        const int i = row < p.Q ? row : p.Q - 1;
         const float* qr = q + b * p.q_b + (int64_t)h * p.q_h + (int64_t)i * p.q_i + hi;
 #pragma unroll
         for (int s = 0; s < D / 2; s++) qreg[s] = qr[2 * s] * p.scale;
     }
-    // what a lane holds of its 16 rows (register e: row 8 (e / 4) + 4 hi + e % 4): the keys each sees, maximum, sum, result
-    int seen[16];
-    float m[16], l[16];
-    f32x16 o[NT];
-#pragma unroll
-    for (int e = 0; e < 16; e++) {
-        const int i = i0 + 8 * (e >> 2) + 4 * hi + (e & 3);
-        seen[e] = i < p.Q ? seen_of(i) : 0;
-        m[e] = -__builtin_inff();
-        l[e] = 0.f;
-    }
+    const int seen = row < p.Q ? seen_of(row) : 0;
+    float m = -__builtin_inff(), l = 0.f;  // the row's maximum so far; the sum over the keys this half of the lanes holds
+    f32x16 o[NT];                          // the row's result, transposed: register e of tile t is feature 32 t + 8 (e / 4) + 4 hi + e % 4
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
         for (int e = 0; e < 16; e++) o[t][e] = 0.f;
 
-    // a thread's part of a tile's keys and values: row tid / 8, elements [PER (tid % 8), + PER)
+    // a thread's part of a tile's keys and values: rows tid / 8 + RP n, elements [PER (tid % 8), + PER)
     const int lrow = tid >> 3, lpart = tid & 7;
     const KV* kbase = k + b * p.k_b + (int64_t)hk * p.k_h + PER * lpart;
     const KV* vbase = v + b * p.v_b + (int64_t)hk * p.v_h + PER * lpart;
     constexpr int VEC = PER * (int)sizeof(KV) / 16;  // 16-byte pieces of a thread's part (the host checks their alignment)
-    uint32_t kreg[4 * VEC], vreg[4 * VEC];
+    uint32_t kreg[NP][4 * VEC], vreg[NP][4 * VEC];
     auto fetch = [&](int j0) {
-        int64_t j = j0 + lrow;
-        j = j < Kt ? j : Kt - 1;  // rows past the last key: never seen, loaded from the last one
 #pragma unroll
-        for (int c = 0; c < VEC; c++) {
-            const u32x4 kw = ((const u32x4*)(kbase + j * p.k_p))[c], vw = ((const u32x4*)(vbase + j * p.v_p))[c];
+        for (int n = 0; n < NP; n++) {
+            int64_t j = j0 + lrow + RP * n;
+            j = j < Kt ? j : Kt - 1;  // rows past the last key: never seen, loaded from the last one
 #pragma unroll
-            for (int w = 0; w < 4; w++) kreg[4 * c + w] = kw[w], vreg[4 * c + w] = vw[w];
+            for (int c = 0; c < VEC; c++) {
+                const u32x4 kw = ((const u32x4*)(kbase + j * p.k_p))[c], vw = ((const u32x4*)(vbase + j * p.v_p))[c];
+#pragma unroll
+                for (int w = 0; w < 4; w++) kreg[n][4 * c + w] = kw[w], vreg[n][4 * c + w] = vw[w];
+            }
         }
     };
     auto stage = [&]() {
 #pragma unroll
-        for (int e = 0; e < PER; e++) ks[lrow * KS + PER * lpart + e] = element<KV>(kreg, e);
+        for (int n = 0; n < NP; n++) {
+            const int r = lrow + RP * n;
 #pragma unroll
-        for (int e = 0; e < PER; e += 4) {
-            const f32x4 f = {element<KV>(vreg, e), element<KV>(vreg, e + 1), element<KV>(vreg, e + 2), element<KV>(vreg, e + 3)};
-            *(f32x4*)(vs + lrow * D + PER * lpart + e) = f;
+            for (int e = 0; e < PER; e++) ks[r * KS + PER * lpart + e] = element<KV>(kreg[n], e);
+#pragma unroll
+            for (int e = 0; e < PER; e += 4) {
+                const f32x4 f = {element<KV>(vreg[n], e), element<KV>(vreg[n], e + 1), element<KV>(vreg[n], e + 2), element<KV>(vreg[n], e + 3)};
+                *(f32x4*)(vs + r * D + PER * lpart + e) = f;
+            }
         }
     };
 
-    float* pw = ps + wave * kRows * PS;
     if (seen_wg > 0) fetch(0);
     for (int j0 = 0; j0 < seen_wg; j0 += kTile) {
         __syncthreads();  // everyone has read the tile before
@@ -147,63 +140,79 @@ __global__ __launch_bounds__(64 * kWaves) void attn_prompt_kernel(const float* _
         if (j0 + kTile < seen_wg) fetch(j0 + kTile);
         if (j0 >= seen_wave) continue;  // nothing of this tile is seen by this wavefront's rows (uniform)
 
-        // scores: lane (key j0 + r32) x 16 rows
+        // scores, transposed (K . Q^T): register e is key j0 + 8 (e / 4) + 4 hi + e % 4 against this lane's row
         f32x16 s;
 #pragma unroll
         for (int e = 0; e < 16; e++) s[e] = 0.f;
 #pragma unroll
-        for (int f = 0; f < D / 2; f++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[f], ks[r32 * KS + 2 * f + hi], s, 0, 0, 0);
-        const int j = j0 + r32;
-        float alpha[16];
+        for (int f = 0; f < D / 2; f++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(ks[r32 * KS + 2 * f + hi], qreg[f], s, 0, 0, 0);
+        float mx = -__builtin_inff();
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-            const float sc = j < seen[e] ? s[e] : -__builtin_inff();
-            const float mx = half_max(sc);
-            const float mn = fmaxf(m[e], mx);
-            float pe = 0.f, al = 1.f;
-            if (mn > -__builtin_inff()) {  // the row has seen a key by now (the same for all its lanes)
-                pe = __builtin_expf(sc - mn);
-                al = __builtin_expf(m[e] - mn);
-            }
-            l[e] = l[e] * al + half_sum(pe);
-            m[e] = mn;
-            alpha[e] = al;
-            pw[(8 * (e >> 2) + 4 * hi + (e & 3)) * PS + r32] = pe;
+            const int j = j0 + 8 * (e >> 2) + 4 * hi + (e & 3);
+            s[e] = j < seen ? s[e] : -__builtin_inff();
+            mx = fmaxf(mx, s[e]);
         }
+        mx = fmaxf(mx, other_half(mx, lane));
+        const float mn = fmaxf(m, mx);
+        float al = 1.f, sum = 0.f;
+        if (mn > -__builtin_inff()) {  // the row has seen a key by now
+            al = __builtin_expf(m - mn);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                s[e] = __builtin_expf(s[e] - mn);
+                sum += s[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; e++) s[e] = 0.f;
+        }
+        l = l * al + sum;
+        m = mn;
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) o[t][e] = o[t][e] * alpha[e];
-        // p . v: p as the first operand, lane (row r32, key 2 f + hi); a wavefront's LDS accesses complete in order
+            for (int e = 0; e < 16; e++) o[t][e] = o[t][e] * al;
+        // result, transposed (V^T . P^T) over the tile's keys in the order the scores' registers hold them: step f takes
+        // key 8 (f / 4) + 4 hi + f % 4 from each half, whose weight for this lane's row is register f
 #pragma unroll
         for (int f = 0; f < kTile / 2; f++) {
-            const float pa = pw[r32 * PS + 2 * f + hi];
+            const int key = 8 * (f >> 2) + 4 * hi + (f & 3);
 #pragma unroll
-            for (int t = 0; t < NT; t++) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa, vs[(2 * f + hi) * D + 32 * t + r32], o[t], 0, 0, 0);
+            for (int t = 0; t < NT; t++) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * D + 32 * t + r32], s[f], o[t], 0, 0, 0);
         }
     }
 
+    l += other_half(l, lane);
+    if (row >= p.Q) return;
+    float* orow = out + b * p.o_b + (int64_t)h * p.o_h + (int64_t)row * p.o_i;
+    const float inv = l == 0.f ? 0.f : 1.0f / l;
+    const bool wide = (((uintptr_t)orow) & 15) == 0;
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-        const int i = i0 + 8 * (e >> 2) + 4 * hi + (e & 3);
-        if (i >= p.Q) continue;
-        float* orow = out + b * p.o_b + (int64_t)h * p.o_h + (int64_t)i * p.o_i;
-        const float inv = l[e] == 0.f ? 0.f : 1.0f / l[e];
+    for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int t = 0; t < NT; t++) orow[32 * t + r32] = l[e] == 0.f ? 0.f : o[t][e] * inv;
-        if (lse && r32 == 0) lse[((int64_t)b * p.H + h) * p.Q + i] = l[e] == 0.f ? -__builtin_inff() : m[e] + __builtin_logf(l[e]);
-    }
+        for (int g = 0; g < 4; g++) {
+            f32x4 r;
+#pragma unroll
+            for (int c = 0; c < 4; c++) r[c] = l == 0.f ? 0.f : o[t][4 * g + c] * inv;
+            float* dst = orow + 32 * t + 8 * g + 4 * hi;
+            if (wide) *(f32x4*)dst = r;
+            else
+#pragma unroll
+                for (int c = 0; c < 4; c++) dst[c] = r[c];
+        }
+    if (lse && hi == 0) lse[((int64_t)b * p.H + h) * p.Q + row] = l == 0.f ? -__builtin_inff() : m + __builtin_logf(l);
 }
 
 std::atomic<int> g_prompt{1};  // measurement aid: 0 keeps every call on the kernel that takes a query row a workgroup
 
-template <typename KV>
+template <typename KV, int WAVES>
 hipError_t launch(const AttnArgs& a, const PromptParams& p, hipStream_t st) {
-    const dim3 grid((unsigned)((a.Q + kWaves * kRows - 1) / (kWaves * kRows)), (unsigned)a.H, (unsigned)a.B);
+    const dim3 grid((unsigned)a.H, (unsigned)a.B, (unsigned)((a.Q + WAVES * kRows - 1) / (WAVES * kRows)));
     if (a.D == 128)
-        hipLaunchKernelGGL((attn_prompt_kernel<KV, 128>), grid, dim3(64 * kWaves), 0, st, a.q, (const KV*)a.k, (const KV*)a.v, a.out, a.lse, p);
+        hipLaunchKernelGGL((attn_prompt_kernel<KV, 128, WAVES>), grid, dim3(64 * WAVES), 0, st, a.q, (const KV*)a.k, (const KV*)a.v, a.out, a.lse, p);
     else
-        hipLaunchKernelGGL((attn_prompt_kernel<KV, 64>), grid, dim3(64 * kWaves), 0, st, a.q, (const KV*)a.k, (const KV*)a.v, a.out, a.lse, p);
+        hipLaunchKernelGGL((attn_prompt_kernel<KV, 64, WAVES>), grid, dim3(64 * WAVES), 0, st, a.q, (const KV*)a.k, (const KV*)a.v, a.out, a.lse, p);
     return hipGetLastError();
 }
 
@@ -217,7 +226,7 @@ bool attention_prompt_ok(const AttnArgs& a) {
     const int DV = a.DV > 0 ? a.DV : a.D;
     const int esz = a.kv_dtype == kF16 ? 2 : 4;
     if (g_prompt == 0 || a.mask || a.dyn_k || a.Q < 64 || a.K < 1 || DV != a.D || (a.D != 64 && a.D != 128) || (a.kv_dtype != kF16 && a.kv_dtype != kF32) ||
-        a.HK <= 0 || a.H % a.HK != 0 || a.B <= 0 || a.B > 65535 || a.H > 65535 || a.Q > (1 << 24) || a.K > (1 << 30))
+        a.HK <= 0 || a.H % a.HK != 0 || a.B <= 0 || a.B > 65535 || a.H > 65535 || a.Q > (1 << 22) || a.K > (1 << 30))
         return false;
     for (int s = 0; s < 3; s++)
         if ((a.k_strides[s] * esz) % 16 != 0 || (a.v_strides[s] * esz) % 16 != 0) return false;
@@ -234,8 +243,11 @@ hipError_t attention_prompt(const AttnArgs& a, hipStream_t st) {
     p.scale = (float)a.scale;
     p.causal = a.causal;
     p.causal_offset = a.causal_offset;
+    // workgroups of two wavefronts where those of four would be fewer than the device holds at two a compute unit
+    const bool two = a.B * a.H * ((a.Q + 4 * kRows - 1) / (4 * kRows)) < 512;
     note_kernel("attn_prompt_kernel");
-    return a.kv_dtype == kF16 ? launch<uint16_t>(a, p, st) : launch<float>(a, p, st);
+    if (a.kv_dtype == kF16) return two ? launch<uint16_t, 2>(a, p, st) : launch<uint16_t, 4>(a, p, st);
+    return two ? launch<float, 2>(a, p, st) : launch<float, 4>(a, p, st);
 }
 
 }  // namespace mimir

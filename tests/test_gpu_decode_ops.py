@@ -313,6 +313,8 @@ def last_kernel():
     (1, 4, 1, 256, 256, 128, capi.F32, True, -40),  # the first 40 rows see no key: zeros and -Inf
     (1, 2, 1, 100, 400, 128, capi.F16, True, 500),  # the offset beyond the keys: every row sees all 400
     (1, 32, 8, 512, 512, 128, capi.F16, True, 0),   # a 512-token prompt of the 8B shape
+    (4, 32, 8, 512, 512, 128, capi.F16, True, 0),   # four of them: enough workgroups of four wavefronts (fewer rows take two)
+    (2, 64, 8, 450, 100, 64, capi.F32, False, 0),   # four wavefronts again: float32 cache, 64 features, ragged, every key seen
 ])
 def test_prompt_attention_on_the_matrix_cores(B, H, HK, Q, K, D, kv_dt, causal, off):
     """Calls of 64 and more query positions go to the kernel that walks tiles of keys with 32 rows a wavefront: against
