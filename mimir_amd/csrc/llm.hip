@@ -173,14 +173,14 @@ mi355x_status convert_for(Model& m, const float* x, int64_t rows, int64_t K, std
 // With resid, y = product + resid (which may be y); only the row kernels of the quantized dtypes add it.
 mi355x_status linear(Model& m, const Weight& w, const float* x, float* y, int64_t rows, const float* resid = nullptr) {
     int cls = act_class(w, rows, m.fx_panel.bytes);
-    if (resid && (cls == kActFx || cls == kActFxPairs || cls == kActNone)) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
+    if (resid && cls == kActNone) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: no residual epilogue for this product");
     QGemvArgs a{w.buf.p, x, m.act[cls].p, y, rows, w.n, w.k, w.k, 0};
     a.resid = resid;
     hipError_t e;
     switch (w.dtype) {
     case kQ4_0:
         e = cls == kActFx || cls == kActFxPairs
-                ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, nullptr, rows, w.n, w.k, cls == kActFxPairs ? m.fx_panel.p : nullptr, m.stream)
+                ? qgemm_q4_0_fx(w.buf.p, m.act[cls].p, y, resid, rows, w.n, w.k, cls == kActFxPairs ? m.fx_panel.p : nullptr, m.stream)
             : cls == kActQ4 ? qgemv_q4_0_act(a, kNoTune, m.stream)
                             : qgemv_q4_0(a, kNoTune, m.stream);
         break;
@@ -221,6 +221,14 @@ static mi355x_status forward(Model& m, int64_t s) {
     float *a = m.a.as<float>(), *o = m.o.as<float>(), *gate = m.gate.as<float>(), *up = m.up.as<float>(), *sw = m.s.as<float>();
     bool done[kActClasses];
     if (mi355x_status st = embed_rows(m, m.tokens_dev.as<int32_t>(), rows, x, device_error_word())) return st;
+    // x += in . W^T: the prompt-sized fixed-point products add x as they store, the others leave it to a launch
+    auto onto_x = [&](const Weight& w, const float* in) -> mi355x_status {
+        const int cls = act_class(w, rows, m.fx_panel.bytes);
+        if (cls == kActFx || cls == kActFxPairs) return linear(m, w, in, x, rows, x);
+        if (mi355x_status st = linear(m, w, in, o, rows)) return st;
+        LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
+        return MI355X_OK;
+    };
     for (int i = 0; i < c.layers; i++) {
         Block& b = m.blocks[i];
         LLM_HIP(rmsnorm(x, b.attn_norm.buf.as<float>(), h, rows, c.embed, c.eps, m.stream), "attn_norm");
@@ -266,16 +274,14 @@ static mi355x_status forward(Model& m, int64_t s) {
         if (need + kAttnTicketBytes > m.act[0].bytes) return capi_fail(MI355X_ERR_INTERNAL, "mi355x: llama: attention scratch of %zu bytes, need %zu", m.act[0].bytes, need);
         LLM_HIP(attention(at, (uint8_t*)m.act[0].p + kAttnTicketBytes, m.stream), "attention");
         if (mi355x_status st = convert_for(m, a, rows, qd, {&b.o}, done)) return st;
-        if (mi355x_status st = linear(m, b.o, a, o, rows)) return st;
-        LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
+        if (mi355x_status st = onto_x(b.o, a)) return st;
         LLM_HIP(rmsnorm(x, b.ffn_norm.buf.as<float>(), h, rows, c.embed, c.eps, m.stream), "ffn_norm");
         if (mi355x_status st = convert_for(m, h, rows, c.embed, {&b.gate, &b.up}, done)) return st;
         if (mi355x_status st = linear(m, b.gate, h, gate, rows)) return st;
         if (mi355x_status st = linear(m, b.up, h, up, rows)) return st;
         LLM_HIP(swiglu(gate, up, sw, rows, c.hidden, c.hidden, m.stream), "swiglu");
         if (mi355x_status st = convert_for(m, sw, rows, c.hidden, {&b.down}, done)) return st;
-        if (mi355x_status st = linear(m, b.down, sw, o, rows)) return st;
-        LLM_HIP(add(x, o, x, rows * c.embed, m.stream), "residual");
+        if (mi355x_status st = onto_x(b.down, sw)) return st;
     }
     m.cache_len = past + s;
     return MI355X_OK;
