@@ -89,7 +89,7 @@ hipError_t rmsnorm_q4act(const float* x, const float* w, float* y, void* act, in
 __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x, float* __restrict__ y, int64_t rows, int s,
                                                    int head_dim, int dim, int interleaved, int64_t x_row_stride,
                                                    int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride,
-                                                   const float* __restrict__ cosv, const float* __restrict__ sinv, int offset) {
+                                                   const float* __restrict__ cosv, const float* __restrict__ sinv, int offset, int period) {
     const int half = dim >> 1, per = half + (head_dim - dim);  // work items per (row, position)
     int64_t total = rows * s * per;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
@@ -106,7 +106,8 @@ __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x, 
         }
         int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
         float a = xi[ia], b = xi[ib];
-        float c = cosv[(int64_t)(offset + q) * half + i], sn = sinv[(int64_t)(offset + q) * half + i];
+        const int64_t at = offset + q % period;  // several sequences' positions in a row: each counts from the offset
+        float c = cosv[at * half + i], sn = sinv[at * half + i];
         float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;
         yo[ia] = ac - bs;
         yo[ib] = interleaved ? as + bc : bc + as;
@@ -115,13 +116,13 @@ __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x, 
 
 hipError_t rope(const float* x, float* y, int64_t rows, int64_t s, int head_dim, int dim, int interleaved, int64_t x_row_stride,
                 int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride, const float* cosv, const float* sinv,
-                int64_t offset, hipStream_t st) {
+                int64_t offset, hipStream_t st, int64_t period) {
     int64_t total = rows * s * (dim / 2 + head_dim - dim);
     if (total == 0) return hipSuccess;
     int64_t groups = (total + 255) / 256;
     if (groups > 65536) groups = 65536;
     hipLaunchKernelGGL(rope_kernel, dim3((unsigned)groups), dim3(256), 0, st, x, y, rows, (int)s, head_dim, dim, interleaved,
-                       x_row_stride, x_pos_stride, y_row_stride, y_pos_stride, cosv, sinv, (int)offset);
+                       x_row_stride, x_pos_stride, y_row_stride, y_pos_stride, cosv, sinv, (int)offset, (int)(period > 0 ? period : s));
     return hipGetLastError();
 }
 

@@ -158,9 +158,11 @@ hipError_t gemv_float(int dt, const void* W, const float* x, float* y, int64_t M
 
 // ---- the other kernels of a decoding step ------------------------------------
 hipError_t rmsnorm(const float* x, const float* w, float* y, int64_t rows, int64_t d, double eps, hipStream_t st);
+// period > 0: the s positions are those of s / period sequences one behind the other, position p turned by the angles of
+// offset + p % period (0: of offset + p).
 hipError_t rope(const float* x, float* y, int64_t rows, int64_t s, int head_dim, int dim, int interleaved, int64_t x_row_stride,
                 int64_t x_pos_stride, int64_t y_row_stride, int64_t y_pos_stride, const float* cosv, const float* sinv,
-                int64_t offset, hipStream_t st);
+                int64_t offset, hipStream_t st, int64_t period = 0);
 hipError_t kv_write(const float* src, void* cache, int cache_dt, int64_t B, int heads, int64_t s, int dim, int64_t cap,
                     int64_t pos, int64_t src_b, int64_t src_h, int64_t src_p, hipStream_t st);
 // RMSNorm that also writes the row converted for the Q4_0 kernel (y may be

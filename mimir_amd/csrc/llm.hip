@@ -250,12 +250,11 @@ static mi355x_status forward(Model& m, int64_t s) {
             LLM_HIP(rope(k, k, B * c.kv_heads, 1, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, kvd, c.head_dim, kvd,
                          m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope k");
         } else {
-            for (int64_t bb = 0; bb < B; bb++) {
-                LLM_HIP(rope(q + bb * s * qd, q + bb * s * qd, c.heads, s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, qd,
-                             c.head_dim, qd, m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope q");
-                LLM_HIP(rope(k + bb * s * kvd, k + bb * s * kvd, c.kv_heads, s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim,
-                             kvd, c.head_dim, kvd, m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream), "rope k");
-            }
+            // the sequences' positions follow one another at the same distance: one launch, each sequence counting from `past`
+            LLM_HIP(rope(q, q, c.heads, B * s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, qd, c.head_dim, qd,
+                         m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream, s), "rope q");
+            LLM_HIP(rope(k, k, c.kv_heads, B * s, c.head_dim, c.rope_dim, c.interleaved, c.head_dim, kvd, c.head_dim, kvd,
+                         m.cos_t.as<float>(), m.sin_t.as<float>(), past, m.stream, s), "rope k");
         }
         LLM_HIP(kv_write(k, m.keys[i].p, c.cache_dtype, B, c.kv_heads, s, c.head_dim, c.context, past, s * kvd, c.head_dim, kvd, m.stream), "cache keys");
         LLM_HIP(kv_write(v, m.values[i].p, c.cache_dtype, B, c.kv_heads, s, c.head_dim, c.context, past, s * kvd, c.head_dim, kvd, m.stream), "cache values");
