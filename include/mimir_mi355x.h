@@ -224,13 +224,9 @@ MI355X_API mi355x_status mi355x_kv_write(const float* src, void* cache, int cach
  * {batch, head, query, key} (0 broadcasts a dimension) and added to the scores;
  * key j is also hidden from query i when causal and j > i + causal_offset. A
  * row that sees no key gets zeros and -Inf; with K == 0 that is every row, and
- * k, v and their strides may be NULL. D and DV at most 256. Calls of 64 and
- * more query positions (see "attention.prompt" under mi355x_tune) multiply whole
- * tiles of keys: a key that causality hides from a row enters that row's sums
- * with weight zero there, so a NaN or infinity in the values of such a key (one
- * of the K the call names, which a later row sees) reaches the earlier rows of
- * its tile too, where the reference, which never reads it, gives finite
- * results. */
+ * k, v and their strides may be NULL. D and DV at most 256. A NaN or an
+ * infinity in the values of a key reaches the rows that see the key and no
+ * other, as in the reference, which reads a row's visible keys only. */
 MI355X_API mi355x_status mi355x_attention(const float* q, const int64_t* q_strides, const void* k, const int64_t* k_strides, const void* v,
                                const int64_t* v_strides, int kv_dtype, const float* mask, const int64_t* mask_strides, float* out,
                                const int64_t* out_strides, float* lse, int64_t B, int H, int HK, int64_t Q, int64_t K, int D, int DV, double scale,

@@ -63,6 +63,7 @@ __global__ __launch_bounds__(64 * WAVES, (sizeof(KV) == 4 && D == 128 && WAVES =
     constexpr int NP = kTile / RP;       // and how often
     __shared__ float ks[kTile * KS];
     __shared__ __align__(16) float vs[kTile * D];
+    __shared__ int vbad[2];              // whether a tile's values hold a NaN or an infinity, for tiles of either parity
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r32 = lane & 31, hi = lane >> 5;
     // the grid is (head, sequence, block of rows), the last rows first: under causality they see the most keys, and
     // workgroups are handed out in this order
@@ -118,7 +119,8 @@ __global__ __launch_bounds__(64 * WAVES, (sizeof(KV) == 4 && D == 128 && WAVES =
             }
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](int parity) {
+        float chk = 0.f;  // 0 * value summed: NaN as soon as a value is a NaN or an infinity
 #pragma unroll
         for (int n = 0; n < NP; n++) {
             const int r = lrow + RP * n;
@@ -128,17 +130,29 @@ __global__ __launch_bounds__(64 * WAVES, (sizeof(KV) == 4 && D == 128 && WAVES =
             for (int e = 0; e < PER; e += 4) {
                 const f32x4 f = {element<KV>(vreg[n], e), element<KV>(vreg[n], e + 1), element<KV>(vreg[n], e + 2), element<KV>(vreg[n], e + 3)};
                 *(f32x4*)(vs + r * D + PER * lpart + e) = f;
+#pragma unroll
+                for (int c = 0; c < 4; c++) chk = __builtin_fmaf(f[c], 0.f, chk);
             }
         }
+        if (__builtin_amdgcn_ballot_w64(chk != chk) != 0 && lane == 0) vbad[parity] = 1;
     };
 
+    // The matrix cores multiply a whole tile of values by the rows' weights, zero for the keys a row does not see: fine
+    // unless such a value is a NaN or an infinity, which the reference never reads for that row. A tile that holds one and
+    // is not seen whole by every row of the wavefront takes the vector units for its second product instead, key by
+    // key and only for the rows that see the key.
+    const int seen_first = i0 < p.Q ? seen_of(i0) : 0;  // the fewest keys a row of this wavefront sees
+    if (tid < 2) vbad[tid] = 0;
     if (seen_wg > 0) fetch(0);
     for (int j0 = 0; j0 < seen_wg; j0 += kTile) {
+        const int parity = (j0 / kTile) & 1;
         __syncthreads();  // everyone has read the tile before
-        stage();
+        stage(parity);
         __syncthreads();
+        if (tid == 0) vbad[parity ^ 1] = 0;  // read last before the first barrier above, set next behind it a tile on
         if (j0 + kTile < seen_wg) fetch(j0 + kTile);
         if (j0 >= seen_wave) continue;  // nothing of this tile is seen by this wavefront's rows (uniform)
+        const bool by_key = vbad[parity] != 0 && j0 + kTile > seen_first;
 
         // scores, transposed (K . Q^T): register e is key j0 + 8 (e / 4) + 4 hi + e % 4 against this lane's row
         f32x16 s;
@@ -175,11 +189,33 @@ __global__ __launch_bounds__(64 * WAVES, (sizeof(KV) == 4 && D == 128 && WAVES =
             for (int e = 0; e < 16; e++) o[t][e] = o[t][e] * al;
         // result, transposed (V^T . P^T) over the tile's keys in the order the scores' registers hold them: step f takes
         // key 8 (f / 4) + 4 hi + f % 4 from each half, whose weight for this lane's row is register f
+        if (!by_key) {
 #pragma unroll
-        for (int f = 0; f < kTile / 2; f++) {
-            const int key = 8 * (f >> 2) + 4 * hi + (f & 3);
+            for (int f = 0; f < kTile / 2; f++) {
+                const int key = 8 * (f >> 2) + 4 * hi + (f & 3);
 #pragma unroll
-            for (int t = 0; t < NT; t++) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * D + 32 * t + r32], s[f], o[t], 0, 0, 0);
+                for (int t = 0; t < NT; t++) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key * D + 32 * t + r32], s[f], o[t], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const float theirs = other_half(s[e], lane);
+#pragma unroll
+                for (int hk = 0; hk < 2; hk++) {  // the key that register e holds in the lanes of half hk
+                    const int key = 8 * (e >> 2) + 4 * hk + (e & 3);
+                    const float pk = hi == hk ? s[e] : theirs;
+                    if (j0 + key < seen) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                const f32x4 vv = *(const f32x4*)(vs + key * D + 32 * t + 8 * g + 4 * hi);
+#pragma unroll
+                                for (int c = 0; c < 4; c++) o[t][4 * g + c] = __builtin_fmaf(pk, vv[c], o[t][4 * g + c]);
+                            }
+                    }
+                }
+            }
         }
     }
 

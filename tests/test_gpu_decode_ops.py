@@ -344,6 +344,50 @@ def test_prompt_attention_on_the_matrix_cores(B, H, HK, Q, K, D, kv_dt, causal, 
         assert not out[:, :, :-off].any() and np.all(lse[:, :, :-off] == -np.inf)
 
 
+@pytest.mark.parametrize("kv_dt,D", [(capi.F16, 128), (capi.F32, 64)])
+def test_prompt_attention_with_nan_and_infinity_among_the_values(kv_dt, D):
+    """A NaN or an infinity in the values of a key reaches the rows that see the key and no row before it (the reference
+    reads a row's visible keys only, backend/cpu/attention.go:437-535), although the kernel multiplies whole tiles of
+    keys: such a tile goes key by key. Also behind the last key, where a tile's rows repeat it."""
+    l = gpu.lib()
+    rng = np.random.default_rng(D)
+    B, H, HK, Q, K = 2, 4, 2, 200, 215
+    off = K - Q
+    q = rng.normal(size=(B, H, Q, D)).astype(np.float32)
+    k = rng.normal(size=(B, HK, K, D)).astype(np.float32); v = rng.normal(size=(B, HK, K, D)).astype(np.float32)
+    v[0, 0, 70, 5] = np.nan      # seen from row 55 on, in the middle of a tile and of a wavefront's rows
+    v[0, 1, 131, 9] = np.inf     # from row 116 on
+    v[1, 0, 214, 3] = -np.inf    # the last key: the last row only
+    v[1, 1, 32, :] = np.nan      # a tile's first key
+    odt = O.F32
+    if kv_dt == capi.F16:
+        k, v, odt = O.f32_to_f16(k), O.f32_to_f16(v), O.F16
+    scale = 1 / np.sqrt(D)
+    def same(got, want, what):
+        bad = ~np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), what
+        assert np.array_equal(got[bad & ~np.isnan(want)], want[bad & ~np.isnan(want)]), what
+        g, w = got[~bad].astype(np.float64), want[~bad]
+        assert np.all(np.abs(g - w) <= ATOL + RTOL * np.abs(w)), what
+    for causal in (True, False):
+        gpu.say(f"prompt attention, NaN and infinities in the values, dt={kv_dt} D={D} causal={causal}")
+        out, lse = attention(q, k, v, scale, causal=causal, offset=off, kv_dt=kv_dt)
+        assert last_kernel() == "attn_prompt_kernel"
+        wo, wl = O.attention(q, k, v, scale, causal=causal, causal_offset=off, kv_dt=odt)
+        same(out, wo, "against the oracle"); close(lse, wl)
+        if causal:  # heads 0, 1 on key head 0 and 2, 3 on key head 1
+            assert np.isfinite(out[0, :2, :55]).all() and np.isnan(out[0, :2, 55:, 5]).all() and np.isfinite(out[0, :2, 55:, 6]).all()
+            assert np.isfinite(out[0, 2:, :116]).all() and not np.isfinite(out[0, 2:, 116:, 9]).any()
+            assert np.isfinite(out[1, :2, :199]).all() and (out[1, :2, 199, 3] == -np.inf).all()
+            assert np.isfinite(out[1, 2:, :17]).all() and np.isnan(out[1, 2:, 17:]).all()
+        try:
+            capi.check(l.mi355x_tune(b"attention.prompt", 0))
+            out2, lse2 = attention(q, k, v, scale, causal=causal, offset=off, kv_dt=kv_dt)
+        finally:
+            capi.check(l.mi355x_tune(b"attention.prompt", 1))
+        same(out, out2, "against the kernel that takes a query row a workgroup"); close(lse, lse2)
+
+
 def test_prompt_attention_leaves_other_calls_where_they_were():
     """Fewer than 64 query positions, values of another width than the keys, a mask, and rows of keys that do not start
     on 16 bytes stay on the other kernels."""
