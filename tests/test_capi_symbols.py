@@ -33,3 +33,18 @@ def test_block_accounting_without_a_device():
         [(32, 34), (256, 144), (256, 210), (32, 18)]
     assert lib.mi355x_bytes(capi.Q4_0, 4096 * 14336) == 4096 * 14336 // 32 * 18
     assert lib.mi355x_bytes(capi.Q8_0, 33) == -1 and lib.mi355x_bytes(capi.F32, 5) == 20 and lib.mi355x_bytes(0, 4) == -1
+
+
+def test_every_tune_key_is_documented_and_every_documented_key_handled():
+    """The keys mi355x_tune compares its argument with (capi.hip) are the keys that the header's comment on
+    mi355x_tune names: a key added to one and not the other fails here."""
+    src = open(os.path.join(ROOT, "mimir_amd", "csrc", "capi.hip")).read()
+    body = src[src.index("mi355x_status mi355x_tune("):]
+    handled = set(re.findall(r'strcmp\(key, "([^"]+)"\)', body))
+    table = re.search(r'static const char\* keys\[\d+\] = \{([^}]*)\}', body)
+    handled |= set(re.findall(r'"([^"]+)"', table.group(1))) if table else set()
+    hdr = open(os.path.join(ROOT, "include", "mimir_mi355x.h")).read()
+    documented = set(re.findall(r'"([a-z0-9_]+\.[a-zA-Z0-9_]+)"', hdr))
+    assert handled and handled == documented, handled ^ documented
+    lib = capi.load()
+    assert lib.mi355x_tune(b"no.such_key", 1) != capi.OK  # and an unknown key is an error, without a device
